@@ -1,0 +1,279 @@
+"""ctypes binding of the CPU oracle (oracle/libegg_oracle.so) and of oracle/_ref.
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py -- never by the product path.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libegg_oracle.so")
+REF_PATH = os.path.join(HERE, "_ref", "libegg_ref.so")
+
+
+class OrcConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "hidden", "head_dim", "n_layers", "seq_len", "vocab", "population",
+        "fixed_point", "sigma_shift", "sigma_shift_vector",
+        "shift_attn", "shift_out", "shift_logit", "shift_mlp_up", "shift_mlp_down",
+        "softmax_scale_bit", "rope_scale_bit", "noise_mask", "host_mask")] + [
+        ("softmax_exp_scale", C.c_double),
+        ("adam_beta1", C.c_float), ("adam_beta2", C.c_float), ("adam_eps", C.c_float),
+        ("adam_weight_decay", C.c_float), ("muon_momentum", C.c_float), ("muon_lr_scale", C.c_float)]
+
+
+class OrcTensor(C.Structure):
+    _fields_ = [("name", C.c_char * 32), ("is_matrix", C.c_int), ("rows", C.c_int), ("cols", C.c_int),
+                ("offset", C.c_int64), ("off_a", C.c_int), ("off_b", C.c_int), ("seed_base", C.c_int),
+                ("lr_scale", C.c_float), ("muon", C.c_int)]
+
+
+class OrcTrace(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("x_emb", "x_init", "q", "k", "v", "ao", "x_attn", "x_mlp",
+                                          "nf", "logits", "loss_t")]
+
+
+class OrcGruConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("hidden", "n_layers", "seq_len", "vocab", "population",
+                                       "fixed_point", "sigma_shift", "update_threshold")]
+
+
+def build(force=False):
+    """(Re)build the oracle library with oracle/Makefile."""
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.check_call(["make", "-C", HERE, "-s"] + (["-B"] if force else []))
+
+
+_lib = None
+_ref = None
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(LIB_PATH)
+        L.orc_hash_rng.restype = C.c_uint32
+        L.orc_hash_rng.argtypes = [C.c_uint32, C.c_uint32]
+        L.orc_noise.restype = C.c_int8
+        L.orc_noise.argtypes = [C.c_uint32, C.c_uint32, C.c_int]
+        L.orc_xorshift32.restype = C.c_uint32
+        L.orc_gen_noise_host.restype = C.c_int8
+        L.orc_clip.restype = C.c_int8
+        L.orc_clip.argtypes = [C.c_int32]
+        L.orc_model_bytes.restype = C.c_int64
+        L.orc_forward_member.restype = C.c_int32
+        L.orc_forward_member.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_uint32,
+                                         C.c_int, C.c_int, C.c_void_p]
+        L.orc_population_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_uint32,
+                                             C.c_int, C.c_int, C.c_void_p]
+        L.orc_perturbed_linear.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_int,
+                                           C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_void_p]
+        L.orc_standard_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_uint32,
+                                        C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+        L.orc_adaptive_normalize.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+        L.orc_rope.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+        L.orc_attention_core.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                         C.c_void_p]
+        L.orc_token_loss.restype = C.c_int64
+        L.orc_token_loss.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int]
+        L.orc_fitness.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        L.orc_adam_apply.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_void_p]
+        L.orc_matrix_votes.restype = C.c_int64
+        L.orc_matrix_votes.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int,
+                                       C.c_uint32, C.c_void_p]
+        for f in (L.orc_update_matrix_adam,):
+            f.restype = C.c_uint64
+            f.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                          C.c_int, C.c_uint32, C.c_float]
+        L.orc_update_vector_adam.restype = C.c_uint64
+        L.orc_update_vector_adam.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                             C.c_void_p, C.c_int, C.c_uint32, C.c_float]
+        L.orc_es_update_adam.restype = C.c_uint64
+        L.orc_es_update_adam.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_float]
+        L.orc_learning_rate.restype = C.c_float
+        L.orc_learning_rate.argtypes = [C.c_long]
+        L.orc_newton_schulz_f32.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
+        L.orc_newton_schulz_f64.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
+        L.orc_update_matrix_muon.restype = C.c_uint64
+        L.orc_update_matrix_muon.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                             C.c_int, C.c_void_p, C.c_int, C.c_uint32, C.c_float, C.c_void_p]
+        L.orc_gru_model_bytes.restype = C.c_int64
+        L.orc_gru_state_bytes.restype = C.c_int64
+        L.orc_gru_matmul_perturbed.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
+                                               C.c_uint32, C.c_int, C.c_int]
+        L.orc_gru_ln.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        L.orc_gru_compute_loss.restype = C.c_int32
+        L.orc_gru_compute_loss.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
+        L.orc_gru_forward.restype = C.c_int32
+        L.orc_gru_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_uint32,
+                                      C.c_int, C.c_void_p]
+        L.orc_gru_population.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_uint32, C.c_int,
+                                         C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.orc_gru_update_matrix.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_uint32, C.c_void_p, C.c_int]
+        L.orc_gru_update_all.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p]
+        L.orc_gru_noise_vector.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        _lib = L
+    return _lib
+
+
+def ref():
+    """oracle/_ref/libegg_ref.so (the reference's own host header, compiled); None if absent."""
+    global _ref
+    if _ref is None:
+        if not os.path.exists(REF_PATH):
+            return None
+        R = C.CDLL(REF_PATH)
+        R.ref_hash_rng.restype = C.c_uint32
+        R.ref_hash_rng.argtypes = [C.c_uint32, C.c_uint32]
+        R.ref_noise_from_hash.restype = C.c_int
+        R.ref_noise_from_hash.argtypes = [C.c_uint32, C.c_uint32]
+        R.ref_clip.restype = C.c_int
+        R.ref_clip.argtypes = [C.c_int32]
+        R.ref_xorshift32_host.restype = C.c_uint32
+        R.ref_gen_noise_host.restype = C.c_int
+        R.ref_ternary_pack_estimate_size.restype = C.c_size_t
+        R.ref_ternary_pack_estimate_size.argtypes = [C.c_size_t]
+        R.ref_ternary_pack.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p]
+        R.ref_ternary_unpack.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p]
+        _ref = R
+    return _ref
+
+
+# ----------------------------------------------------------------------------- helpers
+def config(**kw):
+    c = OrcConfig()
+    lib().orc_default_config(C.byref(c))
+    for k, v in kw.items():
+        if not hasattr(c, k):
+            raise KeyError(k)
+        setattr(c, k, v)
+    return c
+
+
+def gru_config(**kw):
+    c = OrcGruConfig()
+    lib().orc_gru_default_config(C.byref(c))
+    for k, v in kw.items():
+        if not hasattr(c, k):
+            raise KeyError(k)
+        setattr(c, k, v)
+    return c
+
+
+def tables(cfg):
+    exp = np.zeros(256, np.int32)
+    act = np.zeros(256, np.int8)
+    rope = np.zeros(cfg.seq_len * cfg.head_dim, np.int32)
+    lib().orc_tables(C.byref(cfg), _p(exp), _p(act), _p(rope))
+    return exp, act, rope
+
+
+def model_bytes(cfg):
+    return int(lib().orc_model_bytes(C.byref(cfg)))
+
+
+def init_model(cfg, seed=42):
+    m = np.zeros(model_bytes(cfg), np.int8)
+    lib().orc_init_model(C.byref(cfg), _p(m), C.c_uint32(seed))
+    return m
+
+
+def tensor_table(cfg):
+    arr = (OrcTensor * 256)()
+    n = lib().orc_tensor_table(C.byref(cfg), arr, 256)
+    return [dict(name=arr[i].name.decode(), is_matrix=arr[i].is_matrix, rows=arr[i].rows, cols=arr[i].cols,
+                 offset=arr[i].offset, off_a=arr[i].off_a, off_b=arr[i].off_b, seed_base=arr[i].seed_base,
+                 lr_scale=arr[i].lr_scale, muon=arr[i].muon) for i in range(n)]
+
+
+def noise_vec(seed, n, mask=15, first=0):
+    L = lib()
+    return np.array([L.orc_noise(C.c_uint32(seed & 0xFFFFFFFF), C.c_uint32(first + i), mask) for i in range(n)], np.int8)
+
+
+def forward_member(cfg, model, data, start_idx, step_seed, p_idx, ns_override=2, trace=False):
+    T, H, NL, V = cfg.seq_len, cfg.hidden, cfg.n_layers, cfg.vocab
+    tr = None
+    bufs = {}
+    if trace:
+        tr = OrcTrace()
+        shapes = dict(x_emb=(T, H), x_init=(T, H), q=(NL, T, H), k=(NL, T, H), v=(NL, T, H), ao=(NL, T, H),
+                      x_attn=(NL, T, H), x_mlp=(NL, T, H), nf=(T, H))
+        for k, s in shapes.items():
+            bufs[k] = np.zeros(s, np.int8)
+            setattr(tr, k, bufs[k].ctypes.data)
+        bufs["logits"] = np.zeros((T, V), np.int32)
+        tr.logits = bufs["logits"].ctypes.data
+        bufs["loss_t"] = np.zeros(T, np.int64)
+        tr.loss_t = bufs["loss_t"].ctypes.data
+    loss = lib().orc_forward_member(C.byref(cfg), _p(model), _p(data), len(data), start_idx,
+                                    C.c_uint32(step_seed & 0xFFFFFFFF), p_idx, ns_override,
+                                    C.byref(tr) if tr is not None else None)
+    return (loss, bufs) if trace else loss
+
+
+def population_forward(cfg, model, data, start_idx, step_seed, pop_offset=0, count=None):
+    count = cfg.population if count is None else count
+    loss = np.zeros(cfg.population, np.int32)
+    lib().orc_population_forward(C.byref(cfg), _p(model), _p(data), len(data), start_idx,
+                                 C.c_uint32(step_seed & 0xFFFFFFFF), pop_offset, count, _p(loss))
+    return loss
+
+
+def perturbed_linear(cfg, X, Wb, T, K, N, seed, off_a, off_b, shift):
+    rows = X.shape[0]
+    Y = np.zeros((rows, N), np.int32)
+    lib().orc_perturbed_linear(C.byref(cfg), _p(X), _p(Wb), rows, T, K, N, C.c_uint32(seed & 0xFFFFFFFF),
+                               off_a, off_b, shift, _p(Y))
+    return Y
+
+
+def fitness(loss):
+    pairs = len(loss) // 2
+    fit = np.zeros(pairs, np.int32)
+    lib().orc_fitness(_p(np.ascontiguousarray(loss, np.int32)), _p(fit), pairs)
+    return fit
+
+
+ADAM_DTYPE = np.dtype([("m", np.float32), ("v", np.float32), ("acc", np.float32)])
+MUON_DTYPE = np.dtype([("m", np.float32), ("acc", np.float32)])
+
+
+def es_update_adam(cfg, model, state, fit, step_seed, lr):
+    """in place on model (int8) and state (ADAM_DTYPE, one per model byte); returns update count"""
+    return int(lib().orc_es_update_adam(C.byref(cfg), _p(model), _p(state), _p(fit),
+                                        C.c_uint32(step_seed & 0xFFFFFFFF), C.c_float(lr)))
+
+
+def zipf_bytes(n, seed=1234, s=1.1):
+    """Synthetic byte stream: i.i.d. Zipf(s) ranks over a fixed permutation of the 256 byte values.
+    Counter-based SplitMix64 -> inverse CDF (so any slice can be regenerated independently)."""
+    idx = np.arange(1, n + 1, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        z = np.uint64(seed) + idx * np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> np.uint64(31))
+    u = (z >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
+    w = 1.0 / np.arange(1, 257, dtype=np.float64) ** s
+    cdf = np.cumsum(w) / np.sum(w)
+    rank = np.minimum(np.searchsorted(cdf, u, side="right"), 255)
+    # fixed permutation of byte values from the same generator (Fisher-Yates with xorshift32)
+    perm = np.arange(256, dtype=np.uint8)
+    st = np.uint32((seed * 2654435761 + 1) & 0xFFFFFFFF) or np.uint32(1)
+    st = int(st)
+    for i in range(255, 0, -1):
+        st ^= (st << 13) & 0xFFFFFFFF
+        st ^= st >> 17
+        st ^= (st << 5) & 0xFFFFFFFF
+        j = st % (i + 1)
+        perm[i], perm[j] = perm[j], perm[i]
+    return perm[rank].astype(np.uint8)
