@@ -1,0 +1,264 @@
+"""Python host-side binding of libegg_hip.so (the C ABI declared in include/egg_hip.h).
+
+The directory name contains a dot, so load this package with ``load_package()`` from
+``__graft_entry__`` (importlib by path) under the module name ``egg_c_amd``.
+
+There is no CPU fallback: if libegg_hip.so is missing or a call fails, an exception is raised.
+PyTorch is used by callers only to own device memory; this module takes raw device pointers.
+"""
+import ctypes as C
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libegg_hip.so")
+
+
+class EggError(RuntimeError):
+    pass
+
+
+class EggConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "hidden", "head_dim", "n_layers", "seq_len", "vocab", "population",
+        "fixed_point", "sigma_shift", "sigma_shift_vector",
+        "shift_attn", "shift_out", "shift_logit", "shift_mlp_up", "shift_mlp_down",
+        "softmax_scale_bit", "rope_scale_bit", "noise_mask", "host_mask")] + [
+        ("softmax_exp_scale", C.c_double),
+        ("adam_beta1", C.c_float), ("adam_beta2", C.c_float), ("adam_eps", C.c_float),
+        ("adam_weight_decay", C.c_float), ("muon_momentum", C.c_float), ("muon_lr_scale", C.c_float),
+        ("use_muon", C.c_int), ("chunk_members", C.c_int)]
+
+
+class EggTensorInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 32), ("is_matrix", C.c_int), ("rows", C.c_int), ("cols", C.c_int),
+                ("offset", C.c_int64), ("off_a", C.c_int), ("off_b", C.c_int), ("seed_base", C.c_int),
+                ("lr_scale", C.c_float), ("muon", C.c_int)]
+
+
+EXPORTS = [
+    "egg_default_config", "egg_ctx_create", "egg_ctx_destroy", "egg_last_error", "egg_ctx_set_stream", "egg_sync",
+    "egg_model_bytes", "egg_model_init", "egg_model_upload", "egg_model_download",
+    "egg_opt_state_upload", "egg_opt_state_download", "egg_opt_state_reset", "egg_tables_download",
+    "egg_noise_fill", "egg_perturbed_linear", "egg_population_forward", "egg_population_forward_dev",
+    "egg_fitness", "egg_es_update", "egg_update_tensor", "egg_matrix_votes",
+    "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
+    "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses",
+    "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_tap_download",
+]
+
+
+def build(force=True):
+    """Compile libegg_hip.so for gfx950 with hipcc (cross-compiles without a GPU)."""
+    cmd = ["make", "-C", HERE, "-j8", "-s"]
+    if force:
+        cmd.append("-B")
+    subprocess.check_call(cmd)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise EggError("libegg_hip.so is not built (run __graft_entry__.build()); there is no CPU fallback")
+        L = C.CDLL(LIB_PATH)
+        vp, i32, i64, u32 = C.c_void_p, C.c_int, C.c_int64, C.c_uint32
+        L.egg_default_config.argtypes = [vp]
+        L.egg_ctx_create.argtypes = [vp, vp]
+        L.egg_ctx_destroy.argtypes = [vp]
+        L.egg_ctx_destroy.restype = None
+        L.egg_last_error.restype = C.c_char_p
+        L.egg_last_error.argtypes = [vp]
+        L.egg_ctx_set_stream.argtypes = [vp, vp]
+        L.egg_sync.argtypes = [vp]
+        L.egg_model_bytes.restype = i64
+        L.egg_model_bytes.argtypes = [vp]
+        L.egg_model_init.argtypes = [vp, u32]
+        for f in (L.egg_model_upload, L.egg_model_download, L.egg_opt_state_upload, L.egg_opt_state_download):
+            f.argtypes = [vp, vp, C.c_size_t]
+        L.egg_opt_state_reset.argtypes = [vp]
+        L.egg_tables_download.argtypes = [vp, vp, vp, vp]
+        L.egg_noise_fill.argtypes = [vp, u32, u32, i32, vp]
+        L.egg_perturbed_linear.argtypes = [vp, vp, vp, i32, i32, i32, i32, u32, i32, i32, i32, vp, vp]
+        L.egg_population_forward.argtypes = [vp, vp, i64, i64, u32, i32, i32, vp]
+        L.egg_population_forward_dev.argtypes = [vp, vp, i64, vp, vp, i32, i32, vp]
+        L.egg_fitness.argtypes = [vp, vp, vp, i32]
+        L.egg_es_update.argtypes = [vp, vp, vp, vp]
+        L.egg_update_tensor.argtypes = [vp, i32, vp, vp, vp]
+        L.egg_matrix_votes.argtypes = [vp, i32, vp, vp, vp]
+        L.egg_tensor_count.argtypes = [vp]
+        L.egg_tensor_info_get.argtypes = [vp, i32, vp]
+        L.egg_last_update_count.argtypes = [vp, vp]
+        L.egg_step.argtypes = [vp, vp, i64, i64, u32, C.c_float]
+        L.egg_step_capture.argtypes = [vp, vp, i64]
+        L.egg_step_launch.argtypes = [vp, i64, u32, C.c_float]
+        L.egg_step_losses.argtypes = [vp, vp, vp]
+        L.egg_learning_rate.restype = C.c_float
+        L.egg_learning_rate.argtypes = [C.c_long]
+        L.egg_next_seed.restype = u32
+        L.egg_next_seed.argtypes = [u32, C.c_uint64]
+        L.egg_ctx_enable_taps.argtypes = [vp, i32]
+        L.egg_tap_download.argtypes = [vp, C.c_char_p, i32, vp]
+        _lib = L
+    return _lib
+
+
+def default_config(**kw):
+    c = EggConfig()
+    lib().egg_default_config(C.byref(c))
+    for k, v in kw.items():
+        if not hasattr(c, k):
+            raise KeyError(k)
+        setattr(c, k, v)
+    return c
+
+
+def _np_ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Context:
+    """One device context: model + optimizer state + workspace (mirror of the reference's GPUContext,
+    full_cuda_train_transformer_adam_mgpu.cu:1287-1302)."""
+
+    def __init__(self, cfg):
+        self.cfg = cfg
+        self._h = C.c_void_p()
+        rc = lib().egg_ctx_create(C.byref(cfg), C.byref(self._h))
+        if rc != 0:
+            raise EggError(f"egg_ctx_create failed with {rc} (unsupported configuration or HIP error)")
+
+    def close(self):
+        if self._h:
+            lib().egg_ctx_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _ck(self, rc, what):
+        if rc != 0:
+            raise EggError(f"{what} failed with {rc}: {lib().egg_last_error(self._h).decode()}")
+
+    def set_stream(self, stream_handle):
+        self._ck(lib().egg_ctx_set_stream(self._h, C.c_void_p(stream_handle)), "egg_ctx_set_stream")
+
+    def sync(self):
+        self._ck(lib().egg_sync(self._h), "egg_sync")
+
+    def model_bytes(self):
+        return int(lib().egg_model_bytes(self._h))
+
+    def model_init(self, seed=42):
+        self._ck(lib().egg_model_init(self._h, seed), "egg_model_init")
+
+    def model_upload(self, arr):
+        self._ck(lib().egg_model_upload(self._h, _np_ptr(arr), arr.nbytes), "egg_model_upload")
+
+    def model_download(self):
+        import numpy as np
+        out = np.zeros(self.model_bytes(), np.int8)
+        self._ck(lib().egg_model_download(self._h, _np_ptr(out), out.nbytes), "egg_model_download")
+        return out
+
+    def opt_state_upload(self, arr):
+        self._ck(lib().egg_opt_state_upload(self._h, _np_ptr(arr), arr.nbytes), "egg_opt_state_upload")
+
+    def opt_state_download(self):
+        import numpy as np
+        out = np.zeros(self.model_bytes() * 3, np.float32)
+        self._ck(lib().egg_opt_state_download(self._h, _np_ptr(out), out.nbytes), "egg_opt_state_download")
+        return out
+
+    def opt_state_reset(self):
+        self._ck(lib().egg_opt_state_reset(self._h), "egg_opt_state_reset")
+
+    def tables(self):
+        import numpy as np
+        ex = np.zeros(256, np.int32)
+        act = np.zeros(256, np.int8)
+        rope = np.zeros(self.cfg.seq_len * self.cfg.head_dim, np.int32)
+        self._ck(lib().egg_tables_download(self._h, _np_ptr(ex), _np_ptr(act), _np_ptr(rope)), "egg_tables_download")
+        return ex, act, rope
+
+    def noise_fill(self, seed, first, n, d_out):
+        self._ck(lib().egg_noise_fill(self._h, seed & 0xFFFFFFFF, first, n, C.c_void_p(d_out)), "egg_noise_fill")
+
+    def perturbed_linear(self, d_x, d_w, members, T, K, N, seed, off_a, off_b, shift, d_y32=None, d_y8=None):
+        self._ck(lib().egg_perturbed_linear(self._h, C.c_void_p(d_x), C.c_void_p(d_w), members, T, K, N,
+                                            seed & 0xFFFFFFFF, off_a, off_b, shift,
+                                            C.c_void_p(d_y32) if d_y32 else None, C.c_void_p(d_y8) if d_y8 else None),
+                 "egg_perturbed_linear")
+
+    def population_forward(self, d_data, data_len, start_idx, step_seed, pop_offset, pop_count, d_loss):
+        self._ck(lib().egg_population_forward(self._h, C.c_void_p(d_data), data_len, start_idx, step_seed & 0xFFFFFFFF,
+                                              pop_offset, pop_count, C.c_void_p(d_loss)), "egg_population_forward")
+
+    def fitness(self, d_loss, d_fit, pairs):
+        self._ck(lib().egg_fitness(self._h, C.c_void_p(d_loss), C.c_void_p(d_fit), pairs), "egg_fitness")
+
+    def es_update(self, d_fit, d_seed, d_lr):
+        self._ck(lib().egg_es_update(self._h, C.c_void_p(d_fit), C.c_void_p(d_seed), C.c_void_p(d_lr)), "egg_es_update")
+
+    def update_tensor(self, tid, d_fit, d_seed, d_lr):
+        self._ck(lib().egg_update_tensor(self._h, tid, C.c_void_p(d_fit), C.c_void_p(d_seed), C.c_void_p(d_lr)),
+                 "egg_update_tensor")
+
+    def matrix_votes(self, tid, d_fit, d_seed, d_votes):
+        self._ck(lib().egg_matrix_votes(self._h, tid, C.c_void_p(d_fit), C.c_void_p(d_seed), C.c_void_p(d_votes)),
+                 "egg_matrix_votes")
+
+    def tensors(self):
+        out = []
+        for i in range(lib().egg_tensor_count(self._h)):
+            t = EggTensorInfo()
+            self._ck(lib().egg_tensor_info_get(self._h, i, C.byref(t)), "egg_tensor_info_get")
+            out.append(dict(id=i, name=t.name.decode(), is_matrix=t.is_matrix, rows=t.rows, cols=t.cols, offset=t.offset,
+                            off_a=t.off_a, off_b=t.off_b, seed_base=t.seed_base, lr_scale=t.lr_scale, muon=t.muon))
+        return out
+
+    def last_update_count(self):
+        v = C.c_uint64()
+        self._ck(lib().egg_last_update_count(self._h, C.byref(v)), "egg_last_update_count")
+        return int(v.value)
+
+    def step(self, d_data, data_len, start_idx, step_seed, lr):
+        self._ck(lib().egg_step(self._h, C.c_void_p(d_data), data_len, start_idx, step_seed & 0xFFFFFFFF, C.c_float(lr)),
+                 "egg_step")
+
+    def step_capture(self, d_data, data_len):
+        self._ck(lib().egg_step_capture(self._h, C.c_void_p(d_data), data_len), "egg_step_capture")
+
+    def step_launch(self, start_idx, step_seed, lr):
+        self._ck(lib().egg_step_launch(self._h, start_idx, step_seed & 0xFFFFFFFF, C.c_float(lr)), "egg_step_launch")
+
+    def step_losses(self):
+        import numpy as np
+        loss = np.zeros(self.cfg.population, np.int32)
+        fit = np.zeros(self.cfg.population // 2, np.int32)
+        self._ck(lib().egg_step_losses(self._h, _np_ptr(loss), _np_ptr(fit)), "egg_step_losses")
+        return loss, fit
+
+    def enable_taps(self, on=True):
+        self._ck(lib().egg_ctx_enable_taps(self._h, 1 if on else 0), "egg_ctx_enable_taps")
+
+    def tap(self, name, member):
+        import numpy as np
+        T, H = self.cfg.seq_len, self.cfg.hidden
+        out = np.zeros((T, 256), np.int32) if name == "logits" else np.zeros((T, H), np.int8)
+        self._ck(lib().egg_tap_download(self._h, name.encode(), member, _np_ptr(out)), "egg_tap_download")
+        return out
+
+
+def learning_rate(step):
+    return float(lib().egg_learning_rate(step))
+
+
+def next_seed(seed, step):
+    return int(lib().egg_next_seed(seed & 0xFFFFFFFF, step))

@@ -1,0 +1,569 @@
+// egg_api.hip -- the C ABI of libegg_hip.so (declared in include/egg_hip.h): context, model and
+// optimizer-state management, and the host-side sequencing of the forward / fitness / update kernels.
+// Reference host loop: full_cuda_train_transformer_adam_mgpu.cu:1313-1767 ("mgpu.cu").
+#include "../../include/egg_hip.h"
+#include "egg_launch.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+#include <string>
+#include <vector>
+
+// ------------------------------------------------------------------ model layout (TransformerModel, mgpu.cu:284-318)
+struct Layout {
+    int64_t embedding, emb_bias, ln_init, ln_init_bias, w_emb_mlp_up, mlp_emb_bias_up, w_emb_mlp_down,
+        mlp_emb_bias_down, ln_1, ln_1_bias, w_q, w_k, w_v, w_o, ln_2, ln_2_bias, w_up, mlp_bias_up, w_down,
+        mlp_bias_down, ln_f, ln_f_bias, total;
+};
+static Layout make_layout(const egg_config &c) {
+    Layout L; int64_t o = 0, H = c.hidden, V = c.vocab, NL = c.n_layers;
+    auto take = [&](int64_t n) { int64_t r = o; o += n; return r; };
+    L.embedding = take(V * H); L.emb_bias = take(H); L.ln_init = take(H); L.ln_init_bias = take(H);
+    L.w_emb_mlp_up = take(H * 4 * H); L.mlp_emb_bias_up = take(4 * H);
+    L.w_emb_mlp_down = take(4 * H * H); L.mlp_emb_bias_down = take(H);
+    L.ln_1 = take(NL * H); L.ln_1_bias = take(NL * H);
+    L.w_q = take(NL * H * H); L.w_k = take(NL * H * H); L.w_v = take(NL * H * H); L.w_o = take(NL * H * H);
+    L.ln_2 = take(NL * H); L.ln_2_bias = take(NL * H);
+    L.w_up = take(NL * H * 4 * H); L.mlp_bias_up = take(NL * 4 * H);
+    L.w_down = take(NL * 4 * H * H); L.mlp_bias_down = take(NL * H);
+    L.ln_f = take(H); L.ln_f_bias = take(H);
+    L.total = o;
+    return L;
+}
+
+struct Scalars { uint32_t seed; float lr; int64_t start; };
+__global__ void k_set_scalars(Scalars *s, uint32_t seed, float lr, int64_t start) { s->seed = seed; s->lr = lr; s->start = start; }
+
+struct egg_ctx {
+    egg_config cfg;
+    hipStream_t stream = nullptr; bool own_stream = false;
+    Layout L;
+    std::vector<egg_tensor_info> tensors;
+    int8_t *d_model = nullptr; float *d_state = nullptr;
+    int32_t *d_exp = nullptr; int8_t *d_act = nullptr; int32_t *d_rope = nullptr;
+    int chunk = 0;
+    int8_t *d_x = nullptr, *d_q = nullptr, *d_k = nullptr, *d_v = nullptr, *d_ao = nullptr;
+    unsigned long long *d_loss_acc = nullptr, *d_counter = nullptr;
+    int32_t *d_loss = nullptr, *d_fit = nullptr;
+    Scalars *d_scal = nullptr;
+    int8_t *d_panel_a = nullptr, *d_panel_b = nullptr; int pairs_pad = 0;
+    // taps
+    bool taps = false; int8_t *d_tap = nullptr; int32_t *d_tap_logits = nullptr; int tap_members = 0;
+    // graph
+    hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr; bool captured = false;
+    std::string err;
+};
+
+static int fail(egg_ctx *ctx, int code, const char *what, hipError_t e = hipSuccess) {
+    if (ctx) {
+        ctx->err = what;
+        if (e != hipSuccess) { ctx->err += ": "; ctx->err += hipGetErrorString(e); }
+    }
+    return code;
+}
+#define HIP_TRY(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return fail(ctx, EGG_E_HIP, #call, e_); } while (0)
+
+extern "C" void egg_default_config(egg_config *c) {
+    memset(c, 0, sizeof(*c));
+    c->hidden = 256; c->head_dim = 64; c->n_layers = 4; c->seq_len = 32; c->vocab = 256; c->population = 16384 * 4;
+    c->fixed_point = 4; c->sigma_shift = 3; c->sigma_shift_vector = 4;
+    c->shift_attn = 8; c->shift_out = 9; c->shift_logit = 8; c->shift_mlp_up = 8; c->shift_mlp_down = 10;
+    c->softmax_scale_bit = 18; c->rope_scale_bit = 20; c->noise_mask = 15; c->host_mask = 15;
+    c->softmax_exp_scale = 6.0;
+    c->adam_beta1 = 0.9f; c->adam_beta2 = 0.95f; c->adam_eps = 1e-8f; c->adam_weight_decay = 0.01f;
+    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->use_muon = 0; c->chunk_members = 0;
+}
+
+// launch order of mgpu.cu:1603-1643
+static void build_tensor_table(egg_ctx *ctx) {
+    const egg_config &c = ctx->cfg; const Layout &L = ctx->L; int H = c.hidden, V = c.vocab;
+    auto add = [&](const char *name, int l, int is_matrix, int rows, int cols, int64_t off, int oa, int ob, int base, float lrs, int muon) {
+        egg_tensor_info t; memset(&t, 0, sizeof(t));
+        if (l >= 0) snprintf(t.name, sizeof(t.name), "%s.%d", name, l); else snprintf(t.name, sizeof(t.name), "%s", name);
+        t.is_matrix = is_matrix; t.rows = rows; t.cols = cols; t.offset = off; t.off_a = oa; t.off_b = ob;
+        t.seed_base = base; t.lr_scale = lrs; t.muon = muon;
+        ctx->tensors.push_back(t);
+    };
+    for (int l = 0; l < c.n_layers; l++) {
+        int b = l * 1000; int64_t hh = (int64_t)H * H, h4 = (int64_t)H * 4 * H;
+        add("w_q", l, 1, H, H, L.w_q + l * hh, OFF_Q_A, OFF_Q_B, b, 1.f, 1);
+        add("w_k", l, 1, H, H, L.w_k + l * hh, OFF_K_A, OFF_K_B, b, 1.f, 1);
+        add("w_v", l, 1, H, H, L.w_v + l * hh, OFF_V_A, OFF_V_B, b, 1.f, 1);
+        add("w_o", l, 1, H, H, L.w_o + l * hh, OFF_O_A, OFF_O_B, b, 1.f, 1);
+        add("w_up", l, 1, H, 4 * H, L.w_up + l * h4, OFF_MLP_UP_A, OFF_MLP_UP_B, b, 1.f, 1);
+        add("w_down", l, 1, 4 * H, H, L.w_down + l * h4, OFF_MLP_DOWN_A, OFF_MLP_DOWN_B, b, 1.f, 1);
+        add("ln_1", l, 0, 1, H, L.ln_1 + (int64_t)l * H, OFF_LN_1_A, OFF_LN_1_B, b, 1.f, 0);
+        add("ln_1_bias", l, 0, 1, H, L.ln_1_bias + (int64_t)l * H, OFF_LN_1_BIAS_A, OFF_LN_1_BIAS_B, b, 1.f, 0);
+        add("ln_2", l, 0, 1, H, L.ln_2 + (int64_t)l * H, OFF_LN_2_A, OFF_LN_2_B, b, 1.f, 0);
+        add("ln_2_bias", l, 0, 1, H, L.ln_2_bias + (int64_t)l * H, OFF_LN_2_BIAS_A, OFF_LN_2_BIAS_B, b, 1.f, 0);
+        add("mlp_bias_up", l, 0, 1, 4 * H, L.mlp_bias_up + (int64_t)l * 4 * H, OFF_MLP_BIAS_UP_A, OFF_MLP_BIAS_UP_B, b, 1.f, 0);
+        add("mlp_bias_down", l, 0, 1, H, L.mlp_bias_down + (int64_t)l * H, OFF_MLP_BIAS_DOWN_A, OFF_MLP_BIAS_DOWN_B, b, 1.f, 0);
+    }
+    add("ln_f", -1, 0, 1, H, L.ln_f, OFF_LN_F_A, OFF_LN_F_B, 0, 1.f, 0);
+    add("ln_f_bias", -1, 0, 1, H, L.ln_f_bias, OFF_LN_F_BIAS_A, OFF_LN_F_BIAS_B, 0, 1.f, 0);
+    add("ln_init", -1, 0, 1, H, L.ln_init, OFF_LN_INIT_A, OFF_LN_INIT_B, 0, 1.f, 0);
+    add("ln_init_bias", -1, 0, 1, H, L.ln_init_bias, OFF_LN_INIT_BIAS_A, OFF_LN_INIT_BIAS_B, 0, 1.f, 0);
+    add("w_emb_mlp_up", -1, 1, H, 4 * H, L.w_emb_mlp_up, OFF_EMB_MLP_UP_A, OFF_EMB_MLP_UP_B, 0, 1.f, 1);
+    add("mlp_emb_bias_up", -1, 0, 1, 4 * H, L.mlp_emb_bias_up, OFF_EMB_MLP_BIAS_UP_A, OFF_EMB_MLP_BIAS_UP_B, 0, 1.f, 0);
+    add("w_emb_mlp_down", -1, 1, 4 * H, H, L.w_emb_mlp_down, OFF_EMB_MLP_DOWN_A, OFF_EMB_MLP_DOWN_B, 0, 1.f, 1);
+    add("mlp_emb_bias_down", -1, 0, 1, H, L.mlp_emb_bias_down, OFF_EMB_MLP_BIAS_DOWN_A, OFF_EMB_MLP_BIAS_DOWN_B, 0, 1.f, 0);
+    add("emb_bias", -1, 0, 1, H, L.emb_bias, OFF_EMB_BIAS_A, OFF_EMB_BIAS_B, 0, 0.1f, 0);
+    add("embedding", -1, 1, H, V, L.embedding, OFF_EMB, OFF_EMB + H, 0, 1.f, 0);
+}
+
+static void free_all(egg_ctx *ctx) {
+    void *ptrs[] = {ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
+                    ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
+                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits};
+    for (void *p : ptrs) if (p) (void)hipFree(p);
+    if (ctx->gexec) (void)hipGraphExecDestroy(ctx->gexec);
+    if (ctx->graph) (void)hipGraphDestroy(ctx->graph);
+    if (ctx->own_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
+}
+
+extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
+    if (!cfg || !out) return EGG_E_INVALID;
+    *out = nullptr;
+    const egg_config &c = *cfg;
+    if (!(c.hidden == 64 || c.hidden == 128 || c.hidden == 256)) return EGG_E_INVALID;
+    if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return EGG_E_INVALID;
+    if (c.seq_len % 32 || !(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256)) return EGG_E_INVALID;
+    if (c.vocab != 256 || c.n_layers < 1 || c.population < 2 || (c.population & 1)) return EGG_E_INVALID;
+    if (c.use_muon) return EGG_E_INVALID;   // Muon step not available in this build
+    egg_ctx *ctx = new egg_ctx();
+    ctx->cfg = c;
+    ctx->L = make_layout(c);
+    build_tensor_table(ctx);
+    auto bail = [&](int code, const char *what, hipError_t e) { fprintf(stderr, "egg_ctx_create: %s: %s\n", what, hipGetErrorString(e)); free_all(ctx); delete ctx; return code; };
+#define CR(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return bail(EGG_E_HIP, #call, e_); } while (0)
+    CR(hipStreamCreate(&ctx->stream)); ctx->own_stream = true;
+    CR(egg_prepare_forward(c.hidden, c.head_dim, c.seq_len));
+    // lookup tables in double precision on the host, exactly as init_tables (mgpu.cu:394-426)
+    std::vector<int32_t> ex(256), rope((size_t)c.seq_len * c.head_dim); std::vector<int8_t> act(256);
+    for (int i = 0; i < 256; i++) {
+        double val = exp(-(double)i / c.softmax_exp_scale) * (double)(1 << c.softmax_scale_bit);
+        ex[i] = (val >= 1.0) ? (int32_t)round(val) : 0;
+        int8_t input = (int8_t)i;
+        double x = (double)input / (1 << c.fixed_point);
+        double y = 0.5 * x * (1.0 + erf(x / 1.41421356));
+        int v = (int)round(y * (1 << c.fixed_point));
+        act[i] = (int8_t)((v > 127) ? 127 : ((v < -127) ? -127 : v));
+    }
+    for (int t = 0; t < c.seq_len; t++)
+        for (int i = 0; i < c.head_dim / 2; i++) {
+            double theta = pow(10000.0, -2.0 * i / c.head_dim), alpha = t * theta;
+            rope[(size_t)t * c.head_dim + 2 * i] = (int32_t)round(cos(alpha) * (double)(1 << c.rope_scale_bit));
+            rope[(size_t)t * c.head_dim + 2 * i + 1] = (int32_t)round(sin(alpha) * (double)(1 << c.rope_scale_bit));
+        }
+    CR(hipMalloc(&ctx->d_exp, 256 * 4)); CR(hipMalloc(&ctx->d_act, 256)); CR(hipMalloc(&ctx->d_rope, rope.size() * 4));
+    CR(hipMemcpy(ctx->d_exp, ex.data(), 256 * 4, hipMemcpyHostToDevice));
+    CR(hipMemcpy(ctx->d_act, act.data(), 256, hipMemcpyHostToDevice));
+    CR(hipMemcpy(ctx->d_rope, rope.data(), rope.size() * 4, hipMemcpyHostToDevice));
+    CR(hipMalloc(&ctx->d_model, ctx->L.total)); CR(hipMemset(ctx->d_model, 0, ctx->L.total));
+    CR(hipMalloc(&ctx->d_state, ctx->L.total * 12)); CR(hipMemset(ctx->d_state, 0, ctx->L.total * 12));
+    // activation workspace for one chunk of members
+    int chunk = c.chunk_members > 0 ? c.chunk_members : 2048;
+    if (chunk > c.population) chunk = c.population;
+    ctx->chunk = chunk;
+    size_t act_bytes = (size_t)chunk * c.seq_len * c.hidden;
+    CR(hipMalloc(&ctx->d_x, act_bytes)); CR(hipMalloc(&ctx->d_q, act_bytes)); CR(hipMalloc(&ctx->d_k, act_bytes));
+    CR(hipMalloc(&ctx->d_v, act_bytes)); CR(hipMalloc(&ctx->d_ao, act_bytes));
+    CR(hipMalloc(&ctx->d_loss_acc, (size_t)c.population * 8)); CR(hipMalloc(&ctx->d_counter, 8));
+    CR(hipMemset(ctx->d_counter, 0, 8));
+    CR(hipMalloc(&ctx->d_loss, (size_t)c.population * 4)); CR(hipMalloc(&ctx->d_fit, (size_t)(c.population / 2) * 4));
+    CR(hipMalloc(&ctx->d_scal, sizeof(Scalars)));
+    ctx->pairs_pad = ((c.population / 2) + 63) / 64 * 64;
+    CR(hipMalloc(&ctx->d_panel_a, (size_t)4 * c.hidden * ctx->pairs_pad));
+    CR(hipMalloc(&ctx->d_panel_b, (size_t)4 * c.hidden * ctx->pairs_pad));
+#undef CR
+    *out = ctx;
+    return EGG_OK;
+}
+
+extern "C" void egg_ctx_destroy(egg_ctx *ctx) {
+    if (!ctx) return;
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    free_all(ctx);
+    delete ctx;
+}
+extern "C" const char *egg_last_error(const egg_ctx *ctx) { return ctx ? ctx->err.c_str() : "null context"; }
+extern "C" int egg_ctx_set_stream(egg_ctx *ctx, void *s) {
+    if (!ctx) return EGG_E_INVALID;
+    if (ctx->captured) return fail(ctx, EGG_E_STATE, "stream cannot change after egg_step_capture");
+    if (ctx->own_stream && ctx->stream) { (void)hipStreamSynchronize(ctx->stream); (void)hipStreamDestroy(ctx->stream); }
+    ctx->stream = (hipStream_t)s; ctx->own_stream = false;
+    return EGG_OK;
+}
+extern "C" int egg_sync(egg_ctx *ctx) {
+    if (!ctx) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return EGG_OK;
+}
+
+extern "C" int64_t egg_model_bytes(const egg_ctx *ctx) { return ctx ? ctx->L.total : 0; }
+
+// ------------------------------------------------------------------ init_model (mgpu.cu:428-519)
+static inline uint32_t xorshift32_host(uint32_t *st) { uint32_t x = *st; x ^= x << 13; x ^= x >> 17; x ^= x << 5; *st = x; return x; }
+static inline int8_t gen_noise_host(uint32_t *rng, int mask) {
+    uint32_t r = xorshift32_host(rng);
+    return (int8_t)((r & 1 ? 1 : -1) * (int)((r >> 1) & (uint32_t)mask));
+}
+// [In][Out] row-major -> blocked [In/4][Out][4]
+static void repack_matrix(int8_t *dst, const int8_t *src, int rows, int cols) {
+    for (int kq = 0; kq < rows / 4; kq++)
+        for (int n = 0; n < cols; n++)
+            for (int s = 0; s < 4; s++) dst[((size_t)kq * cols + n) * 4 + s] = src[(size_t)(4 * kq + s) * cols + n];
+}
+extern "C" int egg_model_init(egg_ctx *ctx, uint32_t seed) {
+    if (!ctx) return EGG_E_INVALID;
+    const egg_config &c = ctx->cfg; const Layout &L = ctx->L; const int H = c.hidden, V = c.vocab;
+    std::vector<int8_t> m((size_t)L.total, 0), tmp((size_t)H * 4 * H > (size_t)V * H ? (size_t)H * 4 * H : (size_t)V * H);
+    uint32_t rng = seed;
+    auto gen = [&](int8_t *dst, int rows, int cols) {
+        for (size_t i = 0; i < (size_t)rows * cols; i++) tmp[i] = gen_noise_host(&rng, c.host_mask);
+        repack_matrix(dst, tmp.data(), rows, cols);
+    };
+    gen(&m[L.embedding], H, V);
+    for (int i = 0; i < H; i++) m[L.ln_init + i] = 16;
+    gen(&m[L.w_emb_mlp_up], H, 4 * H);
+    gen(&m[L.w_emb_mlp_down], 4 * H, H);
+    for (int l = 0; l < c.n_layers; l++) {
+        for (int i = 0; i < H; i++) { m[L.ln_1 + (int64_t)l * H + i] = 16; m[L.ln_2 + (int64_t)l * H + i] = 16; }
+        gen(&m[L.w_q + (int64_t)l * H * H], H, H); gen(&m[L.w_k + (int64_t)l * H * H], H, H);
+        gen(&m[L.w_v + (int64_t)l * H * H], H, H); gen(&m[L.w_o + (int64_t)l * H * H], H, H);
+        gen(&m[L.w_up + (int64_t)l * H * 4 * H], H, 4 * H); gen(&m[L.w_down + (int64_t)l * 4 * H * H], 4 * H, H);
+    }
+    for (int i = 0; i < H; i++) m[L.ln_f + i] = 16;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemcpy(ctx->d_model, m.data(), m.size(), hipMemcpyHostToDevice));
+    return EGG_OK;
+}
+extern "C" int egg_model_upload(egg_ctx *ctx, const void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != ctx->L.total) return fail(ctx, EGG_E_INVALID, "model size mismatch");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemcpy(ctx->d_model, h, bytes, hipMemcpyHostToDevice));
+    return EGG_OK;
+}
+extern "C" int egg_model_download(egg_ctx *ctx, void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != ctx->L.total) return fail(ctx, EGG_E_INVALID, "model size mismatch");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemcpy(h, ctx->d_model, bytes, hipMemcpyDeviceToHost));
+    return EGG_OK;
+}
+extern "C" int egg_opt_state_upload(egg_ctx *ctx, const void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != ctx->L.total * 12) return fail(ctx, EGG_E_INVALID, "state size mismatch");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemcpy(ctx->d_state, h, bytes, hipMemcpyHostToDevice));
+    return EGG_OK;
+}
+extern "C" int egg_opt_state_download(egg_ctx *ctx, void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != ctx->L.total * 12) return fail(ctx, EGG_E_INVALID, "state size mismatch");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemcpy(h, ctx->d_state, bytes, hipMemcpyDeviceToHost));
+    return EGG_OK;
+}
+extern "C" int egg_opt_state_reset(egg_ctx *ctx) {
+    if (!ctx) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemset(ctx->d_state, 0, ctx->L.total * 12));
+    return EGG_OK;
+}
+extern "C" int egg_tables_download(egg_ctx *ctx, int32_t *ex, int8_t *act, int32_t *rope) {
+    if (!ctx) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (ex) HIP_TRY(hipMemcpy(ex, ctx->d_exp, 256 * 4, hipMemcpyDeviceToHost));
+    if (act) HIP_TRY(hipMemcpy(act, ctx->d_act, 256, hipMemcpyDeviceToHost));
+    if (rope) HIP_TRY(hipMemcpy(rope, ctx->d_rope, (size_t)ctx->cfg.seq_len * ctx->cfg.head_dim * 4, hipMemcpyDeviceToHost));
+    return EGG_OK;
+}
+
+extern "C" int egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first, int n, int8_t *d_out) {
+    if (!ctx || !d_out || n < 0) return fail(ctx, EGG_E_INVALID, "egg_noise_fill arguments");
+    HIP_TRY(egg_launch_noise_fill(seed, first, n, ctx->cfg.noise_mask, d_out, ctx->stream));
+    return EGG_OK;
+}
+
+extern "C" int egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
+                                    uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8) {
+    if (!ctx || !d_X || !d_W || members < 1 || T < 32 || T % 32 || (!d_Y32 && !d_Y8) || shift < 0 || shift > 31)
+        return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear arguments");
+    PlinParams p = {d_X, d_W, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
+                    ctx->cfg.noise_mask, d_Y32, d_Y8};
+    hipError_t e = egg_launch_plinear(p, ctx->stream);
+    if (e == hipErrorInvalidValue) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");
+    HIP_TRY(e);
+    return EGG_OK;
+}
+
+// ------------------------------------------------------------------ forward
+static FwdCommon make_common(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const int64_t *d_start, const uint32_t *d_seed,
+                             int first_member, int nm) {
+    const egg_config &c = ctx->cfg;
+    FwdCommon f;
+    f.data = d_data; f.data_len = len; f.d_start_idx = d_start; f.d_step_seed = d_seed;
+    f.pop_offset = first_member; f.n_members = nm; f.population = c.population;
+    f.T = c.seq_len; f.H = c.hidden; f.head_dim = c.head_dim; f.vocab = c.vocab;
+    f.sigma = c.fixed_point + c.sigma_shift; f.sigma_vec = c.sigma_shift_vector; f.mask = c.noise_mask;
+    f.shift_attn = c.shift_attn; f.shift_out = c.shift_out; f.shift_logit = c.shift_logit;
+    f.shift_mlp_up = c.shift_mlp_up; f.shift_mlp_down = c.shift_mlp_down;
+    f.softmax_scale_bit = c.softmax_scale_bit; f.rope_scale_bit = c.rope_scale_bit;
+    f.exp_lut = ctx->d_exp; f.act_lut = ctx->d_act; f.rope_lut = ctx->d_rope;
+    return f;
+}
+
+// tap buffer: [slot][member][T][H], slots: 0 x_init, then per layer 6: q k v ao x_attn x_mlp
+static int8_t *tap_ptr(egg_ctx *ctx, int slot) {
+    return ctx->d_tap + (size_t)slot * ctx->tap_members * ctx->cfg.seq_len * ctx->cfg.hidden;
+}
+
+static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const int64_t *d_start, const uint32_t *d_seed,
+                         int first_member, int nm) {
+    const egg_config &c = ctx->cfg; const Layout &L = ctx->L; const int8_t *M = ctx->d_model; const int H = c.hidden;
+    hipStream_t s = ctx->stream;
+    const bool taps = ctx->taps && nm <= ctx->tap_members;
+    const size_t act_bytes = (size_t)nm * c.seq_len * H;
+    FwdCommon f = make_common(ctx, d_data, len, d_start, d_seed, first_member, nm);
+    {
+        MlpParams p; memset(&p, 0, sizeof(p)); p.c = f; p.seed_base = 0;
+        p.off_ln_a = OFF_LN_INIT_A; p.off_ln_b = OFF_LN_INIT_B; p.off_lnb_a = OFF_LN_INIT_BIAS_A; p.off_lnb_b = OFF_LN_INIT_BIAS_B;
+        p.off_up_a = OFF_EMB_MLP_UP_A; p.off_up_b = OFF_EMB_MLP_UP_B; p.off_bup_a = OFF_EMB_MLP_BIAS_UP_A; p.off_bup_b = OFF_EMB_MLP_BIAS_UP_B;
+        p.off_dn_a = OFF_EMB_MLP_DOWN_A; p.off_dn_b = OFF_EMB_MLP_DOWN_B; p.off_bdn_a = OFF_EMB_MLP_BIAS_DOWN_A; p.off_bdn_b = OFF_EMB_MLP_BIAS_DOWN_B;
+        p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = M + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
+        p.w_dn = M + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
+        p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
+        HIP_TRY(egg_launch_mlp(p, true, s));
+        if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 0), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
+    }
+    for (int l = 0; l < c.n_layers; l++) {
+        const int64_t hh = (int64_t)H * H, h4 = (int64_t)H * 4 * H;
+        {
+            QkvParams p; memset(&p, 0, sizeof(p)); p.c = f; p.seed_base = l * 1000;
+            p.ln_w = M + L.ln_1 + (int64_t)l * H; p.ln_b = M + L.ln_1_bias + (int64_t)l * H;
+            p.w_q = M + L.w_q + l * hh; p.w_k = M + L.w_k + l * hh; p.w_v = M + L.w_v + l * hh;
+            p.x = ctx->d_x; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v;
+            HIP_TRY(egg_launch_qkv(p, s));
+            if (taps) {
+                HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 0), ctx->d_q, act_bytes, hipMemcpyDeviceToDevice, s));
+                HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 1), ctx->d_k, act_bytes, hipMemcpyDeviceToDevice, s));
+                HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 2), ctx->d_v, act_bytes, hipMemcpyDeviceToDevice, s));
+            }
+        }
+        {
+            AttnParams p; memset(&p, 0, sizeof(p)); p.c = f; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v; p.ao = ctx->d_ao;
+            HIP_TRY(egg_launch_attn(p, s));
+            if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 3), ctx->d_ao, act_bytes, hipMemcpyDeviceToDevice, s));
+        }
+        {
+            MlpParams p; memset(&p, 0, sizeof(p)); p.c = f; p.seed_base = l * 1000;
+            p.off_ln_a = OFF_LN_2_A; p.off_ln_b = OFF_LN_2_B; p.off_lnb_a = OFF_LN_2_BIAS_A; p.off_lnb_b = OFF_LN_2_BIAS_B;
+            p.off_up_a = OFF_MLP_UP_A; p.off_up_b = OFF_MLP_UP_B; p.off_bup_a = OFF_MLP_BIAS_UP_A; p.off_bup_b = OFF_MLP_BIAS_UP_B;
+            p.off_dn_a = OFF_MLP_DOWN_A; p.off_dn_b = OFF_MLP_DOWN_B; p.off_bdn_a = OFF_MLP_BIAS_DOWN_A; p.off_bdn_b = OFF_MLP_BIAS_DOWN_B;
+            p.ln_w = M + L.ln_2 + (int64_t)l * H; p.ln_b = M + L.ln_2_bias + (int64_t)l * H;
+            p.w_up = M + L.w_up + l * h4; p.b_up = M + L.mlp_bias_up + (int64_t)l * 4 * H;
+            p.w_dn = M + L.w_down + l * h4; p.b_dn = M + L.mlp_bias_down + (int64_t)l * H;
+            p.w_o = M + L.w_o + l * hh; p.ao = ctx->d_ao; p.x = ctx->d_x;
+            p.x_mid = taps ? tap_ptr(ctx, 1 + 6 * l + 4) : nullptr;
+            HIP_TRY(egg_launch_mlp(p, false, s));
+            if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 5), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
+        }
+    }
+    {
+        HeadParams p; memset(&p, 0, sizeof(p)); p.c = f;
+        p.ln_w = M + L.ln_f; p.ln_b = M + L.ln_f_bias; p.embedding = M + L.embedding; p.x = ctx->d_x;
+        p.loss_acc = ctx->d_loss_acc; p.logits_tap = taps ? ctx->d_tap_logits : nullptr;
+        HIP_TRY(egg_launch_head(p, s));
+    }
+    return EGG_OK;
+}
+
+static int forward_range(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const int64_t *d_start, const uint32_t *d_seed,
+                         int pop_offset, int pop_count, int32_t *d_loss) {
+    const egg_config &c = ctx->cfg;
+    if (!d_data || !d_loss || pop_offset < 0 || pop_count < 1 || pop_offset + pop_count > c.population)
+        return fail(ctx, EGG_E_INVALID, "population range");
+    if (len <= c.seq_len + 1) return fail(ctx, EGG_E_INVALID, "data_len must exceed seq_len + 1");
+    HIP_TRY(egg_launch_zero_u64(ctx->d_loss_acc + pop_offset, pop_count, ctx->stream));
+    for (int done = 0; done < pop_count; done += ctx->chunk) {
+        int nm = pop_count - done < ctx->chunk ? pop_count - done : ctx->chunk;
+        int rc = forward_chunk(ctx, d_data, len, d_start, d_seed, pop_offset + done, nm);
+        if (rc) return rc;
+    }
+    HIP_TRY(egg_launch_loss_finalize(ctx->d_loss_acc, d_loss, pop_offset, pop_count, ctx->stream));
+    return EGG_OK;
+}
+
+extern "C" int egg_population_forward_dev(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const int64_t *d_start,
+                                          const uint32_t *d_seed, int pop_offset, int pop_count, int32_t *d_loss) {
+    if (!ctx || !d_start || !d_seed) return fail(ctx, EGG_E_INVALID, "null scalar pointer");
+    return forward_range(ctx, d_data, len, d_start, d_seed, pop_offset, pop_count, d_loss);
+}
+extern "C" int egg_population_forward(egg_ctx *ctx, const uint8_t *d_data, int64_t len, int64_t start_idx, uint32_t step_seed,
+                                      int pop_offset, int pop_count, int32_t *d_loss) {
+    if (!ctx) return EGG_E_INVALID;
+    hipLaunchKernelGGL(k_set_scalars, dim3(1), dim3(1), 0, ctx->stream, ctx->d_scal, step_seed, 0.f, start_idx);
+    HIP_TRY(hipGetLastError());
+    return forward_range(ctx, d_data, len, &ctx->d_scal->start, &ctx->d_scal->seed, pop_offset, pop_count, d_loss);
+}
+
+extern "C" int egg_fitness(egg_ctx *ctx, const int32_t *d_loss, int32_t *d_fit, int pairs) {
+    if (!ctx || !d_loss || !d_fit || pairs < 0) return fail(ctx, EGG_E_INVALID, "egg_fitness arguments");
+    HIP_TRY(egg_launch_fitness(d_loss, d_fit, pairs, ctx->stream));
+    return EGG_OK;
+}
+
+// ------------------------------------------------------------------ update
+static UpdParams make_upd(egg_ctx *ctx, const egg_tensor_info &t, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
+    const egg_config &c = ctx->cfg;
+    UpdParams p; memset(&p, 0, sizeof(p));
+    p.W = ctx->d_model + t.offset; p.state = ctx->d_state + t.offset * 3;
+    p.rows = t.rows; p.cols = t.cols; p.off_a = t.off_a; p.off_b = t.off_b; p.seed_base = t.seed_base;
+    p.fit = d_fit; p.pairs = c.population / 2; p.d_seed = d_seed; p.d_lr = d_lr; p.lr_scale = t.lr_scale;
+    p.mask = c.noise_mask; p.beta1 = c.adam_beta1; p.beta2 = c.adam_beta2; p.eps = c.adam_eps; p.wd = c.adam_weight_decay;
+    p.panel_a = ctx->d_panel_a; p.panel_b = ctx->d_panel_b; p.pairs_pad = ctx->pairs_pad; p.counter = ctx->d_counter;
+    return p;
+}
+static int update_one(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
+    const egg_tensor_info &t = ctx->tensors[id];
+    UpdParams p = make_upd(ctx, t, d_fit, d_seed, d_lr);
+    if (t.is_matrix) HIP_TRY(egg_launch_update_matrix(p, ctx->stream));
+    else HIP_TRY(egg_launch_update_vector(p, ctx->stream));
+    return EGG_OK;
+}
+extern "C" int egg_update_tensor(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
+    if (!ctx || id < 0 || id >= (int)ctx->tensors.size() || !d_fit || !d_seed || !d_lr) return fail(ctx, EGG_E_INVALID, "egg_update_tensor arguments");
+    return update_one(ctx, id, d_fit, d_seed, d_lr);
+}
+extern "C" int egg_matrix_votes(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, int32_t *d_votes) {
+    if (!ctx || id < 0 || id >= (int)ctx->tensors.size() || !d_fit || !d_seed || !d_votes || !ctx->tensors[id].is_matrix)
+        return fail(ctx, EGG_E_INVALID, "egg_matrix_votes arguments");
+    UpdParams p = make_upd(ctx, ctx->tensors[id], d_fit, d_seed, nullptr);
+    p.votes_out = d_votes;
+    HIP_TRY(egg_launch_update_matrix(p, ctx->stream));
+    return EGG_OK;
+}
+extern "C" int egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
+    if (!ctx || !d_fit || !d_seed || !d_lr) return fail(ctx, EGG_E_INVALID, "egg_es_update arguments");
+    HIP_TRY(egg_launch_zero_u64(ctx->d_counter, 1, ctx->stream));
+    for (int id = 0; id < (int)ctx->tensors.size(); id++) {
+        int rc = update_one(ctx, id, d_fit, d_seed, d_lr);
+        if (rc) return rc;
+    }
+    return EGG_OK;
+}
+extern "C" int egg_tensor_count(const egg_ctx *ctx) { return ctx ? (int)ctx->tensors.size() : 0; }
+extern "C" int egg_tensor_info_get(const egg_ctx *ctx, int id, egg_tensor_info *out) {
+    if (!ctx || !out || id < 0 || id >= (int)ctx->tensors.size()) return EGG_E_INVALID;
+    *out = ctx->tensors[id];
+    return EGG_OK;
+}
+extern "C" int egg_last_update_count(egg_ctx *ctx, uint64_t *out) {
+    if (!ctx || !out) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    unsigned long long v = 0;
+    HIP_TRY(hipMemcpy(&v, ctx->d_counter, 8, hipMemcpyDeviceToHost));
+    *out = v;
+    return EGG_OK;
+}
+
+// ------------------------------------------------------------------ whole step
+static int enqueue_step(egg_ctx *ctx, const uint8_t *d_data, int64_t len) {
+    int rc = forward_range(ctx, d_data, len, &ctx->d_scal->start, &ctx->d_scal->seed, 0, ctx->cfg.population, ctx->d_loss);
+    if (rc) return rc;
+    HIP_TRY(egg_launch_fitness(ctx->d_loss, ctx->d_fit, ctx->cfg.population / 2, ctx->stream));
+    return egg_es_update(ctx, ctx->d_fit, &ctx->d_scal->seed, &ctx->d_scal->lr);
+}
+extern "C" int egg_step(egg_ctx *ctx, const uint8_t *d_data, int64_t len, int64_t start_idx, uint32_t step_seed, float lr) {
+    if (!ctx) return EGG_E_INVALID;
+    hipLaunchKernelGGL(k_set_scalars, dim3(1), dim3(1), 0, ctx->stream, ctx->d_scal, step_seed, lr, start_idx);
+    HIP_TRY(hipGetLastError());
+    return enqueue_step(ctx, d_data, len);
+}
+extern "C" int egg_step_capture(egg_ctx *ctx, const uint8_t *d_data, int64_t len) {
+    if (!ctx) return EGG_E_INVALID;
+    if (ctx->captured) return fail(ctx, EGG_E_STATE, "step already captured");
+    if (ctx->taps) return fail(ctx, EGG_E_STATE, "disable taps before capturing");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    int rc = enqueue_step(ctx, d_data, len);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+    if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+    if (e != hipSuccess) return fail(ctx, EGG_E_HIP, "hipStreamEndCapture", e);
+    ctx->graph = g;
+    HIP_TRY(hipGraphInstantiate(&ctx->gexec, ctx->graph, nullptr, nullptr, 0));
+    ctx->captured = true;
+    return EGG_OK;
+}
+extern "C" int egg_step_launch(egg_ctx *ctx, int64_t start_idx, uint32_t step_seed, float lr) {
+    if (!ctx) return EGG_E_INVALID;
+    if (!ctx->captured) return fail(ctx, EGG_E_STATE, "egg_step_capture has not been called");
+    hipLaunchKernelGGL(k_set_scalars, dim3(1), dim3(1), 0, ctx->stream, ctx->d_scal, step_seed, lr, start_idx);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipGraphLaunch(ctx->gexec, ctx->stream));
+    return EGG_OK;
+}
+extern "C" int egg_step_losses(egg_ctx *ctx, int32_t *h_loss, int32_t *h_fit) {
+    if (!ctx) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (h_loss) HIP_TRY(hipMemcpy(h_loss, ctx->d_loss, (size_t)ctx->cfg.population * 4, hipMemcpyDeviceToHost));
+    if (h_fit) HIP_TRY(hipMemcpy(h_fit, ctx->d_fit, (size_t)(ctx->cfg.population / 2) * 4, hipMemcpyDeviceToHost));
+    return EGG_OK;
+}
+
+// get_learning_rate (mgpu.cu:217-227)
+extern "C" float egg_learning_rate(long step) {
+    if (step < 300) return 0.3f;
+    if (step < 600) return 0.15f;
+    if (step < 1000) return 0.075f;
+    return 0.05f;
+}
+// current_seed = hash_rng(current_seed, current_step) (d-eggs/src/worker.cu:542)
+extern "C" uint32_t egg_next_seed(uint32_t seed, uint64_t step) {
+    uint32_t x = seed + (uint32_t)step * 0x9e3779b9u;
+    x ^= x >> 16; x *= 0x85ebca6bu; x ^= x >> 13; x *= 0xc2b2ae35u; x ^= x >> 16;
+    return x;
+}
+
+// ------------------------------------------------------------------ taps
+extern "C" int egg_ctx_enable_taps(egg_ctx *ctx, int enable) {
+    if (!ctx) return EGG_E_INVALID;
+    if (ctx->captured) return fail(ctx, EGG_E_STATE, "taps cannot change after capture");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (enable && !ctx->d_tap) {
+        const egg_config &c = ctx->cfg;
+        ctx->tap_members = ctx->chunk < 64 ? ctx->chunk : 64;
+        size_t one = (size_t)ctx->tap_members * c.seq_len * c.hidden;
+        HIP_TRY(hipMalloc(&ctx->d_tap, one * (1 + 6 * c.n_layers)));
+        HIP_TRY(hipMalloc(&ctx->d_tap_logits, (size_t)ctx->tap_members * c.seq_len * 256 * 4));
+    }
+    ctx->taps = enable != 0;
+    return EGG_OK;
+}
+extern "C" int egg_tap_download(egg_ctx *ctx, const char *name, int member, void *host_out) {
+    if (!ctx || !name || !host_out || !ctx->d_tap || member < 0 || member >= ctx->tap_members) return fail(ctx, EGG_E_INVALID, "egg_tap_download arguments");
+    const egg_config &c = ctx->cfg; const int T = c.seq_len, H = c.hidden;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (!strcmp(name, "logits")) {
+        HIP_TRY(hipMemcpy(host_out, ctx->d_tap_logits + (size_t)member * T * 256, (size_t)T * 256 * 4, hipMemcpyDeviceToHost));
+        return EGG_OK;
+    }
+    int slot = -1, layer = 0; char base[32] = {0};
+    const char *dot = strchr(name, '.');
+    if (dot) { size_t n = (size_t)(dot - name); if (n >= sizeof(base)) return EGG_E_INVALID; memcpy(base, name, n); layer = atoi(dot + 1); }
+    else snprintf(base, sizeof(base), "%s", name);
+    if (layer < 0 || layer >= c.n_layers) return fail(ctx, EGG_E_INVALID, "tap layer");
+    const char *names[6] = {"q", "k", "v", "ao", "x_attn", "x_mlp"};
+    if (!strcmp(base, "x_init")) slot = 0;
+    else for (int i = 0; i < 6; i++) if (!strcmp(base, names[i])) slot = 1 + 6 * layer + i;
+    if (slot < 0) return fail(ctx, EGG_E_INVALID, "unknown tap name");
+    std::vector<int8_t> buf((size_t)T * H);
+    HIP_TRY(hipMemcpy(buf.data(), tap_ptr(ctx, slot) + (size_t)member * T * H, buf.size(), hipMemcpyDeviceToHost));
+    int8_t *o = (int8_t *)host_out;
+    for (int t = 0; t < T; t++)
+        for (int n = 0; n < H; n++) {
+            int w = n & 31, q = w >> 3, g = (w >> 2) & 1, e = w & 3;
+            o[(size_t)t * H + n] = buf[(size_t)t * H + (n & ~31) + 16 * g + 4 * q + e];
+        }
+    return EGG_OK;
+}

@@ -1,0 +1,629 @@
+// egg_forward.hip -- Int8NativeFormer population forward on gfx950 (hand-written MFMA kernels).
+//
+// Reference: train_sequence_kernel and its device functions,
+// full_cuda_train_transformer_adam_mgpu.cu:553-1029 ("mgpu.cu"), which runs one member per block,
+// serially over tokens.  Here tokens are the GEMM's free dimension: a wave owns a tile of 32 tokens of
+// one member, four waves share each W block staged in LDS, and a launch covers a chunk of members.
+//   k_mlp<H,true>   embedding stage + initial MLP          (mgpu.cu:901-934, :708-759)
+//   k_qkv<H>        LN1 + Q/K/V projections + RoPE + norms (mgpu.cu:769-784)
+//   k_attn<HD,CT>   causal exp-LUT attention core          (mgpu.cu:787-825)
+//   k_mlp<H,false>  O-projection + residual norm + MLP     (mgpu.cu:827-831, :708-759)
+//   k_head<H>       final norm + tied head + loss          (mgpu.cu:955-1028)
+#include "egg_device.h"
+#include "egg_params.h"
+#include "egg_launch.h"
+
+#pragma clang fp contract(off)
+
+// stream position of a member's pair (mgpu.cu:864-870)
+__device__ __forceinline__ int64_t stream_pos_of(const FwdCommon &c, int member) {
+    int64_t pair = member / 2;
+    int64_t stride = c.data_len / (c.population / 2);
+    return (*c.d_start_idx + pair * stride) % (c.data_len - c.T);
+}
+
+// acc[nt][r] += (sb * At[n]) >> sigma for NT column groups starting at table offset n_off
+template <int NT>
+__device__ __forceinline__ void add_perturb(v16i *acc, int sb, const int *At, int n_off, int sigma, int g) {
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            v4i a4 = *reinterpret_cast<const v4i *>(At + n_off + 32 * nt + 8 * q + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[nt][4 * q + e] += (sb * a4[e]) >> sigma;
+        }
+}
+
+// ============================================================================ MLP block
+template <int H>
+struct MlpLds {
+    // per-wave tables, int32 unless noted
+    static constexpr int I32 = 14 * H;       // ex0[H] ex1[H] lnw[H] lnb[H] upA[4H] bup[4H] dnA[H] bdn[H]
+    static constexpr int I8 = 6 * H;         // exB[H] upB[H] dnB[4H]
+    static constexpr int PER_WAVE = I32 * 4 + I8;
+    static constexpr int WBLOCK = (H < 256 ? H : 256) * (H < 256 ? H : 256);
+    static constexpr int TOTAL = WBLOCK + 256 + EGG_WAVES * PER_WAVE;
+};
+
+template <int H, bool FIRST>
+__global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
+    constexpr int KS = H / 32, NT = H / 32;
+    extern __shared__ __align__(16) int8_t smem[];
+    int8_t *wlds = smem;
+    int8_t *act = smem + MlpLds<H>::WBLOCK;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    int8_t *tb = act + 256 + wave * MlpLds<H>::PER_WAVE;
+    int *ex0 = reinterpret_cast<int *>(tb);   // FIRST: emb_bias + noise   | else: O-proj A noise * ns
+    int *ex1 = ex0 + H;                       // FIRST: b_dim noise * ns    | else: unused
+    int *lnw = ex1 + H, *lnb = lnw + H, *upA = lnb + H, *bup = upA + 4 * H, *dnA = bup + 4 * H, *bdn = dnA + H;
+    int8_t *exB = reinterpret_cast<int8_t *>(bdn + H);   // O-proj B noise
+    int8_t *upB = exB + H, *dnB = upB + H;
+
+    const FwdCommon &c = p.c;
+    const int T = c.T;
+    int mloc = blockIdx.x * EGG_WAVES + wave;
+    const bool valid = mloc < c.n_members;
+    if (!valid) mloc = c.n_members - 1;
+    const int member = c.pop_offset + mloc;
+    const int ns = (member & 1) ? -1 : 1;
+    const uint32_t pair_seed = *c.d_step_seed + (uint32_t)(member / 2);
+    const uint32_t sb_ = pair_seed + (uint32_t)p.seed_base;
+
+    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) act[i] = c.act_lut[i];
+    if (FIRST) {
+        fill_vec_i32(ex0, p.emb_bias, pair_seed + OFF_EMB_BIAS_A, pair_seed + OFF_EMB_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
+        fill_noise_i32(ex1, pair_seed + OFF_EMB + H, H, c.mask, ns, lane);
+    } else {
+        fill_noise_i32(ex0, sb_ + OFF_O_A, H, c.mask, ns, lane);
+        fill_noise_i8(exB, sb_ + OFF_O_B, H, c.mask, lane);
+    }
+    fill_vec_i32(lnw, p.ln_w, sb_ + p.off_ln_a, sb_ + p.off_ln_b, H, c.mask, ns, c.sigma_vec, lane);
+    fill_vec_i32(lnb, p.ln_b, sb_ + p.off_lnb_a, sb_ + p.off_lnb_b, H, c.mask, ns, c.sigma_vec, lane);
+    fill_noise_i32(upA, sb_ + p.off_up_a, 4 * H, c.mask, ns, lane);
+    fill_vec_i32(bup, p.b_up, sb_ + p.off_bup_a, sb_ + p.off_bup_b, 4 * H, c.mask, ns, c.sigma_vec, lane);
+    fill_noise_i32(dnA, sb_ + p.off_dn_a, H, c.mask, ns, lane);
+    fill_vec_i32(bdn, p.b_dn, sb_ + p.off_bdn_a, sb_ + p.off_bdn_b, H, c.mask, ns, c.sigma_vec, lane);
+    fill_noise_i8(upB, sb_ + p.off_up_b, H, c.mask, lane);
+    fill_noise_i8(dnB, sb_ + p.off_dn_b, 4 * H, c.mask, lane);
+    __syncthreads();
+
+    const int64_t spos = FIRST ? stream_pos_of(c, member) : 0;
+
+    for (int pass = 0; pass < T / 32; pass++) {
+        const int t = pass * 32 + j;
+        const size_t row = ((size_t)mloc * T + t) * H;
+        v4i xcur[KS];
+        v16i acc[NT];
+
+        if (FIRST) {
+            // embedding stage (mgpu.cu:901-931)
+            const int tok = c.data[spos + t];
+            const int a_tok = noise_from_hash(pair_seed + OFF_EMB, (uint32_t)tok, c.mask);
+            const uint32_t *E32 = reinterpret_cast<const uint32_t *>(p.embedding);
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int n0 = 32 * ks + 8 * q + 4 * g;
+                    int e4 = (int)E32[(size_t)(n0 >> 2) * c.vocab + tok];
+                    v4i b4 = *reinterpret_cast<const v4i *>(ex0 + n0);
+                    v4i d4 = *reinterpret_cast<const v4i *>(ex1 + n0);
+                    int o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = clip127(sx8(e4, e) + b4[e] + ((a_tok * d4[e]) >> c.sigma));
+                    xcur[ks][q] = pack4(o[0], o[1], o[2], o[3]);
+                }
+        } else {
+            // attention output projection + residual + adaptive norm (mgpu.cu:827-831)
+            v4i aop[KS], xres[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) { aop[ks] = load_op(p.ao + row, ks, g); xres[ks] = load_op(p.x + row, ks, g); }
+            int sbo = dot_noise<KS, false>(aop, exB, 0, g);
+            zero_acc<NT>(acc);
+            gemm_stream<H, H, false>(acc, aop, p.w_o, H, 0, 0, wlds, lane);
+            add_perturb<NT>(acc, sbo, ex0, 0, c.sigma, g);
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[nt][r] = sx8(xres[nt][r >> 2], r & 3) + (acc[nt][r] >> c.shift_out);
+            adaptive_norm<NT>(acc, xcur);
+            if (p.x_mid && valid)
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) store_op(p.x_mid + row, ks, g, xcur[ks]);
+        }
+
+        // MLP (mgpu.cu:708-759)
+        v4i nrm[KS];
+        standard_norm<KS>(xcur, nrm, lnw, lnb, H, g);
+        const int sbu = dot_noise<KS, false>(nrm, upB, 0, g);
+        v16i accd[NT];
+        zero_acc<NT>(accd);
+        int sbd = 0;
+#pragma unroll 1
+        for (int ch = 0; ch < 4; ch++) {
+            zero_acc<NT>(acc);
+            gemm_stream<H, H, false>(acc, nrm, p.w_up, 4 * H, 0, ch * H, wlds, lane);
+            v4i mid[KS];
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int n0 = ch * H + 32 * nt + 8 * q + 4 * g;
+                    v4i a4 = *reinterpret_cast<const v4i *>(upA + n0);
+                    v4i b4 = *reinterpret_cast<const v4i *>(bup + n0);
+                    int o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        int a = acc[nt][4 * q + e] + ((sbu * a4[e]) >> c.sigma);
+                        int v = clip127((a >> c.shift_mlp_up) + b4[e]);
+                        o[e] = act[(uint8_t)v];
+                    }
+                    mid[nt][q] = pack4(o[0], o[1], o[2], o[3]);
+                }
+            {   // partial x.B of the down projection for this chunk (halves combined after the loop)
+                const int *b32 = reinterpret_cast<const int *>(dnB + ch * H);
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) sbd = dot4(mid[ks][q], b32[8 * ks + 2 * q + g], sbd);
+            }
+            gemm_stream<H, H, false>(accd, mid, p.w_dn, H, ch * H, 0, wlds, lane);
+        }
+        sbd += other_half(sbd);
+        add_perturb<NT>(accd, sbd, dnA, 0, c.sigma, g);
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                v4i b4 = *reinterpret_cast<const v4i *>(bdn + 32 * nt + 8 * q + 4 * g);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    accd[nt][4 * q + e] = sx8(xcur[nt][q], e) + (accd[nt][4 * q + e] >> c.shift_mlp_down) + b4[e];
+            }
+        v4i xnew[KS];
+        adaptive_norm<NT>(accd, xnew);
+        if (valid)
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) store_op(p.x + row, ks, g, xnew[ks]);
+    }
+}
+
+// ============================================================================ QKV
+template <int H>
+struct QkvLds {
+    static constexpr int I32 = 5 * H;   // lnw lnb qA kA vA
+    static constexpr int I8 = 3 * H;    // qB kB vB
+    static constexpr int PER_WAVE = I32 * 4 + I8 + (16 - (I8 % 16)) % 16;
+    static constexpr int WBLOCK = (H < 256 ? H : 256) * (H < 256 ? H : 256);
+    static constexpr int TOTAL = WBLOCK + EGG_WAVES * PER_WAVE;
+};
+
+// apply_rope_integer (mgpu.cu:624-644) on the raw accumulators of one token
+template <int NT>
+__device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row, int head_dim, int bit, int g) {
+    const long long half = 1ll << (bit - 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int ep = 0; ep < 2; ep++) {
+                int n = 32 * nt + 8 * q + 4 * g + 2 * ep;           // even element of the pair
+                int pr = (n % head_dim) >> 1;
+                int2 cs = *reinterpret_cast<const int2 *>(rope_row + 2 * pr);
+                long long ve = acc[nt][4 * q + 2 * ep], vo = acc[nt][4 * q + 2 * ep + 1];
+                long long re = (ve * cs.x - vo * cs.y + half) >> bit;
+                long long ro = (ve * cs.y + vo * cs.x + half) >> bit;
+                acc[nt][4 * q + 2 * ep] = (int)re;
+                acc[nt][4 * q + 2 * ep + 1] = (int)ro;
+            }
+}
+
+template <int H>
+__global__ void __launch_bounds__(EGG_THREADS) k_qkv(QkvParams p) {
+    constexpr int KS = H / 32, NT = H / 32;
+    extern __shared__ __align__(16) int8_t smem[];
+    int8_t *wlds = smem;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    int8_t *tb = smem + QkvLds<H>::WBLOCK + wave * QkvLds<H>::PER_WAVE;
+    int *lnw = reinterpret_cast<int *>(tb), *lnb = lnw + H, *qA = lnb + H, *kA = qA + H, *vA = kA + H;
+    int8_t *qB = reinterpret_cast<int8_t *>(vA + H), *kB = qB + H, *vB = kB + H;
+
+    const FwdCommon &c = p.c;
+    const int T = c.T;
+    int mloc = blockIdx.x * EGG_WAVES + wave;
+    const bool valid = mloc < c.n_members;
+    if (!valid) mloc = c.n_members - 1;
+    const int member = c.pop_offset + mloc;
+    const int ns = (member & 1) ? -1 : 1;
+    const uint32_t sb_ = *c.d_step_seed + (uint32_t)(member / 2) + (uint32_t)p.seed_base;
+
+    fill_vec_i32(lnw, p.ln_w, sb_ + OFF_LN_1_A, sb_ + OFF_LN_1_B, H, c.mask, ns, c.sigma_vec, lane);
+    fill_vec_i32(lnb, p.ln_b, sb_ + OFF_LN_1_BIAS_A, sb_ + OFF_LN_1_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
+    fill_noise_i32(qA, sb_ + OFF_Q_A, H, c.mask, ns, lane);
+    fill_noise_i32(kA, sb_ + OFF_K_A, H, c.mask, ns, lane);
+    fill_noise_i32(vA, sb_ + OFF_V_A, H, c.mask, ns, lane);
+    fill_noise_i8(qB, sb_ + OFF_Q_B, H, c.mask, lane);
+    fill_noise_i8(kB, sb_ + OFF_K_B, H, c.mask, lane);
+    fill_noise_i8(vB, sb_ + OFF_V_B, H, c.mask, lane);
+    __syncthreads();
+
+    for (int pass = 0; pass < T / 32; pass++) {
+        const int t = pass * 32 + j;
+        const size_t row = ((size_t)mloc * T + t) * H;
+        v4i x[KS], nrm[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
+        standard_norm<KS>(x, nrm, lnw, lnb, H, g);
+        const int32_t *rope_row = c.rope_lut + (size_t)t * c.head_dim;
+#pragma unroll 1
+        for (int which = 0; which < 3; which++) {
+            const int8_t *W = which == 0 ? p.w_q : (which == 1 ? p.w_k : p.w_v);
+            const int8_t *Bn = which == 0 ? qB : (which == 1 ? kB : vB);
+            const int *An = which == 0 ? qA : (which == 1 ? kA : vA);
+            int8_t *dst = which == 0 ? p.q : (which == 1 ? p.k : p.v);
+            const int sb = dot_noise<KS, false>(nrm, Bn, 0, g);
+            v16i acc[NT];
+            zero_acc<NT>(acc);
+            gemm_stream<H, H, false>(acc, nrm, W, H, 0, 0, wlds, lane);
+            add_perturb<NT>(acc, sb, An, 0, c.sigma, g);
+            if (which < 2) rope_inplace<NT>(acc, rope_row, c.head_dim, c.rope_scale_bit, g);
+            v4i o[KS];
+            adaptive_norm<NT>(acc, o);
+            if (valid)
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) store_op(dst + row, ks, g, o[ks]);
+        }
+    }
+}
+
+// ============================================================================ attention core
+// One wave per (member, head).  S^T = K.Q^T per 32x32 tile (lane = query token), two passes over the
+// causal context (row max, then LUT weights), O^T = V^T.P^T with the 19-bit weights split into three
+// 7-bit planes so the weighted sum stays exact on the int8 MFMA.
+template <int HD, int CT>
+__global__ void __launch_bounds__(EGG_THREADS) k_attn(AttnParams p) {
+    constexpr int KS = HD / 32, DT = HD / 32;
+    constexpr int T = CT * 32;
+    extern __shared__ __align__(16) int8_t smem[];
+    int *lut = reinterpret_cast<int *>(smem);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    int8_t *vl = smem + 1024 + (size_t)wave * T * HD;
+
+    const FwdCommon &c = p.c;
+    const int H = c.H, NH = H / HD;
+    int unit = blockIdx.x * EGG_WAVES + wave;
+    const bool valid = unit < c.n_members * NH;
+    if (!valid) unit = c.n_members * NH - 1;
+    const int mloc = unit / NH, h = unit % NH;
+    const size_t base = (size_t)mloc * T * H + (size_t)h * HD;
+
+    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) lut[i] = c.exp_lut[i];
+    // V tile of this (member, head) -> LDS rows [ctx][HD]
+    for (int i = lane; i < T * HD / 16; i += 64) {
+        int cx = i / (HD / 16), part = i % (HD / 16);
+        *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + part * 16) =
+            *reinterpret_cast<const v4i *>(p.v + base + (size_t)cx * H + part * 16);
+    }
+    __syncthreads();
+    // V^T fragments: A-operand row i = natural head dim d = 32dt + i, stored at slot position 16g'+4q'+e'
+    v4i vt[CT][DT];
+    {
+        const int pos = ((j >> 2) & 1) * 16 + (j >> 3) * 4 + (j & 3);
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int b[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) b[e] = vl[(size_t)(32 * ct + 8 * q + 4 * g + e) * HD + 32 * dt + pos];
+                    vt[ct][dt][q] = pack4(b[0], b[1], b[2], b[3]);
+                }
+    }
+
+#pragma unroll 1
+    for (int qt = 0; qt < CT; qt++) {
+        const int t = qt * 32 + j;
+        v4i qop[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) qop[ks] = load_op(p.q + base + (size_t)t * H, ks, g);
+        // pass 1: per-head maximum score over ctx <= t (mgpu.cu:795-802)
+        int mx = INT_MIN;
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) {
+            if (ct <= qt) {
+                v16i s;
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[r] = 0;
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    v4i kf = load_op(p.k + base + (size_t)(32 * ct + j) * H, ks, g);
+                    s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    int cx = 32 * ct + ((r >> 2) << 3) + (g << 2) + (r & 3);
+                    if (cx <= t) mx = max(mx, s[r]);
+                }
+            }
+        }
+        mx = max(mx, other_half(mx));
+        const int mxs = mx >> c.shift_attn;
+        // pass 2: weights and weighted V sum (mgpu.cu:810-824)
+        v16i o[3][DT];
+#pragma unroll
+        for (int pl = 0; pl < 3; pl++) zero_acc<DT>(o[pl]);
+        int den = 0;
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) {
+            if (ct <= qt) {
+                v16i s;
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[r] = 0;
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    v4i kf = load_op(p.k + base + (size_t)(32 * ct + j) * H, ks, g);
+                    s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
+                }
+                v4i pw[3];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int w0[4], w1[4], w2[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        int r = 4 * q + e;
+                        int cx = 32 * ct + 8 * q + 4 * g + e;
+                        int idx = mxs - (s[r] >> c.shift_attn);
+                        idx = min(255, max(0, idx));
+                        int w = (cx <= t) ? lut[idx] : 0;
+                        den += w;
+                        w0[e] = w & 127; w1[e] = (w >> 7) & 127; w2[e] = w >> 14;
+                    }
+                    pw[0][q] = pack4(w0[0], w0[1], w0[2], w0[3]);
+                    pw[1][q] = pack4(w1[0], w1[1], w1[2], w1[3]);
+                    pw[2][q] = pack4(w2[0], w2[1], w2[2], w2[3]);
+                }
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int pl = 0; pl < 3; pl++)
+                        o[pl][dt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vt[ct][dt], pw[pl], o[pl][dt], 0, 0, 0);
+            }
+        }
+        den += other_half(den);
+        const double dden = (double)(den ? den : 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+            v4i outp;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int ov[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int r = 4 * q + e;
+                    long long num = (long long)o[0][dt][r] + ((long long)o[1][dt][r] << 7) + ((long long)o[2][dt][r] << 14);
+                    // exact truncating quotient: |num/den| <= 127 and a non-integer quotient is at least
+                    // 2^-27 away from an integer, far beyond double rounding
+                    int qv = (int)((double)num / dden);
+                    ov[e] = clip127(qv);
+                }
+                outp[q] = pack4(ov[0], ov[1], ov[2], ov[3]);
+            }
+            if (valid) store_op(p.ao + base + (size_t)t * H, dt, g, outp);
+        }
+    }
+}
+
+// ============================================================================ head + loss
+template <int H>
+struct HeadLds {
+    static constexpr int PER_WAVE = (2 * H + 256) * 4 + H;   // lnw lnb hA[256] + hB[H]
+    static constexpr int WBLOCK = (H < 256 ? H : 256) * 256;
+    static constexpr int TOTAL = WBLOCK + 1024 + EGG_WAVES * PER_WAVE;
+};
+
+template <int H>
+__global__ void __launch_bounds__(EGG_THREADS) k_head(HeadParams p) {
+    constexpr int KS = H / 32, NV = 256 / 32;
+    extern __shared__ __align__(16) int8_t smem[];
+    int8_t *wlds = smem;
+    int *lut = reinterpret_cast<int *>(smem + HeadLds<H>::WBLOCK);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    int8_t *tb = smem + HeadLds<H>::WBLOCK + 1024 + wave * HeadLds<H>::PER_WAVE;
+    int *lnw = reinterpret_cast<int *>(tb), *lnb = lnw + H, *hA = lnb + H;
+    int8_t *hB = reinterpret_cast<int8_t *>(hA + 256);
+
+    const FwdCommon &c = p.c;
+    const int T = c.T;
+    int mloc = blockIdx.x * EGG_WAVES + wave;
+    const bool valid = mloc < c.n_members;
+    if (!valid) mloc = c.n_members - 1;
+    const int member = c.pop_offset + mloc;
+    const int ns = (member & 1) ? -1 : 1;
+    const uint32_t pair_seed = *c.d_step_seed + (uint32_t)(member / 2);
+
+    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) lut[i] = c.exp_lut[i];
+    fill_vec_i32(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane);
+    fill_vec_i32(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
+    fill_noise_i32(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane);
+    fill_noise_i8(hB, pair_seed + OFF_EMB + H, H, c.mask, lane);
+    __syncthreads();
+
+    const int64_t spos = stream_pos_of(c, member);
+    long long wave_loss = 0;
+    for (int pass = 0; pass < T / 32; pass++) {
+        const int t = pass * 32 + j;
+        const size_t row = ((size_t)mloc * T + t) * H;
+        v4i x[KS], nf[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
+        standard_norm<KS>(x, nf, lnw, lnb, H, g);
+        const int sbh = dot_noise<KS, false>(nf, hB, 0, g);
+        v16i acc[NV];
+        zero_acc<NV>(acc);
+        gemm_stream<H, 256, false>(acc, nf, p.embedding, 256, 0, 0, wlds, lane);
+        add_perturb<NV>(acc, sbh, hA, 0, c.sigma, g);
+        // two-pass softmax statistics (mgpu.cu:969-1009)
+        int gmax = INT_MIN;
+#pragma unroll
+        for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) { acc[nt][r] >>= c.shift_logit; gmax = max(gmax, acc[nt][r]); }
+        gmax = max(gmax, other_half(gmax));
+        const int target = c.data[spos + t + 1];
+        long long sum_ex = 0; int tl = 0;
+#pragma unroll
+        for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                int idx = min(255, max(0, gmax - acc[nt][r]));
+                sum_ex += lut[idx];
+                if (col_of(nt, r, g) == target) tl = acc[nt][r];
+            }
+        sum_ex += other_half64(sum_ex);
+        tl += other_half(tl);
+        if (p.logits_tap && valid)
+#pragma unroll
+            for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    v4i o4;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o4[e] = acc[nt][4 * q + e];
+                    *reinterpret_cast<v4i *>(p.logits_tap + ((size_t)mloc * T + t) * 256 + 32 * nt + 8 * q + 4 * g) = o4;
+                }
+        // loss (mgpu.cu:1012-1024)
+        long long log_sum = 0;
+        if (sum_ex > 0) {
+            int pos = 63 - __clzll((unsigned long long)sum_ex);      // floor(log2), same as the reference's shift ladder
+            log_sum = ((long long)pos << 4) - ((long long)c.softmax_scale_bit << 4);
+        }
+        long long lt = (log_sum >> 1) + gmax - tl;
+        if (g == 0) wave_loss += lt;
+    }
+    // sum over the wave's 32 tokens (lanes of half 0), then one atomic per member
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {
+        int lo = __shfl_xor((int)(wave_loss & 0xffffffffll), off, 64);
+        int hi = __shfl_xor((int)(wave_loss >> 32), off, 64);
+        wave_loss += ((long long)hi << 32) | (unsigned int)lo;
+    }
+    if (lane == 0 && valid) atomicAdd(p.loss_acc + member, (unsigned long long)wave_loss);
+}
+
+// ============================================================================ host launchers
+template <int H>
+static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
+    dim3 grid((p.c.n_members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
+    size_t lds = MlpLds<H>::TOTAL;
+    if (first) hipLaunchKernelGGL((k_mlp<H, true>), grid, block, lds, s, p);
+    else hipLaunchKernelGGL((k_mlp<H, false>), grid, block, lds, s, p);
+    return hipGetLastError();
+}
+hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s) {
+    switch (p.c.H) {
+        case 64: return launch_mlp_h<64>(p, first, s);
+        case 128: return launch_mlp_h<128>(p, first, s);
+        case 256: return launch_mlp_h<256>(p, first, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <int H>
+static hipError_t launch_qkv_h(const QkvParams &p, hipStream_t s) {
+    dim3 grid((p.c.n_members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
+    size_t lds = QkvLds<H>::TOTAL;
+    hipLaunchKernelGGL((k_qkv<H>), grid, block, lds, s, p);
+    return hipGetLastError();
+}
+hipError_t egg_launch_qkv(const QkvParams &p, hipStream_t s) {
+    switch (p.c.H) {
+        case 64: return launch_qkv_h<64>(p, s);
+        case 128: return launch_qkv_h<128>(p, s);
+        case 256: return launch_qkv_h<256>(p, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <int HD, int CT>
+static hipError_t launch_attn_t(const AttnParams &p, hipStream_t s) {
+    int units = p.c.n_members * (p.c.H / HD);
+    dim3 grid((units + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
+    size_t lds = 1024 + (size_t)EGG_WAVES * CT * 32 * HD;
+    hipLaunchKernelGGL((k_attn<HD, CT>), grid, block, lds, s, p);
+    return hipGetLastError();
+}
+template <int HD>
+static hipError_t launch_attn_hd(const AttnParams &p, hipStream_t s) {
+    switch (p.c.T / 32) {
+        case 1: return launch_attn_t<HD, 1>(p, s);
+        case 2: return launch_attn_t<HD, 2>(p, s);
+        case 4: return launch_attn_t<HD, 4>(p, s);
+        case 8: return launch_attn_t<HD, 8>(p, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+hipError_t egg_launch_attn(const AttnParams &p, hipStream_t s) {
+    switch (p.c.head_dim) {
+        case 32: return launch_attn_hd<32>(p, s);
+        case 64: return launch_attn_hd<64>(p, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <int H>
+static hipError_t launch_head_h(const HeadParams &p, hipStream_t s) {
+    dim3 grid((p.c.n_members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
+    size_t lds = HeadLds<H>::TOTAL;
+    hipLaunchKernelGGL((k_head<H>), grid, block, lds, s, p);
+    return hipGetLastError();
+}
+hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
+    switch (p.c.H) {
+        case 64: return launch_head_h<64>(p, s);
+        case 128: return launch_head_h<128>(p, s);
+        case 256: return launch_head_h<256>(p, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// ---------------------------------------------------------------- one-time LDS opt-in (not a stream operation,
+// so it is done at context creation and never while a stream is capturing)
+#define SET_LDS(kern, bytes) do { hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)); if (e_ != hipSuccess) return e_; } while (0)
+template <int H>
+static hipError_t prepare_h() {
+    SET_LDS((k_mlp<H, true>), MlpLds<H>::TOTAL);
+    SET_LDS((k_mlp<H, false>), MlpLds<H>::TOTAL);
+    SET_LDS((k_qkv<H>), QkvLds<H>::TOTAL);
+    SET_LDS((k_head<H>), HeadLds<H>::TOTAL);
+    return hipSuccess;
+}
+template <int HD, int CT>
+static hipError_t prepare_attn() {
+    SET_LDS((k_attn<HD, CT>), 1024 + (size_t)EGG_WAVES * CT * 32 * HD);
+    return hipSuccess;
+}
+template <int HD>
+static hipError_t prepare_attn_hd(int ct) {
+    switch (ct) {
+        case 1: return prepare_attn<HD, 1>();
+        case 2: return prepare_attn<HD, 2>();
+        case 4: return prepare_attn<HD, 4>();
+        case 8: return prepare_attn<HD, 8>();
+        default: return hipErrorInvalidValue;
+    }
+}
+hipError_t egg_prepare_forward(int H, int head_dim, int T) {
+    hipError_t e;
+    switch (H) {
+        case 64: e = prepare_h<64>(); break;
+        case 128: e = prepare_h<128>(); break;
+        case 256: e = prepare_h<256>(); break;
+        default: return hipErrorInvalidValue;
+    }
+    if (e != hipSuccess) return e;
+    return head_dim == 32 ? prepare_attn_hd<32>(T / 32) : (head_dim == 64 ? prepare_attn_hd<64>(T / 32) : hipErrorInvalidValue);
+}

@@ -1,0 +1,41 @@
+// egg_launch.h -- host-side launchers of the kernels, one per .hip translation unit.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <limits.h>
+#include "egg_params.h"
+
+hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s);
+hipError_t egg_launch_qkv(const QkvParams &p, hipStream_t s);
+hipError_t egg_launch_attn(const AttnParams &p, hipStream_t s);
+hipError_t egg_launch_head(const HeadParams &p, hipStream_t s);
+hipError_t egg_prepare_forward(int H, int head_dim, int T);
+
+struct PlinParams {
+    const int8_t *X;        // [members*T][K] natural order
+    const int8_t *W;        // blocked [K/4][N][4]
+    int members, T, K, N;
+    uint32_t seed; int off_a, off_b, shift, sigma, mask;
+    int32_t *Y32; int8_t *Y8;
+};
+hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s);
+
+// small utility kernels (egg_update.hip)
+hipError_t egg_launch_noise_fill(uint32_t seed, uint32_t first, int n, int mask, int8_t *out, hipStream_t s);
+hipError_t egg_launch_zero_u64(unsigned long long *p, int64_t n, hipStream_t s);
+hipError_t egg_launch_loss_finalize(const unsigned long long *acc, int32_t *loss, int first, int count, hipStream_t s);
+hipError_t egg_launch_fitness(const int32_t *loss, int32_t *fit, int pairs, hipStream_t s);
+
+struct UpdParams {
+    int8_t *W; float *state;           // tensor weights and optimizer state ({m,v,acc} per element)
+    int rows, cols;                    // matrix: rows = input dim (k), cols = output dim (n); vector: cols = len
+    int off_a, off_b, seed_base;
+    const int32_t *fit; int pairs;
+    const uint32_t *d_seed; const float *d_lr; float lr_scale;
+    int mask; float beta1, beta2, eps, wd;
+    int8_t *panel_a, *panel_b; int pairs_pad;   // workspace: [cols][pairs_pad], [rows][pairs_pad]
+    unsigned long long *counter;
+    int32_t *votes_out;                // optional: only compute votes (blocked order), no update
+};
+hipError_t egg_launch_update_matrix(const UpdParams &p, hipStream_t s);
+hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s);

@@ -1,0 +1,81 @@
+// egg_linear.hip -- one perturbed int8 linear layer over a [members*T][K] activation matrix.
+// Reference: compute_linear_projection, full_cuda_train_transformer_adam_mgpu.cu:553-572, applied to
+// every (member, token) row: acc = x.W + (((x.B) * A[n]) * ns >> sigma), out = acc >> shift.
+// Same tile scheme as the forward kernels (wave = 32 tokens of one member, W blocks through LDS,
+// v_mfma_i32_32x32x32_i8), with the row-major input read in natural k order.
+#include "egg_device.h"
+#include "egg_launch.h"
+
+template <int K, int N>
+struct PlinLds {
+    static constexpr int KB = K < 256 ? K : 256, NB = N < 256 ? N : 256;
+    static constexpr int PER_WAVE = N * 4 + K;
+    static constexpr int TOTAL = KB * NB + EGG_WAVES * PER_WAVE;
+};
+
+template <int K, int N>
+__global__ void __launch_bounds__(EGG_THREADS) k_plinear(PlinParams p) {
+    constexpr int KS = K / 32, NB = PlinLds<K, N>::NB, NTB = NB / 32;
+    extern __shared__ __align__(16) int8_t smem[];
+    int8_t *wlds = smem;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    int8_t *tb = smem + PlinLds<K, N>::KB * NB + wave * PlinLds<K, N>::PER_WAVE;
+    int *At = reinterpret_cast<int *>(tb);
+    int8_t *Bt = reinterpret_cast<int8_t *>(At + N);
+
+    int member = blockIdx.x * EGG_WAVES + wave;
+    const bool valid = member < p.members;
+    if (!valid) member = p.members - 1;
+    const int ns = (member & 1) ? -1 : 1;
+    const uint32_t ps = p.seed + (uint32_t)(member / 2);
+    fill_noise_i32(At, ps + p.off_a, N, p.mask, ns, lane);
+    fill_noise_i8(Bt, ps + p.off_b, K, p.mask, lane);
+    __syncthreads();
+
+    for (int pass = 0; pass < p.T / 32; pass++) {
+        const size_t row = (size_t)member * p.T + pass * 32 + j;
+        v4i xop[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) xop[ks] = load_op(p.X + row * K, ks, g);
+        const int sb = dot_noise<KS, true>(xop, Bt, 0, g);
+#pragma unroll 1
+        for (int nb = 0; nb < N / NB; nb++) {
+            v16i acc[NTB];
+            zero_acc<NTB>(acc);
+            gemm_stream<K, NB, true>(acc, xop, p.W, N, 0, nb * NB, wlds, lane);
+#pragma unroll
+            for (int nt = 0; nt < NTB; nt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int n0 = nb * NB + 32 * nt + 8 * q + 4 * g;
+                    v4i a4 = *reinterpret_cast<const v4i *>(At + n0);
+                    v4i o4;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o4[e] = (acc[nt][4 * q + e] + ((sb * a4[e]) >> p.sigma)) >> p.shift;
+                    if (valid) {
+                        if (p.Y32) *reinterpret_cast<v4i *>(p.Y32 + row * N + n0) = o4;
+                        if (p.Y8) *reinterpret_cast<int *>(p.Y8 + row * N + n0) =
+                            pack4(clip127(o4[0]), clip127(o4[1]), clip127(o4[2]), clip127(o4[3]));
+                    }
+                }
+        }
+    }
+}
+
+template <int K, int N>
+static hipError_t launch_kn(const PlinParams &p, hipStream_t s) {
+    dim3 grid((p.members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
+    size_t lds = PlinLds<K, N>::TOTAL;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_plinear<K, N>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((k_plinear<K, N>), grid, block, lds, s, p);
+    return hipGetLastError();
+}
+
+hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s) {
+#define CASE(K_, N_) if (p.K == K_ && p.N == N_) return launch_kn<K_, N_>(p, s);
+    CASE(64, 64) CASE(64, 256) CASE(256, 64) CASE(128, 128) CASE(128, 512) CASE(512, 128)
+    CASE(256, 256) CASE(256, 1024) CASE(1024, 256) CASE(512, 512)
+#undef CASE
+    return hipErrorInvalidValue;
+}

@@ -1,0 +1,158 @@
+/*
+ * egg_hip.h -- C ABI of libegg_hip.so: the EGGROLL population-evaluation hot path
+ * (Int8NativeFormer forward + fitness + ES update) on one AMD MI355X (gfx950).
+ *
+ * The reference (d0rc/egg.c) exposes no FFI: each trainer is one translation unit
+ * whose main() launches kernels directly.  The functions below are that de-facto
+ * operator surface, one export per thing the reference's host loop does; the
+ * reference site each one replaces is cited.  Shorthand for reference files:
+ *   mgpu.cu = full_cuda_train_transformer_adam_mgpu.cu,  de/ = d-eggs/
+ *
+ * Conventions: every call returns 0 on success or a negative EGG_E_* code and never
+ * exits the process (the reference's CHECK_CUDA does, mgpu.cu:272).  A context owns
+ * one device, one stream, the model, the optimizer state and the activation
+ * workspace.  Calls on one context are not thread-safe; distinct contexts are
+ * independent.  Pointers named d_* are device pointers owned by the caller;
+ * everything is enqueued on the context's stream and no call synchronises unless
+ * it says so.
+ */
+#ifndef EGG_HIP_H
+#define EGG_HIP_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EGG_OK             0
+#define EGG_E_INVALID     -1   /* bad argument / unsupported configuration          */
+#define EGG_E_HIP         -2   /* a HIP runtime call failed (see egg_last_error)     */
+#define EGG_E_NOMEM       -3
+#define EGG_E_STATE       -4   /* call order violated (e.g. launch before capture)   */
+
+typedef struct egg_ctx egg_ctx;
+
+/* Runtime form of the reference's -D macros (mgpu.cu:34-270). */
+typedef struct egg_config {
+    int hidden;              /* HIDDEN_DIM: 64, 128, 256 or 512                       */
+    int head_dim;            /* HEAD_DIM: 32 or 64, divides hidden                    */
+    int n_layers;            /* N_LAYERS                                              */
+    int seq_len;             /* SEQ_LEN: multiple of 32                               */
+    int vocab;               /* VOCAB_SIZE: 256 (byte level)                          */
+    int population;          /* POPULATION_SIZE: even                                 */
+    int fixed_point;         /* 4                                                     */
+    int sigma_shift;         /* 3                                                     */
+    int sigma_shift_vector;  /* 4                                                     */
+    int shift_attn, shift_out, shift_logit, shift_mlp_up, shift_mlp_down;  /* 8 9 8 8 10 */
+    int softmax_scale_bit;   /* 18                                                    */
+    int rope_scale_bit;      /* 20                                                    */
+    int noise_mask;          /* DEVICE_MASK 15                                        */
+    int host_mask;           /* HOST_MASK 15                                          */
+    double softmax_exp_scale;/* 6.0                                                   */
+    float adam_beta1, adam_beta2, adam_eps, adam_weight_decay;   /* .9 .95 1e-8 .01  */
+    float muon_momentum, muon_lr_scale;                          /* .85 1.0          */
+    int use_muon;            /* USE_MUON: 2-D hidden matrices use Muon instead of AdamW */
+    int chunk_members;       /* members evaluated per forward pass over the layers; 0 = auto */
+} egg_config;
+
+void egg_default_config(egg_config *cfg);
+
+/* init_tables + cudaMemcpyToSymbol + per-GPU allocation (mgpu.cu:394-426, :1442-1489) */
+int  egg_ctx_create(const egg_config *cfg, egg_ctx **out);
+void egg_ctx_destroy(egg_ctx *ctx);
+const char *egg_last_error(const egg_ctx *ctx);
+/* run on a caller-provided hipStream_t instead of the context's own (d-eggs update_stream, de/src/worker.cu:352-357) */
+int  egg_ctx_set_stream(egg_ctx *ctx, void *hip_stream);
+int  egg_sync(egg_ctx *ctx);                       /* cudaStreamSynchronize, mgpu.cu:1552 */
+
+/* model blob == the reference's TransformerModel (mgpu.cu:284-318) with runtime sizes; every
+ * matrix in the blocked [K/4][N][4] layout of repack_matrix (mgpu.cu:443-459) */
+int64_t egg_model_bytes(const egg_ctx *ctx);
+int  egg_model_init(egg_ctx *ctx, uint32_t seed);                          /* init_model, mgpu.cu:461-519 */
+int  egg_model_upload(egg_ctx *ctx, const void *host_model, size_t bytes); /* load_model + H2D, mgpu.cu:1373,:1461 */
+int  egg_model_download(egg_ctx *ctx, void *host_model, size_t bytes);     /* D2H before save, mgpu.cu:1734 */
+/* optimizer state == the reference's AdamModel: one {m,v,acc} float triple per model byte (mgpu.cu:321-370) */
+int  egg_opt_state_upload(egg_ctx *ctx, const void *host_state, size_t bytes);
+int  egg_opt_state_download(egg_ctx *ctx, void *host_state, size_t bytes);
+int  egg_opt_state_reset(egg_ctx *ctx);                                    /* calloc'd AdamModel, mgpu.cu:1367 */
+/* lookup tables as uploaded to the device: exp[256], act[256], rope[seq_len*head_dim] (mgpu.cu:394-426) */
+int  egg_tables_download(egg_ctx *ctx, int32_t *exp_lut, int8_t *act_lut, int32_t *rope_lut);
+
+/* noise_from_hash(seed, first_idx + i) for i < n, written to d_out (mgpu.cu:528-538) */
+int  egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first_idx, int n, int8_t *d_out);
+
+/* one perturbed linear layer over a [members*T][K] int8 activation matrix (compute_linear_projection,
+ * mgpu.cu:553-572): row r belongs to member r/T, pair = member/2, ns = +1 (even) / -1 (odd);
+ *   acc[n] = sum_k X[r][k] W[k][n] + (((sum_k X[r][k] B[k]) * A[n]) * ns >> (fixed_point+sigma_shift))
+ *   A[n] = noise(seed + pair + off_a, n), B[k] = noise(seed + pair + off_b, k)
+ * d_Y32 receives acc >> shift as int32 [rows][N] (may be NULL); d_Y8 receives clip(acc >> shift) as int8
+ * [rows][N] (may be NULL).  K, N multiples of 64; T multiple of 32. */
+int  egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocked,
+                          int members, int T, int K, int N, uint32_t seed, int off_a, int off_b,
+                          int shift, int32_t *d_Y32, int8_t *d_Y8);
+
+/* train_sequence_kernel<<<batch,...>>> (mgpu.cu:847-1029, launch :1531): evaluates members
+ * [pop_offset, pop_offset+pop_count) on tokens d_data[stream_pos + t], writes d_loss[member] (int32).
+ * pop_offset and pop_count must be even. */
+int  egg_population_forward(egg_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx,
+                            uint32_t step_seed, int pop_offset, int pop_count, int32_t *d_loss);
+/* same, with the step seed and start index read from device memory when the launch executes
+ * (graph-capturable; mirrors de/include/optimizer/adam.cuh:38-39 passing scalars by device pointer) */
+int  egg_population_forward_dev(egg_ctx *ctx, const uint8_t *d_data, int64_t data_len,
+                                const int64_t *d_start_idx, const uint32_t *d_step_seed,
+                                int pop_offset, int pop_count, int32_t *d_loss);
+
+/* compute_fitness_host / compute_fitness_kernel (mgpu.cu:1305-1311, :1031-1036) */
+int  egg_fitness(egg_ctx *ctx, const int32_t *d_loss, int32_t *d_fit, int pairs);
+
+/* every LAUNCH_ADAM_MATRIX / LAUNCH_ADAM_VECTOR of one step (mgpu.cu:1577-1643); seed and learning
+ * rate by device pointer (de/include/optimizer/adam.cuh:38-39); resets then accumulates the update
+ * counter (mgpu.cu:1574, :1107-1110) */
+int  egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr);
+/* one tensor of the table returned by egg_tensor_info (test hook for update_matrix_adam_kernel,
+ * update_vector_adam_kernel mgpu.cu:1067-1152 and the Muon chain mgpu.cu:1587-1595) */
+int  egg_update_tensor(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr);
+/* int32 votes of one matrix tensor in blocked element order (mgpu.cu:1092-1098), test hook */
+int  egg_matrix_votes(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const uint32_t *d_seed, int32_t *d_votes);
+
+typedef struct egg_tensor_info {
+    char    name[32];
+    int     is_matrix, rows, cols;   /* rows = input dim, cols = output dim (vectors: rows = 1) */
+    int64_t offset;                  /* byte offset in the model blob                           */
+    int     off_a, off_b, seed_base;
+    float   lr_scale;
+    int     muon;
+} egg_tensor_info;
+int  egg_tensor_count(const egg_ctx *ctx);
+int  egg_tensor_info_get(const egg_ctx *ctx, int tensor_id, egg_tensor_info *out);
+
+/* d_total_updates read-back (mgpu.cu:1685); synchronises the stream */
+int  egg_last_update_count(egg_ctx *ctx, uint64_t *out);
+
+/* whole ES step = forward of the full population + fitness + update, enqueued on the stream:
+ * the reference's loop body mgpu.cu:1506-1678 without the host fitness hop */
+int  egg_step(egg_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx,
+              uint32_t step_seed, float lr);
+/* the same step captured once as a hipGraph and replayed (cudaStreamBeginCapture ... cudaGraphLaunch,
+ * de/src/worker.cu:435-533); seed, lr and start index live in device scalars written before each launch */
+int  egg_step_capture(egg_ctx *ctx, const uint8_t *d_data, int64_t data_len);
+int  egg_step_launch(egg_ctx *ctx, int64_t start_idx, uint32_t step_seed, float lr);
+/* losses / fitness of the last egg_step* call, copied to host (synchronises) */
+int  egg_step_losses(egg_ctx *ctx, int32_t *host_loss, int32_t *host_fit);
+
+/* get_learning_rate (mgpu.cu:217-227) and the d-eggs seed chain seed' = hash_rng(seed, step) (de/src/worker.cu:542) */
+float    egg_learning_rate(long step);
+uint32_t egg_next_seed(uint32_t seed, uint64_t step);
+
+/* debug taps (test hook, no reference counterpart beyond EGG_TRACE_STAT, mgpu.cu:723): when enabled, a
+ * forward over at most 64 members keeps every stage's activations; egg_tap_download copies one member's
+ * "x_init", "q.L", "k.L", "v.L", "ao.L", "x_attn.L", "x_mlp.L" (L = layer) or "logits" to the host. */
+int  egg_ctx_enable_taps(egg_ctx *ctx, int enable);
+int  egg_tap_download(egg_ctx *ctx, const char *name, int member, void *host_out /* int8 [T][H] natural order; "logits": int32 [T][256] */);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,274 @@
+"""GPU parity tests: every call goes through the C ABI of libegg_hip.so and is compared bit-for-bit with the
+CPU oracle on the same seeded inputs."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SMALL = dict(hidden=64, head_dim=32, n_layers=2, seq_len=32, population=8)
+
+
+def _t(dev, arr):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+
+
+def _mapping_hint(got, exp):
+    """When a row of `got` is a column permutation of `exp`, say which one (layout debugging aid)."""
+    hints = []
+    for r in range(min(2, got.shape[0])):
+        e, g = exp[r], got[r]
+        if len(set(e.tolist())) < len(e) * 0.9:
+            continue
+        pos = {int(v): i for i, v in enumerate(g.tolist())}
+        m = [pos.get(int(v), -1) for v in e.tolist()]
+        hints.append(f"row {r}: expected col i found at gpu col {m[:64]}")
+    return "\n".join(hints)
+
+
+def test_tables_and_model_init(pkg, orc, dev):
+    for kw in (SMALL, dict(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=4)):
+        ctx = pkg.Context(pkg.default_config(**kw))
+        ocfg = orc.config(**kw)
+        ex, act, rope = ctx.tables()
+        oex, oact, orope = orc.tables(ocfg)
+        assert np.array_equal(ex, oex) and np.array_equal(act, oact) and np.array_equal(rope, orope)
+        ctx.model_init(42)
+        assert np.array_equal(ctx.model_download(), orc.init_model(ocfg, 42))
+        names = [t["name"] for t in ctx.tensors()]
+        assert names == [t["name"] for t in orc.tensor_table(ocfg)]
+        for a, b in zip(ctx.tensors(), orc.tensor_table(ocfg)):
+            for k in ("is_matrix", "rows", "cols", "offset", "off_a", "off_b", "seed_base", "muon"):
+                assert a[k] == b[k], (a, b)
+        ctx.close()
+
+
+def test_noise_fill(pkg, orc, dev):
+    import torch
+    ctx = pkg.Context(pkg.default_config(**SMALL))
+    for seed, first, n in ((42, 0, 1000), (0xFFFFFFFF, 7, 513), (123456789, 4000000000, 64)):
+        out = torch.zeros(n, dtype=torch.int8, device=dev)
+        ctx.noise_fill(seed, first, n, out.data_ptr())
+        ctx.sync()
+        assert np.array_equal(out.cpu().numpy(), orc.noise_vec(seed, n, 15, first)), (seed, first)
+    ctx.close()
+
+
+@pytest.mark.parametrize("K,N,members,T", [(64, 64, 4, 32), (256, 256, 6, 64), (512, 512, 8, 32), (256, 1024, 3, 32),
+                                           (1024, 256, 2, 32)])
+def test_perturbed_linear(pkg, orc, dev, K, N, members, T):
+    import torch
+    rng = np.random.default_rng(K * 7 + N)
+    ctx = pkg.Context(pkg.default_config(**SMALL))
+    ocfg = orc.config(**SMALL)
+    X = rng.integers(-127, 128, size=(members * T, K), dtype=np.int8)
+    W = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    Wb = np.zeros(K * N, np.int8)
+    orc.lib().orc_repack(Wb.ctypes.data_as(C.c_void_p), W.ctypes.data_as(C.c_void_p), K, N)
+    for shift in (0, 8):
+        ref = orc.perturbed_linear(ocfg, X, Wb, T, K, N, 3, 200, 201, shift)
+        dX, dW = _t(dev, X), _t(dev, Wb)
+        y32 = torch.zeros((members * T, N), dtype=torch.int32, device=dev)
+        y8 = torch.zeros((members * T, N), dtype=torch.int8, device=dev)
+        ctx.perturbed_linear(dX.data_ptr(), dW.data_ptr(), members, T, K, N, 3, 200, 201, shift, y32.data_ptr(), y8.data_ptr())
+        ctx.sync()
+        got = y32.cpu().numpy()
+        if not np.array_equal(got, ref):
+            bad = np.argwhere(got != ref)
+            plain = (X.astype(np.int64) @ W.astype(np.int64))
+            raise AssertionError(
+                f"perturbed linear K={K} N={N} shift={shift}: {len(bad)} of {ref.size} differ; first {bad[:5].tolist()}\n"
+                f"gpu[0,:16]={got[0, :16].tolist()}\nref[0,:16]={ref[0, :16].tolist()}\nplain xW>>s[0,:16]={(plain[0, :16] >> shift).tolist()}\n"
+                + _mapping_hint(got, ref))
+        assert np.array_equal(y8.cpu().numpy(), np.clip(ref, -127, 127).astype(np.int8))
+    ctx.close()
+
+
+STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao", "x_attn", "x_mlp")]
+
+
+@pytest.mark.parametrize("kw", [SMALL,
+                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=64, population=6),
+                                dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4)],
+                         ids=["h64", "h128", "h256"])
+def test_forward_stages_and_loss(pkg, orc, dev, kw):
+    """Every stage tap of every member against the oracle's trace, then the per-member losses."""
+    data = orc.zipf_bytes(1 << 15)
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    # make biases / gains non-trivial so every term of the arithmetic is exercised
+    rng = np.random.default_rng(5)
+    for t in orc.tensor_table(ocfg):
+        if not t["is_matrix"]:
+            sl = slice(t["offset"], t["offset"] + t["cols"])
+            model[sl] = rng.integers(-20, 21, t["cols"]).astype(np.int8) + (16 if t["name"].startswith("ln_") and "bias" not in t["name"] else 0)
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_upload(model)
+    ctx.enable_taps(True)
+    import torch
+    d_data = _t(dev, data)
+    P = kw["population"]
+    d_loss = torch.zeros(P, dtype=torch.int32, device=dev)
+    seed, start = 987654321, 3 * kw["seq_len"]
+    ctx.population_forward(d_data.data_ptr(), len(data), start, seed, 0, P, d_loss.data_ptr())
+    ctx.sync()
+    problems = []
+    for m in range(P):
+        ref_loss, tr = orc.forward_member(ocfg, model, data, start, seed, m, trace=True)
+        stages = ["x_init"] + [f"{n}.{l}" for l in range(kw["n_layers"]) for n in ("q", "k", "v", "ao", "x_attn", "x_mlp")]
+        for st in stages:
+            got = ctx.tap(st, m)
+            if "." in st:
+                base, l = st.split(".")
+                exp = tr[base][int(l)]
+            else:
+                exp = tr[st]
+            if not np.array_equal(got, exp):
+                bad = np.argwhere(got != exp)
+                problems.append(f"member {m} stage {st}: {len(bad)}/{exp.size} differ, first at {bad[0].tolist()} "
+                                f"gpu {got[tuple(bad[0])]} ref {exp[tuple(bad[0])]}; gpu row {got[bad[0][0], :12].tolist()} ref row {exp[bad[0][0], :12].tolist()}")
+                break   # later stages of this member inherit the error
+        else:
+            got = ctx.tap("logits", m)
+            if not np.array_equal(got, tr["logits"]):
+                bad = np.argwhere(got != tr["logits"])
+                problems.append(f"member {m} logits: {len(bad)} differ, first {bad[0].tolist()} gpu {got[tuple(bad[0])]} ref {tr['logits'][tuple(bad[0])]}")
+            elif int(d_loss[m].item()) != ref_loss:
+                problems.append(f"member {m} loss gpu {int(d_loss[m].item())} ref {ref_loss}")
+    ctx.close()
+    assert not problems, "\n".join(problems[:12])
+
+
+def test_forward_chunked_and_offsets(pkg, orc, dev):
+    """Chunked evaluation (chunk smaller than the population, odd tail) and a sub-range give the same losses."""
+    import torch
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=22)
+    data = orc.zipf_bytes(1 << 14)
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 7)
+    ref = orc.population_forward(ocfg, model, data, 64, 555)
+    ctx = pkg.Context(pkg.default_config(chunk_members=6, **kw))
+    ctx.model_upload(model)
+    d_data = _t(dev, data)
+    d_loss = torch.full((22,), -1, dtype=torch.int32, device=dev)
+    ctx.population_forward(d_data.data_ptr(), len(data), 64, 555, 0, 22, d_loss.data_ptr())
+    ctx.sync()
+    assert np.array_equal(d_loss.cpu().numpy(), ref)
+    d_loss.fill_(-1)
+    ctx.population_forward(d_data.data_ptr(), len(data), 64, 555, 4, 10, d_loss.data_ptr())
+    ctx.sync()
+    got = d_loss.cpu().numpy()
+    assert np.array_equal(got[4:14], ref[4:14]) and (got[:4] == -1).all() and (got[14:] == -1).all()
+    ctx.close()
+
+
+def test_fitness(pkg, orc, dev):
+    import torch
+    ctx = pkg.Context(pkg.default_config(**SMALL))
+    loss = np.array([5, 7, 7, 5, 3, 3, -2**31, 2**31 - 1, 0, -1], np.int32)
+    d_loss = _t(dev, loss)
+    d_fit = torch.zeros(5, dtype=torch.int32, device=dev)
+    ctx.fitness(d_loss.data_ptr(), d_fit.data_ptr(), 5)
+    ctx.sync()
+    assert d_fit.cpu().tolist() == [1, -1, 0, 1, -1] == orc.fitness(loss).tolist()
+    ctx.close()
+
+
+@pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=200),
+                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=66)], ids=["p200", "p66"])
+def test_votes_and_adam_update(pkg, orc, dev, kw):
+    import torch
+    ocfg = orc.config(**kw)
+    cfg = pkg.default_config(**kw)
+    ctx = pkg.Context(cfg)
+    rng = np.random.default_rng(11)
+    pairs = kw["population"] // 2
+    fit = rng.integers(-1, 2, pairs).astype(np.int32)
+    model = orc.init_model(ocfg, 42)
+    model[rng.integers(0, model.size, 50)] = 127      # saturated weights exercise the accumulator clamp
+    model[rng.integers(0, model.size, 50)] = -127
+    state = np.zeros(model.size, orc.ADAM_DTYPE)
+    ctx.model_upload(model)
+    d_fit = _t(dev, fit)
+    seed = 2024
+    d_seed = _t(dev, np.array([seed], np.uint32).view(np.int32))
+    d_lr = _t(dev, np.array([0.3], np.float32))
+    # votes of each matrix
+    for t in ctx.tensors():
+        if not t["is_matrix"]:
+            continue
+        n = t["rows"] * t["cols"]
+        d_votes = torch.zeros(n, dtype=torch.int32, device=dev)
+        ctx.matrix_votes(t["id"], d_fit.data_ptr(), d_seed.data_ptr(), d_votes.data_ptr())
+        ctx.sync()
+        ref = np.zeros(n, np.int32)
+        orc.lib().orc_matrix_votes(C.byref(ocfg), t["rows"], t["cols"], t["off_a"], t["off_b"], t["seed_base"],
+                                   fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed), ref.ctypes.data_as(C.c_void_p))
+        assert np.array_equal(d_votes.cpu().numpy(), ref), t["name"]
+    # several full updates: weights, float state and update counter bit-exact
+    for step in range(4):
+        lr = 0.3 if step < 2 else 5.0      # the large rate drives accumulators through the +-1 thresholds
+        d_lr.fill_(lr)
+        fit = rng.integers(-1, 2, pairs).astype(np.int32)
+        d_fit.copy_(_t(dev, fit))
+        s = seed + 17 * step
+        d_seed.copy_(_t(dev, np.array([s], np.uint32).view(np.int32)))
+        ctx.es_update(d_fit.data_ptr(), d_seed.data_ptr(), d_lr.data_ptr())
+        n_ref = orc.es_update_adam(ocfg, model, state, fit, s, lr)
+        got_m = ctx.model_download()
+        got_s = ctx.opt_state_download().view(orc.ADAM_DTYPE)
+        assert np.array_equal(got_m, model), f"step {step}: {np.count_nonzero(got_m != model)} weights differ"
+        for f in ("m", "v", "acc"):
+            a, b = got_s[f], state[f]
+            assert np.array_equal(a.view(np.int32), b.view(np.int32)), \
+                f"step {step} state.{f}: {np.count_nonzero(a != b)} differ, max rel {np.max(np.abs(a - b) / (np.abs(b) + 1e-30))}"
+        assert ctx.last_update_count() == n_ref
+    ctx.close()
+
+
+def test_full_step_eager_and_graph(pkg, orc, dev):
+    """Whole ES steps (forward + fitness + update): eager and hipGraph replays follow the oracle's weight trajectory."""
+    kw = dict(hidden=64, head_dim=32, n_layers=2, seq_len=32, population=16)
+    data = orc.zipf_bytes(1 << 15)
+    ocfg = orc.config(**kw)
+    d_data = _t(dev, data)
+    for mode in ("eager", "graph"):
+        model = orc.init_model(ocfg, 42)
+        state = np.zeros(model.size, orc.ADAM_DTYPE)
+        ctx = pkg.Context(pkg.default_config(**kw))
+        ctx.model_init(42)
+        if mode == "graph":
+            ctx.step_capture(d_data.data_ptr(), len(data))
+        seed = 42
+        for step in range(5):
+            lr = 2.0
+            start = step * kw["seq_len"]
+            if mode == "graph":
+                ctx.step_launch(start, seed, lr)
+            else:
+                ctx.step(d_data.data_ptr(), len(data), start, seed, lr)
+            loss, fit = ctx.step_losses()
+            ref_loss = orc.population_forward(ocfg, model, data, start, seed)
+            assert np.array_equal(loss, ref_loss), f"{mode} step {step} losses"
+            ref_fit = orc.fitness(ref_loss)
+            assert np.array_equal(fit, ref_fit)
+            n_ref = orc.es_update_adam(ocfg, model, state, ref_fit, seed, lr)
+            assert np.array_equal(ctx.model_download(), model), f"{mode} step {step} weights"
+            assert ctx.last_update_count() == n_ref
+            seed = pkg.next_seed(seed, step + 1)
+        ctx.close()
+
+
+def test_error_paths(pkg, dev):
+    with pytest.raises(pkg.EggError):
+        pkg.Context(pkg.default_config(hidden=100))
+    with pytest.raises(pkg.EggError):
+        pkg.Context(pkg.default_config(seq_len=48))
+    ctx = pkg.Context(pkg.default_config(**SMALL))
+    with pytest.raises(pkg.EggError):
+        ctx.step_launch(0, 1, 0.1)            # launch before capture
+    with pytest.raises(pkg.EggError):
+        ctx.model_upload(np.zeros(3, np.int8))
+    ctx.close()
