@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Benchmark of the EGGROLL hot path on one MI355X.
+
+A step is one full ES step of the Int8NativeFormer (N=4 layers, H=256, 4 heads, T=256) at population 40,960:
+forward of every member + fitness + vote reconstruction + AdamW, through the C ABI of libegg_hip.so, on a
+synthetic Zipf(1.1) byte stream that is resident in HBM before the timed region starts.
+Prints one JSON line (metric member-tokens/s) carrying `roofline` for the dominant kernel and `cpu_baseline`.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_OPS = 5.0e15      # MI355X dense int8 MFMA, published
+PEAK_HBM = 8.0e12
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--population", type=int, default=40960)
+    ap.add_argument("--chunk", type=int, default=0, help="members per forward chunk (0 = library default)")
+    ap.add_argument("--data-mib", type=int, default=64)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="skip the hipGraph replay leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (--gpus 1); no multi-GPU figure is produced", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    orc = entry.load_oracle()          # only for the synthetic data generator and the cpu_baseline leg
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+
+    H, L, T, HD, P = 256, 4, 256, 64, args.population
+    kw = dict(hidden=H, head_dim=HD, n_layers=L, seq_len=T, population=P)
+    cfg = pkg.default_config(chunk_members=args.chunk, **kw)
+    ctx = pkg.Context(cfg)
+    ctx.set_stream(torch.cuda.current_stream().cuda_stream)
+    ctx.model_init(42)
+    data = orc.zipf_bytes(args.data_mib << 20, seed=1234)
+    d_data = torch.from_numpy(data).to(dev)
+    n = len(data)
+
+    def run_steps(k, first_step, seed, graph):
+        for i in range(k):
+            step = first_step + i
+            lr = pkg.learning_rate(step)
+            if graph:
+                ctx.step_launch(step * T, seed, lr)
+            else:
+                ctx.step(d_data.data_ptr(), n, step * T, seed, lr)
+            seed = pkg.next_seed(seed, step + 1)
+        return seed
+
+    # ---- timed region: eager launches with a hipEvent pair around every kernel
+    seed = run_steps(args.warmup, 0, 42, False)
+    ctx.enable_timing(True)
+    ctx.timing_reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    seed = run_steps(args.steps, args.warmup, seed, False)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    timing = ctx.timing()
+    ctx.enable_timing(False)
+    ms_per_step = dt * 1e3 / args.steps
+    value = P * T * args.steps / dt
+    updates = ctx.last_update_count()
+    loss, _ = ctx.step_losses()
+    mean_loss = float(loss.astype(np.int64).sum()) / (P * T * 16.0)
+
+    # ---- dominant kernel: O-projection + MLP block (k_mlp), MFMA-bound
+    per_class = {k: {"launches": v[0], "avg_ms": (v[1] / v[0] if v[0] else None), "total_ms": v[1]} for k, v in timing.items()}
+    dom = max(("mlp", "qkv", "attn", "mlp_first", "head"), key=lambda k: timing[k][1])
+    chunk = min(P, args.chunk if args.chunk > 0 else 2048)
+    ops_per_token = {"mlp": 2 * (H * H + 2 * H * 4 * H), "mlp_first": 2 * (2 * H * 4 * H), "qkv": 2 * 3 * H * H,
+                     "head": 2 * H * 256, "attn": 2 * 2 * H * (T + 1) // 2}
+    launches, tot_ms = timing[dom]
+    tokens_per_launch = P * T * args.steps * (L if dom in ("mlp", "qkv", "attn") else 1) / max(launches, 1)
+    achieved = ops_per_token[dom] * tokens_per_launch / (tot_ms / launches * 1e-3) if launches else 0.0
+    roofline = {"kernel": "k_" + dom, "bound": "mfma", "achieved": achieved / 1e12, "peak": PEAK_INT8_OPS / 1e12,
+                "unit": "TOP/s", "frac": achieved / PEAK_INT8_OPS, "traffic": None,
+                "avg_launch_ms": tot_ms / launches if launches else None, "launches": launches}
+
+    # ---- the same steps replayed as one captured hipGraph per step
+    graph_ms = None
+    if not args.no_graph:
+        ctx.step_capture(d_data.data_ptr(), n)
+        seed = run_steps(1, args.warmup + args.steps, seed, True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(args.steps, args.warmup + args.steps + 1, seed, True)
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- perturbed-linear microbenchmark (P=8192, T=128, K=N=512), int32 output
+    mb = {}
+    try:
+        members, Tm, K, N = 8192, 128, 512, 512
+        X = torch.randint(-127, 128, (members * Tm, K), dtype=torch.int8, device=dev)
+        W = torch.randint(-127, 128, (K * N,), dtype=torch.int8, device=dev)
+        Y = torch.empty((members * Tm, N), dtype=torch.int32, device=dev)
+        Y8 = torch.empty((members * Tm, N), dtype=torch.int8, device=dev)
+        for name, y32, y8, bytes_row in (("int32_out", Y.data_ptr(), None, K + 4 * N), ("int8_out", None, Y8.data_ptr(), K + N)):
+            ctx.perturbed_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 3, 200, 201, 8, y32, y8)
+            ctx.enable_timing(True); ctx.timing_reset()
+            for _ in range(5):
+                ctx.perturbed_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 3, 200, 201, 8, y32, y8)
+            nl, ms = ctx.timing()["plinear"]
+            ctx.enable_timing(False)
+            sec = ms / nl * 1e-3
+            mb[name] = {"ms": ms / nl, "TOP/s": 2.0 * K * N * members * Tm / sec / 1e12,
+                        "frac_mfma": 2.0 * K * N * members * Tm / sec / PEAK_INT8_OPS,
+                        "GB/s": bytes_row * members * Tm / sec / 1e9, "frac_hbm": bytes_row * members * Tm / sec / PEAK_HBM}
+        del X, W, Y, Y8
+    except Exception as e:   # the microbenchmark must not take the headline down
+        mb = {"error": str(e)}
+
+    # ---- CPU baseline: the oracle's restatement of the same forward on a bounded sample of members
+    cpu = None
+    cpu_ref_path = None
+    if not args.no_cpu:
+        threads = orc.lib().orc_num_threads()
+        ocfg = orc.config(**kw)
+        model = orc.init_model(ocfg, 42)
+        sample = 8 * threads
+        t0 = time.perf_counter()
+        orc.population_forward(ocfg, model, data, 0, 42, 0, sample)
+        sec = time.perf_counter() - t0
+        cpu = {"value": sample * T / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
+               "sample": f"forward only of {sample} of {P} members (T={T}) of the same model, scalar C++/OpenMP oracle, {sec:.1f}s"}
+        # the reference's CPU program (full_trained_egg.c: GRU LM, H=512, L=4, P=128), scalar/OpenMP restatement
+        g = orc.gru_config(seq_len=1024)
+        gm = orc.gru_init_model(g, 42)
+        states = np.zeros(g.population * g.n_layers * g.hidden, np.int8)
+        npairs = min(64, 2 * threads)
+        t0 = time.perf_counter()
+        orc.gru_population(g, gm, data, 0, 42, 0, npairs, states)
+        sec = time.perf_counter() - t0
+        cpu_ref_path = {"value": 2 * npairs * g.seq_len / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
+                        "sample": f"full_trained_egg.c defaults (GRU H=512 L=4), forward of {npairs} pairs x {g.seq_len} tokens, {sec:.1f}s"}
+
+    out = {
+        "metric": "member-tokens/sec on 1 MI355X (pop 40,960) + % int8 MFMA peak",
+        "value": value, "unit": "member-tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 (int32 accumulate), f32 optimizer state", "data": "synthetic Zipf(1.1) bytes, seed 1234",
+        "config": {"workload": f"full ES step: Int8NativeFormer L={L} H={H} heads={H // HD} T={T}, population {P}, "
+                               f"forward+fitness+vote+AdamW, eager launches (chunk {chunk} members)",
+                   "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss},
+        "roofline": roofline, "kernels": per_class, "microbench_c2": mb,
+        "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
+    }
+    print(json.dumps(out))
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

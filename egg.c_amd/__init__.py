@@ -45,7 +45,9 @@ EXPORTS = [
     "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
     "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_tap_download",
+    "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
 ]
+KCLASSES = ["mlp_first", "qkv", "attn", "mlp", "head", "update_matrix", "update_vector", "plinear"]
 
 
 def build(force=True):
@@ -102,6 +104,9 @@ def lib():
         L.egg_next_seed.argtypes = [u32, C.c_uint64]
         L.egg_ctx_enable_taps.argtypes = [vp, i32]
         L.egg_tap_download.argtypes = [vp, C.c_char_p, i32, vp]
+        L.egg_ctx_enable_timing.argtypes = [vp, i32]
+        L.egg_timing_reset.argtypes = [vp]
+        L.egg_timing_get.argtypes = [vp, i32, vp, vp]
         _lib = L
     return _lib
 
@@ -254,6 +259,29 @@ class Context:
         out = np.zeros((T, 256), np.int32) if name == "logits" else np.zeros((T, H), np.int8)
         self._ck(lib().egg_tap_download(self._h, name.encode(), member, _np_ptr(out)), "egg_tap_download")
         return out
+
+
+def _enable_timing(self, on=True):
+    self._ck(lib().egg_ctx_enable_timing(self._h, 1 if on else 0), "egg_ctx_enable_timing")
+
+
+def _timing_reset(self):
+    self._ck(lib().egg_timing_reset(self._h), "egg_timing_reset")
+
+
+def _timing(self):
+    """{kernel class: (launches, total_ms)} measured with hipEvents on the context's stream"""
+    out = {}
+    for i, name in enumerate(KCLASSES):
+        n, ms = C.c_int64(), C.c_double()
+        self._ck(lib().egg_timing_get(self._h, i, C.byref(n), C.byref(ms)), "egg_timing_get")
+        out[name] = (int(n.value), float(ms.value))
+    return out
+
+
+Context.enable_timing = _enable_timing
+Context.timing_reset = _timing_reset
+Context.timing = _timing
 
 
 def learning_rate(step):

@@ -50,6 +50,11 @@ struct egg_ctx {
     int8_t *d_panel_a = nullptr, *d_panel_b = nullptr; int pairs_pad = 0;
     // taps
     bool taps = false; int8_t *d_tap = nullptr; int32_t *d_tap_logits = nullptr; int tap_members = 0;
+    // per-kernel-class event timing (egg_ctx_enable_timing)
+    bool timing = false;
+    struct Span { int cls; hipEvent_t a, b; };
+    std::vector<Span> spans; size_t spans_used = 0;
+    double t_ms[EGG_KCLASS_COUNT] = {0}; long t_n[EGG_KCLASS_COUNT] = {0};
     // graph
     hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr; bool captured = false;
     std::string err;
@@ -63,6 +68,30 @@ static int fail(egg_ctx *ctx, int code, const char *what, hipError_t e = hipSucc
     return code;
 }
 #define HIP_TRY(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return fail(ctx, EGG_E_HIP, #call, e_); } while (0)
+
+// event pair around one kernel launch of class `cls`; no-ops unless timing is enabled
+static void span_begin(egg_ctx *ctx, int cls) {
+    if (!ctx->timing) return;
+    if (ctx->spans_used == ctx->spans.size()) {
+        egg_ctx::Span sp; sp.cls = cls;
+        if (hipEventCreate(&sp.a) != hipSuccess || hipEventCreate(&sp.b) != hipSuccess) { ctx->timing = false; return; }
+        ctx->spans.push_back(sp);
+    }
+    ctx->spans[ctx->spans_used].cls = cls;
+    (void)hipEventRecord(ctx->spans[ctx->spans_used].a, ctx->stream);
+}
+static void span_end(egg_ctx *ctx) {
+    if (!ctx->timing) return;
+    (void)hipEventRecord(ctx->spans[ctx->spans_used].b, ctx->stream);
+    ctx->spans_used++;
+}
+static void spans_collect(egg_ctx *ctx) {
+    for (size_t i = 0; i < ctx->spans_used; i++) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, ctx->spans[i].a, ctx->spans[i].b) == hipSuccess) { ctx->t_ms[ctx->spans[i].cls] += ms; ctx->t_n[ctx->spans[i].cls]++; }
+    }
+    ctx->spans_used = 0;
+}
 
 extern "C" void egg_default_config(egg_config *c) {
     memset(c, 0, sizeof(*c));
@@ -117,6 +146,7 @@ static void free_all(egg_ctx *ctx) {
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
                     ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits};
     for (void *p : ptrs) if (p) (void)hipFree(p);
+    for (auto &sp : ctx->spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
     if (ctx->gexec) (void)hipGraphExecDestroy(ctx->gexec);
     if (ctx->graph) (void)hipGraphDestroy(ctx->graph);
     if (ctx->own_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -290,7 +320,9 @@ extern "C" int egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_
         return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear arguments");
     PlinParams p = {d_X, d_W, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
                     ctx->cfg.noise_mask, d_Y32, d_Y8};
+    span_begin(ctx, EGG_K_PLINEAR);
     hipError_t e = egg_launch_plinear(p, ctx->stream);
+    span_end(ctx);
     if (e == hipErrorInvalidValue) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");
     HIP_TRY(e);
     return EGG_OK;
@@ -332,7 +364,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = M + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
         p.w_dn = M + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
         p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
-        HIP_TRY(egg_launch_mlp(p, true, s));
+        span_begin(ctx, EGG_K_MLP_FIRST); HIP_TRY(egg_launch_mlp(p, true, s)); span_end(ctx);
         if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 0), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
     }
     for (int l = 0; l < c.n_layers; l++) {
@@ -342,7 +374,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
             p.ln_w = M + L.ln_1 + (int64_t)l * H; p.ln_b = M + L.ln_1_bias + (int64_t)l * H;
             p.w_q = M + L.w_q + l * hh; p.w_k = M + L.w_k + l * hh; p.w_v = M + L.w_v + l * hh;
             p.x = ctx->d_x; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v;
-            HIP_TRY(egg_launch_qkv(p, s));
+            span_begin(ctx, EGG_K_QKV); HIP_TRY(egg_launch_qkv(p, s)); span_end(ctx);
             if (taps) {
                 HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 0), ctx->d_q, act_bytes, hipMemcpyDeviceToDevice, s));
                 HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 1), ctx->d_k, act_bytes, hipMemcpyDeviceToDevice, s));
@@ -351,7 +383,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         }
         {
             AttnParams p; memset(&p, 0, sizeof(p)); p.c = f; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v; p.ao = ctx->d_ao;
-            HIP_TRY(egg_launch_attn(p, s));
+            span_begin(ctx, EGG_K_ATTN); HIP_TRY(egg_launch_attn(p, s)); span_end(ctx);
             if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 3), ctx->d_ao, act_bytes, hipMemcpyDeviceToDevice, s));
         }
         {
@@ -364,7 +396,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
             p.w_dn = M + L.w_down + l * h4; p.b_dn = M + L.mlp_bias_down + (int64_t)l * H;
             p.w_o = M + L.w_o + l * hh; p.ao = ctx->d_ao; p.x = ctx->d_x;
             p.x_mid = taps ? tap_ptr(ctx, 1 + 6 * l + 4) : nullptr;
-            HIP_TRY(egg_launch_mlp(p, false, s));
+            span_begin(ctx, EGG_K_MLP); HIP_TRY(egg_launch_mlp(p, false, s)); span_end(ctx);
             if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 5), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
         }
     }
@@ -372,7 +404,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         HeadParams p; memset(&p, 0, sizeof(p)); p.c = f;
         p.ln_w = M + L.ln_f; p.ln_b = M + L.ln_f_bias; p.embedding = M + L.embedding; p.x = ctx->d_x;
         p.loss_acc = ctx->d_loss_acc; p.logits_tap = taps ? ctx->d_tap_logits : nullptr;
-        HIP_TRY(egg_launch_head(p, s));
+        span_begin(ctx, EGG_K_HEAD); HIP_TRY(egg_launch_head(p, s)); span_end(ctx);
     }
     return EGG_OK;
 }
@@ -426,8 +458,8 @@ static UpdParams make_upd(egg_ctx *ctx, const egg_tensor_info &t, const int32_t 
 static int update_one(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
     const egg_tensor_info &t = ctx->tensors[id];
     UpdParams p = make_upd(ctx, t, d_fit, d_seed, d_lr);
-    if (t.is_matrix) HIP_TRY(egg_launch_update_matrix(p, ctx->stream));
-    else HIP_TRY(egg_launch_update_vector(p, ctx->stream));
+    if (t.is_matrix) { span_begin(ctx, EGG_K_UPDATE_MATRIX); HIP_TRY(egg_launch_update_matrix(p, ctx->stream)); span_end(ctx); }
+    else { span_begin(ctx, EGG_K_UPDATE_VECTOR); HIP_TRY(egg_launch_update_vector(p, ctx->stream)); span_end(ctx); }
     return EGG_OK;
 }
 extern "C" int egg_update_tensor(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
@@ -483,6 +515,7 @@ extern "C" int egg_step_capture(egg_ctx *ctx, const uint8_t *d_data, int64_t len
     if (!ctx) return EGG_E_INVALID;
     if (ctx->captured) return fail(ctx, EGG_E_STATE, "step already captured");
     if (ctx->taps) return fail(ctx, EGG_E_STATE, "disable taps before capturing");
+    if (ctx->timing) return fail(ctx, EGG_E_STATE, "disable timing before capturing");
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     int rc = enqueue_step(ctx, d_data, len);
@@ -565,5 +598,29 @@ extern "C" int egg_tap_download(egg_ctx *ctx, const char *name, int member, void
             int w = n & 31, q = w >> 3, g = (w >> 2) & 1, e = w & 3;
             o[(size_t)t * H + n] = buf[(size_t)t * H + (n & ~31) + 16 * g + 4 * q + e];
         }
+    return EGG_OK;
+}
+
+// ------------------------------------------------------------------ per-kernel timing
+extern "C" int egg_ctx_enable_timing(egg_ctx *ctx, int enable) {
+    if (!ctx) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    spans_collect(ctx);
+    ctx->timing = enable != 0;
+    return EGG_OK;
+}
+extern "C" int egg_timing_reset(egg_ctx *ctx) {
+    if (!ctx) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    ctx->spans_used = 0;
+    for (int i = 0; i < EGG_KCLASS_COUNT; i++) { ctx->t_ms[i] = 0; ctx->t_n[i] = 0; }
+    return EGG_OK;
+}
+extern "C" int egg_timing_get(egg_ctx *ctx, int kclass, int64_t *launches, double *total_ms) {
+    if (!ctx || kclass < 0 || kclass >= EGG_KCLASS_COUNT) return EGG_E_INVALID;
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    spans_collect(ctx);
+    if (launches) *launches = ctx->t_n[kclass];
+    if (total_ms) *total_ms = ctx->t_ms[kclass];
     return EGG_OK;
 }

@@ -152,6 +152,14 @@ uint32_t egg_next_seed(uint32_t seed, uint64_t step);
 int  egg_ctx_enable_taps(egg_ctx *ctx, int enable);
 int  egg_tap_download(egg_ctx *ctx, const char *name, int member, void *host_out /* int8 [T][H] natural order; "logits": int32 [T][256] */);
 
+/* per-kernel-class timing with hipEvent pairs recorded on the context's stream around each launch (the
+ * reference only splits Fwd/Host/Upd wall time, full_cuda_train_egg.cu:1116-1126).  Not usable while capturing. */
+enum { EGG_K_MLP_FIRST = 0, EGG_K_QKV = 1, EGG_K_ATTN = 2, EGG_K_MLP = 3, EGG_K_HEAD = 4,
+       EGG_K_UPDATE_MATRIX = 5, EGG_K_UPDATE_VECTOR = 6, EGG_K_PLINEAR = 7, EGG_KCLASS_COUNT = 8 };
+int  egg_ctx_enable_timing(egg_ctx *ctx, int enable);
+int  egg_timing_reset(egg_ctx *ctx);
+int  egg_timing_get(egg_ctx *ctx, int kclass, int64_t *launches, double *total_ms);   /* synchronises */
+
 #ifdef __cplusplus
 }
 #endif

@@ -106,6 +106,19 @@ def lib():
         L.orc_update_matrix_muon.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                                              C.c_int, C.c_void_p, C.c_int, C.c_uint32, C.c_float, C.c_void_p]
         L.orc_gru_model_bytes.restype = C.c_int64
+        L.orc_gru_model_bytes.argtypes = [C.c_void_p]
+        L.orc_gru_state_bytes.argtypes = [C.c_void_p]
+        L.orc_gru_init_model.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32]
+        L.orc_init_model.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32]
+        L.orc_model_bytes.argtypes = [C.c_void_p]
+        L.orc_tables.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.orc_tensor_table.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+        L.orc_repack.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int]
+        L.orc_unpack.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int]
+        L.orc_xorshift32.argtypes = [C.c_void_p]
+        L.orc_gen_noise_host.argtypes = [C.c_void_p, C.c_int]
+        L.orc_default_config.argtypes = [C.c_void_p]
+        L.orc_gru_default_config.argtypes = [C.c_void_p]
         L.orc_gru_state_bytes.restype = C.c_int64
         L.orc_gru_matmul_perturbed.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
                                                C.c_uint32, C.c_int, C.c_int]
@@ -251,6 +264,21 @@ def es_update_adam(cfg, model, state, fit, step_seed, lr):
     """in place on model (int8) and state (ADAM_DTYPE, one per model byte); returns update count"""
     return int(lib().orc_es_update_adam(C.byref(cfg), _p(model), _p(state), _p(fit),
                                         C.c_uint32(step_seed & 0xFFFFFFFF), C.c_float(lr)))
+
+
+def gru_init_model(gcfg, seed=42):
+    m = np.zeros(int(lib().orc_gru_model_bytes(C.byref(gcfg))), np.int8)
+    lib().orc_gru_init_model(C.byref(gcfg), _p(m), seed)
+    return m
+
+
+def gru_population(gcfg, model, data, start_idx, step_seed, pair0, npairs, states):
+    """forward +/- for pairs [pair0, pair0+npairs); returns (loss[population], fit[population/2]) (only those pairs written)"""
+    loss = np.zeros(gcfg.population, np.int32)
+    fit = np.zeros(gcfg.population // 2, np.int32)
+    lib().orc_gru_population(C.byref(gcfg), _p(model), _p(data), len(data), start_idx, C.c_uint32(step_seed & 0xFFFFFFFF),
+                             pair0, npairs, _p(states), _p(loss), _p(fit))
+    return loss, fit
 
 
 def zipf_bytes(n, seed=1234, s=1.1):
