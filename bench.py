@@ -46,7 +46,11 @@ def main():
     kw = dict(hidden=H, head_dim=HD, n_layers=L, seq_len=T, population=P)
     cfg = pkg.default_config(chunk_members=args.chunk, **kw)
     ctx = pkg.Context(cfg)
-    ctx.set_stream(torch.cuda.current_stream().cuda_stream)
+    # one non-default stream for everything (the legacy default stream cannot be captured into a hipGraph);
+    # torch.cuda.Event / synchronize below therefore see the stream the kernels run on
+    stream = torch.cuda.Stream()
+    torch.cuda.set_stream(stream)
+    ctx.set_stream(stream.cuda_stream)
     ctx.model_init(42)
     data = orc.zipf_bytes(args.data_mib << 20, seed=1234)
     d_data = torch.from_numpy(data).to(dev)
