@@ -1,0 +1,477 @@
+"""CPU tests that pin the oracle (oracle/egg_oracle.cpp, oracle/egg_gru_oracle.cpp) against things it does not
+itself define: the reference's own host header compiled into oracle/_ref, known answers, closed forms, brute
+force in numpy and algebraic special cases.  A plausible slip (dropped term, wrong sign / index / shift,
+transposed operand) fails at least one of them."""
+import ctypes as C
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLD = json.load(open(os.path.join(HERE, "golden", "reference_known_answers.json")))
+
+
+def P(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def np_noise(seed, idx, mask=15):
+    """murmur3 fmix32 of (seed + idx*golden) -> sign * ((r>>1)&mask), written independently in numpy"""
+    x = (np.uint64(seed) + np.asarray(idx, np.uint64) * np.uint64(0x9E3779B9)) & np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(16); x = (x * np.uint64(0x85EBCA6B)) & np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(13); x = (x * np.uint64(0xC2B2AE35)) & np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(16)
+    mag = ((x >> np.uint64(1)) & np.uint64(mask)).astype(np.int64)
+    return np.where(x & np.uint64(1), mag, -mag)
+
+
+# ------------------------------------------------------------------ RNG
+def test_hash_known_answers(orc):
+    L = orc.lib()
+    for s, i, v in GOLD["hash_rng"]:
+        assert L.orc_hash_rng(s, i) == int(v, 16)
+    assert [int(x) for x in orc.noise_vec(42, 16)] == GOLD["noise_from_hash_seed42_idx0_15"]
+    st = C.c_uint32(42)
+    assert [hex(L.orc_xorshift32(C.byref(st))) for _ in range(3)] == GOLD["xorshift32_from_42"]
+    st = C.c_uint32(42)
+    assert [int(L.orc_gen_noise_host(C.byref(st), 15)) for _ in range(16)] == GOLD["gen_noise_host_from_42"]
+    st = C.c_uint32(0)          # state 0 is absorbing
+    assert [int(L.orc_gen_noise_host(C.byref(st), 15)) for _ in range(4)] == [0, 0, 0, 0]
+
+
+def test_rng_against_reference_header(orc):
+    R = orc.ref()
+    if R is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    L = orc.lib()
+    rng = np.random.default_rng(0)
+    for s, i in rng.integers(0, 2**32, size=(4000, 2), dtype=np.uint64):
+        s, i = int(s), int(i)
+        assert L.orc_hash_rng(s, i) == R.ref_hash_rng(s, i)
+        assert int(L.orc_noise(s, i, 15)) == R.ref_noise_from_hash(s, i)
+    for a in (-2**31, -1000, -128, -127, -1, 0, 1, 126, 127, 128, 5000, 2**31 - 1):
+        assert int(L.orc_clip(a)) == R.ref_clip(a)
+    a, b = C.c_uint32(12345), C.c_uint32(12345)
+    for _ in range(2000):
+        assert int(L.orc_gen_noise_host(C.byref(a), 15)) == R.ref_gen_noise_host(C.byref(b))
+    assert a.value == b.value
+
+
+def test_noise_matches_independent_numpy(orc):
+    for seed in (0, 42, 0xFFFFFFFF, 123456789):
+        assert np.array_equal(orc.noise_vec(seed, 300).astype(np.int64), np_noise(seed, np.arange(300)))
+
+
+# ------------------------------------------------------------------ tables
+def test_tables_closed_forms(orc):
+    cfg = orc.config(seq_len=64)
+    ex, act, rope = orc.tables(cfg)
+    for i, v in GOLD["exp_lut_scale6"].items():
+        assert ex[int(i)] == v
+    assert (ex[75:] == 0).all() and ex[74] == 1
+    assert all(ex[i] == int(round(math.exp(-i / 6.0) * 2**18)) for i in range(75))
+    for i, v in GOLD["gelu_lut"].items():
+        assert act[np.uint8(np.int8(int(i)))] == v
+    # screenshot of the reference's debugger (SOFTMAX_EXP_SCALE=8): wt = round(exp(-i/8) 2^18)
+    ex8, _, _ = orc.tables(orc.config(softmax_exp_scale=8.0))
+    for i, v in GOLD["exp_lut_scale8_screenshot"].items():
+        assert ex8[int(i)] == v
+    r = rope.reshape(64, 32, 2).astype(np.int64)
+    assert (r[0, :, 0] == 2**20).all() and (r[0, :, 1] == 0).all()
+    assert np.abs(r[..., 0] ** 2 + r[..., 1] ** 2 - 2**40).max() <= 2**21 + 2
+    assert r[1, 0, 0] == round(math.cos(1.0) * 2**20) and r[1, 0, 1] == round(math.sin(1.0) * 2**20)
+    assert r[5, 3, 1] == round(math.sin(5 * 10000.0 ** (-6 / 64)) * 2**20)
+
+
+# ------------------------------------------------------------------ layout / init
+def test_repack_roundtrip_and_embedding_access(orc):
+    rng = np.random.default_rng(1)
+    K, N = 64, 256
+    W = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    Wb = np.zeros(K * N, np.int8); back = np.zeros((K, N), np.int8)
+    orc.lib().orc_repack(P(Wb), P(W), K, N)
+    orc.lib().orc_unpack(P(back), P(Wb), K, N)
+    assert np.array_equal(back, W)
+    # get_embedding_byte: byte ((h>>2)*V + tok)*4 + (h&3) is logical E[h][tok]
+    for h, tok in ((0, 0), (5, 17), (63, 255), (34, 128)):
+        assert Wb[((h >> 2) * N + tok) * 4 + (h & 3)] == W[h, tok]
+
+
+def test_init_model_stream_order(orc):
+    cfg = orc.config(hidden=64, head_dim=32, n_layers=2, seq_len=32, population=8)
+    m = orc.init_model(cfg, 42)
+    tt = {t["name"]: t for t in orc.tensor_table(cfg)}
+    st = C.c_uint32(42)
+    draw = lambda n: np.array([int(orc.lib().orc_gen_noise_host(C.byref(st), 15)) for _ in range(n)], np.int8)
+
+    def logical(name):
+        t = tt[name]; out = np.zeros((t["rows"], t["cols"]), np.int8)
+        orc.lib().orc_unpack(P(out), P(np.ascontiguousarray(m[t["offset"]:t["offset"] + t["rows"] * t["cols"]])), t["rows"], t["cols"])
+        return out
+    H = 64
+    assert np.array_equal(logical("embedding").ravel(), draw(H * 256))
+    assert np.array_equal(logical("w_emb_mlp_up").ravel(), draw(H * 4 * H))
+    assert np.array_equal(logical("w_emb_mlp_down").ravel(), draw(H * 4 * H))
+    for l in range(2):
+        for n in ("w_q", "w_k", "w_v", "w_o", "w_up", "w_down"):
+            assert np.array_equal(logical(f"{n}.{l}").ravel(), draw(tt[f"{n}.{l}"]["rows"] * tt[f"{n}.{l}"]["cols"])), (n, l)
+    for name, t in tt.items():
+        if not t["is_matrix"]:
+            want = 16 if name.split(".")[0] in ("ln_1", "ln_2", "ln_f", "ln_init") else 0
+            assert (m[t["offset"]:t["offset"] + t["cols"]] == want).all(), name
+    assert sum(t["rows"] * t["cols"] for t in tt.values()) == m.size
+
+
+# ------------------------------------------------------------------ perturbed linear
+def test_perturbed_linear_brute_force_and_special_cases(orc):
+    cfg = orc.config()
+    rng = np.random.default_rng(2)
+    T, K, N, members = 4, 32, 48, 6
+    X = rng.integers(-127, 128, (members * T, K), dtype=np.int8)
+    W = rng.integers(-127, 128, (K, N), dtype=np.int8)
+    Wb = np.zeros(K * N, np.int8); orc.lib().orc_repack(P(Wb), P(W), K, N)
+    seed, oa, ob, shift = 77, 200, 201, 3
+    Y = orc.perturbed_linear(cfg, X, Wb, T, K, N, seed, oa, ob, shift)
+    xw = X.astype(np.int64) @ W.astype(np.int64)
+    for r in range(members * T):
+        member = r // T; pair = member // 2; ns = 1 if member % 2 == 0 else -1
+        A = np_noise(seed + pair + oa, np.arange(N)); B = np_noise(seed + pair + ob, np.arange(K))
+        sb = int((X[r].astype(np.int64) * B).sum())
+        exp = (xw[r] + ((sb * A * ns) >> 7)) >> shift
+        assert np.array_equal(Y[r], exp), r
+    # antithetic identity: acc(+) + acc(-) = 2 xW + (q>>7) + (-q>>7)  in {2xW, 2xW-1}
+    Y0 = orc.perturbed_linear(cfg, X, Wb, T, K, N, seed, oa, ob, 0)
+    for m in range(0, members, 2):
+        # rows of member m and m+1 differ in X, so use X of member m for both via a duplicated input
+        Xd = np.concatenate([X[m * T:(m + 1) * T]] * 2)
+        Yd = orc.perturbed_linear(cfg, Xd, Wb, T, K, N, seed + m // 2, oa, ob, 0)
+        s = Yd[:T].astype(np.int64) + Yd[T:].astype(np.int64) - 2 * xw[m * T:(m + 1) * T]
+        assert set(np.unique(s)) <= {0, -1}
+    assert Y0.dtype == np.int32
+
+
+def test_gemm_without_noise_is_plain_matmul(orc):
+    """noise mask 0 makes every noise value 0: the path must reduce to an exact integer matmul"""
+    cfg = orc.config(noise_mask=0)
+    rng = np.random.default_rng(3)
+    X = rng.integers(-127, 128, (8, 64), dtype=np.int8); W = rng.integers(-127, 128, (64, 32), dtype=np.int8)
+    Wb = np.zeros(64 * 32, np.int8); orc.lib().orc_repack(P(Wb), P(W), 64, 32)
+    Y = orc.perturbed_linear(cfg, X, Wb, 4, 64, 32, 5, 1, 2, 0)
+    assert np.array_equal(Y, (X.astype(np.int64) @ W.astype(np.int64)).astype(np.int32))
+
+
+# ------------------------------------------------------------------ norms / rope / attention / loss
+def test_standard_norm(orc):
+    cfg = orc.config(); H = 64
+    rng = np.random.default_rng(4)
+    for ns in (0, 1, -1):
+        x = rng.integers(-127, 128, H, dtype=np.int8); w = rng.integers(-30, 31, H, dtype=np.int8); b = rng.integers(-9, 10, H, dtype=np.int8)
+        out = np.zeros(H, np.int8)
+        orc.lib().orc_standard_norm(C.byref(cfg), P(x), P(w), P(b), H, 1000, 100, 101, 110, 111, ns, P(out))
+        mn = max(int(np.abs(x.astype(np.int64)).sum()) // H, 1)
+        wm = w.astype(np.int64) + ((np_noise(1100, np.arange(H)) * np_noise(1101, np.arange(H)) * ns) >> 4)
+        bm = b.astype(np.int64) + ((np_noise(1110, np.arange(H)) * np_noise(1111, np.arange(H)) * ns) >> 4)
+        prod = x.astype(np.int64) * wm
+        q = np.sign(prod) * (np.abs(prod) // mn)          # C division truncates toward zero
+        assert np.array_equal(out, np.clip(q + bm, -127, 127))
+    z = np.zeros(H, np.int8); out = np.ones(H, np.int8)
+    orc.lib().orc_standard_norm(C.byref(cfg), P(z), P(w), P(z), H, 0, 0, 0, 0, 0, 0, P(out))
+    assert (out == 0).all()
+
+
+def test_adaptive_normalize(orc):
+    rng = np.random.default_rng(5)
+    for scale in (3, 300, 40000, 5000000):
+        v = rng.integers(-scale, scale + 1, 256).astype(np.int32)
+        out = np.zeros(256, np.int8)
+        orc.lib().orc_adaptive_normalize(P(v), 256, P(out))
+        mx = np.abs(v).max()
+        assert np.abs(out.astype(int)).max() == 127
+        s = np.float32(127.0) / (np.float32(mx) + np.float32(1e-9))
+        sf = v.astype(np.float32) * s
+        exp = np.clip(np.trunc(sf + np.copysign(np.float32(0.5), sf)).astype(np.int64), -127, 127)
+        ties = np.abs(np.abs(sf - np.trunc(sf)) - 0.5) < 1e-6
+        assert np.array_equal(out[~ties], exp[~ties])
+        assert np.array_equal(-out, _neg_norm(orc, v))          # sign symmetric
+    z = np.zeros(8, np.int32); out = np.ones(8, np.int8)
+    orc.lib().orc_adaptive_normalize(P(z), 8, P(out))
+    assert (out == 0).all()
+    v = np.array([127, -127, 64, 0], np.int32)                   # already spanning +-127: identity
+    orc.lib().orc_adaptive_normalize(P(v), 4, P(out))
+    assert out[:4].tolist() == [127, -127, 64, 0]
+    v = np.array([254, 1, 3, -1, -3], np.int32)                  # exact .5 ties round away from zero
+    orc.lib().orc_adaptive_normalize(P(v), 5, P(out))
+    assert out[:5].tolist() == [127, 1, 2, -1, -2]
+
+
+def _neg_norm(orc, v):
+    out = np.zeros(len(v), np.int8)
+    orc.lib().orc_adaptive_normalize(P(np.ascontiguousarray(-v)), len(v), P(out))
+    return out
+
+
+def test_rope(orc):
+    cfg = orc.config(hidden=64, head_dim=32, seq_len=64)
+    _, _, rope = orc.tables(cfg)
+    rng = np.random.default_rng(6)
+    v = rng.integers(-4000000, 4000000, 64).astype(np.int32)
+    out = np.zeros(64, np.int32)
+    orc.lib().orc_rope(C.byref(cfg), P(rope), P(v), 0, 64, P(out))
+    assert np.array_equal(out, v)                                 # t = 0 is the identity
+    t = 37
+    orc.lib().orc_rope(C.byref(cfg), P(rope), P(v), t, 64, P(out))
+    r = rope.reshape(64, 16, 2).astype(np.int64)
+    for n in range(0, 64, 2):
+        c, s = r[t, (n % 32) // 2]
+        assert out[n] == (int(v[n]) * c - int(v[n + 1]) * s + 2**19) >> 20
+        assert out[n + 1] == (int(v[n]) * s + int(v[n + 1]) * c + 2**19) >> 20
+    # a rotation preserves the norm up to rounding
+    assert abs(np.hypot(out[0], out[1]) - np.hypot(v[0], v[1])) < 2
+
+
+def test_attention_core(orc):
+    cfg = orc.config(hidden=64, head_dim=32)
+    ex, _, _ = orc.tables(cfg)
+    rng = np.random.default_rng(7)
+    H, T = 64, 9
+    q = rng.integers(-127, 128, H, dtype=np.int8); k = rng.integers(-127, 128, (T, H), dtype=np.int8); v = rng.integers(-127, 128, (T, H), dtype=np.int8)
+    ao = np.zeros(H, np.int8)
+    orc.lib().orc_attention_core(C.byref(cfg), P(ex), P(q), P(k), P(v), 0, H, P(ao))
+    assert np.array_equal(ao, v[0])                               # T = 1: output is V[0]
+    t = T - 1
+    orc.lib().orc_attention_core(C.byref(cfg), P(ex), P(q), P(k), P(v), t, H, P(ao))
+    for h in range(2):
+        sl = slice(32 * h, 32 * h + 32)
+        s = k[:, sl].astype(np.int64) @ q[sl].astype(np.int64)
+        w = ex[np.clip((s.max() >> 8) - (s >> 8), 0, 255)].astype(np.int64)
+        num = (w[:, None] * v[:, sl].astype(np.int64)).sum(0); den = max(int(w.sum()), 1)
+        exp = np.sign(num) * (np.abs(num) // den)
+        assert np.array_equal(ao[sl], np.clip(exp, -127, 127))
+    # equal scores -> integer mean of V truncated toward zero
+    kz = np.zeros((T, H), np.int8)
+    orc.lib().orc_attention_core(C.byref(cfg), P(ex), P(q), P(kz), P(v), t, H, P(ao))
+    sm = v.astype(np.int64).sum(0) * 2**18
+    assert np.array_equal(ao, np.sign(sm) * (np.abs(sm) // (T * 2**18)))
+    # a key 75*256 below the maximum has weight zero
+    q1 = np.zeros(H, np.int8); q1[0] = 127; q1[32] = 127
+    k2 = np.zeros((2, H), np.int8); k2[0, 0] = 127; k2[0, 32] = 127; k2[1, 0] = -127; k2[1, 32] = -127
+    orc.lib().orc_attention_core(C.byref(cfg), P(ex), P(q1), P(k2), P(v[:2].copy()), 1, H, P(ao))
+    assert np.array_equal(ao, v[0])
+
+
+def test_token_loss(orc):
+    cfg = orc.config()
+    ex, _, _ = orc.tables(cfg)
+    lg = np.full(256, 5, np.int32)
+    assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), 256, 3) == 64       # uniform: log2(256)*16/2
+    lg = np.full(256, -1000, np.int32); lg[7] = 300
+    assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), 256, 7) == 0        # one dominant logit, target hit
+    assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), 256, 8) == 1300     # G - logit_target
+    rng = np.random.default_rng(8)
+    lg = rng.integers(-40, 40, 256).astype(np.int32)
+    S = int(ex[np.clip(lg.max() - lg, 0, 255)].astype(np.int64).sum())
+    exp = ((((S.bit_length() - 1) << 4) - (18 << 4)) >> 1) + int(lg.max()) - int(lg[11])
+    assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), 256, 11) == exp
+
+
+def test_forward_invariants(orc):
+    """ns = 0 ignores the seed; with all noise zero the two members of a pair score the same; trace is consistent"""
+    kw = dict(hidden=64, head_dim=32, n_layers=2, seq_len=8, population=4)
+    cfg = orc.config(**kw); data = orc.zipf_bytes(4096); m = orc.init_model(cfg, 42)
+    a = orc.forward_member(cfg, m, data, 0, 111, 0, ns_override=0)
+    b = orc.forward_member(cfg, m, data, 0, 999, 0, ns_override=0)
+    assert a == b
+    cz = orc.config(noise_mask=0, **kw)
+    assert orc.forward_member(cz, m, data, 0, 5, 0) == orc.forward_member(cz, m, data, 0, 5, 1) == a
+    loss, tr = orc.forward_member(cfg, m, data, 16, 5, 3, trace=True)
+    assert loss == int(tr["loss_t"].sum())
+    assert loss != orc.forward_member(cfg, m, data, 16, 5, 2)      # antithetic members differ
+    # causal: changing a later token leaves earlier per-token losses unchanged
+    d2 = data.copy(); pos = (16 + 1 * (len(data) // 2)) % (len(data) - 8)
+    d2[pos + 6] ^= 0x55
+    _, tr2 = orc.forward_member(cfg, m, d2, 16, 5, 3, trace=True)
+    assert np.array_equal(tr["loss_t"][:5], tr2["loss_t"][:5]) and not np.array_equal(tr["loss_t"], tr2["loss_t"])
+    pl = orc.population_forward(cfg, m, data, 16, 5)
+    assert pl[3] == loss and pl[2] == orc.forward_member(cfg, m, data, 16, 5, 2)
+
+
+# ------------------------------------------------------------------ fitness / votes / AdamW
+def test_fitness_truth_table(orc):
+    assert orc.fitness(np.array([1, 2, 2, 1, 3, 3], np.int32)).tolist() == [1, -1, 0]
+
+
+def test_votes_identity(orc):
+    cfg = orc.config()
+    rng = np.random.default_rng(9)
+    rows, cols, pairs, seed, oa, ob, base = 8, 12, 40, 31337, 400, 401, 2000
+    fit = rng.integers(-1, 2, pairs).astype(np.int32)
+    votes = np.zeros(rows * cols, np.int32)
+    orc.lib().orc_matrix_votes(C.byref(cfg), rows, cols, oa, ob, base, P(fit), pairs, seed, P(votes))
+    A = np.stack([np_noise(seed + p + base + oa, np.arange(cols)) for p in range(pairs)])
+    B = np.stack([np_noise(seed + p + base + ob, np.arange(rows)) for p in range(pairs)])
+    full = B.T @ (fit[:, None] * A)                                # [k][n]
+    blocked = np.zeros(rows * cols, np.int64)
+    for k in range(rows):
+        for n in range(cols):
+            blocked[((k >> 2) * cols + n) * 4 + (k & 3)] = full[k, n]
+    assert np.array_equal(votes, blocked)
+    v2 = np.zeros_like(votes)
+    orc.lib().orc_matrix_votes(C.byref(cfg), rows, cols, oa, ob, base, P(np.ascontiguousarray(-fit)), pairs, seed, P(v2))
+    assert np.array_equal(v2, -votes)
+    orc.lib().orc_matrix_votes(C.byref(cfg), rows, cols, oa, ob, base, P(np.zeros(pairs, np.int32)), pairs, seed, P(v2))
+    assert (v2 == 0).all()
+
+
+def test_adam_apply(orc):
+    cfg = orc.config()
+    f32 = np.float32
+
+    def step(m, v, acc, w, g, lr):
+        st = np.array([(m, v, acc)], orc.ADAM_DTYPE); wv = np.array([w], np.int8); ch = C.c_int(0)
+        orc.lib().orc_adam_apply(C.byref(cfg), P(st), P(wv), C.c_float(g), C.c_float(lr), C.byref(ch))
+        return st[0], int(wv[0]), ch.value
+    st, w, ch = step(0, 0, 0, 0, 0.0, 0.3)                        # g = 0, w = 0: nothing moves
+    assert (st["m"], st["v"], st["acc"], w, ch) == (0, 0, 0, 0, 0)
+    st, w, ch = step(-1000, 1, 0.5, 127, -100.0, 1.0)             # saturated weight: acc clamps to exactly 1
+    assert w == 127 and ch == 0 and st["acc"] == f32(1.0)
+    st, w, ch = step(1000, 1, -0.5, -127, 100.0, 1.0)
+    assert w == -127 and ch == 0 and st["acc"] == f32(-1.0)
+    # generic step against numpy float32 arithmetic, one rounding per operation
+    m0, v0, a0, w0, g, lr = f32(0.3), f32(2.0), f32(0.96), 5, f32(-7.0), f32(0.3)
+    st, w, ch = step(m0, v0, a0, w0, g, lr)
+    m1 = f32(f32(0.9) * m0) + f32(f32(f32(1.0) - f32(0.9)) * g)
+    v1 = f32(f32(0.95) * v0) + f32(f32(f32(1.0) - f32(0.95)) * f32(g * g))
+    stp = f32(-lr) * f32(f32(m1 / f32(np.sqrt(v1) + f32(1e-8))) + f32(f32(0.01) * f32(w0)))
+    acc = f32(a0 + stp)
+    assert st["m"] == m1 and st["v"] == v1
+    assert (w, ch) == (6, 1) and st["acc"] == f32(acc - f32(1.0))
+    # no bias correction: first step from zero state moves acc by -lr*(0.1 g / (sqrt(0.05 g^2)+eps))
+    st, w, ch = step(0, 0, 0, 0, 4.0, 0.3)
+    assert abs(st["acc"] + 0.3 * 0.1 / math.sqrt(0.05)) < 1e-6
+    assert orc.lib().orc_learning_rate(0) == f32(0.3) and orc.lib().orc_learning_rate(300) == f32(0.15)
+    assert orc.lib().orc_learning_rate(999) == f32(0.075) and orc.lib().orc_learning_rate(1000) == f32(0.05)
+
+
+def test_vector_update_matches_definition(orc):
+    cfg = orc.config()
+    rng = np.random.default_rng(10)
+    n, pairs, seed = 16, 30, 99
+    fit = rng.integers(-1, 2, pairs).astype(np.int32)
+    V = np.zeros(n, np.int8); st = np.zeros(n, orc.ADAM_DTYPE)
+    orc.lib().orc_update_vector_adam(C.byref(cfg), P(V), P(st), n, 100, 101, 3000, P(fit), pairs, seed, C.c_float(0.3))
+    vote = sum(int(fit[p]) * np_noise(seed + p + 3000 + 100, np.arange(n)) * np_noise(seed + p + 3000 + 101, np.arange(n)) for p in range(pairs))
+    g = -vote.astype(np.float32)
+    assert np.allclose(st["m"], np.float32(1 - np.float32(0.9)) * g)
+
+
+# ------------------------------------------------------------------ Muon
+def test_newton_schulz(orc):
+    rng = np.random.default_rng(11)
+    for rows, cols in ((16, 16), (8, 24), (24, 8)):
+        X = rng.standard_normal((rows, cols))
+        X64 = X.copy(); orc.lib().orc_newton_schulz_f64(P(X64), rows, cols, 5)
+        # numpy restatement: X/||X||_F then X <- 0.5 X (3I - X^T X) on the short side
+        Y = X / np.linalg.norm(X)
+        for _ in range(5):
+            Y = 0.5 * (3 * np.eye(rows) - Y @ Y.T) @ Y if rows < cols else 0.5 * Y @ (3 * np.eye(cols) - Y.T @ Y)
+        assert np.allclose(X64, Y, rtol=1e-10, atol=1e-12)
+        X32 = X.astype(np.float32); orc.lib().orc_newton_schulz_f32(P(X32), rows, cols, 5)
+        assert np.linalg.norm(X32 - Y) / np.linalg.norm(Y) < 1e-5
+        # singular values move monotonically toward 1
+        s0 = np.linalg.svd(X / np.linalg.norm(X), compute_uv=False); s5 = np.linalg.svd(Y, compute_uv=False)
+        assert (s5 >= s0 - 1e-12).all() and (s5 <= 1 + 1e-9).all()
+    Q, _ = np.linalg.qr(rng.standard_normal((12, 12)))
+    Q *= math.sqrt(12)        # after Frobenius normalisation Q/sqrt(12)... orthogonal rows scaled: fixed direction
+    Z = (Q / math.sqrt(12)).copy()
+    orc.lib().orc_newton_schulz_f64(P(Z), 12, 12, 0)
+    assert np.allclose(Z, Q / math.sqrt(12) / np.linalg.norm(Q / math.sqrt(12)))
+
+
+# ------------------------------------------------------------------ CPU GRU path (full_trained_egg.c)
+def test_gru_noise_vector_draw_pattern(orc):
+    """4 draws discarded before each block of 16, none for padded slots (full_trained_egg.c:88-104)"""
+    L = orc.lib()
+    for count in (16, 20, 512):
+        st = C.c_uint32(777); out = np.zeros(count, np.int8)
+        L.orc_gru_noise_vector(C.byref(st), P(out), count)
+        ref = C.c_uint32(777); exp = []
+        for i in range(0, count, 16):
+            for _ in range(4):
+                L.orc_xorshift32(C.byref(ref))
+            for j in range(min(16, count - i)):
+                r = L.orc_xorshift32(C.byref(ref)); exp.append((1 if r & 1 else -1) * ((r >> 1) & 31))
+        assert out.tolist() == exp and st.value == ref.value
+
+
+def test_gru_matmul_and_loss(orc):
+    g = orc.gru_config(hidden=32, n_layers=1, seq_len=4, population=4)
+    rng = np.random.default_rng(12)
+    rows, cols = 48, 32
+    x = rng.integers(-127, 128, cols, dtype=np.int8); W = rng.integers(-127, 128, (rows, cols), dtype=np.int8)
+    out = np.zeros(rows, np.int8)
+    L = orc.lib()
+    L.orc_gru_matmul_perturbed(C.byref(g), P(x), P(W), P(out), rows, cols, 4242, -1, 8)
+    st = C.c_uint32(4242); A = np.zeros(rows, np.int8); B = np.zeros(cols, np.int8)
+    L.orc_gru_noise_vector(C.byref(st), P(A), rows); L.orc_gru_noise_vector(C.byref(st), P(B), cols)
+    xB = int((x.astype(np.int64) * B).sum())
+    acc = W.astype(np.int64) @ x.astype(np.int64) + ((xB * A.astype(np.int64) * -1) >> 8)
+    assert np.array_equal(out, np.clip(acc >> 8, -127, 127))
+    L.orc_gru_matmul_perturbed(C.byref(g), P(x), P(W), P(out), rows, cols, 4242, 0, 8)
+    assert np.array_equal(out, np.clip((W.astype(np.int64) @ x.astype(np.int64)) >> 8, -127, 127))
+    for i, v in GOLD["exp2_table"].items():
+        assert int(2.0 ** (int(i) / 16) * 16) == v
+    lg = np.zeros(256, np.int8)                                    # uniform logits: sum = 256*4096 = 2^20
+    assert L.orc_gru_compute_loss(P(lg), 256, 5, 4) == (20 << 4) - 64 - 128
+    lg = rng.integers(-127, 128, 256).astype(np.int8)
+    S = sum(int(2.0 ** ((int(v) + 128) / 16) * 16) for v in lg)
+    k = S.bit_length() - 1
+    assert L.orc_gru_compute_loss(P(lg), 256, 9, 4) == (k << 4) + ((S - (1 << k)) >> (k - 4)) - 64 - (int(lg[9]) + 128)
+
+
+def test_gru_forward_and_update(orc):
+    g = orc.gru_config(hidden=32, n_layers=2, seq_len=6, population=8)
+    L = orc.lib()
+    m = orc.gru_init_model(g, 42)
+    data = orc.zipf_bytes(2048)
+    states = np.zeros(8 * 2 * 32, np.int8)
+    loss, fit = orc.gru_population(g, m, data, 0, 1000, 0, 4, states)
+    assert np.array_equal(fit, orc.fitness(loss))
+    # noise_sign = 0 is seed independent and leaves both members of a pair equal
+    s1 = np.zeros(64, np.int8); s2 = np.zeros(64, np.int8)
+    a = L.orc_gru_forward(C.byref(g), P(m), P(data), P(data[1:].copy()), 6, None, 1, 0, P(s1))
+    b = L.orc_gru_forward(C.byref(g), P(m), P(data), P(data[1:].copy()), 6, None, 2, 0, P(s2))
+    assert a == b and np.array_equal(s1, s2) and s1.any()
+    # the recurrent state persists: a second call continues from it
+    c = L.orc_gru_forward(C.byref(g), P(m), P(data), P(data[1:].copy()), 6, None, 1, 0, P(s1))
+    assert c != a or not np.array_equal(s1, s2)
+    # update: vote = sum_p fit_p A_p[r] B_p[c], +-1 beyond the threshold
+    rows, cols = 16, 32
+    W = np.zeros((rows, cols), np.int8)
+    g2 = orc.gru_config(hidden=32, n_layers=1, seq_len=4, population=64, update_threshold=40)
+    fit = np.random.default_rng(13).integers(-1, 2, 32).astype(np.int32)
+    L.orc_gru_update_matrix(C.byref(g2), P(W), rows, cols, 555, P(fit), 64)
+    vote = np.zeros((rows, cols), np.int64)
+    for p in range(32):
+        st = C.c_uint32(555 + p); A = np.zeros(rows, np.int8); B = np.zeros(cols, np.int8)
+        L.orc_gru_noise_vector(C.byref(st), P(A), rows); L.orc_gru_noise_vector(C.byref(st), P(B), cols)
+        vote += int(fit[p]) * np.outer(A.astype(np.int64), B.astype(np.int64))
+    assert np.array_equal(W, np.where(vote > 40, 1, np.where(vote < -40, -1, 0)))
+    assert W.any()
+
+
+def test_ternary_pack_reference_vectors(orc):
+    """the only test the reference ships (d-eggs/test_ternary.cpp): its two round-trip vectors, through the
+    reference's own header when oracle/_ref is built"""
+    R = orc.ref()
+    if R is None:
+        pytest.skip("oracle/_ref not built")
+    for vec in GOLD["ternary_vectors"]:
+        src = np.array(vec, np.int32)
+        n = R.ref_ternary_pack_estimate_size(len(src))
+        assert n == (len(src) + 4) // 5
+        buf = np.zeros(n, np.uint8); back = np.zeros(len(src), np.int32)
+        R.ref_ternary_pack(P(src), len(src), P(buf)); R.ref_ternary_unpack(P(buf), len(src), P(back))
+        assert np.array_equal(back, src)
