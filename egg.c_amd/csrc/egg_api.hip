@@ -41,6 +41,8 @@ struct egg_ctx {
     Layout L;
     std::vector<egg_tensor_info> tensors;
     int8_t *d_model = nullptr; float *d_state = nullptr;
+    int8_t *d_wfrag = nullptr;      // fragment-major copy of every matrix, same offsets as the model blob
+    int8_t *d_plin_frag = nullptr; size_t plin_frag_bytes = 0;
     int32_t *d_exp = nullptr; int8_t *d_act = nullptr; int32_t *d_rope = nullptr;
     int chunk = 0;
     int8_t *d_x = nullptr, *d_q = nullptr, *d_k = nullptr, *d_v = nullptr, *d_ao = nullptr;
@@ -142,7 +144,7 @@ static void build_tensor_table(egg_ctx *ctx) {
 }
 
 static void free_all(egg_ctx *ctx) {
-    void *ptrs[] = {ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
+    void *ptrs[] = {ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
                     ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits};
     for (void *p : ptrs) if (p) (void)hipFree(p);
@@ -191,6 +193,7 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     CR(hipMemcpy(ctx->d_act, act.data(), 256, hipMemcpyHostToDevice));
     CR(hipMemcpy(ctx->d_rope, rope.data(), rope.size() * 4, hipMemcpyHostToDevice));
     CR(hipMalloc(&ctx->d_model, ctx->L.total)); CR(hipMemset(ctx->d_model, 0, ctx->L.total));
+    CR(hipMalloc(&ctx->d_wfrag, ctx->L.total)); CR(hipMemset(ctx->d_wfrag, 0, ctx->L.total));
     CR(hipMalloc(&ctx->d_state, ctx->L.total * 12)); CR(hipMemset(ctx->d_state, 0, ctx->L.total * 12));
     // activation workspace for one chunk of members
     int chunk = c.chunk_members > 0 ? c.chunk_members : 2048;
@@ -208,6 +211,17 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     CR(hipMalloc(&ctx->d_panel_b, (size_t)4 * c.hidden * ctx->pairs_pad));
 #undef CR
     *out = ctx;
+    return EGG_OK;
+}
+
+// refresh the fragment-major copy of one matrix (tensor id) or of all matrices (id < 0); enqueued on the stream
+static int refresh_frag(egg_ctx *ctx, int id) {
+    const int B = ctx->cfg.hidden < 256 ? ctx->cfg.hidden : 256;
+    for (int i = 0; i < (int)ctx->tensors.size(); i++) {
+        const egg_tensor_info &t = ctx->tensors[i];
+        if (!t.is_matrix || (id >= 0 && i != id)) continue;
+        HIP_TRY(egg_launch_swizzle(ctx->d_model + t.offset, ctx->d_wfrag + t.offset, t.rows, t.cols, B, 0, ctx->stream));
+    }
     return EGG_OK;
 }
 
@@ -267,13 +281,13 @@ extern "C" int egg_model_init(egg_ctx *ctx, uint32_t seed) {
     for (int i = 0; i < H; i++) m[L.ln_f + i] = 16;
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     HIP_TRY(hipMemcpy(ctx->d_model, m.data(), m.size(), hipMemcpyHostToDevice));
-    return EGG_OK;
+    return refresh_frag(ctx, -1);
 }
 extern "C" int egg_model_upload(egg_ctx *ctx, const void *h, size_t bytes) {
     if (!ctx || !h || (int64_t)bytes != ctx->L.total) return fail(ctx, EGG_E_INVALID, "model size mismatch");
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     HIP_TRY(hipMemcpy(ctx->d_model, h, bytes, hipMemcpyHostToDevice));
-    return EGG_OK;
+    return refresh_frag(ctx, -1);
 }
 extern "C" int egg_model_download(egg_ctx *ctx, void *h, size_t bytes) {
     if (!ctx || !h || (int64_t)bytes != ctx->L.total) return fail(ctx, EGG_E_INVALID, "model size mismatch");
@@ -318,10 +332,21 @@ extern "C" int egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_
                                     uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8) {
     if (!ctx || !d_X || !d_W || members < 1 || T < 32 || T % 32 || (!d_Y32 && !d_Y8) || shift < 0 || shift > 31)
         return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear arguments");
-    PlinParams p = {d_X, d_W, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
+    if (K < 64 || N < 64 || K % 64 || N % 64) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: K and N must be multiples of 64");
+    if ((size_t)K * N > ctx->plin_frag_bytes) {
+        HIP_TRY(hipStreamSynchronize(ctx->stream));
+        if (ctx->d_plin_frag) (void)hipFree(ctx->d_plin_frag);
+        ctx->d_plin_frag = nullptr; ctx->plin_frag_bytes = 0;
+        HIP_TRY(hipMalloc(&ctx->d_plin_frag, (size_t)K * N));
+        ctx->plin_frag_bytes = (size_t)K * N;
+    }
+    PlinParams p = {d_X, ctx->d_plin_frag, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
                     ctx->cfg.noise_mask, d_Y32, d_Y8};
+    const int PB = egg_plinear_block(K, N);
+    if (K % PB || N % PB) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");
     span_begin(ctx, EGG_K_PLINEAR);
-    hipError_t e = egg_launch_plinear(p, ctx->stream);
+    hipError_t e = egg_launch_swizzle(d_W, ctx->d_plin_frag, K, N, PB, 1, ctx->stream);
+    if (e == hipSuccess) e = egg_launch_plinear(p, ctx->stream);
     span_end(ctx);
     if (e == hipErrorInvalidValue) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");
     HIP_TRY(e);
@@ -352,6 +377,7 @@ static int8_t *tap_ptr(egg_ctx *ctx, int slot) {
 static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const int64_t *d_start, const uint32_t *d_seed,
                          int first_member, int nm) {
     const egg_config &c = ctx->cfg; const Layout &L = ctx->L; const int8_t *M = ctx->d_model; const int H = c.hidden;
+    const int8_t *F = ctx->d_wfrag;
     hipStream_t s = ctx->stream;
     const bool taps = ctx->taps && nm <= ctx->tap_members;
     const size_t act_bytes = (size_t)nm * c.seq_len * H;
@@ -361,8 +387,8 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.off_ln_a = OFF_LN_INIT_A; p.off_ln_b = OFF_LN_INIT_B; p.off_lnb_a = OFF_LN_INIT_BIAS_A; p.off_lnb_b = OFF_LN_INIT_BIAS_B;
         p.off_up_a = OFF_EMB_MLP_UP_A; p.off_up_b = OFF_EMB_MLP_UP_B; p.off_bup_a = OFF_EMB_MLP_BIAS_UP_A; p.off_bup_b = OFF_EMB_MLP_BIAS_UP_B;
         p.off_dn_a = OFF_EMB_MLP_DOWN_A; p.off_dn_b = OFF_EMB_MLP_DOWN_B; p.off_bdn_a = OFF_EMB_MLP_BIAS_DOWN_A; p.off_bdn_b = OFF_EMB_MLP_BIAS_DOWN_B;
-        p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = M + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
-        p.w_dn = M + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
+        p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = F + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
+        p.w_dn = F + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
         p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
         span_begin(ctx, EGG_K_MLP_FIRST); HIP_TRY(egg_launch_mlp(p, true, s)); span_end(ctx);
         if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 0), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
@@ -372,7 +398,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         {
             QkvParams p; memset(&p, 0, sizeof(p)); p.c = f; p.seed_base = l * 1000;
             p.ln_w = M + L.ln_1 + (int64_t)l * H; p.ln_b = M + L.ln_1_bias + (int64_t)l * H;
-            p.w_q = M + L.w_q + l * hh; p.w_k = M + L.w_k + l * hh; p.w_v = M + L.w_v + l * hh;
+            p.w_q = F + L.w_q + l * hh; p.w_k = F + L.w_k + l * hh; p.w_v = F + L.w_v + l * hh;
             p.x = ctx->d_x; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v;
             span_begin(ctx, EGG_K_QKV); HIP_TRY(egg_launch_qkv(p, s)); span_end(ctx);
             if (taps) {
@@ -392,9 +418,9 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
             p.off_up_a = OFF_MLP_UP_A; p.off_up_b = OFF_MLP_UP_B; p.off_bup_a = OFF_MLP_BIAS_UP_A; p.off_bup_b = OFF_MLP_BIAS_UP_B;
             p.off_dn_a = OFF_MLP_DOWN_A; p.off_dn_b = OFF_MLP_DOWN_B; p.off_bdn_a = OFF_MLP_BIAS_DOWN_A; p.off_bdn_b = OFF_MLP_BIAS_DOWN_B;
             p.ln_w = M + L.ln_2 + (int64_t)l * H; p.ln_b = M + L.ln_2_bias + (int64_t)l * H;
-            p.w_up = M + L.w_up + l * h4; p.b_up = M + L.mlp_bias_up + (int64_t)l * 4 * H;
-            p.w_dn = M + L.w_down + l * h4; p.b_dn = M + L.mlp_bias_down + (int64_t)l * H;
-            p.w_o = M + L.w_o + l * hh; p.ao = ctx->d_ao; p.x = ctx->d_x;
+            p.w_up = F + L.w_up + l * h4; p.b_up = M + L.mlp_bias_up + (int64_t)l * 4 * H;
+            p.w_dn = F + L.w_down + l * h4; p.b_dn = M + L.mlp_bias_down + (int64_t)l * H;
+            p.w_o = F + L.w_o + l * hh; p.ao = ctx->d_ao; p.x = ctx->d_x;
             p.x_mid = taps ? tap_ptr(ctx, 1 + 6 * l + 4) : nullptr;
             span_begin(ctx, EGG_K_MLP); HIP_TRY(egg_launch_mlp(p, false, s)); span_end(ctx);
             if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 5), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
@@ -402,7 +428,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
     }
     {
         HeadParams p; memset(&p, 0, sizeof(p)); p.c = f;
-        p.ln_w = M + L.ln_f; p.ln_b = M + L.ln_f_bias; p.embedding = M + L.embedding; p.x = ctx->d_x;
+        p.ln_w = M + L.ln_f; p.ln_b = M + L.ln_f_bias; p.embedding_frag = F + L.embedding; p.x = ctx->d_x;
         p.loss_acc = ctx->d_loss_acc; p.logits_tap = taps ? ctx->d_tap_logits : nullptr;
         span_begin(ctx, EGG_K_HEAD); HIP_TRY(egg_launch_head(p, s)); span_end(ctx);
     }
@@ -458,7 +484,11 @@ static UpdParams make_upd(egg_ctx *ctx, const egg_tensor_info &t, const int32_t 
 static int update_one(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
     const egg_tensor_info &t = ctx->tensors[id];
     UpdParams p = make_upd(ctx, t, d_fit, d_seed, d_lr);
-    if (t.is_matrix) { span_begin(ctx, EGG_K_UPDATE_MATRIX); HIP_TRY(egg_launch_update_matrix(p, ctx->stream)); span_end(ctx); }
+    if (t.is_matrix) {
+        span_begin(ctx, EGG_K_UPDATE_MATRIX); HIP_TRY(egg_launch_update_matrix(p, ctx->stream)); span_end(ctx);
+        int rc = refresh_frag(ctx, id);
+        if (rc) return rc;
+    }
     else { span_begin(ctx, EGG_K_UPDATE_VECTOR); HIP_TRY(egg_launch_update_vector(p, ctx->stream)); span_end(ctx); }
     return EGG_OK;
 }

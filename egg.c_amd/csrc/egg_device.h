@@ -68,68 +68,76 @@ __device__ __forceinline__ int sumabs4(int a, int c) {
     return c + abs(sx8(a, 0)) + abs(sx8(a, 1)) + abs(sx8(a, 2)) + abs(sx8(a, 3));
 }
 
-// truncating division of a by a divisor in [1,127] for |a| < 2^24, via a per-token magic number
-struct MagicDiv { uint32_t m; int one; };
-__device__ __forceinline__ MagicDiv make_magic(int d) {
-    MagicDiv r; r.one = (d == 1);
-    r.m = r.one ? 0u : (uint32_t)(0x100000000ull / (uint32_t)d) + 1u;
-    return r;
+// full-rate 24-bit multiply (both operands must fit in 24 signed bits, the product in 32)
+__device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
+
+// C truncating division a / d for |a| <= 40000 and d in [1,127], with rcp = 1.0f / (float)d:
+// trunc((a + copysign(0.5, a)) * rcp).  a/d is a multiple of 1/d, so (a +- 0.5)/d stays at least 0.5/d away
+// from the next integer while the float error is below 0.007/d; checked exhaustively on the CPU.
+__device__ __forceinline__ int div_trunc(int a, float rcp) {
+    float af = (float)a;
+    return (int)((af + __builtin_copysignf(0.5f, af)) * rcp);
 }
-__device__ __forceinline__ int div_trunc(int a, MagicDiv md) {
-    int sg = a >> 31; uint32_t ua = (uint32_t)((a ^ sg) - sg);
-    uint32_t uq = md.one ? ua : __umulhi(ua, md.m);
-    return ((int)uq ^ sg) - sg;
+// (int)roundf(x) (half away from zero) for |x| <= 4096: trunc(x + copysign(0.5 - 2^-25, x)); checked
+// exhaustively on the CPU against roundf for every float in that range.
+__device__ __forceinline__ int round_half_away(float x) {
+    return (int)(x + __builtin_copysignf(0x1.fffffep-2f, x));
 }
 
 // ---------------------------------------------------------------- W block staging
-// Copies the block rows [k0, k0+KB) x cols [n0, n0+NB) of a blocked [K/4][N][4] matrix into LDS as
-// [KB/16][NB][16 bytes]: entry (p = 2*ks + g, n) holds the 16 k-bytes lane half g consumes in k-step ks,
-// i.e. dwords kq = 8ks + 2q + g (slot order) or 8ks + 4g + q (natural order), q = 0..3.
-template <int KB, int NB, bool NAT>
-__device__ __forceinline__ void stage_w_block(int8_t *lds, const int8_t *Wg, int n_total, int k0, int n0) {
-    const uint32_t *W32 = reinterpret_cast<const uint32_t *>(Wg);
-    constexpr int ITEMS = (KB / 16) * NB;
-    for (int it = threadIdx.x; it < ITEMS; it += EGG_THREADS) {
-        int n = it % NB, p = it / NB, ks = p >> 1, g = p & 1;
-        v4i v;
+// Weights are consumed from a "fragment-major" copy of each matrix (built by k_swizzle whenever the canonical
+// blocked weights change): the matrix is cut into B x B blocks, B = min(hidden, 256); block (kb, nb) is stored
+// contiguously at ((kb * (N/B)) + nb) * B*B as [B/16][B][16 bytes], where entry (p = 2*ks + g, n) holds the
+// 16 k-bytes lane half g consumes in k-step ks for output column n: canonical dwords kq = 8ks + 2q + g (slot
+// order) or 8ks + 4g + q (natural order), q = 0..3.  A block is therefore exactly its LDS image and staging
+// is a straight 16-byte-per-lane copy with every load in flight before the first LDS write.
+template <int B>
+__device__ __forceinline__ void stage_w_block(int8_t *lds, const int8_t *blk) {
+    constexpr int CHUNKS = B * B / 16;
+    constexpr int PER = (CHUNKS + EGG_THREADS - 1) / EGG_THREADS;
+    v4i v[PER];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            int kq = (k0 >> 2) + 8 * ks + (NAT ? (4 * g + q) : (2 * q + g));
-            v[q] = (int)W32[(size_t)kq * n_total + n0 + n];
-        }
-        *reinterpret_cast<v4i *>(lds + ((size_t)p * NB + n) * 16) = v;
+    for (int i = 0; i < PER; i++) {
+        int c = threadIdx.x + i * EGG_THREADS;
+        if (CHUNKS % EGG_THREADS == 0 || c < CHUNKS) v[i] = *reinterpret_cast<const v4i *>(blk + (size_t)c * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        int c = threadIdx.x + i * EGG_THREADS;
+        if (CHUNKS % EGG_THREADS == 0 || c < CHUNKS) *reinterpret_cast<v4i *>(lds + (size_t)c * 16) = v[i];
     }
 }
 
 // acc[nt] += W_block^T . xop for one staged block; xop[ks] is the token operand of k-step ks of the block
-template <int KB, int NB>
+template <int B>
 __device__ __forceinline__ void mfma_block(v16i *acc, const v4i *xop, const int8_t *lds, int lane) {
     const int i = lane & 31, g = lane >> 5;
 #pragma unroll
-    for (int ks = 0; ks < KB / 32; ks++) {
+    for (int ks = 0; ks < B / 32; ks++) {
 #pragma unroll
-        for (int nt = 0; nt < NB / 32; nt++) {
-            v4i a = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * NB + nt * 32 + i) * 16);
+        for (int nt = 0; nt < B / 32; nt++) {
+            v4i a = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * B + nt * 32 + i) * 16);
             acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, xop[ks], acc[nt], 0, 0, 0);
         }
     }
 }
 
-// Full GEMM for one tile: acc[NOUT/32] (+)= W[k_off.., n_off..]^T . xop[KTOT/32], W streamed through LDS
-// in blocks of at most 256 x 256.  Every wave of the workgroup must call it (it synchronises).
-template <int KTOT, int NOUT, bool NAT>
-__device__ __forceinline__ void gemm_stream(v16i *acc, const v4i *xop, const int8_t *Wg, int n_total,
+// Full GEMM for one tile: acc[NOUT/32] (+)= W[k_off.., n_off..]^T . xop[KTOT/32], W blocks (fragment-major)
+// streamed through LDS.  Every wave of the workgroup must call it (it synchronises).
+template <int KTOT, int NOUT, int B>
+__device__ __forceinline__ void gemm_stream(v16i *acc, const v4i *xop, const int8_t *Wf, int n_total,
                                             int k_off, int n_off, int8_t *wlds, int lane) {
-    constexpr int KB = KTOT < 256 ? KTOT : 256;
-    constexpr int NB = NOUT < 256 ? NOUT : 256;
+    static_assert(KTOT % B == 0 && NOUT % B == 0, "block size must divide the GEMM");
+    const int nblk_n = n_total / B;
 #pragma unroll
-    for (int nb = 0; nb < NOUT / NB; nb++) {
+    for (int nb = 0; nb < NOUT / B; nb++) {
 #pragma unroll
-        for (int kb = 0; kb < KTOT / KB; kb++) {
+        for (int kb = 0; kb < KTOT / B; kb++) {
+            const int8_t *blk = Wf + ((size_t)(k_off / B + kb) * nblk_n + (n_off / B + nb)) * (B * B);
             __syncthreads();
-            stage_w_block<KB, NB, NAT>(wlds, Wg, n_total, k_off + kb * KB, n_off + nb * NB);
+            stage_w_block<B>(wlds, blk);
             __syncthreads();
-            mfma_block<KB, NB>(acc + nb * (NB / 32), xop + kb * (KB / 32), wlds, lane);
+            mfma_block<B>(acc + nb * (B / 32), xop + kb * (B / 32), wlds, lane);
         }
     }
 }
@@ -184,7 +192,8 @@ __device__ __forceinline__ int dot_noise(const v4i *xop, const int8_t *btab, int
 // ---------------------------------------------------------------- norms on a token held as a packed operand
 // apply_standard_norm (mgpu.cu:646-678): wt / bt are int32 tables already holding w + noise, b + noise
 template <int KS>
-__device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int *wt, const int *bt, int H, int g) {
+__device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int *wt, const int *bt, int g) {
+    constexpr int H = 32 * KS;
     int tot = 0;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++)
@@ -192,7 +201,7 @@ __device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int 
         for (int q = 0; q < 4; q++) tot = sumabs4(x[ks][q], tot);
     tot += other_half(tot);
     int mn = tot / H; if (!mn) mn = 1;
-    MagicDiv md = make_magic(mn);
+    const float md = 1.0f / (float)mn;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++)
 #pragma unroll
@@ -202,7 +211,7 @@ __device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int 
             v4i b4 = *reinterpret_cast<const v4i *>(bt + n0);
             int o[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(sx8(x[ks][q], e) * w4[e], md) + b4[e]);
+            for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(mul24(sx8(x[ks][q], e), w4[e]), md) + b4[e]);
             out[ks][q] = pack4(o[0], o[1], o[2], o[3]);
         }
 }
@@ -210,11 +219,15 @@ __device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int 
 // adaptive_*_normalize (egg_adaptive_normalize.h:10-103) over NT column groups held in acc; result packed
 template <int NT>
 __device__ __forceinline__ void adaptive_norm(const v16i *val, v4i *out) {
-    int mx = 0;
+    int hi = 0, lo = 0;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) mx = max(mx, abs(val[nt][r]));
+        for (int r = 0; r < 16; r += 2) {
+            hi = max(max(hi, val[nt][r]), val[nt][r + 1]);
+            lo = min(min(lo, val[nt][r]), val[nt][r + 1]);
+        }
+    int mx = max(hi, -lo);
     mx = max(mx, other_half(mx));
     float scale = 127.0f / ((float)mx + 1e-9f);
 #pragma unroll
@@ -225,8 +238,7 @@ __device__ __forceinline__ void adaptive_norm(const v16i *val, v4i *out) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 float sf = (float)val[nt][4 * q + e] * scale;
-                int s = (int)roundf(sf);
-                o[e] = min(127, max(-127, s));
+                o[e] = clip127(round_half_away(sf));
             }
             out[nt][q] = pack4(o[0], o[1], o[2], o[3]);
         }

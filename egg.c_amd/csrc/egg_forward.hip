@@ -31,7 +31,7 @@ __device__ __forceinline__ void add_perturb(v16i *acc, int sb, const int *At, in
         for (int q = 0; q < 4; q++) {
             v4i a4 = *reinterpret_cast<const v4i *>(At + n_off + 32 * nt + 8 * q + 4 * g);
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc[nt][4 * q + e] += (sb * a4[e]) >> sigma;
+            for (int e = 0; e < 4; e++) acc[nt][4 * q + e] += mul24(sb, a4[e]) >> sigma;
         }
 }
 
@@ -48,7 +48,7 @@ struct MlpLds {
 
 template <int H, bool FIRST>
 __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
-    constexpr int KS = H / 32, NT = H / 32;
+    constexpr int KS = H / 32, NT = H / 32, BLK = H < 256 ? H : 256;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *wlds = smem;
     int8_t *act = smem + MlpLds<H>::WBLOCK;
@@ -111,7 +111,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
                     v4i d4 = *reinterpret_cast<const v4i *>(ex1 + n0);
                     int o[4];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = clip127(sx8(e4, e) + b4[e] + ((a_tok * d4[e]) >> c.sigma));
+                    for (int e = 0; e < 4; e++) o[e] = clip127(sx8(e4, e) + b4[e] + (mul24(a_tok, d4[e]) >> c.sigma));
                     xcur[ks][q] = pack4(o[0], o[1], o[2], o[3]);
                 }
         } else {
@@ -121,7 +121,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
             for (int ks = 0; ks < KS; ks++) { aop[ks] = load_op(p.ao + row, ks, g); xres[ks] = load_op(p.x + row, ks, g); }
             int sbo = dot_noise<KS, false>(aop, exB, 0, g);
             zero_acc<NT>(acc);
-            gemm_stream<H, H, false>(acc, aop, p.w_o, H, 0, 0, wlds, lane);
+            gemm_stream<H, H, BLK>(acc, aop, p.w_o, H, 0, 0, wlds, lane);
             add_perturb<NT>(acc, sbo, ex0, 0, c.sigma, g);
 #pragma unroll
             for (int nt = 0; nt < NT; nt++)
@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
 
         // MLP (mgpu.cu:708-759)
         v4i nrm[KS];
-        standard_norm<KS>(xcur, nrm, lnw, lnb, H, g);
+        standard_norm<KS>(xcur, nrm, lnw, lnb, g);
         const int sbu = dot_noise<KS, false>(nrm, upB, 0, g);
         v16i accd[NT];
         zero_acc<NT>(accd);
@@ -143,7 +143,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
 #pragma unroll 1
         for (int ch = 0; ch < 4; ch++) {
             zero_acc<NT>(acc);
-            gemm_stream<H, H, false>(acc, nrm, p.w_up, 4 * H, 0, ch * H, wlds, lane);
+            gemm_stream<H, H, BLK>(acc, nrm, p.w_up, 4 * H, 0, ch * H, wlds, lane);
             v4i mid[KS];
 #pragma unroll
             for (int nt = 0; nt < NT; nt++)
@@ -155,7 +155,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
                     int o[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        int a = acc[nt][4 * q + e] + ((sbu * a4[e]) >> c.sigma);
+                        int a = acc[nt][4 * q + e] + (mul24(sbu, a4[e]) >> c.sigma);
                         int v = clip127((a >> c.shift_mlp_up) + b4[e]);
                         o[e] = act[(uint8_t)v];
                     }
@@ -168,7 +168,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
 #pragma unroll
                     for (int q = 0; q < 4; q++) sbd = dot4(mid[ks][q], b32[8 * ks + 2 * q + g], sbd);
             }
-            gemm_stream<H, H, false>(accd, mid, p.w_dn, H, ch * H, 0, wlds, lane);
+            gemm_stream<H, H, BLK>(accd, mid, p.w_dn, H, ch * H, 0, wlds, lane);
         }
         sbd += other_half(sbd);
         add_perturb<NT>(accd, sbd, dnA, 0, c.sigma, g);
@@ -222,7 +222,7 @@ __device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row,
 
 template <int H>
 __global__ void __launch_bounds__(EGG_THREADS) k_qkv(QkvParams p) {
-    constexpr int KS = H / 32, NT = H / 32;
+    constexpr int KS = H / 32, NT = H / 32, BLK = H < 256 ? H : 256;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *wlds = smem;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
@@ -255,7 +255,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_qkv(QkvParams p) {
         v4i x[KS], nrm[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
-        standard_norm<KS>(x, nrm, lnw, lnb, H, g);
+        standard_norm<KS>(x, nrm, lnw, lnb, g);
         const int32_t *rope_row = c.rope_lut + (size_t)t * c.head_dim;
 #pragma unroll 1
         for (int which = 0; which < 3; which++) {
@@ -266,7 +266,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_qkv(QkvParams p) {
             const int sb = dot_noise<KS, false>(nrm, Bn, 0, g);
             v16i acc[NT];
             zero_acc<NT>(acc);
-            gemm_stream<H, H, false>(acc, nrm, W, H, 0, 0, wlds, lane);
+            gemm_stream<H, H, BLK>(acc, nrm, W, H, 0, 0, wlds, lane);
             add_perturb<NT>(acc, sb, An, 0, c.sigma, g);
             if (which < 2) rope_inplace<NT>(acc, rope_row, c.head_dim, c.rope_scale_bit, g);
             v4i o[KS];
@@ -421,13 +421,13 @@ __global__ void __launch_bounds__(EGG_THREADS) k_attn(AttnParams p) {
 template <int H>
 struct HeadLds {
     static constexpr int PER_WAVE = (2 * H + 256) * 4 + H;   // lnw lnb hA[256] + hB[H]
-    static constexpr int WBLOCK = (H < 256 ? H : 256) * 256;
+    static constexpr int WBLOCK = (H < 256 ? H : 256) * (H < 256 ? H : 256);
     static constexpr int TOTAL = WBLOCK + 1024 + EGG_WAVES * PER_WAVE;
 };
 
 template <int H>
 __global__ void __launch_bounds__(EGG_THREADS) k_head(HeadParams p) {
-    constexpr int KS = H / 32, NV = 256 / 32;
+    constexpr int KS = H / 32, NV = 256 / 32, BLK = H < 256 ? H : 256;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *wlds = smem;
     int *lut = reinterpret_cast<int *>(smem + HeadLds<H>::WBLOCK);
@@ -460,11 +460,11 @@ __global__ void __launch_bounds__(EGG_THREADS) k_head(HeadParams p) {
         v4i x[KS], nf[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
-        standard_norm<KS>(x, nf, lnw, lnb, H, g);
+        standard_norm<KS>(x, nf, lnw, lnb, g);
         const int sbh = dot_noise<KS, false>(nf, hB, 0, g);
         v16i acc[NV];
         zero_acc<NV>(acc);
-        gemm_stream<H, 256, false>(acc, nf, p.embedding, 256, 0, 0, wlds, lane);
+        gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, wlds, lane);
         add_perturb<NV>(acc, sbh, hA, 0, c.sigma, g);
         // two-pass softmax statistics (mgpu.cu:969-1009)
         int gmax = INT_MIN;

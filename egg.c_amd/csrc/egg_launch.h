@@ -13,12 +13,15 @@ hipError_t egg_prepare_forward(int H, int head_dim, int T);
 
 struct PlinParams {
     const int8_t *X;        // [members*T][K] natural order
-    const int8_t *W;        // blocked [K/4][N][4]
+    const int8_t *Wfrag;    // fragment-major copy of W (natural k order), block size egg_plinear_block(K, N)
     int members, T, K, N;
     uint32_t seed; int off_a, off_b, shift, sigma, mask;
     int32_t *Y32; int8_t *Y8;
 };
 hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s);
+int egg_plinear_block(int K, int N);
+// canonical blocked [K/4][N][4] -> fragment-major (see egg_device.h); nat = natural k order inside a k-step
+hipError_t egg_launch_swizzle(const int8_t *W_blocked, int8_t *W_frag, int K, int N, int B, int nat, hipStream_t s);
 
 // small utility kernels (egg_update.hip)
 hipError_t egg_launch_noise_fill(uint32_t seed, uint32_t first, int n, int mask, int8_t *out, hipStream_t s);

@@ -8,18 +8,20 @@
 
 template <int K, int N>
 struct PlinLds {
-    static constexpr int KB = K < 256 ? K : 256, NB = N < 256 ? N : 256;
+    static constexpr int MINKN = K < N ? K : N;
+    static constexpr int B = MINKN < 256 ? MINKN : 256;      // fragment block size
+    static constexpr int NB = N < 256 ? N : 256;             // output columns per epilogue
     static constexpr int PER_WAVE = N * 4 + K;
-    static constexpr int TOTAL = KB * NB + EGG_WAVES * PER_WAVE;
+    static constexpr int TOTAL = B * B + EGG_WAVES * PER_WAVE;
 };
 
 template <int K, int N>
 __global__ void __launch_bounds__(EGG_THREADS) k_plinear(PlinParams p) {
-    constexpr int KS = K / 32, NB = PlinLds<K, N>::NB, NTB = NB / 32;
+    constexpr int KS = K / 32, NB = PlinLds<K, N>::NB, NTB = NB / 32, B = PlinLds<K, N>::B;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *wlds = smem;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    int8_t *tb = smem + PlinLds<K, N>::KB * NB + wave * PlinLds<K, N>::PER_WAVE;
+    int8_t *tb = smem + B * B + wave * PlinLds<K, N>::PER_WAVE;
     int *At = reinterpret_cast<int *>(tb);
     int8_t *Bt = reinterpret_cast<int8_t *>(At + N);
 
@@ -42,7 +44,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_plinear(PlinParams p) {
         for (int nb = 0; nb < N / NB; nb++) {
             v16i acc[NTB];
             zero_acc<NTB>(acc);
-            gemm_stream<K, NB, true>(acc, xop, p.W, N, 0, nb * NB, wlds, lane);
+            gemm_stream<K, NB, B>(acc, xop, p.Wfrag, N, 0, nb * NB, wlds, lane);
 #pragma unroll
             for (int nt = 0; nt < NTB; nt++)
 #pragma unroll
@@ -51,7 +53,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_plinear(PlinParams p) {
                     v4i a4 = *reinterpret_cast<const v4i *>(At + n0);
                     v4i o4;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o4[e] = (acc[nt][4 * q + e] + ((sb * a4[e]) >> p.sigma)) >> p.shift;
+                    for (int e = 0; e < 4; e++) o4[e] = (acc[nt][4 * q + e] + (mul24(sb, a4[e]) >> p.sigma)) >> p.shift;
                     if (valid) {
                         if (p.Y32) *reinterpret_cast<v4i *>(p.Y32 + row * N + n0) = o4;
                         if (p.Y8) *reinterpret_cast<int *>(p.Y8 + row * N + n0) =
@@ -71,6 +73,8 @@ static hipError_t launch_kn(const PlinParams &p, hipStream_t s) {
     hipLaunchKernelGGL((k_plinear<K, N>), grid, block, lds, s, p);
     return hipGetLastError();
 }
+
+int egg_plinear_block(int K, int N) { int m = K < N ? K : N; return m < 256 ? m : 256; }
 
 hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s) {
 #define CASE(K_, N_) if (p.K == K_ && p.N == N_) return launch_kn<K_, N_>(p, s);

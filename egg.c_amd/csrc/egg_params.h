@@ -45,11 +45,12 @@ struct MlpParams {
     // seed offsets of the block (MlpConfig, mgpu.cu:680-706)
     int off_ln_a, off_ln_b, off_lnb_a, off_lnb_b, off_up_a, off_up_b, off_bup_a, off_bup_b,
         off_dn_a, off_dn_b, off_bdn_a, off_bdn_b;
-    const int8_t *ln_w, *ln_b, *w_up, *b_up, *w_dn, *b_dn;
+    const int8_t *ln_w, *ln_b, *b_up, *b_dn;   // canonical model blob
+    const int8_t *w_up, *w_dn;                 // fragment-major copies
     // FIRST: embedding stage inputs
     const int8_t *embedding, *emb_bias;
     // !FIRST: attention output projection inputs
-    const int8_t *w_o;
+    const int8_t *w_o;           // fragment-major copy
     const int8_t *ao;            // [n_members][T][H] slot order
     int8_t *x;                   // [n_members][T][H] slot order, read (if !FIRST) and written
     int8_t *x_mid;               // optional tap: residual stream after attention (may be null)
@@ -58,7 +59,8 @@ struct MlpParams {
 struct QkvParams {
     FwdCommon c;
     int seed_base;
-    const int8_t *ln_w, *ln_b, *w_q, *w_k, *w_v;
+    const int8_t *ln_w, *ln_b;   // canonical
+    const int8_t *w_q, *w_k, *w_v;   // fragment-major copies
     const int8_t *x;
     int8_t *q, *k, *v;           // [n_members][T][H] slot order
 };
@@ -71,7 +73,8 @@ struct AttnParams {
 
 struct HeadParams {
     FwdCommon c;
-    const int8_t *ln_w, *ln_b, *embedding;
+    const int8_t *ln_w, *ln_b;
+    const int8_t *embedding_frag; // fragment-major copy of the tied embedding [H][vocab]
     const int8_t *x;
     unsigned long long *loss_acc; // [population] two's-complement int64 accumulators
     int32_t *logits_tap;          // optional [n_members][T][vocab] natural order (may be null)

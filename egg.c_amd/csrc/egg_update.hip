@@ -184,3 +184,26 @@ hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s) {
     hipLaunchKernelGGL(k_vector_adam, dim3((p.cols + EGG_WAVES - 1) / EGG_WAVES), dim3(EGG_THREADS), 0, s, p);
     return hipGetLastError();
 }
+
+// canonical blocked weights -> fragment-major copy consumed by the GEMM kernels (layout in egg_device.h)
+__global__ void k_swizzle(const uint32_t *src, v4i *dst, int K, int N, int B, int nat) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= K * N / 16) return;
+    const int per_block = B * B / 16;
+    int block = c / per_block, idx = c % per_block;
+    int p = idx / B, n = idx % B, kb = block / (N / B), nb = block % (N / B), ks = p >> 1, g = p & 1;
+    v4i v;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        int kq = (kb * B) / 4 + 8 * ks + (nat ? (4 * g + q) : (2 * q + g));
+        v[q] = (int)src[(size_t)kq * N + nb * B + n];
+    }
+    dst[c] = v;
+}
+hipError_t egg_launch_swizzle(const int8_t *W, int8_t *Wf, int K, int N, int B, int nat, hipStream_t s) {
+    if (K % B || N % B || B % 32) return hipErrorInvalidValue;
+    int chunks = K * N / 16;
+    hipLaunchKernelGGL(k_swizzle, dim3((chunks + 255) / 256), dim3(256), 0, s, reinterpret_cast<const uint32_t *>(W),
+                       reinterpret_cast<v4i *>(Wf), K, N, B, nat);
+    return hipGetLastError();
+}
