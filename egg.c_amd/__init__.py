@@ -46,6 +46,7 @@ EXPORTS = [
     "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
+    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz",
 ]
 KCLASSES = ["mlp_first", "qkv", "attn", "mlp", "head", "update_matrix", "update_vector", "plinear"]
 
@@ -107,6 +108,11 @@ def lib():
         L.egg_ctx_enable_timing.argtypes = [vp, i32]
         L.egg_timing_reset.argtypes = [vp]
         L.egg_timing_get.argtypes = [vp, i32, vp, vp]
+        L.egg_opt_state_bytes.restype = i64
+        L.egg_opt_state_bytes.argtypes = [vp]
+        L.egg_tensor_state_offset.restype = i64
+        L.egg_tensor_state_offset.argtypes = [vp, i32]
+        L.egg_newton_schulz.argtypes = [vp, vp, i32, i32, i32]
         _lib = L
     return _lib
 
@@ -177,9 +183,15 @@ class Context:
 
     def opt_state_download(self):
         import numpy as np
-        out = np.zeros(self.model_bytes() * 3, np.float32)
+        out = np.zeros(int(lib().egg_opt_state_bytes(self._h)) // 4, np.float32)
         self._ck(lib().egg_opt_state_download(self._h, _np_ptr(out), out.nbytes), "egg_opt_state_download")
         return out
+
+    def tensor_state_offset(self, tid):
+        return int(lib().egg_tensor_state_offset(self._h, tid))
+
+    def newton_schulz(self, d_x, rows, cols, iters=5):
+        self._ck(lib().egg_newton_schulz(self._h, C.c_void_p(d_x), rows, cols, iters), "egg_newton_schulz")
 
     def opt_state_reset(self):
         self._ck(lib().egg_opt_state_reset(self._h), "egg_opt_state_reset")

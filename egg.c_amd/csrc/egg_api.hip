@@ -7,6 +7,7 @@
 #include <math.h>
 #include <stdio.h>
 #include <string.h>
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -40,7 +41,9 @@ struct egg_ctx {
     hipStream_t stream = nullptr; bool own_stream = false;
     Layout L;
     std::vector<egg_tensor_info> tensors;
-    int8_t *d_model = nullptr; float *d_state = nullptr;
+    int8_t *d_model = nullptr;
+    uint8_t *d_state = nullptr; int64_t state_bytes = 0; std::vector<int64_t> t_state_off;   // optimizer state (AdamModel layout)
+    MuonWork muon = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     int8_t *d_wfrag = nullptr;      // fragment-major copy of every matrix, same offsets as the model blob
     int8_t *d_plin_frag = nullptr; size_t plin_frag_bytes = 0;
     int32_t *d_exp = nullptr; int8_t *d_act = nullptr; int32_t *d_rope = nullptr;
@@ -144,7 +147,8 @@ static void build_tensor_table(egg_ctx *ctx) {
 }
 
 static void free_all(egg_ctx *ctx) {
-    void *ptrs[] = {ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
+    void *ptrs[] = {ctx->muon.x, ctx->muon.swap, ctx->muon.bterm, ctx->muon.partials, ctx->muon.norm,
+                    ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
                     ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits};
     for (void *p : ptrs) if (p) (void)hipFree(p);
@@ -162,7 +166,6 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return EGG_E_INVALID;
     if (c.seq_len % 32 || !(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256)) return EGG_E_INVALID;
     if (c.vocab != 256 || c.n_layers < 1 || c.population < 2 || (c.population & 1)) return EGG_E_INVALID;
-    if (c.use_muon) return EGG_E_INVALID;   // Muon step not available in this build
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
     ctx->L = make_layout(c);
@@ -194,7 +197,27 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     CR(hipMemcpy(ctx->d_rope, rope.data(), rope.size() * 4, hipMemcpyHostToDevice));
     CR(hipMalloc(&ctx->d_model, ctx->L.total)); CR(hipMemset(ctx->d_model, 0, ctx->L.total));
     CR(hipMalloc(&ctx->d_wfrag, ctx->L.total)); CR(hipMemset(ctx->d_wfrag, 0, ctx->L.total));
-    CR(hipMalloc(&ctx->d_state, ctx->L.total * 12)); CR(hipMemset(ctx->d_state, 0, ctx->L.total * 12));
+    {   // optimizer state in the field order of AdamModel (mgpu.cu:337-370): {m,v,acc} per element, or {m,acc} for
+        // the matrices that use Muon (HIDDEN_OPT_TYPE, mgpu.cu:327-335)
+        std::vector<int> order(ctx->tensors.size());
+        for (size_t i = 0; i < order.size(); i++) order[i] = (int)i;
+        std::sort(order.begin(), order.end(), [&](int a, int b) { return ctx->tensors[a].offset < ctx->tensors[b].offset; });
+        ctx->t_state_off.assign(ctx->tensors.size(), 0);
+        int64_t so = 0;
+        for (int id : order) {
+            const egg_tensor_info &t = ctx->tensors[id];
+            ctx->t_state_off[id] = so;
+            so += (int64_t)t.rows * t.cols * ((c.use_muon && t.muon) ? 8 : 12);
+        }
+        ctx->state_bytes = so;
+    }
+    CR(hipMalloc(&ctx->d_state, ctx->state_bytes)); CR(hipMemset(ctx->d_state, 0, ctx->state_bytes));
+    if (c.use_muon) {
+        size_t mx = (size_t)4 * c.hidden * c.hidden;
+        CR(hipMalloc(&ctx->muon.x, mx * 4)); CR(hipMalloc(&ctx->muon.swap, mx * 4));
+        CR(hipMalloc(&ctx->muon.bterm, (size_t)c.hidden * c.hidden * 4));
+        CR(hipMalloc(&ctx->muon.partials, 1024 * 4)); CR(hipMalloc(&ctx->muon.norm, 16));
+    }
     // activation workspace for one chunk of members
     int chunk = c.chunk_members > 0 ? c.chunk_members : 2048;
     if (chunk > c.population) chunk = c.population;
@@ -296,13 +319,13 @@ extern "C" int egg_model_download(egg_ctx *ctx, void *h, size_t bytes) {
     return EGG_OK;
 }
 extern "C" int egg_opt_state_upload(egg_ctx *ctx, const void *h, size_t bytes) {
-    if (!ctx || !h || (int64_t)bytes != ctx->L.total * 12) return fail(ctx, EGG_E_INVALID, "state size mismatch");
+    if (!ctx || !h || (int64_t)bytes != ctx->state_bytes) return fail(ctx, EGG_E_INVALID, "state size mismatch");
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     HIP_TRY(hipMemcpy(ctx->d_state, h, bytes, hipMemcpyHostToDevice));
     return EGG_OK;
 }
 extern "C" int egg_opt_state_download(egg_ctx *ctx, void *h, size_t bytes) {
-    if (!ctx || !h || (int64_t)bytes != ctx->L.total * 12) return fail(ctx, EGG_E_INVALID, "state size mismatch");
+    if (!ctx || !h || (int64_t)bytes != ctx->state_bytes) return fail(ctx, EGG_E_INVALID, "state size mismatch");
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     HIP_TRY(hipMemcpy(h, ctx->d_state, bytes, hipMemcpyDeviceToHost));
     return EGG_OK;
@@ -310,7 +333,7 @@ extern "C" int egg_opt_state_download(egg_ctx *ctx, void *h, size_t bytes) {
 extern "C" int egg_opt_state_reset(egg_ctx *ctx) {
     if (!ctx) return EGG_E_INVALID;
     HIP_TRY(hipStreamSynchronize(ctx->stream));
-    HIP_TRY(hipMemset(ctx->d_state, 0, ctx->L.total * 12));
+    HIP_TRY(hipMemset(ctx->d_state, 0, ctx->state_bytes));
     return EGG_OK;
 }
 extern "C" int egg_tables_download(egg_ctx *ctx, int32_t *ex, int8_t *act, int32_t *rope) {
@@ -471,10 +494,11 @@ extern "C" int egg_fitness(egg_ctx *ctx, const int32_t *d_loss, int32_t *d_fit, 
 }
 
 // ------------------------------------------------------------------ update
-static UpdParams make_upd(egg_ctx *ctx, const egg_tensor_info &t, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
+static UpdParams make_upd(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
+    const egg_tensor_info &t = ctx->tensors[id];
     const egg_config &c = ctx->cfg;
     UpdParams p; memset(&p, 0, sizeof(p));
-    p.W = ctx->d_model + t.offset; p.state = ctx->d_state + t.offset * 3;
+    p.W = ctx->d_model + t.offset; p.state = reinterpret_cast<float *>(ctx->d_state + ctx->t_state_off[id]);
     p.rows = t.rows; p.cols = t.cols; p.off_a = t.off_a; p.off_b = t.off_b; p.seed_base = t.seed_base;
     p.fit = d_fit; p.pairs = c.population / 2; p.d_seed = d_seed; p.d_lr = d_lr; p.lr_scale = t.lr_scale;
     p.mask = c.noise_mask; p.beta1 = c.adam_beta1; p.beta2 = c.adam_beta2; p.eps = c.adam_eps; p.wd = c.adam_weight_decay;
@@ -483,8 +507,19 @@ static UpdParams make_upd(egg_ctx *ctx, const egg_tensor_info &t, const int32_t 
 }
 static int update_one(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
     const egg_tensor_info &t = ctx->tensors[id];
-    UpdParams p = make_upd(ctx, t, d_fit, d_seed, d_lr);
-    if (t.is_matrix) {
+    UpdParams p = make_upd(ctx, id, d_fit, d_seed, d_lr);
+    if (t.is_matrix && t.muon && ctx->cfg.use_muon) {
+        // LAUNCH_ADAM_MATRIX under USE_MUON (mgpu.cu:1587-1595)
+        span_begin(ctx, EGG_K_UPDATE_MATRIX);
+        p.muon_momentum = ctx->cfg.muon_momentum; p.muon_x = ctx->muon.x;
+        HIP_TRY(egg_launch_muon_momentum(p, ctx->stream));
+        HIP_TRY(egg_launch_newton_schulz(ctx->muon, t.rows, t.cols, 5, ctx->stream));
+        p.lr_scale = t.lr_scale * ctx->cfg.muon_lr_scale;
+        HIP_TRY(egg_launch_muon_apply(p, ctx->cfg.adam_weight_decay, ctx->stream));
+        span_end(ctx);
+        int rc = refresh_frag(ctx, id);
+        if (rc) return rc;
+    } else if (t.is_matrix) {
         span_begin(ctx, EGG_K_UPDATE_MATRIX); HIP_TRY(egg_launch_update_matrix(p, ctx->stream)); span_end(ctx);
         int rc = refresh_frag(ctx, id);
         if (rc) return rc;
@@ -499,7 +534,7 @@ extern "C" int egg_update_tensor(egg_ctx *ctx, int id, const int32_t *d_fit, con
 extern "C" int egg_matrix_votes(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, int32_t *d_votes) {
     if (!ctx || id < 0 || id >= (int)ctx->tensors.size() || !d_fit || !d_seed || !d_votes || !ctx->tensors[id].is_matrix)
         return fail(ctx, EGG_E_INVALID, "egg_matrix_votes arguments");
-    UpdParams p = make_upd(ctx, ctx->tensors[id], d_fit, d_seed, nullptr);
+    UpdParams p = make_upd(ctx, id, d_fit, d_seed, nullptr);
     p.votes_out = d_votes;
     HIP_TRY(egg_launch_update_matrix(p, ctx->stream));
     return EGG_OK;
@@ -511,6 +546,21 @@ extern "C" int egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t 
         int rc = update_one(ctx, id, d_fit, d_seed, d_lr);
         if (rc) return rc;
     }
+    return EGG_OK;
+}
+extern "C" int64_t egg_opt_state_bytes(const egg_ctx *ctx) { return ctx ? ctx->state_bytes : 0; }
+extern "C" int64_t egg_tensor_state_offset(const egg_ctx *ctx, int id) {
+    return (ctx && id >= 0 && id < (int)ctx->tensors.size()) ? ctx->t_state_off[id] : -1;
+}
+// Newton-Schulz orthogonalisation of a row-major [rows][cols] fp32 device matrix, in place (test hook for
+// perform_newton_schulz, muon_internal.cuh:182-342)
+extern "C" int egg_newton_schulz(egg_ctx *ctx, float *d_X, int rows, int cols, int iters) {
+    if (!ctx || !d_X || rows < 32 || cols < 32 || rows % 32 || cols % 32) return fail(ctx, EGG_E_INVALID, "egg_newton_schulz arguments");
+    if (!ctx->muon.x) return fail(ctx, EGG_E_STATE, "context was created without use_muon");
+    if ((size_t)rows * cols > (size_t)4 * ctx->cfg.hidden * ctx->cfg.hidden || (rows < cols ? rows : cols) > ctx->cfg.hidden)
+        return fail(ctx, EGG_E_INVALID, "matrix larger than the Muon workspace");
+    MuonWork w = ctx->muon; w.x = d_X;
+    HIP_TRY(egg_launch_newton_schulz(w, rows, cols, iters, ctx->stream));
     return EGG_OK;
 }
 extern "C" int egg_tensor_count(const egg_ctx *ctx) { return ctx ? (int)ctx->tensors.size() : 0; }

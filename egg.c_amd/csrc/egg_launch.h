@@ -39,6 +39,15 @@ struct UpdParams {
     int8_t *panel_a, *panel_b; int pairs_pad;   // workspace: [cols][pairs_pad], [rows][pairs_pad]
     unsigned long long *counter;
     int32_t *votes_out;                // optional: only compute votes (blocked order), no update
+    // Muon (state is {m, acc} per element): momentum pass writes m and the row-major gather buffer
+    float muon_momentum; float *muon_x; // [rows][cols] row-major
 };
 hipError_t egg_launch_update_matrix(const UpdParams &p, hipStream_t s);
 hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s);
+
+// Muon chain (muon_internal.cuh:15-342): momentum + gather (vote GEMM epilogue), Frobenius normalisation,
+// 5 Newton-Schulz iterations on fp32 MFMA, quantised apply.
+hipError_t egg_launch_muon_momentum(const UpdParams &p, hipStream_t s);
+struct MuonWork { float *x, *swap, *gram, *bterm, *partials, *norm; };   // x/swap: rows*cols, gram/bterm: K*K, partials: 1024
+hipError_t egg_launch_newton_schulz(const MuonWork &w, int rows, int cols, int iters, hipStream_t s);
+hipError_t egg_launch_muon_apply(const UpdParams &p, float wd, hipStream_t s);

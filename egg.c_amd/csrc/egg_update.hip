@@ -108,6 +108,25 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vote_adam(UpdParams p) {
     }
     // lane (n = n0 + j, half g), register 4q+e -> k = k0 + 8q + 4g + e ; blocked index of (k, n) (mgpu.cu:1085-1089)
     const int n = n0 + j;
+    if (p.muon_x) {
+        // muon_momentum_update_kernel + muon_gather_m_kernel (muon_internal.cuh:15-74): m = mu*m + vote
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const size_t idx0 = ((size_t)((k0 >> 2) + 2 * q + g) * p.cols + n) * 4;
+            float4 *sp = reinterpret_cast<float4 *>(p.state + idx0 * 2);
+            float4 s0 = sp[0], s1 = sp[1];
+            float mv[4] = {s0.x, s0.z, s1.x, s1.z};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float t = p.muon_momentum * mv[e];
+                mv[e] = t + (float)acc[4 * q + e];
+                p.muon_x[(size_t)(k0 + 8 * q + 4 * g + e) * p.cols + n] = mv[e];
+            }
+            sp[0] = make_float4(mv[0], s0.y, mv[1], s0.w);
+            sp[1] = make_float4(mv[2], s1.y, mv[3], s1.w);
+        }
+        return;
+    }
     const float lr = p.votes_out ? 0.f : (*p.d_lr) * p.lr_scale;
     const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd};
     int changes = 0;
@@ -205,5 +224,120 @@ hipError_t egg_launch_swizzle(const int8_t *W, int8_t *Wf, int K, int N, int B, 
     int chunks = K * N / 16;
     hipLaunchKernelGGL(k_swizzle, dim3((chunks + 255) / 256), dim3(256), 0, s, reinterpret_cast<const uint32_t *>(W),
                        reinterpret_cast<v4i *>(Wf), K, N, B, nat);
+    return hipGetLastError();
+}
+
+hipError_t egg_launch_muon_momentum(const UpdParams &p, hipStream_t s) {
+    if (!p.muon_x) return hipErrorInvalidValue;
+    return egg_launch_update_matrix(p, s);
+}
+
+// ---------------------------------------------------------------- Newton-Schulz (muon_internal.cuh:182-342)
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// sum of squares in two deterministic stages (cublasSnrm2 in the reference)
+__global__ void __launch_bounds__(256) k_sumsq_partial(const float *x, int n, float *partials) {
+    __shared__ float sh[256];
+    float s = 0.f;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) { float v = x[i]; s += v * v; }
+    sh[threadIdx.x] = s; __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) { if (threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o]; __syncthreads(); }
+    if (threadIdx.x == 0) partials[blockIdx.x] = sh[0];
+}
+__global__ void __launch_bounds__(256) k_norm_finish(const float *partials, int n, float *norm) {
+    __shared__ float sh[256];
+    float s = 0.f;
+    for (int i = threadIdx.x; i < n; i += 256) s += partials[i];
+    sh[threadIdx.x] = s; __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) { if (threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o]; __syncthreads(); }
+    if (threadIdx.x == 0) norm[0] = sqrtf(sh[0]);
+}
+// muon_scale_by_norm_kernel (muon_internal.cuh:77-87)
+__global__ void k_scale_by_norm(float *x, const float *norm, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) { float nv = *norm; if (nv > 1e-6f) x[i] /= nv; }
+}
+
+// C[M][N] (row-major, ldc = N) = epilogue(sum_k A(i,k) B(k,j)), generic strides, one wave per 32x32 tile on
+// v_mfma_f32_32x32x2_f32.  mode 0: C = alpha * acc.  mode 1: C = (i == j ? 3 : 0) - acc  (3I - G, muon_internal.cuh:91-109).
+__global__ void __launch_bounds__(EGG_THREADS) k_sgemm(const float *A, long sa_i, long sa_k, const float *B, long sb_k, long sb_j,
+                                                      float *C, int M, int N, int K, float alpha, int mode) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int tiles_n = N / 32, tile = blockIdx.x * EGG_WAVES + wave;
+    if (tile >= (M / 32) * tiles_n) return;
+    const int i0 = (tile / tiles_n) * 32, j0 = (tile % tiles_n) * 32;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    const float *ap = A + (long)(i0 + j) * sa_i + (long)g * sa_k;
+    const float *bp = B + (long)g * sb_k + (long)(j0 + j) * sb_j;
+    for (int k = 0; k < K; k += 2) {
+        float a = ap[(long)k * sa_k], b = bp[(long)k * sb_k];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        int i = i0 + ((r >> 2) << 3) + (g << 2) + (r & 3), jj = j0 + j;
+        float v = (mode == 1) ? ((i == jj ? 3.0f : 0.0f) - acc[r]) : alpha * acc[r];
+        C[(size_t)i * N + jj] = v;
+    }
+}
+static void sgemm(const float *A, long sa_i, long sa_k, const float *B, long sb_k, long sb_j, float *C, int M, int N, int K,
+                  float alpha, int mode, hipStream_t s) {
+    int tiles = (M / 32) * (N / 32);
+    hipLaunchKernelGGL(k_sgemm, dim3((tiles + EGG_WAVES - 1) / EGG_WAVES), dim3(EGG_THREADS), 0, s, A, sa_i, sa_k, B, sb_k, sb_j, C, M, N, K, alpha, mode);
+}
+__global__ void k_copy_f32(float *dst, const float *src, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
+hipError_t egg_launch_newton_schulz(const MuonWork &w, int rows, int cols, int iters, hipStream_t s) {
+    if (rows % 32 || cols % 32) return hipErrorInvalidValue;
+    const int n = rows * cols;
+    const bool use_rows = rows < cols;
+    const int K = use_rows ? rows : cols;
+    hipLaunchKernelGGL(k_sumsq_partial, dim3(256), dim3(256), 0, s, w.x, n, w.partials);
+    hipLaunchKernelGGL(k_norm_finish, dim3(1), dim3(256), 0, s, w.partials, 256, w.norm);
+    hipLaunchKernelGGL(k_scale_by_norm, dim3((n + 255) / 256), dim3(256), 0, s, w.x, w.norm, n);
+    for (int it = 0; it < iters; it++) {
+        if (use_rows) {
+            // G = X X^T (rows x rows); X <- 0.5 (3I - G) X
+            sgemm(w.x, cols, 1, w.x, 1, cols, w.bterm, K, K, cols, 1.f, 1, s);
+            sgemm(w.bterm, K, 1, w.x, cols, 1, w.swap, rows, cols, K, 0.5f, 0, s);
+        } else {
+            // G = X^T X (cols x cols); X <- 0.5 X (3I - G)
+            sgemm(w.x, 1, cols, w.x, cols, 1, w.bterm, K, K, rows, 1.f, 1, s);
+            sgemm(w.x, cols, 1, w.bterm, K, 1, w.swap, rows, cols, K, 0.5f, 0, s);
+        }
+        hipLaunchKernelGGL(k_copy_f32, dim3((n + 255) / 256), dim3(256), 0, s, w.x, w.swap, n);
+    }
+    return hipGetLastError();
+}
+
+// muon_apply_update_kernel (muon_internal.cuh:112-170)
+__global__ void __launch_bounds__(256) k_muon_apply(UpdParams p, float wd) {
+    int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    int change = 0;
+    if (idx < p.rows * p.cols) {
+        int byte_off = idx & 3, word = idx >> 2, n = word % p.cols, k = (word / p.cols) * 4 + byte_off;
+        int w = p.W[idx];
+        float *st = p.state + (size_t)idx * 2;
+        float acc = st[1];
+        float u = p.muon_x[(size_t)k * p.cols + n];
+        float lr = (*p.d_lr) * p.lr_scale;
+        float wdw = wd * (float)w;
+        float step = (-lr) * (u + wdw);
+        acc += step;
+        if (acc >= 1.0f) { if (w < 127) { w++; change = 1; acc -= 1.0f; } else acc = 1.0f; }
+        else if (acc <= -1.0f) { if (w > -127) { w--; change = 1; acc += 1.0f; } else acc = -1.0f; }
+        p.W[idx] = (int8_t)w; st[1] = acc;
+    }
+    unsigned long long m = __ballot(change);
+    if ((threadIdx.x & 63) == 0 && m) atomicAdd(p.counter, (unsigned long long)__popcll(m));
+}
+hipError_t egg_launch_muon_apply(const UpdParams &p, float wd, hipStream_t s) {
+    int n = p.rows * p.cols;
+    hipLaunchKernelGGL(k_muon_apply, dim3((n + 255) / 256), dim3(256), 0, s, p, wd);
     return hipGetLastError();
 }

@@ -73,7 +73,10 @@ int64_t egg_model_bytes(const egg_ctx *ctx);
 int  egg_model_init(egg_ctx *ctx, uint32_t seed);                          /* init_model, mgpu.cu:461-519 */
 int  egg_model_upload(egg_ctx *ctx, const void *host_model, size_t bytes); /* load_model + H2D, mgpu.cu:1373,:1461 */
 int  egg_model_download(egg_ctx *ctx, void *host_model, size_t bytes);     /* D2H before save, mgpu.cu:1734 */
-/* optimizer state == the reference's AdamModel: one {m,v,acc} float triple per model byte (mgpu.cu:321-370) */
+/* optimizer state == the reference's AdamModel (mgpu.cu:321-370): in model field order, one {m,v,acc} float triple
+ * per element; with use_muon the 2-D hidden matrices hold {m,acc} pairs instead (HIDDEN_OPT_TYPE, mgpu.cu:327-335) */
+int64_t egg_opt_state_bytes(const egg_ctx *ctx);
+int64_t egg_tensor_state_offset(const egg_ctx *ctx, int tensor_id);   /* byte offset of a tensor's state */
 int  egg_opt_state_upload(egg_ctx *ctx, const void *host_state, size_t bytes);
 int  egg_opt_state_download(egg_ctx *ctx, void *host_state, size_t bytes);
 int  egg_opt_state_reset(egg_ctx *ctx);                                    /* calloc'd AdamModel, mgpu.cu:1367 */
@@ -116,6 +119,10 @@ int  egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t *d_seed, c
 int  egg_update_tensor(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr);
 /* int32 votes of one matrix tensor in blocked element order (mgpu.cu:1092-1098), test hook */
 int  egg_matrix_votes(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const uint32_t *d_seed, int32_t *d_votes);
+
+/* perform_newton_schulz (muon_internal.cuh:182-342) on a row-major fp32 [rows][cols] device matrix, in place:
+ * X /= ||X||_F, then `iters` times X <- 0.5 X (3I - X^T X) on the short side.  Needs a use_muon context. */
+int  egg_newton_schulz(egg_ctx *ctx, float *d_X, int rows, int cols, int iters);
 
 typedef struct egg_tensor_info {
     char    name[32];

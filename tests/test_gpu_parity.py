@@ -272,3 +272,78 @@ def test_error_paths(pkg, dev):
     with pytest.raises(pkg.EggError):
         ctx.model_upload(np.zeros(3, np.int8))
     ctx.close()
+
+
+def test_newton_schulz_gpu(pkg, orc, dev):
+    """fp32 MFMA Newton-Schulz against the fp64 restatement (the reference's cuBLAS summation order is unspecified,
+    so this is a tolerance check: relative Frobenius error <= 1e-5) plus the orthogonality it is meant to reach."""
+    import torch
+    ctx = pkg.Context(pkg.default_config(use_muon=1, hidden=256, head_dim=64, n_layers=1, seq_len=32, population=8))
+    rng = np.random.default_rng(21)
+    for rows, cols in ((256, 256), (256, 1024), (1024, 256), (64, 96)):
+        X = (rng.integers(-300, 301, (rows, cols))).astype(np.float32)
+        ref = X.astype(np.float64)
+        orc.lib().orc_newton_schulz_f64(ref.ctypes.data_as(C.c_void_p), rows, cols, 5)
+        d = _t(dev, X)
+        ctx.newton_schulz(d.data_ptr(), rows, cols, 5)
+        ctx.sync()
+        got = d.cpu().numpy().astype(np.float64)
+        err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+        assert err < 1e-5, (rows, cols, err)
+    ctx.close()
+
+
+def test_muon_update(pkg, orc, dev):
+    """Muon chain per matrix: momentum state is bit-exact (integer votes, two float ops); the orthogonalised step
+    goes through fp32 GEMMs, so weights may differ from the oracle only where an accumulator sits within rounding
+    distance of the +-1 threshold."""
+    import torch
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=120)
+    ocfg = orc.config(**kw)
+    ctx = pkg.Context(pkg.default_config(use_muon=1, **kw))
+    rng = np.random.default_rng(22)
+    pairs = kw["population"] // 2
+    model = orc.init_model(ocfg, 42)
+    ctx.model_upload(model)
+    seed, lr = 777, 40.0          # a large rate so many accumulators cross the threshold
+    d_seed = _t(dev, np.array([seed], np.uint32).view(np.int32))
+    d_lr = _t(dev, np.array([lr], np.float32))
+    st_bytes = ctx.opt_state_download().nbytes
+    tensors = ctx.tensors()
+    assert st_bytes == sum(t["rows"] * t["cols"] * (8 if t["muon"] else 12) for t in tensors)
+    ref_states = {t["id"]: np.zeros(t["rows"] * t["cols"], orc.MUON_DTYPE) for t in tensors if t["muon"]}
+    for step in range(3):
+        fit = rng.integers(-1, 2, pairs).astype(np.int32)
+        d_fit = _t(dev, fit)
+        for t in tensors:
+            if not t["muon"]:
+                continue
+            n = t["rows"] * t["cols"]
+            ctx.update_tensor(t["id"], d_fit.data_ptr(), d_seed.data_ptr(), d_lr.data_ptr())
+            W = model[t["offset"]:t["offset"] + n]
+            st = ref_states[t["id"]]
+            orc.lib().orc_update_matrix_muon(C.byref(ocfg), W.ctypes.data_as(C.c_void_p), st.ctypes.data_as(C.c_void_p),
+                                             t["rows"], t["cols"], t["off_a"], t["off_b"], t["seed_base"],
+                                             fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed), C.c_float(lr), None)
+            got_m = ctx.model_download()[t["offset"]:t["offset"] + n]
+            raw = ctx.opt_state_download().view(np.uint8)
+            off = ctx.tensor_state_offset(t["id"])
+            got_st = raw[off:off + 8 * n].view(orc.MUON_DTYPE)
+            assert np.array_equal(got_st["m"].view(np.int32), st["m"].view(np.int32)), (t["name"], step)
+            diff = np.flatnonzero(got_m != W)
+            # any disagreement must be a threshold crossing decided by float rounding in the GEMMs
+            assert len(diff) <= max(2, n // 500), (t["name"], step, len(diff))
+            for i in diff:
+                assert abs(int(got_m[i]) - int(W[i])) == 1
+            same = got_m == W
+            assert np.allclose(got_st["acc"][same], st["acc"][same], atol=2e-3), t["name"]
+            # keep both sides on the same trajectory for the next step
+            if len(diff):
+                m2 = ctx.model_download(); m2[t["offset"]:t["offset"] + n] = W; ctx.model_upload(m2)
+                raw2 = raw.copy(); raw2[off:off + 8 * n] = st.view(np.uint8); ctx.opt_state_upload(raw2)
+            else:
+                raw2 = raw.copy(); raw2[off:off + 8 * n] = st.view(np.uint8); ctx.opt_state_upload(raw2)
+        seed += 1
+        d_seed.copy_(_t(dev, np.array([seed], np.uint32).view(np.int32)))
+    assert ctx.last_update_count() >= 0
+    ctx.close()
