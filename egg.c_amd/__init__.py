@@ -56,7 +56,7 @@ def build(force=True):
     cmd = ["make", "-C", HERE, "-j8", "-s"]
     if force:
         cmd.append("-B")
-    subprocess.check_call(cmd)
+    subprocess.check_call(cmd + ["all", "host"])
 
 
 _lib = None

@@ -1,0 +1,103 @@
+// egg_train.cpp -- the reference's training loop (full_cuda_train_transformer_adam_mgpu.cu:1313-1767) written
+// against the C ABI of libegg_hip.so: load or synthesise the byte stream, init the model, then per step
+// forward + fitness + update (one egg_step / egg_step_launch), read the update counter and the losses, print
+// the reference's status line.  Differences by design: the step seed is an explicit argument chained with
+// hash_rng (d-eggs/src/worker.cu:542) instead of time(NULL); no remote logging; errors return instead of exit(1)
+// inside the library.
+//
+// usage: egg_train [--data FILE] [--steps N] [--population P] [--seq T] [--hidden H] [--layers L] [--graph]
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+#include <algorithm>
+#include <vector>
+
+#include "../../include/egg_hip.h"
+
+#define CK(call) do { int rc_ = (call); if (rc_ != EGG_OK) { fprintf(stderr, "%s failed (%d): %s\n", #call, rc_, egg_last_error(ctx)); return 1; } } while (0)
+#define HK(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) { fprintf(stderr, "%s: %s\n", #call, hipGetErrorString(e_)); return 1; } } while (0)
+
+// i.i.d. Zipf(s) ranks over a fixed permutation of the 256 byte values; counter-based SplitMix64 -> inverse CDF
+static std::vector<uint8_t> zipf_bytes(size_t n, uint64_t seed, double s) {
+    std::vector<double> cdf(256); double tot = 0;
+    for (int r = 0; r < 256; r++) { tot += 1.0 / pow((double)(r + 1), s); cdf[r] = tot; }
+    for (double &c : cdf) c /= tot;
+    uint8_t perm[256]; for (int i = 0; i < 256; i++) perm[i] = (uint8_t)i;
+    uint32_t st = (uint32_t)((seed * 2654435761ull + 1ull) & 0xffffffffull); if (!st) st = 1;
+    for (int i = 255; i > 0; i--) { st ^= st << 13; st ^= st >> 17; st ^= st << 5; int j = (int)(st % (uint32_t)(i + 1)); std::swap(perm[i], perm[j]); }
+    std::vector<uint8_t> out(n);
+    for (size_t i = 0; i < n; i++) {
+        uint64_t z = seed + (uint64_t)(i + 1) * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull; z = (z ^ (z >> 27)) * 0x94D049BB133111EBull; z ^= z >> 31;
+        double u = (double)(z >> 11) * (1.0 / 9007199254740992.0);
+        int r = (int)(std::upper_bound(cdf.begin(), cdf.end(), u) - cdf.begin());
+        out[i] = perm[r > 255 ? 255 : r];
+    }
+    return out;
+}
+
+int main(int argc, char **argv) {
+    egg_config cfg; egg_default_config(&cfg);
+    cfg.seq_len = 256; cfg.population = 40960;
+    const char *data_file = nullptr; long steps = 10; bool graph = false; size_t synth_bytes = 64u << 20;
+    for (int i = 1; i < argc; i++) {
+        auto next = [&](const char *name) -> const char * { if (i + 1 >= argc) { fprintf(stderr, "%s needs a value\n", name); exit(2); } return argv[++i]; };
+        if (!strcmp(argv[i], "--data")) data_file = next("--data");
+        else if (!strcmp(argv[i], "--steps")) steps = atol(next("--steps"));
+        else if (!strcmp(argv[i], "--population")) cfg.population = atoi(next("--population"));
+        else if (!strcmp(argv[i], "--seq")) cfg.seq_len = atoi(next("--seq"));
+        else if (!strcmp(argv[i], "--hidden")) cfg.hidden = atoi(next("--hidden"));
+        else if (!strcmp(argv[i], "--layers")) cfg.n_layers = atoi(next("--layers"));
+        else if (!strcmp(argv[i], "--muon")) cfg.use_muon = 1;
+        else if (!strcmp(argv[i], "--graph")) graph = true;
+        else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
+    }
+    std::vector<uint8_t> data;
+    if (data_file) {
+        FILE *f = fopen(data_file, "rb");
+        if (!f) { fprintf(stderr, "cannot open %s\n", data_file); return 1; }
+        fseek(f, 0, SEEK_END); long len = ftell(f); fseek(f, 0, SEEK_SET);
+        data.resize((size_t)len);
+        if (fread(data.data(), 1, (size_t)len, f) != (size_t)len) { fprintf(stderr, "short read\n"); return 1; }
+        fclose(f);
+    } else {
+        data = zipf_bytes(synth_bytes, 1234, 1.1);
+    }
+    printf("data: %zu bytes (%s)\n", data.size(), data_file ? data_file : "synthetic Zipf(1.1)");
+
+    egg_ctx *ctx = nullptr;
+    int rc = egg_ctx_create(&cfg, &ctx);
+    if (rc != EGG_OK) { fprintf(stderr, "egg_ctx_create failed (%d): unsupported configuration or no GPU\n", rc); return 1; }
+    CK(egg_model_init(ctx, 42));
+    uint8_t *d_data = nullptr;
+    HK(hipMalloc(&d_data, data.size()));
+    HK(hipMemcpy(d_data, data.data(), data.size(), hipMemcpyHostToDevice));
+    if (graph) CK(egg_step_capture(ctx, d_data, (int64_t)data.size()));
+
+    std::vector<int32_t> loss((size_t)cfg.population), fit((size_t)cfg.population / 2);
+    uint32_t seed = 42;
+    long max_steps = (long)((data.size() - 1) / (size_t)cfg.seq_len);
+    for (long step = 0; step < steps && step < max_steps; step++) {
+        struct timespec t0, t1; clock_gettime(CLOCK_MONOTONIC, &t0);
+        float lr = egg_learning_rate(step);
+        if (graph) CK(egg_step_launch(ctx, step * cfg.seq_len, seed, lr));
+        else CK(egg_step(ctx, d_data, (int64_t)data.size(), step * cfg.seq_len, seed, lr));
+        uint64_t updates = 0;
+        CK(egg_last_update_count(ctx, &updates));          // synchronises, like the reference's cudaMemcpy of d_total_updates
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        CK(egg_step_losses(ctx, loss.data(), fit.data()));
+        double ms = (t1.tv_sec - t0.tv_sec) * 1e3 + (t1.tv_nsec - t0.tv_nsec) / 1e6;
+        long long total = 0; for (int32_t l : loss) total += l;
+        double avg = (double)total / ((double)cfg.population * cfg.seq_len * 16.0);
+        printf("Step %ld | Loss: %.4f | Time: %.2f ms | Updates: %llu | Speed: %.2f tok/s | LR: %.3f\n", step, avg, ms,
+               (unsigned long long)updates, (double)cfg.population * cfg.seq_len / (ms / 1e3), lr);
+        seed = egg_next_seed(seed, (uint64_t)(step + 1));
+    }
+    (void)hipFree(d_data);
+    egg_ctx_destroy(ctx);
+    return 0;
+}

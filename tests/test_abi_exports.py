@@ -1,0 +1,47 @@
+"""CPU checks of the drop-in boundary: the C-ABI library loads without a GPU and exports every function that
+include/egg_hip.h declares; nothing under the product package touches the oracle."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "egg_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(egg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    lib = pkg.lib()
+    names = declared_functions()
+    assert len(names) > 30
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    assert set(pkg.EXPORTS) <= set(names), sorted(set(pkg.EXPORTS) - set(names))
+
+
+def test_default_config_matches_reference_defaults(pkg):
+    c = pkg.default_config()
+    assert (c.hidden, c.head_dim, c.n_layers, c.vocab) == (256, 64, 4, 256)
+    assert (c.fixed_point, c.sigma_shift, c.sigma_shift_vector) == (4, 3, 4)
+    assert (c.shift_attn, c.shift_out, c.shift_logit, c.shift_mlp_up, c.shift_mlp_down) == (8, 9, 8, 8, 10)
+    assert c.softmax_scale_bit == 18 and c.rope_scale_bit == 20 and c.noise_mask == 15
+    assert abs(c.adam_beta1 - 0.9) < 1e-7 and abs(c.adam_beta2 - 0.95) < 1e-7 and abs(c.muon_momentum - 0.85) < 1e-7
+    assert pkg.learning_rate(0) == ctypes.c_float(0.3).value and pkg.learning_rate(1000) == ctypes.c_float(0.05).value
+    # d-eggs seed chain == murmur3 fmix32(seed + step * golden)
+    assert pkg.next_seed(42, 0) == 0x087FCD5C and pkg.next_seed(42, 1) == 0x3805EA2C
+
+
+def test_product_sources_do_not_reference_the_oracle():
+    bad = []
+    for base, _, files in os.walk(os.path.join(ROOT, "egg.c_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp", "Makefile")):
+                txt = open(os.path.join(base, f), errors="ignore").read()
+                if "oracle" in txt.lower() and f != "__init__.py":
+                    bad.append(f)
+                if f == "__init__.py" and re.search(r"import\s+oracle|oracle_py|libegg_oracle", txt):
+                    bad.append(f)
+    assert not bad, bad
