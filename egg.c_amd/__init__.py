@@ -47,6 +47,9 @@ EXPORTS = [
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
     "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz",
+    "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
+    "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
+    "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
 ]
 KCLASSES = ["mlp_first", "qkv", "attn", "mlp", "head", "update_matrix", "update_vector", "plinear"]
 
@@ -113,6 +116,21 @@ def lib():
         L.egg_tensor_state_offset.restype = i64
         L.egg_tensor_state_offset.argtypes = [vp, i32]
         L.egg_newton_schulz.argtypes = [vp, vp, i32, i32, i32]
+        L.egg_gru_default_config.argtypes = [vp]
+        L.egg_gru_create.argtypes = [vp, vp]
+        L.egg_gru_destroy.argtypes = [vp]
+        L.egg_gru_destroy.restype = None
+        L.egg_gru_last_error.restype = C.c_char_p
+        L.egg_gru_last_error.argtypes = [vp]
+        L.egg_gru_model_bytes.restype = i64
+        L.egg_gru_model_bytes.argtypes = [vp]
+        L.egg_gru_model_init.argtypes = [vp, u32]
+        L.egg_gru_model_upload.argtypes = [vp, vp, C.c_size_t]
+        L.egg_gru_model_download.argtypes = [vp, vp, C.c_size_t]
+        L.egg_gru_state_reset.argtypes = [vp]
+        L.egg_gru_state_download.argtypes = [vp, vp, C.c_size_t]
+        L.egg_gru_step.argtypes = [vp, vp, i64, i64, u32, i32]
+        L.egg_gru_losses.argtypes = [vp, vp, vp]
         _lib = L
     return _lib
 
@@ -302,3 +320,80 @@ def learning_rate(step):
 
 def next_seed(seed, step):
     return int(lib().egg_next_seed(seed & 0xFFFFFFFF, step))
+
+
+class EggGruConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("hidden", "n_layers", "seq_len", "vocab", "population",
+                                       "fixed_point", "sigma_shift", "update_threshold")]
+
+
+def gru_default_config(**kw):
+    c = EggGruConfig()
+    lib().egg_gru_default_config(C.byref(c))
+    for k, v in kw.items():
+        if not hasattr(c, k):
+            raise KeyError(k)
+        setattr(c, k, v)
+    return c
+
+
+class GruContext:
+    """The reference's CPU program (full_trained_egg.c) on the GPU: model, recurrent states and one-step driver."""
+
+    def __init__(self, cfg):
+        self.cfg = cfg
+        self._h = C.c_void_p()
+        rc = lib().egg_gru_create(C.byref(cfg), C.byref(self._h))
+        if rc != 0:
+            raise EggError(f"egg_gru_create failed with {rc} (unsupported configuration or HIP error)")
+
+    def close(self):
+        if self._h:
+            lib().egg_gru_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _ck(self, rc, what):
+        if rc != 0:
+            raise EggError(f"{what} failed with {rc}: {lib().egg_gru_last_error(self._h).decode()}")
+
+    def model_bytes(self):
+        return int(lib().egg_gru_model_bytes(self._h))
+
+    def model_init(self, seed=42):
+        self._ck(lib().egg_gru_model_init(self._h, seed), "egg_gru_model_init")
+
+    def model_upload(self, arr):
+        self._ck(lib().egg_gru_model_upload(self._h, _np_ptr(arr), arr.nbytes), "egg_gru_model_upload")
+
+    def model_download(self):
+        import numpy as np
+        out = np.zeros(self.model_bytes(), np.int8)
+        self._ck(lib().egg_gru_model_download(self._h, _np_ptr(out), out.nbytes), "egg_gru_model_download")
+        return out
+
+    def state_reset(self):
+        self._ck(lib().egg_gru_state_reset(self._h), "egg_gru_state_reset")
+
+    def state_download(self):
+        import numpy as np
+        c = self.cfg
+        out = np.zeros(c.population * c.n_layers * c.hidden, np.int8)
+        self._ck(lib().egg_gru_state_download(self._h, _np_ptr(out), out.nbytes), "egg_gru_state_download")
+        return out
+
+    def step(self, d_data, data_len, start_idx, step_seed, do_update=True):
+        self._ck(lib().egg_gru_step(self._h, C.c_void_p(d_data), data_len, start_idx, step_seed & 0xFFFFFFFF,
+                                    1 if do_update else 0), "egg_gru_step")
+
+    def losses(self):
+        import numpy as np
+        loss = np.zeros(self.cfg.population, np.int32)
+        fit = np.zeros(self.cfg.population // 2, np.int32)
+        self._ck(lib().egg_gru_losses(self._h, _np_ptr(loss), _np_ptr(fit)), "egg_gru_losses")
+        return loss, fit

@@ -1,0 +1,558 @@
+// egg_gru.hip -- the reference's CPU program (full_trained_egg.c, "egg.c": GRU-style recurrent byte LM with
+// sequential-xorshift rank-1 noise and the +-1 threshold update) on gfx950.
+//
+// The model is recurrent, so tokens are serial; the GEMM's free dimension is the population.  A workgroup of 16
+// waves owns 32 members (16 antithetic pairs): every perturbed matmul (egg.c:108-177) is one
+// v_mfma_i32_32x32x32_i8 strip per wave (A operand = 32 output rows of W read straight from the fragment-major
+// copy in L2, B operand = the 32 members' input vectors in LDS), output rows are split over the waves and the
+// int8 results go back to LDS as the next matmul's input.  Noise vectors of all (pair, matrix) are generated once
+// per step by replaying the reference's xorshift stream (4 discarded draws per block of 16, egg.c:87-105).
+#include "egg_device.h"
+#include "egg_launch.h"
+#include "../../include/egg_hip.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+#include <string>
+#include <vector>
+
+#define GRU_WAVES 16
+#define GRU_THREADS (GRU_WAVES * 64)
+
+struct GruMat {            // one weight matrix, W[rows = out][cols = in] row-major (egg.c:42-50)
+    long long w_off;       // byte offset in the model blob (and in the fragment copy)
+    int rows, cols;
+    long long a_off, b_off;   // offsets of the per-pair noise vectors (slot order), [pair][rows] / [pair][cols]
+    long long pa_off, pb_off; // offsets of the update panels [rows][pairs_pad] / [cols][pairs_pad]
+    int seed_off;          // 100*l + k, or 999 for the head (egg.c:242-290)
+    int shift;
+};
+
+struct GruParams {
+    const GruMat *mats;
+    const int8_t *model;      // canonical blob (embedding, biases, ln weights)
+    const int8_t *frag;       // fragment-major copies of the matrices
+    const int8_t *noise;      // per-pair noise vectors
+    const uint8_t *data; long long data_len; long long start_idx;
+    int8_t *states;           // [population][L][H]
+    int32_t *loss;            // [population]
+    int H, L, T, V, population, sigma;   // sigma = fixed_point + sigma_shift
+    long long off_emb, off_gru_b, off_ln_w, off_ln_out;
+    const int32_t *exp2;      // [256]
+};
+
+__device__ __forceinline__ uint32_t xorshift32(uint32_t &x) { x ^= x << 13; x ^= x >> 17; x ^= x << 5; return x; }
+__device__ __forceinline__ int slot_pos(int n) { int w = n & 31; return (n & ~31) + 16 * ((w >> 2) & 1) + 4 * (w >> 3) + (w & 3); }
+
+// gen_noise_vector_neon (egg.c:87-105) for every (matrix, pair): A[rows] then B[cols] from one stream seeded
+// step_seed + pair + seed_off.  Writes the vectors in slot order for the forward and the raw panels for the vote.
+__global__ void k_gru_noise(const GruMat *mats, int n_mats, int pairs, int pairs_pad, uint32_t step_seed,
+                            int8_t *noise, int8_t *panels) {
+    int id = blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= n_mats * pairs) return;
+    const GruMat m = mats[id / pairs]; const int p = id % pairs;
+    uint32_t rng = step_seed + (uint32_t)p + (uint32_t)m.seed_off;
+    for (int part = 0; part < 2; part++) {
+        const int count = part ? m.cols : m.rows;
+        int8_t *vec = noise + (part ? m.b_off + (long long)p * m.cols : m.a_off + (long long)p * m.rows);
+        int8_t *pan = panels + (part ? m.pb_off : m.pa_off);
+        for (int i = 0; i < count; i += 16) {
+            xorshift32(rng); xorshift32(rng); xorshift32(rng); xorshift32(rng);
+            for (int jj = 0; jj < 16 && i + jj < count; jj++) {
+                uint32_t r = xorshift32(rng);
+                int v = (int)((r >> 1) & 31u); if (!(r & 1)) v = -v;
+                vec[slot_pos(i + jj)] = (int8_t)v;
+                pan[(long long)(i + jj) * pairs_pad + p] = (int8_t)v;
+            }
+        }
+    }
+}
+
+// W[rows][cols] row-major -> [rows/32][cols/16][32][16 B]: entry (nt, 2ks+g, i) holds W[32nt+i][32ks + 8q+4g+e]
+__global__ void k_gru_swizzle(const int8_t *W, int8_t *F, int rows, int cols) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= rows * cols / 16) return;
+    int i = c & 31, p = (c >> 5) % (cols / 16), nt = (c >> 5) / (cols / 16), ks = p >> 1, g = p & 1;
+    const int *src = reinterpret_cast<const int *>(W + (size_t)(32 * nt + i) * cols + 32 * ks);
+    v4i v;
+#pragma unroll
+    for (int q = 0; q < 4; q++) v[q] = src[2 * q + g];
+    reinterpret_cast<v4i *>(F)[c] = v;
+}
+
+// one 32-row strip: acc += W[32nt.., :] . in, in = LDS [32 members][K (+16 pad)] in slot order
+template <int DUMMY = 0>
+__device__ __forceinline__ void gru_strip(v16i &acc, const int8_t *ftile, const int8_t *ldsB, int K, int lane) {
+    const int i = lane & 31, g = lane >> 5, stride = K + 16;
+    for (int ks = 0; ks < K / 32; ks++) {
+        v4i a = *reinterpret_cast<const v4i *>(ftile + ((size_t)(2 * ks + g) * 32 + i) * 16);
+        v4i b = *reinterpret_cast<const v4i *>(ldsB + (size_t)i * stride + 32 * ks + 16 * g);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+    }
+}
+// xB = sum_c in[c] * B[c] for the lane's member (egg.c:122-140)
+__device__ __forceinline__ int gru_xb(const int8_t *ldsB, const int8_t *bvec, int K, int lane) {
+    const int j = lane & 31, g = lane >> 5, stride = K + 16;
+    int s = 0;
+    for (int ks = 0; ks < K / 32; ks++) {
+        v4i b = *reinterpret_cast<const v4i *>(ldsB + (size_t)j * stride + 32 * ks + 16 * g);
+        v4i n = *reinterpret_cast<const v4i *>(bvec + 32 * ks + 16 * g);
+#pragma unroll
+        for (int q = 0; q < 4; q++) s = dot4(b[q], n[q], s);
+    }
+    return s + other_half(s);
+}
+// rank-1 term, shift and clamp of one strip (egg.c:167-175); returns the 16 int8 results packed in slot order
+__device__ __forceinline__ v4i gru_finish(const v16i &acc, int xb, const int8_t *avec, int nt, int ns, int sigma, int shift, int g) {
+    v4i a4 = *reinterpret_cast<const v4i *>(avec + 32 * nt + 16 * g);
+    v4i out;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        int o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            int noise = (xb * sx8(a4[q], e)) * ns;
+            o[e] = clip127((acc[4 * q + e] + (noise >> sigma)) >> shift);
+        }
+        out[q] = pack4(o[0], o[1], o[2], o[3]);
+    }
+    return out;
+}
+__device__ __forceinline__ int cadd(int a, int b) { return clip127(a + b); }   // clipped_add, egg.c:62-67
+
+template <int H>
+__global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
+    constexpr int NTH = H / 32;                 // strips of an H-wide output
+    constexpr int NT4 = 4 * H / 32;
+    constexpr int MAXT4 = (NT4 + GRU_WAVES - 1) / GRU_WAVES;
+    constexpr int SH = H + 16, S4 = 4 * H + 16; // padded LDS row strides
+    extern __shared__ __align__(16) int8_t smem[];
+    int8_t *XN = smem, *HB = XN + 32 * SH, *MB = HB + 32 * SH;
+    int *psum = reinterpret_cast<int *>(MB + 32 * S4);          // [GRU_WAVES][32]
+    int *tl = psum + GRU_WAVES * 32;                            // [32]
+    int *lut = tl + 32;                                         // [256]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const bool own = wave < NTH;
+    const int member = blockIdx.x * 32 + j, pair = member >> 1, ns = (member & 1) ? -1 : 1;
+    const int L = p.L, V = p.V;
+    for (int i = threadIdx.x; i < 256; i += GRU_THREADS) lut[i] = p.exp2[i];
+
+    // stream position of the pair (egg.c:553-554)
+    const long long stride = p.data_len / (p.population / 2);
+    const long long spos = (p.start_idx + (long long)pair * stride) % (p.data_len - p.T);
+
+    // the recurrent state (egg.c:515-517, persists across steps) stays in global memory; a lane re-reads and
+    // rewrites only the 16 bytes of its own strip, once per layer and token
+    int loss = 0;
+    __syncthreads();
+
+    auto put = [&](int8_t *buf, int strideb, int nt, v4i v) { *reinterpret_cast<v4i *>(buf + (size_t)j * strideb + 32 * nt + 16 * g) = v; };
+    // egg_ln (egg.c:180-210) of the H-wide vector whose own strip is x; result packed
+    auto layer_norm = [&](v4i x, const int8_t *w) -> v4i {
+        int part = 0;
+        if (own) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) part = sumabs4(x[q], part);
+            part += other_half(part);
+            if (g == 0) psum[wave * 32 + j] = part;
+        }
+        __syncthreads();
+        int sum = 0;
+        for (int w2 = 0; w2 < NTH; w2++) sum += psum[w2 * 32 + j];
+        if (sum == 0) sum = 1;
+        int mean = sum / H; if (mean == 0) mean = 1;
+        const float rcp = 1.0f / (float)mean;
+        v4i out = {0, 0, 0, 0};
+        if (own) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int w4 = *reinterpret_cast<const int *>(w + 32 * wave + 8 * q + 4 * g);
+                int o[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(sx8(x[q], e) * sx8(w4, e), rcp));
+                out[q] = pack4(o[0], o[1], o[2], o[3]);
+            }
+        }
+        return out;
+    };
+    // perturbed matmul of an H-wide output: the own strip's packed result
+    auto matmul_h = [&](int mi, const int8_t *in, int K) -> v4i {
+        v4i r = {0, 0, 0, 0};
+        if (own) {
+            const GruMat m = p.mats[mi];
+            const int xb = gru_xb(in, p.noise + m.b_off + (long long)pair * K, K, lane);
+            v16i acc;
+#pragma unroll
+            for (int t = 0; t < 16; t++) acc[t] = 0;
+            gru_strip(acc, p.frag + m.w_off + (size_t)wave * 32 * K, in, K, lane);
+            r = gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, wave, ns, p.sigma, m.shift, g);
+        }
+        return r;
+    };
+
+    for (int t = 0; t < p.T; t++) {
+        const int tok = p.data[spos + t];
+        v4i x = {0, 0, 0, 0}, resid = {0, 0, 0, 0};
+        if (own) {
+            const int *e = reinterpret_cast<const int *>(p.model + p.off_emb + (size_t)tok * H + 32 * wave);
+#pragma unroll
+            for (int q = 0; q < 4; q++) x[q] = e[2 * q + g];
+        }
+        for (int l = 0; l < L; l++) {
+            const int8_t *lnw = p.model + p.off_ln_w + (size_t)l * 2 * H;
+            const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
+            resid = x;
+            int *hptr = reinterpret_cast<int *>(p.states + ((size_t)member * L + l) * H + 32 * wave);
+            v4i hcur = {0, 0, 0, 0};
+            if (own)
+#pragma unroll
+                for (int q = 0; q < 4; q++) hcur[q] = hptr[2 * q + g];
+            v4i xn = layer_norm(x, lnw);
+            if (own) { put(XN, SH, wave, xn); put(HB, SH, wave, hcur); }
+            __syncthreads();
+            v4i b1 = matmul_h(6 * l + 0, XN, H);
+            v4i b2 = matmul_h(6 * l + 1, HB, H);
+            v4i ft = {0, 0, 0, 0}, gated = {0, 0, 0, 0};
+            if (own) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int bf4 = *reinterpret_cast<const int *>(gb + 32 * wave + 8 * q + 4 * g);
+                    int f[4], gp[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        f[e] = cadd(cadd(sx8(b1[q], e), sx8(b2[q], e)), sx8(bf4, e));
+                        gp[e] = ((f[e] + 127) * sx8(hcur[q], e)) >> 8;
+                    }
+                    ft[q] = pack4(f[0], f[1], f[2], f[3]); gated[q] = pack4(gp[0], gp[1], gp[2], gp[3]);
+                }
+            }
+            __syncthreads();                       // every wave has finished reading HB (old state)
+            if (own) put(HB, SH, wave, gated);
+            __syncthreads();
+            b1 = matmul_h(6 * l + 2, XN, H);
+            b2 = matmul_h(6 * l + 3, HB, H);
+            if (own) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int bh4 = *reinterpret_cast<const int *>(gb + H + 32 * wave + 8 * q + 4 * g);
+                    int hn[4], xo[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        int ht = cadd(cadd(sx8(b1[q], e), sx8(b2[q], e)), sx8(bh4, e));
+                        int hv = sx8(hcur[q], e);
+                        int upd = ((sx8(ft[q], e) + 127) * (ht - hv)) >> 8;
+                        hn[e] = cadd(hv, upd);
+                        xo[e] = cadd(hn[e], sx8(resid[q], e));
+                    }
+                    hptr[2 * q + g] = pack4(hn[0], hn[1], hn[2], hn[3]); x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
+                }
+            }
+            // MLP (egg.c:273-285)
+            resid = x;
+            xn = layer_norm(x, lnw + H);             // its barrier also orders the XN reads above before the write below
+            if (own) put(XN, SH, wave, xn);
+            __syncthreads();
+            {
+                const GruMat m = p.mats[6 * l + 4];
+                const int xb = gru_xb(XN, p.noise + m.b_off + (long long)pair * H, H, lane);
+                for (int ti = 0; ti < MAXT4; ti++) {
+                    const int nt = wave + GRU_WAVES * ti;
+                    if (nt < NT4) {
+                        v16i acc;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[r] = 0;
+                        gru_strip(acc, p.frag + m.w_off + (size_t)nt * 32 * H, XN, H, lane);
+                        put(MB, S4, nt, gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g));
+                    }
+                }
+            }
+            __syncthreads();
+            v4i pr = matmul_h(6 * l + 5, MB, 4 * H);
+            if (own)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int xo[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) xo[e] = cadd(sx8(pr[q], e), sx8(resid[q], e));
+                    x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
+                }
+        }
+        // head + loss (egg.c:288-294, :321-330)
+        v4i xn = layer_norm(x, p.model + p.off_ln_out);
+        if (own) put(XN, SH, wave, xn);
+        __syncthreads();
+        const int target = p.data[spos + t + 1];
+        int part = 0;
+        if (wave < V / 32) {
+            const GruMat m = p.mats[6 * L];
+            const int xb = gru_xb(XN, p.noise + m.b_off + (long long)pair * H, H, lane);
+            v16i acc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = 0;
+            gru_strip(acc, p.frag + m.w_off + (size_t)wave * 32 * H, XN, H, lane);
+            v4i lg = gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, wave, ns, p.sigma, m.shift, g);
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int v = sx8(lg[q], e);
+                    part += lut[v + 128];
+                    if (32 * wave + 8 * q + 4 * g + e == target) tl[j] = v;
+                }
+            part += other_half(part);
+        }
+        if (g == 0) psum[wave * 32 + j] = part;
+        __syncthreads();
+        {
+            int sum_exp = 0;
+            for (int w2 = 0; w2 < V / 32; w2++) sum_exp += psum[w2 * 32 + j];
+            // log2_fixed (egg.c:309-319)
+            int lg2 = 0;
+            if (sum_exp > 0) {
+                int k = 31 - __clz(sum_exp);
+                int frac = (k >= 4) ? ((sum_exp - (1 << k)) >> (k - 4)) : ((sum_exp - (1 << k)) << (4 - k));
+                lg2 = (k << 4) + frac - 64;
+            }
+            loss += lg2 - (tl[j] + 128);
+        }
+        __syncthreads();                           // psum is rewritten by the next token's first norm
+    }
+    if (wave == 0 && g == 0) p.loss[member] = loss;
+}
+
+// A panel *= fitness of the pair (A_T[r][p] = A[r] * f, egg.c:362-366)
+__global__ void k_gru_scale_panel(int8_t *panel, long long n, int pairs_pad, int pairs, const int32_t *fit) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int pp = (int)(i % pairs_pad);
+    panel[i] = (pp < pairs) ? (int8_t)(panel[i] * fit[pp]) : (int8_t)0;
+}
+
+// update_matrix (egg.c:332-409): vote[r][c] = sum_p A_T[r][p] B_T[c][p] on the MFMA, then the +-1 threshold rule
+__global__ void __launch_bounds__(256) k_gru_vote_update(int8_t *W, const int8_t *pa, const int8_t *pb, int rows, int cols,
+                                                        int pairs_pad, int threshold) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int tiles_c = cols / 32, tile = blockIdx.x * 4 + wave;
+    if (tile >= (rows / 32) * tiles_c) return;
+    const int r0 = (tile / tiles_c) * 32, c0 = (tile % tiles_c) * 32;
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+    for (int s = 0; s < pairs_pad; s += 32) {
+        v4i a = *reinterpret_cast<const v4i *>(pb + (size_t)(c0 + j) * pairs_pad + s + 16 * g);   // rows of the MFMA = input index c
+        v4i b = *reinterpret_cast<const v4i *>(pa + (size_t)(r0 + j) * pairs_pad + s + 16 * g);   // columns = output row r
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+    }
+    // lane (r = r0 + j, half g), register 4q+e -> c = c0 + 8q + 4g + e
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        int *wp = reinterpret_cast<int *>(W + (size_t)(r0 + j) * cols + c0 + 8 * q + 4 * g);
+        int w4 = *wp, o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            int w = sx8(w4, e), vote = acc[4 * q + e];
+            if (vote > threshold && w < 127) w++;
+            else if (vote < -threshold && w > -127) w--;
+            o[e] = w;
+        }
+        *wp = pack4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------- host side / C ABI
+struct egg_gru_ctx {
+    egg_gru_config cfg;
+    hipStream_t stream = nullptr;
+    std::vector<GruMat> mats;
+    long long model_bytes = 0, noise_bytes = 0, panel_bytes = 0, off_emb = 0, off_gru_w = 0, off_gru_b = 0, off_mlp_w = 0,
+              off_head = 0, off_ln_w = 0, off_ln_out = 0;
+    int pairs_pad = 0;
+    int8_t *d_model = nullptr, *d_frag = nullptr, *d_noise = nullptr, *d_panels = nullptr, *d_states = nullptr;
+    GruMat *d_mats = nullptr; int32_t *d_loss = nullptr, *d_fit = nullptr, *d_exp2 = nullptr;
+    std::string err;
+};
+static int gfail(egg_gru_ctx *c, int code, const char *what, hipError_t e = hipSuccess) {
+    if (c) { c->err = what; if (e != hipSuccess) { c->err += ": "; c->err += hipGetErrorString(e); } }
+    return code;
+}
+#define GTRY(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return gfail(ctx, EGG_E_HIP, #call, e_); } while (0)
+
+extern "C" void egg_gru_default_config(egg_gru_config *c) {
+    c->hidden = 512; c->n_layers = 4; c->seq_len = 4096; c->vocab = 256; c->population = 128;
+    c->fixed_point = 4; c->sigma_shift = 4; c->update_threshold = 160;
+}
+
+static size_t gru_lds_bytes(int H) { return (size_t)32 * (H + 16) * 2 + (size_t)32 * (4 * H + 16) + (GRU_WAVES * 32 + 32 + 256) * 4; }
+
+template <int H>
+static hipError_t gru_prepare() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(&k_gru_forward<H>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)gru_lds_bytes(H));
+}
+
+static int gru_refresh_frag(egg_gru_ctx *ctx) {
+    for (const GruMat &m : ctx->mats) {
+        int chunks = m.rows * m.cols / 16;
+        hipLaunchKernelGGL(k_gru_swizzle, dim3((chunks + 255) / 256), dim3(256), 0, ctx->stream, ctx->d_model + m.w_off,
+                           ctx->d_frag + m.w_off, m.rows, m.cols);
+    }
+    GTRY(hipGetLastError());
+    return EGG_OK;
+}
+
+extern "C" int egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out) {
+    if (!cfg || !out) return EGG_E_INVALID;
+    *out = nullptr;
+    const egg_gru_config &c = *cfg;
+    if (!(c.hidden == 64 || c.hidden == 128 || c.hidden == 256 || c.hidden == 512)) return EGG_E_INVALID;
+    if (c.vocab != 256 || c.n_layers < 1 || c.n_layers > 8 || c.population < 32 || c.population % 32 || c.seq_len < 1) return EGG_E_INVALID;
+    egg_gru_ctx *ctx = new egg_gru_ctx(); ctx->cfg = c;
+    const long long H = c.hidden, V = c.vocab, L = c.n_layers;
+    long long o = 0;
+    ctx->off_emb = o; o += V * H;
+    ctx->off_gru_w = o; o += L * 4 * H * H;
+    ctx->off_gru_b = o; o += L * 2 * H;
+    ctx->off_mlp_w = o; o += L * 2 * H * 4 * H;
+    ctx->off_head = o; o += H * V;
+    ctx->off_ln_w = o; o += L * 2 * H;
+    ctx->off_ln_out = o; o += H;
+    ctx->model_bytes = o;
+    const int pairs = c.population / 2;
+    ctx->pairs_pad = (pairs + 31) / 32 * 32;
+    long long no = 0, po = 0;
+    auto add = [&](long long w_off, int rows, int cols, int seed_off, int shift) {
+        GruMat m; m.w_off = w_off; m.rows = rows; m.cols = cols; m.seed_off = seed_off; m.shift = shift;
+        m.a_off = no; no += (long long)pairs * rows; m.b_off = no; no += (long long)pairs * cols;
+        m.pa_off = po; po += (long long)rows * ctx->pairs_pad; m.pb_off = po; po += (long long)cols * ctx->pairs_pad;
+        ctx->mats.push_back(m);
+    };
+    for (int l = 0; l < L; l++) {
+        for (int g = 0; g < 4; g++) add(ctx->off_gru_w + ((long long)l * 4 + g) * H * H, (int)H, (int)H, 100 * l + 1 + g, 8);
+        add(ctx->off_mlp_w + ((long long)l * 2) * H * 4 * H, (int)(4 * H), (int)H, 100 * l + 5, 8);
+        add(ctx->off_mlp_w + ((long long)l * 2 + 1) * H * 4 * H, (int)H, (int)(4 * H), 100 * l + 6, 9);
+    }
+    add(ctx->off_head, (int)V, (int)H, 999, 8);
+    ctx->noise_bytes = no; ctx->panel_bytes = po;
+    auto bail = [&](const char *what, hipError_t e) { fprintf(stderr, "egg_gru_create: %s: %s\n", what, hipGetErrorString(e)); delete ctx; return EGG_E_HIP; };
+#define CR(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return bail(#call, e_); } while (0)
+    CR(hipStreamCreate(&ctx->stream));
+    switch (c.hidden) {
+        case 64: CR(gru_prepare<64>()); break;
+        case 128: CR(gru_prepare<128>()); break;
+        case 256: CR(gru_prepare<256>()); break;
+        default: CR(gru_prepare<512>()); break;
+    }
+    CR(hipMalloc(&ctx->d_model, ctx->model_bytes)); CR(hipMemset(ctx->d_model, 0, ctx->model_bytes));
+    CR(hipMalloc(&ctx->d_frag, ctx->model_bytes));
+    CR(hipMalloc(&ctx->d_noise, ctx->noise_bytes)); CR(hipMalloc(&ctx->d_panels, ctx->panel_bytes));
+    CR(hipMemset(ctx->d_panels, 0, ctx->panel_bytes));
+    CR(hipMalloc(&ctx->d_states, (size_t)c.population * L * H)); CR(hipMemset(ctx->d_states, 0, (size_t)c.population * L * H));
+    CR(hipMalloc(&ctx->d_mats, ctx->mats.size() * sizeof(GruMat)));
+    CR(hipMemcpy(ctx->d_mats, ctx->mats.data(), ctx->mats.size() * sizeof(GruMat), hipMemcpyHostToDevice));
+    CR(hipMalloc(&ctx->d_loss, (size_t)c.population * 4)); CR(hipMalloc(&ctx->d_fit, (size_t)pairs * 4));
+    int32_t ex[256];
+    for (int i = 0; i < 256; i++) ex[i] = (int32_t)(pow(2.0, (double)i / (1 << c.fixed_point)) * (1 << c.fixed_point));   // egg.c:57-60
+    CR(hipMalloc(&ctx->d_exp2, 1024)); CR(hipMemcpy(ctx->d_exp2, ex, 1024, hipMemcpyHostToDevice));
+#undef CR
+    *out = ctx;
+    return EGG_OK;
+}
+extern "C" void egg_gru_destroy(egg_gru_ctx *ctx) {
+    if (!ctx) return;
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    void *ptrs[] = {ctx->d_model, ctx->d_frag, ctx->d_noise, ctx->d_panels, ctx->d_states, ctx->d_mats, ctx->d_loss, ctx->d_fit, ctx->d_exp2};
+    for (void *q : ptrs) if (q) (void)hipFree(q);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+extern "C" const char *egg_gru_last_error(const egg_gru_ctx *ctx) { return ctx ? ctx->err.c_str() : "null context"; }
+extern "C" int64_t egg_gru_model_bytes(const egg_gru_ctx *ctx) { return ctx ? ctx->model_bytes : 0; }
+
+// model init of egg.c:487-509: one xorshift32 stream, noise magnitude mask 31
+extern "C" int egg_gru_model_init(egg_gru_ctx *ctx, uint32_t seed) {
+    if (!ctx) return EGG_E_INVALID;
+    const long long H = ctx->cfg.hidden, V = ctx->cfg.vocab, L = ctx->cfg.n_layers;
+    std::vector<int8_t> m((size_t)ctx->model_bytes, 0);
+    uint32_t rng = seed;
+    auto draw = [&]() { uint32_t x = rng; x ^= x << 13; x ^= x >> 17; x ^= x << 5; rng = x; return (int8_t)((x & 1 ? 1 : -1) * (int)((x >> 1) & 31)); };
+    for (long long i = 0; i < V * H; i++) m[ctx->off_emb + i] = draw();
+    for (long long i = 0; i < H * V; i++) m[ctx->off_head + i] = draw();
+    for (long long l = 0; l < L; l++) {
+        for (long long i = 0; i < 4 * H * H; i++) m[ctx->off_gru_w + l * 4 * H * H + i] = draw();
+        for (long long i = 0; i < 2 * H * 4 * H; i++) m[ctx->off_mlp_w + l * 2 * H * 4 * H + i] = draw();
+    }
+    for (long long i = 0; i < L * 2 * H; i++) m[ctx->off_ln_w + i] = 16;
+    for (long long i = 0; i < H; i++) m[ctx->off_ln_out + i] = 16;
+    GTRY(hipStreamSynchronize(ctx->stream));
+    GTRY(hipMemcpy(ctx->d_model, m.data(), m.size(), hipMemcpyHostToDevice));
+    return gru_refresh_frag(ctx);
+}
+extern "C" int egg_gru_model_upload(egg_gru_ctx *ctx, const void *h, size_t bytes) {
+    if (!ctx || !h || (long long)bytes != ctx->model_bytes) return gfail(ctx, EGG_E_INVALID, "model size mismatch");
+    GTRY(hipStreamSynchronize(ctx->stream));
+    GTRY(hipMemcpy(ctx->d_model, h, bytes, hipMemcpyHostToDevice));
+    return gru_refresh_frag(ctx);
+}
+extern "C" int egg_gru_model_download(egg_gru_ctx *ctx, void *h, size_t bytes) {
+    if (!ctx || !h || (long long)bytes != ctx->model_bytes) return gfail(ctx, EGG_E_INVALID, "model size mismatch");
+    GTRY(hipStreamSynchronize(ctx->stream));
+    GTRY(hipMemcpy(h, ctx->d_model, bytes, hipMemcpyDeviceToHost));
+    return EGG_OK;
+}
+extern "C" int egg_gru_state_reset(egg_gru_ctx *ctx) {
+    if (!ctx) return EGG_E_INVALID;
+    GTRY(hipStreamSynchronize(ctx->stream));
+    GTRY(hipMemset(ctx->d_states, 0, (size_t)ctx->cfg.population * ctx->cfg.n_layers * ctx->cfg.hidden));
+    return EGG_OK;
+}
+extern "C" int egg_gru_state_download(egg_gru_ctx *ctx, void *h, size_t bytes) {
+    size_t want = (size_t)ctx->cfg.population * ctx->cfg.n_layers * ctx->cfg.hidden;
+    if (!ctx || !h || bytes != want) return gfail(ctx, EGG_E_INVALID, "state size mismatch");
+    GTRY(hipStreamSynchronize(ctx->stream));
+    GTRY(hipMemcpy(h, ctx->d_states, want, hipMemcpyDeviceToHost));
+    return EGG_OK;
+}
+
+extern "C" int egg_gru_step(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx, uint32_t step_seed, int do_update) {
+    if (!ctx || !d_data || data_len <= ctx->cfg.seq_len + 1) return gfail(ctx, EGG_E_INVALID, "egg_gru_step arguments");
+    const egg_gru_config &c = ctx->cfg;
+    const int pairs = c.population / 2, nm = (int)ctx->mats.size();
+    hipLaunchKernelGGL(k_gru_noise, dim3((nm * pairs + 63) / 64), dim3(64), 0, ctx->stream, ctx->d_mats, nm, pairs, ctx->pairs_pad,
+                       step_seed, ctx->d_noise, ctx->d_panels);
+    GruParams p;
+    p.mats = ctx->d_mats; p.model = ctx->d_model; p.frag = ctx->d_frag; p.noise = ctx->d_noise;
+    p.data = d_data; p.data_len = data_len; p.start_idx = start_idx; p.states = ctx->d_states; p.loss = ctx->d_loss;
+    p.H = c.hidden; p.L = c.n_layers; p.T = c.seq_len; p.V = c.vocab; p.population = c.population; p.sigma = c.fixed_point + c.sigma_shift;
+    p.off_emb = ctx->off_emb; p.off_gru_b = ctx->off_gru_b; p.off_ln_w = ctx->off_ln_w; p.off_ln_out = ctx->off_ln_out; p.exp2 = ctx->d_exp2;
+    dim3 grid(c.population / 32), block(GRU_THREADS);
+    size_t lds = gru_lds_bytes(c.hidden);
+    switch (c.hidden) {
+        case 64: hipLaunchKernelGGL((k_gru_forward<64>), grid, block, lds, ctx->stream, p); break;
+        case 128: hipLaunchKernelGGL((k_gru_forward<128>), grid, block, lds, ctx->stream, p); break;
+        case 256: hipLaunchKernelGGL((k_gru_forward<256>), grid, block, lds, ctx->stream, p); break;
+        default: hipLaunchKernelGGL((k_gru_forward<512>), grid, block, lds, ctx->stream, p); break;
+    }
+    GTRY(hipGetLastError());
+    // pair fitness (egg.c:559-561) has the same rule as the transformer's
+    GTRY(egg_launch_fitness(ctx->d_loss, ctx->d_fit, pairs, ctx->stream));
+    if (do_update) {
+        for (const GruMat &m : ctx->mats) {
+            long long n = (long long)m.rows * ctx->pairs_pad;
+            hipLaunchKernelGGL(k_gru_scale_panel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, ctx->d_panels + m.pa_off, n,
+                               ctx->pairs_pad, pairs, ctx->d_fit);
+            int tiles = (m.rows / 32) * (m.cols / 32);
+            hipLaunchKernelGGL(k_gru_vote_update, dim3((tiles + 3) / 4), dim3(256), 0, ctx->stream, ctx->d_model + m.w_off,
+                               ctx->d_panels + m.pa_off, ctx->d_panels + m.pb_off, m.rows, m.cols, ctx->pairs_pad, c.update_threshold);
+        }
+        GTRY(hipGetLastError());
+        return gru_refresh_frag(ctx);
+    }
+    return EGG_OK;
+}
+extern "C" int egg_gru_losses(egg_gru_ctx *ctx, int32_t *h_loss, int32_t *h_fit) {
+    if (!ctx) return EGG_E_INVALID;
+    GTRY(hipStreamSynchronize(ctx->stream));
+    if (h_loss) GTRY(hipMemcpy(h_loss, ctx->d_loss, (size_t)ctx->cfg.population * 4, hipMemcpyDeviceToHost));
+    if (h_fit) GTRY(hipMemcpy(h_fit, ctx->d_fit, (size_t)(ctx->cfg.population / 2) * 4, hipMemcpyDeviceToHost));
+    return EGG_OK;
+}

@@ -159,6 +159,35 @@ uint32_t egg_next_seed(uint32_t seed, uint64_t step);
 int  egg_ctx_enable_taps(egg_ctx *ctx, int enable);
 int  egg_tap_download(egg_ctx *ctx, const char *name, int member, void *host_out /* int8 [T][H] natural order; "logits": int32 [T][256] */);
 
+/* ---- the reference's CPU program on the GPU (full_trained_egg.c: GRU-style recurrent byte LM, sequential
+ * xorshift noise, +-1 threshold update).  Model blob == EggModel (full_trained_egg.c:42-50) with runtime sizes,
+ * every matrix row-major [out][in]; recurrent states [population][n_layers][hidden] persist across steps. ---- */
+typedef struct egg_gru_ctx egg_gru_ctx;
+typedef struct egg_gru_config {
+    int hidden;            /* HIDDEN_DIM 512 (64, 128, 256 or 512)          full_trained_egg.c:12 */
+    int n_layers;          /* N_LAYERS 4                                    :13 */
+    int seq_len;           /* SEQ_LEN 4096                                  :14 */
+    int vocab;             /* VOCAB_SIZE 256                                :11 */
+    int population;        /* POPULATION_SIZE 128 (multiple of 32)          :15 */
+    int fixed_point;       /* 4                                             :17 */
+    int sigma_shift;       /* 4                                             :18 */
+    int update_threshold;  /* 160                                           :19 */
+} egg_gru_config;
+void egg_gru_default_config(egg_gru_config *cfg);
+int  egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out);          /* init_tables + allocations, :479-518 */
+void egg_gru_destroy(egg_gru_ctx *ctx);
+const char *egg_gru_last_error(const egg_gru_ctx *ctx);
+int64_t egg_gru_model_bytes(const egg_gru_ctx *ctx);
+int  egg_gru_model_init(egg_gru_ctx *ctx, uint32_t seed);                    /* :487-509 */
+int  egg_gru_model_upload(egg_gru_ctx *ctx, const void *host_model, size_t bytes);
+int  egg_gru_model_download(egg_gru_ctx *ctx, void *host_model, size_t bytes);
+int  egg_gru_state_reset(egg_gru_ctx *ctx);                                  /* memset(pop_states), :517 */
+int  egg_gru_state_download(egg_gru_ctx *ctx, void *host_states, size_t bytes);
+/* one training step: forward_pass(+1) and forward_pass(-1) of every pair with pair fitness (:547-562), then, if
+ * do_update, update_matrix on every GRU / MLP / head matrix (:564-574) */
+int  egg_gru_step(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx, uint32_t step_seed, int do_update);
+int  egg_gru_losses(egg_gru_ctx *ctx, int32_t *host_loss, int32_t *host_fit);  /* synchronises */
+
 /* per-kernel-class timing with hipEvent pairs recorded on the context's stream around each launch (the
  * reference only splits Fwd/Host/Upd wall time, full_cuda_train_egg.cu:1116-1126).  Not usable while capturing. */
 enum { EGG_K_MLP_FIRST = 0, EGG_K_QKV = 1, EGG_K_ATTN = 2, EGG_K_MLP = 3, EGG_K_HEAD = 4,

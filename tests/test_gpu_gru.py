@@ -1,0 +1,60 @@
+"""GPU parity of the reference's CPU program (full_trained_egg.c) on the GPU, through the C ABI, against the
+scalar restatement in oracle/egg_gru_oracle.cpp: per-member losses, pair fitness, recurrent states and the
+updated int8 weights, bit for bit, over consecutive steps (the recurrent state carries over)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(dev, arr):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+
+
+@pytest.mark.parametrize("kw,steps", [
+    (dict(hidden=64, n_layers=2, seq_len=6, population=32, update_threshold=12), 3),
+    (dict(hidden=128, n_layers=1, seq_len=5, population=64, update_threshold=20), 2),
+    (dict(hidden=512, n_layers=4, seq_len=3, population=32, update_threshold=10), 2),
+], ids=["h64", "h128", "h512"])
+def test_gru_steps(pkg, orc, dev, kw, steps):
+    import ctypes as C
+    g = orc.gru_config(**kw)
+    data = orc.zipf_bytes(1 << 14)
+    model = orc.gru_init_model(g, 42)
+    rng = np.random.default_rng(3)
+    # non-trivial biases so clipped_add and the gates see every term
+    L, H = kw["n_layers"], kw["hidden"]
+    off_b = 256 * H + L * 4 * H * H
+    model[off_b:off_b + L * 2 * H] = rng.integers(-30, 31, L * 2 * H).astype(np.int8)
+    ctx = pkg.GruContext(pkg.gru_default_config(**kw))
+    assert ctx.model_bytes() == model.size
+    ctx.model_init(42)
+    got0 = ctx.model_download()
+    ref0 = orc.gru_init_model(g, 42)
+    assert np.array_equal(got0, ref0)
+    ctx.model_upload(model)
+    d_data = _t(dev, data)
+    P = kw["population"]
+    states = np.zeros(P * L * H, np.int8)
+    for step in range(steps):
+        seed = 1000 + 77 * step
+        start = step * kw["seq_len"]
+        ctx.step(d_data.data_ptr(), len(data), start, seed, True)
+        loss, fit = ctx.losses()
+        ref_loss, ref_fit = orc.gru_population(g, model, data, start, seed, 0, P // 2, states)
+        assert np.array_equal(loss, ref_loss), f"step {step}: gpu {loss[:8]} ref {ref_loss[:8]}"
+        assert np.array_equal(fit, ref_fit)
+        assert np.array_equal(ctx.state_download(), states), f"step {step} recurrent states"
+        orc.lib().orc_gru_update_all(C.byref(g), model.ctypes.data_as(C.c_void_p), C.c_uint32(seed), ref_fit.ctypes.data_as(C.c_void_p))
+        got = ctx.model_download()
+        assert np.array_equal(got, model), f"step {step}: {np.count_nonzero(got != model)} weights differ"
+    assert np.count_nonzero(model != ref0) > 0
+    ctx.close()
+
+
+def test_gru_config_errors(pkg, dev):
+    with pytest.raises(pkg.EggError):
+        pkg.GruContext(pkg.gru_default_config(hidden=100))
+    with pytest.raises(pkg.EggError):
+        pkg.GruContext(pkg.gru_default_config(population=30))
