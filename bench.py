@@ -131,6 +131,24 @@ def main():
     except Exception as e:   # the microbenchmark must not take the headline down
         mb = {"error": str(e)}
 
+    # ---- the reference's CPU configuration (full_trained_egg.c defaults: GRU H=512 L=4 T=4096 P=128) on the GPU
+    gru = None
+    try:
+        gcfg = pkg.gru_default_config()
+        gctx = pkg.GruContext(gcfg)
+        gctx.model_init(42)
+        gctx.step(d_data.data_ptr(), n, 0, 42, True)
+        gctx.losses()
+        t0 = time.perf_counter()
+        gctx.step(d_data.data_ptr(), n, gcfg.seq_len, 43, True)
+        gctx.losses()
+        sec = time.perf_counter() - t0
+        gru = {"value": gcfg.population * gcfg.seq_len / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3,
+               "workload": "full_trained_egg.c defaults, one full step (forward of 128 members x 4096 tokens + update)"}
+        gctx.close()
+    except Exception as e:
+        gru = {"error": str(e)}
+
     # ---- CPU baseline: the oracle's restatement of the same forward on a bounded sample of members
     cpu = None
     cpu_ref_path = None
@@ -164,7 +182,7 @@ def main():
                                f"forward+fitness+vote+AdamW, eager launches (chunk {chunk} members)",
                    "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss},
         "roofline": roofline, "kernels": per_class, "microbench_c2": mb,
-        "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
+        "gru_c1_gpu": gru, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }
     print(json.dumps(out))
     ctx.close()

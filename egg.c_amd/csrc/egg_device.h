@@ -91,29 +91,57 @@ __device__ __forceinline__ int round_half_away(float x) {
 // 16 k-bytes lane half g consumes in k-step ks for output column n: canonical dwords kq = 8ks + 2q + g (slot
 // order) or 8ks + 4g + q (natural order), q = 0..3.  A block is therefore exactly its LDS image and staging
 // is a straight 16-byte-per-lane copy with every load in flight before the first LDS write.
+// A block is streamed in units of UK = min(B,128) k-rows (a contiguous slice of the block) through two LDS
+// buffers with global_load_lds_dwordx4 (global -> LDS without passing through registers): while the waves run the
+// MFMAs of unit i, the copy of unit i+1 is in flight.  One barrier per unit: it proves both that unit i has landed
+// for every wave and that every wave is done with the buffer unit i+1 is about to overwrite.
 template <int B>
-__device__ __forceinline__ void stage_w_block(int8_t *lds, const int8_t *blk) {
-    constexpr int CHUNKS = B * B / 16;
-    constexpr int PER = (CHUNKS + EGG_THREADS - 1) / EGG_THREADS;
-    v4i v[PER];
+struct WUnit {
+    static constexpr int UK = B < 128 ? B : 128;
+    static constexpr int BYTES = UK * B;
+    static constexpr int PER_BLOCK = B / UK;
+};
+struct WStream {
+    int8_t *fill;          // buffer the next prefetch writes
+    int8_t *other;
+};
+__device__ __forceinline__ void wstream_init(WStream &s, int8_t *lds, int unit_bytes) { s.fill = lds; s.other = lds + unit_bytes; }
+
+template <int B>
+__device__ __forceinline__ void w_prefetch(WStream &s, const int8_t *unit) {
+    if (unit == nullptr) return;
+    constexpr int CHUNKS = WUnit<B>::BYTES / 16;                 // 16-byte chunks, 64 per wave instruction
+    constexpr int PER = (CHUNKS / 64 + EGG_WAVES - 1) / EGG_WAVES;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    int8_t *dst = s.fill;
 #pragma unroll
     for (int i = 0; i < PER; i++) {
-        int c = threadIdx.x + i * EGG_THREADS;
-        if (CHUNKS % EGG_THREADS == 0 || c < CHUNKS) v[i] = *reinterpret_cast<const v4i *>(blk + (size_t)c * 16);
-    }
-#pragma unroll
-    for (int i = 0; i < PER; i++) {
-        int c = threadIdx.x + i * EGG_THREADS;
-        if (CHUNKS % EGG_THREADS == 0 || c < CHUNKS) *reinterpret_cast<v4i *>(lds + (size_t)c * 16) = v[i];
+        const int c0 = (i * EGG_WAVES + wave) * 64;
+        if (CHUNKS / 64 % EGG_WAVES == 0 || c0 < CHUNKS)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(unit + (size_t)(c0 + lane) * 16),
+                                             (__attribute__((address_space(3))) void *)(dst + (size_t)c0 * 16), 16, 0, 0);
     }
 }
-
-// acc[nt] += W_block^T . xop for one staged block; xop[ks] is the token operand of k-step ks of the block
+// wait for the unit prefetched last, make it visible to the workgroup, and hand it out
+__device__ __forceinline__ const int8_t *w_acquire(WStream &s) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int8_t *p = s.fill;
+    s.fill = s.other; s.other = p;
+    return p;
+}
 template <int B>
-__device__ __forceinline__ void mfma_block(v16i *acc, const v4i *xop, const int8_t *lds, int lane) {
+__device__ __forceinline__ const int8_t *w_unit_ptr(const int8_t *Wf, int n_total, int k_off, int n_off, int unit) {
+    const int kb = unit / WUnit<B>::PER_BLOCK, h = unit % WUnit<B>::PER_BLOCK;
+    return Wf + ((size_t)(k_off / B + kb) * (n_total / B) + n_off / B) * (B * B) + (size_t)h * WUnit<B>::BYTES;
+}
+
+// acc[nt] += W_unit^T . xop for one staged unit; xop[ks] is the token operand of k-step ks of the unit
+template <int B>
+__device__ __forceinline__ void mfma_unit(v16i *acc, const v4i *xop, const int8_t *lds, int lane) {
     const int i = lane & 31, g = lane >> 5;
 #pragma unroll
-    for (int ks = 0; ks < B / 32; ks++) {
+    for (int ks = 0; ks < WUnit<B>::UK / 32; ks++) {
 #pragma unroll
         for (int nt = 0; nt < B / 32; nt++) {
             v4i a = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * B + nt * 32 + i) * 16);
@@ -122,25 +150,77 @@ __device__ __forceinline__ void mfma_block(v16i *acc, const v4i *xop, const int8
     }
 }
 
-// Full GEMM for one tile: acc[NOUT/32] (+)= W[k_off.., n_off..]^T . xop[KTOT/32], W blocks (fragment-major)
-// streamed through LDS.  Every wave of the workgroup must call it (it synchronises).
+// Full GEMM for one tile: acc[NOUT/32] (+)= W[k_off.., n_off..]^T . xop[KTOT/32].  The first unit must already
+// have been prefetched; `next` is the first unit of whatever GEMM follows (nullptr if none) and is prefetched while
+// the last unit is consumed.  Every wave of the workgroup must call it (it synchronises).
 template <int KTOT, int NOUT, int B>
 __device__ __forceinline__ void gemm_stream(v16i *acc, const v4i *xop, const int8_t *Wf, int n_total,
-                                            int k_off, int n_off, int8_t *wlds, int lane) {
+                                            int k_off, int n_off, WStream &ws, const int8_t *next, int lane) {
     static_assert(KTOT % B == 0 && NOUT % B == 0, "block size must divide the GEMM");
-    const int nblk_n = n_total / B;
+    constexpr int UPB = WUnit<B>::PER_BLOCK, KU = (KTOT / B) * UPB;
 #pragma unroll
     for (int nb = 0; nb < NOUT / B; nb++) {
 #pragma unroll
-        for (int kb = 0; kb < KTOT / B; kb++) {
-            const int8_t *blk = Wf + ((size_t)(k_off / B + kb) * nblk_n + (n_off / B + nb)) * (B * B);
-            __syncthreads();
-            stage_w_block<B>(wlds, blk);
-            __syncthreads();
-            mfma_block<B>(acc + nb * (B / 32), xop + kb * (B / 32), wlds, lane);
+        for (int u = 0; u < KU; u++) {
+            const int8_t *cur = w_acquire(ws);
+            const int8_t *nx = (u + 1 < KU) ? w_unit_ptr<B>(Wf, n_total, k_off, n_off + nb * B, u + 1)
+                             : ((nb + 1 < NOUT / B) ? w_unit_ptr<B>(Wf, n_total, k_off, n_off + (nb + 1) * B, 0) : next);
+            w_prefetch<B>(ws, nx);
+            mfma_unit<B>(acc + nb * (B / 32), xop + u * (WUnit<B>::UK / 32), cur, lane);
         }
     }
 }
+
+// ---- generic units for the register-lean kernels: NP p-rows (p = 2*kstep + half) x COLS output columns of a
+// fragment-major block whose rows hold src_cols columns.  LDS image: [NP][COLS][16 bytes].
+template <int NP, int COLS>
+__device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, int src_cols) {
+    if (src == nullptr) return;
+    static_assert(COLS % 64 == 0, "a wave instruction copies 64 columns");
+    constexpr int SEG = COLS / 64, INSTR = NP * SEG, PER = (INSTR + EGG_WAVES - 1) / EGG_WAVES;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    int8_t *dst = s.fill;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+        const int id = i * EGG_WAVES + wave;
+        if (INSTR % EGG_WAVES == 0 || id < INSTR) {
+            const int pr = id / SEG, seg = id % SEG;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + ((size_t)pr * src_cols + seg * 64 + lane) * 16),
+                                             (__attribute__((address_space(3))) void *)(dst + ((size_t)pr * COLS + seg * 64) * 16), 16, 0, 0);
+        }
+    }
+}
+// acc[nt] += unit^T . xop for a unit of KSU k-steps x NTU column groups
+template <int KSU, int NTU>
+__device__ __forceinline__ void mfma_unit2(v16i *acc, const v4i *xop, const int8_t *lds, int lane) {
+    const int i = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int ks = 0; ks < KSU; ks++)
+#pragma unroll
+        for (int nt = 0; nt < NTU; nt++) {
+            v4i a = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * (NTU * 32) + nt * 32 + i) * 16);
+            acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, xop[ks], acc[nt], 0, 0, 0);
+        }
+}
+
+// How the four waves of a workgroup map to (member, tile) for a sequence of T tokens: with at least four tiles
+// per member the whole workgroup serves one member (one shared set of noise tables) and walks its tiles in
+// passes of four; with two tiles it serves two members, with one tile four.
+struct TileMap {
+    int sets;        // members (= noise table sets) per workgroup
+    int passes;
+    int set;         // table set of this wave
+    int mloc;        // member index within the chunk (may be >= n_members for a padding wave)
+    int tile0;       // tile of this wave in pass 0; later passes add 4
+};
+__device__ __forceinline__ TileMap tile_map(int T, int wave, int block) {
+    TileMap m; const int tpm = T / 32;
+    if (tpm >= 4) { m.sets = 1; m.passes = tpm / 4; m.set = 0; m.mloc = block; m.tile0 = wave; }
+    else if (tpm == 2) { m.sets = 2; m.passes = 1; m.set = wave >> 1; m.mloc = block * 2 + (wave >> 1); m.tile0 = wave & 1; }
+    else { m.sets = 4; m.passes = 1; m.set = wave; m.mloc = block * 4 + wave; m.tile0 = 0; }
+    return m;
+}
+static inline int tile_map_sets(int T) { int tpm = T / 32; return tpm >= 4 ? 1 : (tpm == 2 ? 2 : 4); }
 
 template <int N>
 __device__ __forceinline__ void zero_acc(v16i *acc) {
@@ -151,17 +231,17 @@ __device__ __forceinline__ void zero_acc(v16i *acc) {
 }
 
 // ---------------------------------------------------------------- per-member noise tables (one wave fills its own)
-__device__ __forceinline__ void fill_noise_i8(int8_t *dst, uint32_t seed, int n, int mask, int lane) {
-    for (int i = lane; i < n; i += 64) dst[i] = (int8_t)noise_from_hash(seed, i, mask);
+__device__ __forceinline__ void fill_noise_i8(int8_t *dst, uint32_t seed, int n, int mask, int lane, int nthr = 64) {
+    for (int i = lane; i < n; i += nthr) dst[i] = (int8_t)noise_from_hash(seed, i, mask);
 }
 // dst[i] = noise(seed, i) * mult
-__device__ __forceinline__ void fill_noise_i32(int *dst, uint32_t seed, int n, int mask, int mult, int lane) {
-    for (int i = lane; i < n; i += 64) dst[i] = noise_from_hash(seed, i, mask) * mult;
+__device__ __forceinline__ void fill_noise_i32(int *dst, uint32_t seed, int n, int mask, int mult, int lane, int nthr = 64) {
+    for (int i = lane; i < n; i += nthr) dst[i] = noise_from_hash(seed, i, mask) * mult;
 }
 // dst[i] = base[i] + ((noise(seed_a,i) * noise(seed_b,i) * ns) >> shift)       (mgpu.cu:666-675, :733-735)
 __device__ __forceinline__ void fill_vec_i32(int *dst, const int8_t *base, uint32_t seed_a, uint32_t seed_b,
-                                             int n, int mask, int ns, int shift, int lane) {
-    for (int i = lane; i < n; i += 64) {
+                                             int n, int mask, int ns, int shift, int lane, int nthr = 64) {
+    for (int i = lane; i < n; i += nthr) {
         int v = base[i];
         if (ns != 0) v += (noise_from_hash(seed_a, i, mask) * noise_from_hash(seed_b, i, mask) * ns) >> shift;
         dst[i] = v;

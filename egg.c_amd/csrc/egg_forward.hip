@@ -36,65 +36,82 @@ __device__ __forceinline__ void add_perturb(v16i *acc, int sb, const int *At, in
 }
 
 // ============================================================================ MLP block
+// Register-lean form (<= 256 VGPRs, two workgroups per CU): the 4H-wide intermediate is produced 64 columns at a
+// time (up GEMM on a [H x 64] unit, GELU epilogue, immediately consumed as two k-steps of the down GEMM on a
+// [64 x H] unit), so only the H-wide down accumulator, the normalised input and a 64-column accumulator are live.
+// W units (64*H bytes) stream through two LDS buffers.  The residual is parked in the x buffer and re-read at the end.
 template <int H>
 struct MlpLds {
-    // per-wave tables, int32 unless noted
     static constexpr int I32 = 14 * H;       // ex0[H] ex1[H] lnw[H] lnb[H] upA[4H] bup[4H] dnA[H] bdn[H]
     static constexpr int I8 = 6 * H;         // exB[H] upB[H] dnB[4H]
-    static constexpr int PER_WAVE = I32 * 4 + I8;
-    static constexpr int WBLOCK = (H < 256 ? H : 256) * (H < 256 ? H : 256);
-    static constexpr int TOTAL = WBLOCK + 256 + EGG_WAVES * PER_WAVE;
+    static constexpr int PER_SET = I32 * 4 + I8;
+    static constexpr int UNIT = 64 * H;
+    static constexpr int WBYTES = 2 * UNIT;
+    static int total(int sets) { return WBYTES + 256 + sets * PER_SET; }
 };
 
 template <int H, bool FIRST>
-__global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
-    constexpr int KS = H / 32, NT = H / 32, BLK = H < 256 ? H : 256;
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_mlp(MlpParams p) {
+    constexpr int KS = H / 32, NT = H / 32, PR = H / 16;      // k-steps, column groups, p-rows of a full-K unit
     extern __shared__ __align__(16) int8_t smem[];
-    int8_t *wlds = smem;
-    int8_t *act = smem + MlpLds<H>::WBLOCK;
+    int8_t *act = smem + MlpLds<H>::WBYTES;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    int8_t *tb = act + 256 + wave * MlpLds<H>::PER_WAVE;
+    const FwdCommon &c = p.c;
+    const int T = c.T;
+    const TileMap tm = tile_map(T, wave, blockIdx.x);
+    int8_t *tb = act + 256 + tm.set * MlpLds<H>::PER_SET;
     int *ex0 = reinterpret_cast<int *>(tb);   // FIRST: emb_bias + noise   | else: O-proj A noise * ns
     int *ex1 = ex0 + H;                       // FIRST: b_dim noise * ns    | else: unused
     int *lnw = ex1 + H, *lnb = lnw + H, *upA = lnb + H, *bup = upA + 4 * H, *dnA = bup + 4 * H, *bdn = dnA + H;
     int8_t *exB = reinterpret_cast<int8_t *>(bdn + H);   // O-proj B noise
     int8_t *upB = exB + H, *dnB = upB + H;
 
-    const FwdCommon &c = p.c;
-    const int T = c.T;
-    int mloc = blockIdx.x * EGG_WAVES + wave;
+    WStream ws; wstream_init(ws, smem, MlpLds<H>::UNIT);
+    // unit sources inside the fragment-major copies (block size B == H for H <= 256)
+    auto up_unit = [&](int sidx) { return p.w_up + (size_t)((64 * sidx) / H) * H * H + (size_t)((64 * sidx) % H) * 16; };
+    auto dn_unit = [&](int sidx) { return p.w_dn + (size_t)((64 * sidx) / H) * H * H + (size_t)(((64 * sidx) % H) / 16) * H * 16; };
+    auto o_unit = [&](int u) { return p.w_o + (size_t)(4 * u) * H * 16; };
+    const int8_t *pass_first = FIRST ? up_unit(0) : o_unit(0);
+    if (FIRST) w_prefetch2<PR, 64>(ws, pass_first, H); else w_prefetch2<4, H>(ws, pass_first, H);
+
+    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) act[i] = c.act_lut[i];
+    for (int ss = 0; ss < tm.sets; ss++) {
+        int ml = blockIdx.x * tm.sets + ss; if (ml >= c.n_members) ml = c.n_members - 1;
+        const int mem = c.pop_offset + ml, nsx = (mem & 1) ? -1 : 1;
+        const uint32_t pseed = *c.d_step_seed + (uint32_t)(mem / 2), sbx = pseed + (uint32_t)p.seed_base;
+        int8_t *t2 = act + 256 + ss * MlpLds<H>::PER_SET;
+        int *e0 = reinterpret_cast<int *>(t2), *e1 = e0 + H, *lw = e1 + H, *lb = lw + H, *uA = lb + H, *bu = uA + 4 * H, *dA = bu + 4 * H, *bd = dA + H;
+        int8_t *eB = reinterpret_cast<int8_t *>(bd + H), *uB = eB + H, *dB = uB + H;
+        const int tid = threadIdx.x;
+        if (FIRST) {
+            fill_vec_i32(e0, p.emb_bias, pseed + OFF_EMB_BIAS_A, pseed + OFF_EMB_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+            fill_noise_i32(e1, pseed + OFF_EMB + H, H, c.mask, nsx, tid, EGG_THREADS);
+        } else {
+            fill_noise_i32(e0, sbx + OFF_O_A, H, c.mask, nsx, tid, EGG_THREADS);
+            fill_noise_i8(eB, sbx + OFF_O_B, H, c.mask, tid, EGG_THREADS);
+        }
+        fill_vec_i32(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        fill_vec_i32(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        fill_noise_i32(uA, sbx + p.off_up_a, 4 * H, c.mask, nsx, tid, EGG_THREADS);
+        fill_vec_i32(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        fill_noise_i32(dA, sbx + p.off_dn_a, H, c.mask, nsx, tid, EGG_THREADS);
+        fill_vec_i32(bd, p.b_dn, sbx + p.off_bdn_a, sbx + p.off_bdn_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        fill_noise_i8(uB, sbx + p.off_up_b, H, c.mask, tid, EGG_THREADS);
+        fill_noise_i8(dB, sbx + p.off_dn_b, 4 * H, c.mask, tid, EGG_THREADS);
+    }
+    __syncthreads();
+
+    int mloc = tm.mloc;
     const bool valid = mloc < c.n_members;
     if (!valid) mloc = c.n_members - 1;
     const int member = c.pop_offset + mloc;
-    const int ns = (member & 1) ? -1 : 1;
     const uint32_t pair_seed = *c.d_step_seed + (uint32_t)(member / 2);
-    const uint32_t sb_ = pair_seed + (uint32_t)p.seed_base;
-
-    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) act[i] = c.act_lut[i];
-    if (FIRST) {
-        fill_vec_i32(ex0, p.emb_bias, pair_seed + OFF_EMB_BIAS_A, pair_seed + OFF_EMB_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
-        fill_noise_i32(ex1, pair_seed + OFF_EMB + H, H, c.mask, ns, lane);
-    } else {
-        fill_noise_i32(ex0, sb_ + OFF_O_A, H, c.mask, ns, lane);
-        fill_noise_i8(exB, sb_ + OFF_O_B, H, c.mask, lane);
-    }
-    fill_vec_i32(lnw, p.ln_w, sb_ + p.off_ln_a, sb_ + p.off_ln_b, H, c.mask, ns, c.sigma_vec, lane);
-    fill_vec_i32(lnb, p.ln_b, sb_ + p.off_lnb_a, sb_ + p.off_lnb_b, H, c.mask, ns, c.sigma_vec, lane);
-    fill_noise_i32(upA, sb_ + p.off_up_a, 4 * H, c.mask, ns, lane);
-    fill_vec_i32(bup, p.b_up, sb_ + p.off_bup_a, sb_ + p.off_bup_b, 4 * H, c.mask, ns, c.sigma_vec, lane);
-    fill_noise_i32(dnA, sb_ + p.off_dn_a, H, c.mask, ns, lane);
-    fill_vec_i32(bdn, p.b_dn, sb_ + p.off_bdn_a, sb_ + p.off_bdn_b, H, c.mask, ns, c.sigma_vec, lane);
-    fill_noise_i8(upB, sb_ + p.off_up_b, H, c.mask, lane);
-    fill_noise_i8(dnB, sb_ + p.off_dn_b, 4 * H, c.mask, lane);
-    __syncthreads();
-
     const int64_t spos = FIRST ? stream_pos_of(c, member) : 0;
 
-    for (int pass = 0; pass < T / 32; pass++) {
-        const int t = pass * 32 + j;
+    for (int pass = 0; pass < tm.passes; pass++) {
+        const int t = (tm.tile0 + 4 * pass) * 32 + j;
         const size_t row = ((size_t)mloc * T + t) * H;
         v4i xcur[KS];
-        v16i acc[NT];
 
         if (FIRST) {
             // embedding stage (mgpu.cu:901-931)
@@ -116,22 +133,34 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
                 }
         } else {
             // attention output projection + residual + adaptive norm (mgpu.cu:827-831)
-            v4i aop[KS], xres[KS];
+            v4i aop[KS];
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) { aop[ks] = load_op(p.ao + row, ks, g); xres[ks] = load_op(p.x + row, ks, g); }
-            int sbo = dot_noise<KS, false>(aop, exB, 0, g);
+            for (int ks = 0; ks < KS; ks++) aop[ks] = load_op(p.ao + row, ks, g);
+            const int sbo = dot_noise<KS, false>(aop, exB, 0, g);
+            v16i acc[NT];
             zero_acc<NT>(acc);
-            gemm_stream<H, H, BLK>(acc, aop, p.w_o, H, 0, 0, wlds, lane);
+#pragma unroll
+            for (int u = 0; u < H / 64; u++) {
+                const int8_t *cur = w_acquire(ws);
+                if (u + 1 < H / 64) w_prefetch2<4, H>(ws, o_unit(u + 1), H); else w_prefetch2<PR, 64>(ws, up_unit(0), H);
+                mfma_unit2<2, NT>(acc, aop + 2 * u, cur, lane);
+            }
             add_perturb<NT>(acc, sbo, ex0, 0, c.sigma, g);
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++)
+            for (int nt = 0; nt < NT; nt++) {
+                v4i xr = load_op(p.x + row, nt, g);
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc[nt][r] = sx8(xres[nt][r >> 2], r & 3) + (acc[nt][r] >> c.shift_out);
+                for (int r = 0; r < 16; r++) acc[nt][r] = sx8(xr[r >> 2], r & 3) + (acc[nt][r] >> c.shift_out);
+            }
             adaptive_norm<NT>(acc, xcur);
             if (p.x_mid && valid)
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) store_op(p.x_mid + row, ks, g, xcur[ks]);
         }
+        // park the residual (this wave owns the row; invalid padding waves only recompute)
+        if (valid)
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) store_op(p.x + row, ks, g, xcur[ks]);
 
         // MLP (mgpu.cu:708-759)
         v4i nrm[KS];
@@ -140,47 +169,57 @@ __global__ void __launch_bounds__(EGG_THREADS) k_mlp(MlpParams p) {
         v16i accd[NT];
         zero_acc<NT>(accd);
         int sbd = 0;
+        constexpr int NSUB = 4 * H / 64;
 #pragma unroll 1
-        for (int ch = 0; ch < 4; ch++) {
-            zero_acc<NT>(acc);
-            gemm_stream<H, H, BLK>(acc, nrm, p.w_up, 4 * H, 0, ch * H, wlds, lane);
-            v4i mid[KS];
+        for (int sidx = 0; sidx < NSUB; sidx++) {
+            v16i au[2];
+            zero_acc<2>(au);
+            {
+                const int8_t *cur = w_acquire(ws);
+                w_prefetch2<4, H>(ws, dn_unit(sidx), H);
+                mfma_unit2<KS, 2>(au, nrm, cur, lane);
+            }
+            v4i mid[2];
+            const int *dnb32 = reinterpret_cast<const int *>(dnB + 64 * sidx);
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++)
+            for (int nt = 0; nt < 2; nt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    int n0 = ch * H + 32 * nt + 8 * q + 4 * g;
+                    int n0 = 64 * sidx + 32 * nt + 8 * q + 4 * g;
                     v4i a4 = *reinterpret_cast<const v4i *>(upA + n0);
                     v4i b4 = *reinterpret_cast<const v4i *>(bup + n0);
                     int o[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        int a = acc[nt][4 * q + e] + (mul24(sbu, a4[e]) >> c.sigma);
+                        int a = au[nt][4 * q + e] + (mul24(sbu, a4[e]) >> c.sigma);
                         int v = clip127((a >> c.shift_mlp_up) + b4[e]);
                         o[e] = act[(uint8_t)v];
                     }
                     mid[nt][q] = pack4(o[0], o[1], o[2], o[3]);
+                    sbd = dot4(mid[nt][q], dnb32[8 * nt + 2 * q + g], sbd);
                 }
-            {   // partial x.B of the down projection for this chunk (halves combined after the loop)
-                const int *b32 = reinterpret_cast<const int *>(dnB + ch * H);
-#pragma unroll
-                for (int ks = 0; ks < KS; ks++)
-#pragma unroll
-                    for (int q = 0; q < 4; q++) sbd = dot4(mid[ks][q], b32[8 * ks + 2 * q + g], sbd);
+            {
+                const int8_t *cur = w_acquire(ws);
+                const int8_t *nx = (sidx + 1 < NSUB) ? up_unit(sidx + 1) : nullptr;
+                if (nx) w_prefetch2<PR, 64>(ws, nx, H);
+                else if (pass + 1 < tm.passes) { if (FIRST) w_prefetch2<PR, 64>(ws, pass_first, H); else w_prefetch2<4, H>(ws, pass_first, H); }
+                mfma_unit2<2, NT>(accd, mid, cur, lane);
             }
-            gemm_stream<H, H, BLK>(accd, mid, p.w_dn, H, ch * H, 0, wlds, lane);
         }
         sbd += other_half(sbd);
         add_perturb<NT>(accd, sbd, dnA, 0, c.sigma, g);
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++)
+        for (int nt = 0; nt < NT; nt++) {
+            v4i xr = load_op(p.x + row, nt, g);          // the parked residual (for a padding wave: someone else's row, unused)
+            if (!valid) xr = xcur[nt];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 v4i b4 = *reinterpret_cast<const v4i *>(bdn + 32 * nt + 8 * q + 4 * g);
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    accd[nt][4 * q + e] = sx8(xcur[nt][q], e) + (accd[nt][4 * q + e] >> c.shift_mlp_down) + b4[e];
+                    accd[nt][4 * q + e] = sx8(xr[q], e) + (accd[nt][4 * q + e] >> c.shift_mlp_down) + b4[e];
             }
+        }
         v4i xnew[KS];
         adaptive_norm<NT>(accd, xnew);
         if (valid)
@@ -194,79 +233,110 @@ template <int H>
 struct QkvLds {
     static constexpr int I32 = 5 * H;   // lnw lnb qA kA vA
     static constexpr int I8 = 3 * H;    // qB kB vB
-    static constexpr int PER_WAVE = I32 * 4 + I8 + (16 - (I8 % 16)) % 16;
-    static constexpr int WBLOCK = (H < 256 ? H : 256) * (H < 256 ? H : 256);
-    static constexpr int TOTAL = WBLOCK + EGG_WAVES * PER_WAVE;
+    static constexpr int PER_SET = I32 * 4 + I8 + (16 - (I8 % 16)) % 16;
+    static constexpr int UNIT = 64 * H;
+    static constexpr int WBYTES = 2 * UNIT;
+    static int total(int sets) { return WBYTES + sets * PER_SET; }
 };
 
-// apply_rope_integer (mgpu.cu:624-644) on the raw accumulators of one token
+// apply_rope_integer (mgpu.cu:624-644) on the raw accumulators of one token.  The (cos, sin) pairs repeat every
+// head, so a lane needs only the head_dim/32 * 8 pairs of its own slots; they are loaded once and reused.
 template <int NT>
 __device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row, int head_dim, int bit, int g) {
     const long long half = 1ll << (bit - 1);
+    int2 cs[2][4][2];
+    const int hdt = head_dim >> 5;                 // column groups per head: 1 or 2
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int ep = 0; ep < 2; ep++) {
+                int n = 32 * (h2 < hdt ? h2 : 0) + 8 * q + 4 * g + 2 * ep;
+                cs[h2][q][ep] = *reinterpret_cast<const int2 *>(rope_row + 2 * (n >> 1));
+            }
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
         for (int q = 0; q < 4; q++)
 #pragma unroll
             for (int ep = 0; ep < 2; ep++) {
-                int n = 32 * nt + 8 * q + 4 * g + 2 * ep;           // even element of the pair
-                int pr = (n % head_dim) >> 1;
-                int2 cs = *reinterpret_cast<const int2 *>(rope_row + 2 * pr);
+                const int2 c2 = (hdt == 2) ? cs[nt & 1][q][ep] : cs[0][q][ep];
                 long long ve = acc[nt][4 * q + 2 * ep], vo = acc[nt][4 * q + 2 * ep + 1];
-                long long re = (ve * cs.x - vo * cs.y + half) >> bit;
-                long long ro = (ve * cs.y + vo * cs.x + half) >> bit;
+                long long re = (ve * c2.x - vo * c2.y + half) >> bit;
+                long long ro = (ve * c2.y + vo * c2.x + half) >> bit;
                 acc[nt][4 * q + 2 * ep] = (int)re;
                 acc[nt][4 * q + 2 * ep + 1] = (int)ro;
             }
 }
 
 template <int H>
-__global__ void __launch_bounds__(EGG_THREADS) k_qkv(QkvParams p) {
-    constexpr int KS = H / 32, NT = H / 32, BLK = H < 256 ? H : 256;
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
+    constexpr int KS = H / 32, NT = H / 32;
     extern __shared__ __align__(16) int8_t smem[];
-    int8_t *wlds = smem;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    int8_t *tb = smem + QkvLds<H>::WBLOCK + wave * QkvLds<H>::PER_WAVE;
+    const FwdCommon &c = p.c;
+    const int T = c.T;
+    const TileMap tm = tile_map(T, wave, blockIdx.x);
+    int8_t *tb = smem + QkvLds<H>::WBYTES + tm.set * QkvLds<H>::PER_SET;
     int *lnw = reinterpret_cast<int *>(tb), *lnb = lnw + H, *qA = lnb + H, *kA = qA + H, *vA = kA + H;
     int8_t *qB = reinterpret_cast<int8_t *>(vA + H), *kB = qB + H, *vB = kB + H;
 
-    const FwdCommon &c = p.c;
-    const int T = c.T;
-    int mloc = blockIdx.x * EGG_WAVES + wave;
-    const bool valid = mloc < c.n_members;
-    if (!valid) mloc = c.n_members - 1;
-    const int member = c.pop_offset + mloc;
-    const int ns = (member & 1) ? -1 : 1;
-    const uint32_t sb_ = *c.d_step_seed + (uint32_t)(member / 2) + (uint32_t)p.seed_base;
+    WStream ws; wstream_init(ws, smem, QkvLds<H>::UNIT);
+    auto w_unit = [&](const int8_t *W, int u) { return W + (size_t)(4 * u) * H * 16; };     // k rows [64u, 64u+64)
+    w_prefetch2<4, H>(ws, w_unit(p.w_q, 0), H);
 
-    fill_vec_i32(lnw, p.ln_w, sb_ + OFF_LN_1_A, sb_ + OFF_LN_1_B, H, c.mask, ns, c.sigma_vec, lane);
-    fill_vec_i32(lnb, p.ln_b, sb_ + OFF_LN_1_BIAS_A, sb_ + OFF_LN_1_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
-    fill_noise_i32(qA, sb_ + OFF_Q_A, H, c.mask, ns, lane);
-    fill_noise_i32(kA, sb_ + OFF_K_A, H, c.mask, ns, lane);
-    fill_noise_i32(vA, sb_ + OFF_V_A, H, c.mask, ns, lane);
-    fill_noise_i8(qB, sb_ + OFF_Q_B, H, c.mask, lane);
-    fill_noise_i8(kB, sb_ + OFF_K_B, H, c.mask, lane);
-    fill_noise_i8(vB, sb_ + OFF_V_B, H, c.mask, lane);
+    for (int ss = 0; ss < tm.sets; ss++) {
+        int ml = blockIdx.x * tm.sets + ss; if (ml >= c.n_members) ml = c.n_members - 1;
+        const int mem = c.pop_offset + ml, nsx = (mem & 1) ? -1 : 1;
+        const uint32_t sbx = *c.d_step_seed + (uint32_t)(mem / 2) + (uint32_t)p.seed_base;
+        int8_t *t2 = smem + QkvLds<H>::WBYTES + ss * QkvLds<H>::PER_SET;
+        int *lw = reinterpret_cast<int *>(t2), *lb = lw + H, *a0 = lb + H, *a1 = a0 + H, *a2 = a1 + H;
+        int8_t *b0 = reinterpret_cast<int8_t *>(a2 + H), *b1 = b0 + H, *b2 = b1 + H;
+        const int tid = threadIdx.x;
+        fill_vec_i32(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        fill_vec_i32(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        fill_noise_i32(a0, sbx + OFF_Q_A, H, c.mask, nsx, tid, EGG_THREADS);
+        fill_noise_i32(a1, sbx + OFF_K_A, H, c.mask, nsx, tid, EGG_THREADS);
+        fill_noise_i32(a2, sbx + OFF_V_A, H, c.mask, nsx, tid, EGG_THREADS);
+        fill_noise_i8(b0, sbx + OFF_Q_B, H, c.mask, tid, EGG_THREADS);
+        fill_noise_i8(b1, sbx + OFF_K_B, H, c.mask, tid, EGG_THREADS);
+        fill_noise_i8(b2, sbx + OFF_V_B, H, c.mask, tid, EGG_THREADS);
+    }
     __syncthreads();
 
-    for (int pass = 0; pass < T / 32; pass++) {
-        const int t = pass * 32 + j;
+    int mloc = tm.mloc;
+    const bool valid = mloc < c.n_members;
+    if (!valid) mloc = c.n_members - 1;
+
+    for (int pass = 0; pass < tm.passes; pass++) {
+        const int t = (tm.tile0 + 4 * pass) * 32 + j;
         const size_t row = ((size_t)mloc * T + t) * H;
-        v4i x[KS], nrm[KS];
+        v4i nrm[KS];
+        {
+            v4i x[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
-        standard_norm<KS>(x, nrm, lnw, lnb, g);
+            for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
+            standard_norm<KS>(x, nrm, lnw, lnb, g);
+        }
         const int32_t *rope_row = c.rope_lut + (size_t)t * c.head_dim;
 #pragma unroll 1
         for (int which = 0; which < 3; which++) {
             const int8_t *W = which == 0 ? p.w_q : (which == 1 ? p.w_k : p.w_v);
+            const int8_t *nw = which == 0 ? p.w_k : (which == 1 ? p.w_v : ((pass + 1 < tm.passes) ? p.w_q : nullptr));
             const int8_t *Bn = which == 0 ? qB : (which == 1 ? kB : vB);
             const int *An = which == 0 ? qA : (which == 1 ? kA : vA);
             int8_t *dst = which == 0 ? p.q : (which == 1 ? p.k : p.v);
             const int sb = dot_noise<KS, false>(nrm, Bn, 0, g);
             v16i acc[NT];
             zero_acc<NT>(acc);
-            gemm_stream<H, H, BLK>(acc, nrm, W, H, 0, 0, wlds, lane);
+#pragma unroll
+            for (int u = 0; u < H / 64; u++) {
+                const int8_t *cur = w_acquire(ws);
+                if (u + 1 < H / 64) w_prefetch2<4, H>(ws, w_unit(W, u + 1), H);
+                else if (nw) w_prefetch2<4, H>(ws, w_unit(nw, 0), H);
+                mfma_unit2<2, NT>(acc, nrm + 2 * u, cur, lane);
+            }
             add_perturb<NT>(acc, sb, An, 0, c.sigma, g);
             if (which < 2) rope_inplace<NT>(acc, rope_row, c.head_dim, c.rope_scale_bit, g);
             v4i o[KS];
@@ -283,7 +353,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_qkv(QkvParams p) {
 // causal context (row max, then LUT weights), O^T = V^T.P^T with the 19-bit weights split into three
 // 7-bit planes so the weighted sum stays exact on the int8 MFMA.
 template <int HD, int CT>
-__global__ void __launch_bounds__(EGG_THREADS) k_attn(AttnParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_attn(AttnParams p) {
     constexpr int KS = HD / 32, DT = HD / 32;
     constexpr int T = CT * 32;
     extern __shared__ __align__(16) int8_t smem[];
@@ -421,12 +491,12 @@ __global__ void __launch_bounds__(EGG_THREADS) k_attn(AttnParams p) {
 template <int H>
 struct HeadLds {
     static constexpr int PER_WAVE = (2 * H + 256) * 4 + H;   // lnw lnb hA[256] + hB[H]
-    static constexpr int WBLOCK = (H < 256 ? H : 256) * (H < 256 ? H : 256);
+    static constexpr int WBLOCK = 2 * WUnit<(H < 256 ? H : 256)>::BYTES;   // double-buffered W units
     static constexpr int TOTAL = WBLOCK + 1024 + EGG_WAVES * PER_WAVE;
 };
 
 template <int H>
-__global__ void __launch_bounds__(EGG_THREADS) k_head(HeadParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_head(HeadParams p) {
     constexpr int KS = H / 32, NV = 256 / 32, BLK = H < 256 ? H : 256;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *wlds = smem;
@@ -445,6 +515,8 @@ __global__ void __launch_bounds__(EGG_THREADS) k_head(HeadParams p) {
     const int ns = (member & 1) ? -1 : 1;
     const uint32_t pair_seed = *c.d_step_seed + (uint32_t)(member / 2);
 
+    WStream ws; wstream_init(ws, wlds, WUnit<BLK>::BYTES);
+    w_prefetch<BLK>(ws, w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0));
     for (int i = threadIdx.x; i < 256; i += EGG_THREADS) lut[i] = c.exp_lut[i];
     fill_vec_i32(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane);
     fill_vec_i32(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
@@ -464,7 +536,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_head(HeadParams p) {
         const int sbh = dot_noise<KS, false>(nf, hB, 0, g);
         v16i acc[NV];
         zero_acc<NV>(acc);
-        gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, wlds, lane);
+        gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, ws, (pass + 1 < T / 32) ? w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0) : nullptr, lane);
         add_perturb<NV>(acc, sbh, hA, 0, c.sigma, g);
         // two-pass softmax statistics (mgpu.cu:969-1009)
         int gmax = INT_MIN;
@@ -517,8 +589,9 @@ __global__ void __launch_bounds__(EGG_THREADS) k_head(HeadParams p) {
 // ============================================================================ host launchers
 template <int H>
 static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
-    dim3 grid((p.c.n_members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
-    size_t lds = MlpLds<H>::TOTAL;
+    const int sets = tile_map_sets(p.c.T);
+    dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
+    size_t lds = MlpLds<H>::total(sets);
     if (first) hipLaunchKernelGGL((k_mlp<H, true>), grid, block, lds, s, p);
     else hipLaunchKernelGGL((k_mlp<H, false>), grid, block, lds, s, p);
     return hipGetLastError();
@@ -534,8 +607,9 @@ hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s) {
 
 template <int H>
 static hipError_t launch_qkv_h(const QkvParams &p, hipStream_t s) {
-    dim3 grid((p.c.n_members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
-    size_t lds = QkvLds<H>::TOTAL;
+    const int sets = tile_map_sets(p.c.T);
+    dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
+    size_t lds = QkvLds<H>::total(sets);
     hipLaunchKernelGGL((k_qkv<H>), grid, block, lds, s, p);
     return hipGetLastError();
 }
@@ -595,9 +669,9 @@ hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
 #define SET_LDS(kern, bytes) do { hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)); if (e_ != hipSuccess) return e_; } while (0)
 template <int H>
 static hipError_t prepare_h() {
-    SET_LDS((k_mlp<H, true>), MlpLds<H>::TOTAL);
-    SET_LDS((k_mlp<H, false>), MlpLds<H>::TOTAL);
-    SET_LDS((k_qkv<H>), QkvLds<H>::TOTAL);
+    SET_LDS((k_mlp<H, true>), MlpLds<H>::total(4));
+    SET_LDS((k_mlp<H, false>), MlpLds<H>::total(4));
+    SET_LDS((k_qkv<H>), QkvLds<H>::total(4));
     SET_LDS((k_head<H>), HeadLds<H>::TOTAL);
     return hipSuccess;
 }

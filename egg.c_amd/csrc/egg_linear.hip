@@ -12,16 +12,17 @@ struct PlinLds {
     static constexpr int B = MINKN < 256 ? MINKN : 256;      // fragment block size
     static constexpr int NB = N < 256 ? N : 256;             // output columns per epilogue
     static constexpr int PER_WAVE = N * 4 + K;
-    static constexpr int TOTAL = B * B + EGG_WAVES * PER_WAVE;
+    static constexpr int WBYTES = 2 * WUnit<B>::BYTES;       // double-buffered W units
+    static constexpr int TOTAL = WBYTES + EGG_WAVES * PER_WAVE;
 };
 
 template <int K, int N>
-__global__ void __launch_bounds__(EGG_THREADS) k_plinear(PlinParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
     constexpr int KS = K / 32, NB = PlinLds<K, N>::NB, NTB = NB / 32, B = PlinLds<K, N>::B;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *wlds = smem;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    int8_t *tb = smem + B * B + wave * PlinLds<K, N>::PER_WAVE;
+    int8_t *tb = smem + PlinLds<K, N>::WBYTES + wave * PlinLds<K, N>::PER_WAVE;
     int *At = reinterpret_cast<int *>(tb);
     int8_t *Bt = reinterpret_cast<int8_t *>(At + N);
 
@@ -30,6 +31,8 @@ __global__ void __launch_bounds__(EGG_THREADS) k_plinear(PlinParams p) {
     if (!valid) member = p.members - 1;
     const int ns = (member & 1) ? -1 : 1;
     const uint32_t ps = p.seed + (uint32_t)(member / 2);
+    WStream ws; wstream_init(ws, wlds, WUnit<B>::BYTES);
+    w_prefetch<B>(ws, w_unit_ptr<B>(p.Wfrag, N, 0, 0, 0));
     fill_noise_i32(At, ps + p.off_a, N, p.mask, ns, lane);
     fill_noise_i8(Bt, ps + p.off_b, K, p.mask, lane);
     __syncthreads();
@@ -44,7 +47,9 @@ __global__ void __launch_bounds__(EGG_THREADS) k_plinear(PlinParams p) {
         for (int nb = 0; nb < N / NB; nb++) {
             v16i acc[NTB];
             zero_acc<NTB>(acc);
-            gemm_stream<K, NB, B>(acc, xop, p.Wfrag, N, 0, nb * NB, wlds, lane);
+            const int8_t *nx = (nb + 1 < N / NB) ? w_unit_ptr<B>(p.Wfrag, N, 0, (nb + 1) * NB, 0)
+                                                 : ((pass + 1 < p.T / 32) ? w_unit_ptr<B>(p.Wfrag, N, 0, 0, 0) : nullptr);
+            gemm_stream<K, NB, B>(acc, xop, p.Wfrag, N, 0, nb * NB, ws, nx, lane);
 #pragma unroll
             for (int nt = 0; nt < NTB; nt++)
 #pragma unroll
