@@ -162,9 +162,10 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (!cfg || !out) return EGG_E_INVALID;
     *out = nullptr;
     const egg_config &c = *cfg;
-    if (!(c.hidden == 64 || c.hidden == 128 || c.hidden == 256)) return EGG_E_INVALID;
+    if (!(c.hidden == 64 || c.hidden == 128 || c.hidden == 256 || c.hidden == 512)) return EGG_E_INVALID;
     if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return EGG_E_INVALID;
-    if (c.seq_len % 32 || !(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256)) return EGG_E_INVALID;
+    if (!(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256 || c.seq_len == 512)) return EGG_E_INVALID;
+    if (c.hidden == 512 && c.seq_len < 128) return EGG_E_INVALID;      // the per-member LDS tables of hidden 512 fit once per workgroup
     if (c.vocab != 256 || c.n_layers < 1 || c.population < 2 || (c.population & 1)) return EGG_E_INVALID;
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
@@ -239,10 +240,11 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
 
 // refresh the fragment-major copy of one matrix (tensor id) or of all matrices (id < 0); enqueued on the stream
 static int refresh_frag(egg_ctx *ctx, int id) {
-    const int B = ctx->cfg.hidden < 256 ? ctx->cfg.hidden : 256;
     for (int i = 0; i < (int)ctx->tensors.size(); i++) {
         const egg_tensor_info &t = ctx->tensors[i];
         if (!t.is_matrix || (id >= 0 && i != id)) continue;
+        // hidden x hidden blocks for the layer matrices; the embedding (hidden x 256) is cut into <= 256-wide blocks
+        const int B = (t.cols == ctx->cfg.vocab && t.rows == ctx->cfg.hidden && ctx->cfg.hidden > 256) ? 256 : ctx->cfg.hidden;
         HIP_TRY(egg_launch_swizzle(ctx->d_model + t.offset, ctx->d_wfrag + t.offset, t.rows, t.cols, B, 0, ctx->stream));
     }
     return EGG_OK;

@@ -51,7 +51,7 @@ struct MlpLds {
 };
 
 template <int H, bool FIRST>
-__global__ void __launch_bounds__(EGG_THREADS, 2) k_mlp(MlpParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_mlp(MlpParams p) {
     constexpr int KS = H / 32, NT = H / 32, PR = H / 16;      // k-steps, column groups, p-rows of a full-K unit
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *act = smem + MlpLds<H>::WBYTES;
@@ -271,7 +271,7 @@ __device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row,
 }
 
 template <int H>
-__global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_qkv(QkvParams p) {
     constexpr int KS = H / 32, NT = H / 32;
     extern __shared__ __align__(16) int8_t smem[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
@@ -353,7 +353,7 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
 // causal context (row max, then LUT weights), O^T = V^T.P^T with the 19-bit weights split into three
 // 7-bit planes so the weighted sum stays exact on the int8 MFMA.
 template <int HD, int CT>
-__global__ void __launch_bounds__(EGG_THREADS, 2) k_attn(AttnParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnParams p) {
     constexpr int KS = HD / 32, DT = HD / 32;
     constexpr int T = CT * 32;
     extern __shared__ __align__(16) int8_t smem[];
@@ -496,7 +496,7 @@ struct HeadLds {
 };
 
 template <int H>
-__global__ void __launch_bounds__(EGG_THREADS, 2) k_head(HeadParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadParams p) {
     constexpr int KS = H / 32, NV = 256 / 32, BLK = H < 256 ? H : 256;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *wlds = smem;
@@ -601,6 +601,7 @@ hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s) {
         case 64: return launch_mlp_h<64>(p, first, s);
         case 128: return launch_mlp_h<128>(p, first, s);
         case 256: return launch_mlp_h<256>(p, first, s);
+        case 512: return launch_mlp_h<512>(p, first, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -618,6 +619,7 @@ hipError_t egg_launch_qkv(const QkvParams &p, hipStream_t s) {
         case 64: return launch_qkv_h<64>(p, s);
         case 128: return launch_qkv_h<128>(p, s);
         case 256: return launch_qkv_h<256>(p, s);
+        case 512: return launch_qkv_h<512>(p, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -637,6 +639,7 @@ static hipError_t launch_attn_hd(const AttnParams &p, hipStream_t s) {
         case 2: return launch_attn_t<HD, 2>(p, s);
         case 4: return launch_attn_t<HD, 4>(p, s);
         case 8: return launch_attn_t<HD, 8>(p, s);
+        case 16: return launch_attn_t<HD, 16>(p, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -660,6 +663,7 @@ hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
         case 64: return launch_head_h<64>(p, s);
         case 128: return launch_head_h<128>(p, s);
         case 256: return launch_head_h<256>(p, s);
+        case 512: return launch_head_h<512>(p, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -668,10 +672,11 @@ hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
 // so it is done at context creation and never while a stream is capturing)
 #define SET_LDS(kern, bytes) do { hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)); if (e_ != hipSuccess) return e_; } while (0)
 template <int H>
-static hipError_t prepare_h() {
-    SET_LDS((k_mlp<H, true>), MlpLds<H>::total(4));
-    SET_LDS((k_mlp<H, false>), MlpLds<H>::total(4));
-    SET_LDS((k_qkv<H>), QkvLds<H>::total(4));
+static hipError_t prepare_h(int T) {
+    const int sets = tile_map_sets(T);
+    SET_LDS((k_mlp<H, true>), MlpLds<H>::total(sets));
+    SET_LDS((k_mlp<H, false>), MlpLds<H>::total(sets));
+    SET_LDS((k_qkv<H>), QkvLds<H>::total(sets));
     SET_LDS((k_head<H>), HeadLds<H>::TOTAL);
     return hipSuccess;
 }
@@ -687,15 +692,17 @@ static hipError_t prepare_attn_hd(int ct) {
         case 2: return prepare_attn<HD, 2>();
         case 4: return prepare_attn<HD, 4>();
         case 8: return prepare_attn<HD, 8>();
+        case 16: return prepare_attn<HD, 16>();
         default: return hipErrorInvalidValue;
     }
 }
 hipError_t egg_prepare_forward(int H, int head_dim, int T) {
     hipError_t e;
     switch (H) {
-        case 64: e = prepare_h<64>(); break;
-        case 128: e = prepare_h<128>(); break;
-        case 256: e = prepare_h<256>(); break;
+        case 64: e = prepare_h<64>(T); break;
+        case 128: e = prepare_h<128>(T); break;
+        case 256: e = prepare_h<256>(T); break;
+        case 512: e = prepare_h<512>(T); break;
         default: return hipErrorInvalidValue;
     }
     if (e != hipSuccess) return e;

@@ -91,8 +91,10 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
 
 @pytest.mark.parametrize("kw", [SMALL,
                                 dict(hidden=128, head_dim=32, n_layers=1, seq_len=64, population=6),
-                                dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4)],
-                         ids=["h64", "h128", "h256"])
+                                dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4),
+                                dict(hidden=512, head_dim=64, n_layers=1, seq_len=128, population=4),
+                                dict(hidden=512, head_dim=64, n_layers=2, seq_len=512, population=2)],
+                         ids=["h64", "h128", "h256", "h512_t128", "h512_t512"])
 def test_forward_stages_and_loss(pkg, orc, dev, kw):
     """Every stage tap of every member against the oracle's trace, then the per-member losses."""
     data = orc.zipf_bytes(1 << 15)
@@ -177,7 +179,9 @@ def test_fitness(pkg, orc, dev):
 
 
 @pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=200),
-                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=66)], ids=["p200", "p66"])
+                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=66),
+                                dict(hidden=512, head_dim=64, n_layers=1, seq_len=128, population=40)],
+                         ids=["p200", "p66", "h512"])
 def test_votes_and_adam_update(pkg, orc, dev, kw):
     import torch
     ocfg = orc.config(**kw)
@@ -266,6 +270,8 @@ def test_error_paths(pkg, dev):
         pkg.Context(pkg.default_config(hidden=100))
     with pytest.raises(pkg.EggError):
         pkg.Context(pkg.default_config(seq_len=48))
+    with pytest.raises(pkg.EggError):
+        pkg.Context(pkg.default_config(hidden=512, seq_len=64))
     ctx = pkg.Context(pkg.default_config(**SMALL))
     with pytest.raises(pkg.EggError):
         ctx.step_launch(0, 1, 0.1)            # launch before capture
@@ -278,9 +284,9 @@ def test_newton_schulz_gpu(pkg, orc, dev):
     """fp32 MFMA Newton-Schulz against the fp64 restatement (the reference's cuBLAS summation order is unspecified,
     so this is a tolerance check: relative Frobenius error <= 1e-5) plus the orthogonality it is meant to reach."""
     import torch
-    ctx = pkg.Context(pkg.default_config(use_muon=1, hidden=256, head_dim=64, n_layers=1, seq_len=32, population=8))
+    ctx = pkg.Context(pkg.default_config(use_muon=1, hidden=512, head_dim=64, n_layers=1, seq_len=128, population=8))
     rng = np.random.default_rng(21)
-    for rows, cols in ((256, 256), (256, 1024), (1024, 256), (64, 96)):
+    for rows, cols in ((256, 256), (256, 1024), (1024, 256), (64, 96), (512, 512), (512, 2048), (2048, 512)):
         X = (rng.integers(-300, 301, (rows, cols))).astype(np.float32)
         ref = X.astype(np.float64)
         orc.lib().orc_newton_schulz_f64(ref.ctypes.data_as(C.c_void_p), rows, cols, 5)
