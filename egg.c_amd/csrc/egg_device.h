@@ -112,14 +112,19 @@ __device__ __forceinline__ void w_prefetch(WStream &s, const int8_t *unit) {
     if (unit == nullptr) return;
     constexpr int CHUNKS = WUnit<B>::BYTES / 16;                 // 16-byte chunks, 64 per wave instruction
     constexpr int PER = (CHUNKS / 64 + EGG_WAVES - 1) / EGG_WAVES;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // the wave index is read through readfirstlane so that the compiler keeps every address part that does not
+    // depend on the lane in scalar registers (LDS destination in M0, global base in an SGPR pair)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lane16 = (threadIdx.x & 63u) * 16u;
     int8_t *dst = s.fill;
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int c0 = (i * EGG_WAVES + wave) * 64;
-        if (CHUNKS / 64 % EGG_WAVES == 0 || c0 < CHUNKS)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(unit + (size_t)(c0 + lane) * 16),
+        if (CHUNKS / 64 % EGG_WAVES == 0 || c0 < CHUNKS) {
+            const int8_t *ubase = unit + (size_t)c0 * 16;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ubase + lane16),
                                              (__attribute__((address_space(3))) void *)(dst + (size_t)c0 * 16), 16, 0, 0);
+        }
     }
 }
 // wait for the unit prefetched last, make it visible to the workgroup, and hand it out
@@ -178,14 +183,16 @@ __device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, int s
     if (src == nullptr) return;
     static_assert(COLS % 64 == 0, "a wave instruction copies 64 columns");
     constexpr int SEG = COLS / 64, INSTR = NP * SEG, PER = (INSTR + EGG_WAVES - 1) / EGG_WAVES;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lane16 = (threadIdx.x & 63u) * 16u;
     int8_t *dst = s.fill;
 #pragma unroll
     for (int i = 0; i < PER; i++) {
         const int id = i * EGG_WAVES + wave;
         if (INSTR % EGG_WAVES == 0 || id < INSTR) {
             const int pr = id / SEG, seg = id % SEG;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + ((size_t)pr * src_cols + seg * 64 + lane) * 16),
+            const int8_t *ubase = src + ((size_t)pr * src_cols + seg * 64) * 16;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ubase + lane16),
                                              (__attribute__((address_space(3))) void *)(dst + ((size_t)pr * COLS + seg * 64) * 16), 16, 0, 0);
         }
     }
