@@ -165,7 +165,6 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (!(c.hidden == 64 || c.hidden == 128 || c.hidden == 256 || c.hidden == 512)) return EGG_E_INVALID;
     if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return EGG_E_INVALID;
     if (!(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256 || c.seq_len == 512)) return EGG_E_INVALID;
-    if (c.hidden == 512 && c.seq_len < 128) return EGG_E_INVALID;      // the per-member LDS tables of hidden 512 fit once per workgroup
     if (c.vocab != 256 || c.n_layers < 1 || c.population < 2 || (c.population & 1)) return EGG_E_INVALID;
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;

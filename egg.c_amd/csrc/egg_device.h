@@ -210,24 +210,65 @@ __device__ __forceinline__ void mfma_unit2(v16i *acc, const v4i *xop, const int8
         }
 }
 
-// How the four waves of a workgroup map to (member, tile) for a sequence of T tokens: with at least four tiles
-// per member the whole workgroup serves one member (one shared set of noise tables) and walks its tiles in
-// passes of four; with two tiles it serves two members, with one tile four.
+// acc[nt] += unit^T . xop for the NTW column groups starting at column `colbase` of a staged unit that is
+// KSU k-steps deep and `cols` columns wide
+template <int KSU, int NTW>
+__device__ __forceinline__ void mfma_cols(v16i *acc, const v4i *xop, const int8_t *lds, int cols, int colbase, int lane) {
+    const int i = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int ks = 0; ks < KSU; ks++)
+#pragma unroll
+        for (int nt = 0; nt < NTW; nt++) {
+            v4i a = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * cols + colbase + nt * 32 + i) * 16);
+            acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, xop[ks], acc[nt], 0, 0, 0);
+        }
+}
+
+// Column split: for hidden sizes above 128 the H-wide accumulators of one 32-token tile do not fit one wave next to
+// its operands, so CS = H/128 waves share a tile and each owns H/CS output columns (and 32*NTU of every sub-chunk
+// of the MLP intermediate).  Per-token row statistics and the operands of the next GEMM are exchanged through LDS.
+template <int H>
+struct Shape {
+    static constexpr int CS = H <= 128 ? 1 : H / 128;
+    static constexpr int TPW = EGG_WAVES / CS;            // token tiles a workgroup covers per pass
+    static constexpr int HS = H / CS, NTS = HS / 32, KS = H / 32;
+};
+
+// How the waves of a workgroup map to (member, tile, column slice) for a sequence of T tokens: with at least TPW
+// tiles per member the whole workgroup serves one member (one shared set of noise tables) and walks its tiles in
+// passes of TPW; with fewer it serves TPW / tiles members at once.
 struct TileMap {
     int sets;        // members (= noise table sets) per workgroup
     int passes;
     int set;         // table set of this wave
     int mloc;        // member index within the chunk (may be >= n_members for a padding wave)
-    int tile0;       // tile of this wave in pass 0; later passes add 4
+    int tile0;       // tile of this wave in pass 0; later passes add TPW
+    int tslot;       // which of the workgroup's TPW tiles this wave works on
+    int cs;          // column slice of this wave
 };
+template <int CS>
 __device__ __forceinline__ TileMap tile_map(int T, int wave, int block) {
+    constexpr int TPW = EGG_WAVES / CS;
     TileMap m; const int tpm = T / 32;
-    if (tpm >= 4) { m.sets = 1; m.passes = tpm / 4; m.set = 0; m.mloc = block; m.tile0 = wave; }
-    else if (tpm == 2) { m.sets = 2; m.passes = 1; m.set = wave >> 1; m.mloc = block * 2 + (wave >> 1); m.tile0 = wave & 1; }
-    else { m.sets = 4; m.passes = 1; m.set = wave; m.mloc = block * 4 + wave; m.tile0 = 0; }
+    m.tslot = wave / CS; m.cs = wave % CS;
+    if (tpm >= TPW) { m.sets = 1; m.passes = tpm / TPW; m.set = 0; m.mloc = block; m.tile0 = m.tslot; }
+    else { m.sets = TPW / tpm; m.passes = 1; m.set = m.tslot / tpm; m.mloc = block * m.sets + m.set; m.tile0 = m.tslot % tpm; }
     return m;
 }
-static inline int tile_map_sets(int T) { int tpm = T / 32; return tpm >= 4 ? 1 : (tpm == 2 ? 2 : 4); }
+static inline int tile_map_sets(int T, int cs) { int tpm = T / 32, tpw = EGG_WAVES / cs; return tpm >= tpw ? 1 : tpw / tpm; }
+
+// Combine a per-token value over the CS waves sharing a tile.  `site` is an LDS area of EGG_WAVES*64 ints that no
+// other exchange uses until every wave has passed another barrier.  Every wave of the workgroup must call it.
+template <int CS, bool IS_MAX>
+__device__ __forceinline__ int xreduce(int v, int *site, const TileMap &tm, int lane) {
+    if (CS == 1) return v;
+    site[(tm.tslot * CS + tm.cs) * 64 + lane] = v;
+    __syncthreads();
+    int r = site[(tm.tslot * CS) * 64 + lane];
+#pragma unroll
+    for (int c = 1; c < CS; c++) { int o = site[(tm.tslot * CS + c) * 64 + lane]; r = IS_MAX ? max(r, o) : r + o; }
+    return r;
+}
 
 template <int N>
 __device__ __forceinline__ void zero_acc(v16i *acc) {
@@ -238,8 +279,8 @@ __device__ __forceinline__ void zero_acc(v16i *acc) {
 }
 
 // ---------------------------------------------------------------- per-member noise tables (one wave fills its own)
-__device__ __forceinline__ void fill_noise_i8(int8_t *dst, uint32_t seed, int n, int mask, int lane, int nthr = 64) {
-    for (int i = lane; i < n; i += nthr) dst[i] = (int8_t)noise_from_hash(seed, i, mask);
+__device__ __forceinline__ void fill_noise_i8(int8_t *dst, uint32_t seed, int n, int mask, int lane, int nthr = 64, int mult = 1) {
+    for (int i = lane; i < n; i += nthr) dst[i] = (int8_t)(noise_from_hash(seed, i, mask) * mult);
 }
 // dst[i] = noise(seed, i) * mult
 __device__ __forceinline__ void fill_noise_i32(int *dst, uint32_t seed, int n, int mask, int mult, int lane, int nthr = 64) {
@@ -277,23 +318,26 @@ __device__ __forceinline__ int dot_noise(const v4i *xop, const int8_t *btab, int
 }
 
 // ---------------------------------------------------------------- norms on a token held as a packed operand
-// apply_standard_norm (mgpu.cu:646-678): wt / bt are int32 tables already holding w + noise, b + noise
-template <int KS>
-__device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int *wt, const int *bt, int g) {
-    constexpr int H = 32 * KS;
+// apply_standard_norm (mgpu.cu:646-678) in two parts so that the row sum can be combined across waves:
+// sum of |x| over N column groups (this lane's half only), then the scaling of N groups whose first column is col0.
+// wt / bt are int32 tables already holding w + noise, b + noise.
+template <int N>
+__device__ __forceinline__ int sumabs_groups(const v4i *x) {
     int tot = 0;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++)
+    for (int ks = 0; ks < N; ks++)
 #pragma unroll
         for (int q = 0; q < 4; q++) tot = sumabs4(x[ks][q], tot);
-    tot += other_half(tot);
-    int mn = tot / H; if (!mn) mn = 1;
+    return tot;
+}
+template <int N>
+__device__ __forceinline__ void standard_scale(const v4i *x, v4i *out, int mn, const int *wt, const int *bt, int col0, int g) {
     const float md = 1.0f / (float)mn;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++)
+    for (int ks = 0; ks < N; ks++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            int n0 = 32 * ks + 8 * q + 4 * g;
+            int n0 = col0 + 32 * ks + 8 * q + 4 * g;
             v4i w4 = *reinterpret_cast<const v4i *>(wt + n0);
             v4i b4 = *reinterpret_cast<const v4i *>(bt + n0);
             int o[4];
@@ -302,10 +346,19 @@ __device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int 
             out[ks][q] = pack4(o[0], o[1], o[2], o[3]);
         }
 }
+template <int KS>
+__device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int *wt, const int *bt, int g) {
+    int tot = sumabs_groups<KS>(x);
+    tot += other_half(tot);
+    int mn = tot / (32 * KS); if (!mn) mn = 1;
+    standard_scale<KS>(x, out, mn, wt, bt, 0, g);
+}
 
-// adaptive_*_normalize (egg_adaptive_normalize.h:10-103) over NT column groups held in acc; result packed
+// adaptive_*_normalize (egg_adaptive_normalize.h:10-103), also in two parts: max |val| over NT column groups
+// (both lane halves of the token combined), then the scaling.  The reference's final clamp to +-127 never binds:
+// |val| <= mx, so (float)val * (127.0f / (float)mx) <= 127 * (1 + 2^-23) and rounds to at most 127.
 template <int NT>
-__device__ __forceinline__ void adaptive_norm(const v16i *val, v4i *out) {
+__device__ __forceinline__ int absmax_groups(const v16i *val) {
     int hi = 0, lo = 0;
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
@@ -315,20 +368,24 @@ __device__ __forceinline__ void adaptive_norm(const v16i *val, v4i *out) {
             lo = min(min(lo, val[nt][r]), val[nt][r + 1]);
         }
     int mx = max(hi, -lo);
-    mx = max(mx, other_half(mx));
-    float scale = 127.0f / ((float)mx + 1e-9f);
+    return max(mx, other_half(mx));
+}
+template <int NT>
+__device__ __forceinline__ void adaptive_scale(const v16i *val, int mx, v4i *out) {
+    const float scale = 127.0f / ((float)mx + 1e-9f);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             int o[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                float sf = (float)val[nt][4 * q + e] * scale;
-                o[e] = clip127(round_half_away(sf));
-            }
+            for (int e = 0; e < 4; e++) o[e] = round_half_away((float)val[nt][4 * q + e] * scale);
             out[nt][q] = pack4(o[0], o[1], o[2], o[3]);
         }
+}
+template <int NT>
+__device__ __forceinline__ void adaptive_norm(const v16i *val, v4i *out) {
+    adaptive_scale<NT>(val, absmax_groups<NT>(val), out);
 }
 
 // 128-bit load/store of a token's 16 bytes of column group `grp` in a slot-ordered [.][H] int8 buffer

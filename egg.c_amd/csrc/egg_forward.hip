@@ -35,66 +35,112 @@ __device__ __forceinline__ void add_perturb(v16i *acc, int sb, const int *At, in
         }
 }
 
+// same with the output-side noise kept as int8, already multiplied by the member's sign
+template <int NT>
+__device__ __forceinline__ void add_perturb8(v16i *acc, int sb, const int8_t *At, int n_off, int sigma, int g) {
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            int a4 = *reinterpret_cast<const int *>(At + n_off + 32 * nt + 8 * q + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[nt][4 * q + e] += mul24(sb, sx8(a4, e)) >> sigma;
+        }
+}
+
+// exchange of packed 32-column groups between the waves sharing a tile: group k of tile slot ts, 16 bytes per lane
+__device__ __forceinline__ void xch_put(int8_t *xch, int groups, int ts, int k, int lane, v4i v) {
+    *reinterpret_cast<v4i *>(xch + ((size_t)(ts * groups + k) * 64 + lane) * 16) = v;
+}
+__device__ __forceinline__ v4i xch_get(const int8_t *xch, int groups, int ts, int k, int lane) {
+    return *reinterpret_cast<const v4i *>(xch + ((size_t)(ts * groups + k) * 64 + lane) * 16);
+}
+
 // ============================================================================ MLP block
-// Register-lean form (<= 256 VGPRs, two workgroups per CU): the 4H-wide intermediate is produced 64 columns at a
-// time (up GEMM on a [H x 64] unit, GELU epilogue, immediately consumed as two k-steps of the down GEMM on a
-// [64 x H] unit), so only the H-wide down accumulator, the normalised input and a 64-column accumulator are live.
-// W units (64*H bytes) stream through two LDS buffers.  The residual is parked in the x buffer and re-read at the end.
+// The 4H-wide intermediate is produced SC columns at a time (up GEMM, GELU epilogue, immediately consumed as k-steps
+// of the down GEMM), so only the down accumulator of the wave's column slice, the normalised input and one
+// sub-chunk accumulator are live.  W streams through two LDS buffers in units of at most 16 KB.  The residual is
+// parked in the x buffer and re-read at the end.
 template <int H>
-struct MlpLds {
-    static constexpr int I32 = 14 * H;       // ex0[H] ex1[H] lnw[H] lnb[H] upA[4H] bup[4H] dnA[H] bdn[H]
-    static constexpr int I8 = 6 * H;         // exB[H] upB[H] dnB[4H]
-    static constexpr int PER_SET = I32 * 4 + I8;
-    static constexpr int UNIT = 64 * H;
+struct MlpCfg {
+    typedef Shape<H> S;
+    static constexpr int CS = S::CS, TPW = S::TPW, HS = S::HS, NTS = S::NTS, KS = S::KS;
+    static constexpr int NTU = CS == 1 ? 2 : 1;          // up-GEMM column groups per wave and sub-chunk
+    static constexpr int SC = 32 * CS * NTU;             // intermediate columns per sub-chunk
+    static constexpr int NSUB = 4 * H / SC;
+    static constexpr int cmin(int a, int b) { return a < b ? a : b; }
+    static constexpr int cmax(int a, int b) { return a > b ? a : b; }
+    // p-rows (16 k-bytes each, two per k-step) per staged unit and units per GEMM
+    static constexpr int PRO = cmin(H / 16, 1024 / H), OU = (H / 16) / PRO;         // O projection  [H x H]
+    static constexpr int PRUP = cmin(H / 16, 1024 / SC), UPU = (H / 16) / PRUP;     // up sub-chunk  [H x SC]
+    static constexpr int PRDN = cmin(SC / 16, 1024 / H), DNU = (SC / 16) / PRDN;    // down sub-chunk [SC x H]
+    static constexpr int UNIT = 16 * cmax(PRO * H, cmax(PRUP * SC, PRDN * H));
     static constexpr int WBYTES = 2 * UNIT;
-    static int total(int sets) { return WBYTES + 256 + sets * PER_SET; }
+    static constexpr int I32 = 9 * H;        // ex0[H] ex1[H] lnw[H] lnb[H] bup[4H] bdn[H]
+    static constexpr int I8 = 11 * H;        // exB[H] upB[H] dnB[4H] upA[4H] dnA[H]   (A noise already times the sign)
+    static constexpr int PER_SET = I32 * 4 + I8;
+    static constexpr int XCHG = CS > 1 ? TPW * 32 * H : 0;          // normalised input / intermediate exchange
+    static constexpr int SITE = EGG_WAVES * 64;                       // ints per reduction site
+    static constexpr int RED = CS > 1 ? 4 * SITE * 4 : 0;
+    static int total(int sets) { return WBYTES + 256 + sets * PER_SET + XCHG + RED; }
 };
 
 template <int H, bool FIRST>
-__global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_mlp(MlpParams p) {
-    constexpr int KS = H / 32, NT = H / 32, PR = H / 16;      // k-steps, column groups, p-rows of a full-K unit
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_mlp(MlpParams p) {
+    typedef MlpCfg<H> M;
+    constexpr int CS = M::CS, KS = M::KS, NTS = M::NTS, HS = M::HS, NTU = M::NTU, SC = M::SC;
     extern __shared__ __align__(16) int8_t smem[];
-    int8_t *act = smem + MlpLds<H>::WBYTES;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    int8_t *act = smem + M::WBYTES;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const FwdCommon &c = p.c;
     const int T = c.T;
-    const TileMap tm = tile_map(T, wave, blockIdx.x);
-    int8_t *tb = act + 256 + tm.set * MlpLds<H>::PER_SET;
-    int *ex0 = reinterpret_cast<int *>(tb);   // FIRST: emb_bias + noise   | else: O-proj A noise * ns
-    int *ex1 = ex0 + H;                       // FIRST: b_dim noise * ns    | else: unused
-    int *lnw = ex1 + H, *lnb = lnw + H, *upA = lnb + H, *bup = upA + 4 * H, *dnA = bup + 4 * H, *bdn = dnA + H;
+    const TileMap tm = tile_map<CS>(T, wave, blockIdx.x);
+    const int col0 = tm.cs * HS;                      // first output column of this wave's slice
+    int8_t *tb = act + 256 + tm.set * M::PER_SET;
+    int *ex0 = reinterpret_cast<int *>(tb);           // FIRST: emb_bias + noise   | else: O-proj A noise * ns as int8
+    int *ex1 = ex0 + H;                               // FIRST: b_dim noise * ns    | else: unused
+    int *lnw = ex1 + H, *lnb = lnw + H, *bup = lnb + H, *bdn = bup + 4 * H;
     int8_t *exB = reinterpret_cast<int8_t *>(bdn + H);   // O-proj B noise
-    int8_t *upB = exB + H, *dnB = upB + H;
+    int8_t *upB = exB + H, *dnB = upB + H, *upA = dnB + 4 * H, *dnA = upA + 4 * H;
+    const int8_t *oA = reinterpret_cast<const int8_t *>(ex0);
+    int8_t *xch = act + 256 + tm.sets * M::PER_SET;
+    int *red = reinterpret_cast<int *>(xch + M::XCHG);
 
-    WStream ws; wstream_init(ws, smem, MlpLds<H>::UNIT);
-    // unit sources inside the fragment-major copies (block size B == H for H <= 256)
-    auto up_unit = [&](int sidx) { return p.w_up + (size_t)((64 * sidx) / H) * H * H + (size_t)((64 * sidx) % H) * 16; };
-    auto dn_unit = [&](int sidx) { return p.w_dn + (size_t)((64 * sidx) / H) * H * H + (size_t)(((64 * sidx) % H) / 16) * H * 16; };
-    auto o_unit = [&](int u) { return p.w_o + (size_t)(4 * u) * H * 16; };
-    const int8_t *pass_first = FIRST ? up_unit(0) : o_unit(0);
-    if (FIRST) w_prefetch2<PR, 64>(ws, pass_first, H); else w_prefetch2<4, H>(ws, pass_first, H);
+    WStream ws; wstream_init(ws, smem, M::UNIT);
+    // unit sources inside the fragment-major copies (block size == H)
+    auto pf_up = [&](int s, int ku) {
+        const int n = s * SC;
+        w_prefetch2<M::PRUP, SC>(ws, p.w_up + (size_t)(n / H) * H * H + ((size_t)ku * M::PRUP * H + n % H) * 16, H);
+    };
+    auto pf_dn = [&](int s, int du) {
+        const int k = s * SC;
+        w_prefetch2<M::PRDN, H>(ws, p.w_dn + (size_t)(k / H) * H * H + (size_t)((k % H) / 16 + du * M::PRDN) * H * 16, H);
+    };
+    auto pf_o = [&](int u) { w_prefetch2<M::PRO, H>(ws, p.w_o + (size_t)u * M::PRO * H * 16, H); };
+    auto pf_pass_first = [&]() { if (FIRST) pf_up(0, 0); else pf_o(0); };
+    pf_pass_first();
 
     for (int i = threadIdx.x; i < 256; i += EGG_THREADS) act[i] = c.act_lut[i];
     for (int ss = 0; ss < tm.sets; ss++) {
         int ml = blockIdx.x * tm.sets + ss; if (ml >= c.n_members) ml = c.n_members - 1;
         const int mem = c.pop_offset + ml, nsx = (mem & 1) ? -1 : 1;
         const uint32_t pseed = *c.d_step_seed + (uint32_t)(mem / 2), sbx = pseed + (uint32_t)p.seed_base;
-        int8_t *t2 = act + 256 + ss * MlpLds<H>::PER_SET;
-        int *e0 = reinterpret_cast<int *>(t2), *e1 = e0 + H, *lw = e1 + H, *lb = lw + H, *uA = lb + H, *bu = uA + 4 * H, *dA = bu + 4 * H, *bd = dA + H;
-        int8_t *eB = reinterpret_cast<int8_t *>(bd + H), *uB = eB + H, *dB = uB + H;
+        int8_t *t2 = act + 256 + ss * M::PER_SET;
+        int *e0 = reinterpret_cast<int *>(t2), *e1 = e0 + H, *lw = e1 + H, *lb = lw + H, *bu = lb + H, *bd = bu + 4 * H;
+        int8_t *eB = reinterpret_cast<int8_t *>(bd + H), *uB = eB + H, *dB = uB + H, *uA = dB + 4 * H, *dA = uA + 4 * H;
         const int tid = threadIdx.x;
         if (FIRST) {
             fill_vec_i32(e0, p.emb_bias, pseed + OFF_EMB_BIAS_A, pseed + OFF_EMB_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
             fill_noise_i32(e1, pseed + OFF_EMB + H, H, c.mask, nsx, tid, EGG_THREADS);
         } else {
-            fill_noise_i32(e0, sbx + OFF_O_A, H, c.mask, nsx, tid, EGG_THREADS);
+            fill_noise_i8(reinterpret_cast<int8_t *>(e0), sbx + OFF_O_A, H, c.mask, tid, EGG_THREADS, nsx);
             fill_noise_i8(eB, sbx + OFF_O_B, H, c.mask, tid, EGG_THREADS);
         }
         fill_vec_i32(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_vec_i32(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
-        fill_noise_i32(uA, sbx + p.off_up_a, 4 * H, c.mask, nsx, tid, EGG_THREADS);
+        fill_noise_i8(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx);
         fill_vec_i32(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
-        fill_noise_i32(dA, sbx + p.off_dn_a, H, c.mask, nsx, tid, EGG_THREADS);
+        fill_noise_i8(dA, sbx + p.off_dn_a, H, c.mask, tid, EGG_THREADS, nsx);
         fill_vec_i32(bd, p.b_dn, sbx + p.off_bdn_a, sbx + p.off_bdn_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_noise_i8(uB, sbx + p.off_up_b, H, c.mask, tid, EGG_THREADS);
         fill_noise_i8(dB, sbx + p.off_dn_b, 4 * H, c.mask, tid, EGG_THREADS);
@@ -109,9 +155,10 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_mlp(MlpParam
     const int64_t spos = FIRST ? stream_pos_of(c, member) : 0;
 
     for (int pass = 0; pass < tm.passes; pass++) {
-        const int t = (tm.tile0 + 4 * pass) * 32 + j;
+        const int t = (tm.tile0 + M::TPW * pass) * 32 + j;
         const size_t row = ((size_t)mloc * T + t) * H;
-        v4i xcur[KS];
+        int8_t *xrow = p.x + row + col0;                 // this wave's slice of the residual row
+        v4i xs[NTS];
 
         if (FIRST) {
             // embedding stage (mgpu.cu:901-931)
@@ -119,128 +166,168 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_mlp(MlpParam
             const int a_tok = noise_from_hash(pair_seed + OFF_EMB, (uint32_t)tok, c.mask);
             const uint32_t *E32 = reinterpret_cast<const uint32_t *>(p.embedding);
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++)
+            for (int nt = 0; nt < NTS; nt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    int n0 = 32 * ks + 8 * q + 4 * g;
+                    int n0 = col0 + 32 * nt + 8 * q + 4 * g;
                     int e4 = (int)E32[(size_t)(n0 >> 2) * c.vocab + tok];
                     v4i b4 = *reinterpret_cast<const v4i *>(ex0 + n0);
                     v4i d4 = *reinterpret_cast<const v4i *>(ex1 + n0);
                     int o[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) o[e] = clip127(sx8(e4, e) + b4[e] + (mul24(a_tok, d4[e]) >> c.sigma));
-                    xcur[ks][q] = pack4(o[0], o[1], o[2], o[3]);
+                    xs[nt][q] = pack4(o[0], o[1], o[2], o[3]);
                 }
         } else {
             // attention output projection + residual + adaptive norm (mgpu.cu:827-831)
-            v4i aop[KS];
+            v16i acc[NTS];
+            zero_acc<NTS>(acc);
+            int sbo;
+            {
+                v4i aop[KS];
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) aop[ks] = load_op(p.ao + row, ks, g);
-            const int sbo = dot_noise<KS, false>(aop, exB, 0, g);
-            v16i acc[NT];
-            zero_acc<NT>(acc);
+                for (int ks = 0; ks < KS; ks++) aop[ks] = load_op(p.ao + row, ks, g);
+                sbo = dot_noise<KS, false>(aop, exB, 0, g);
 #pragma unroll
-            for (int u = 0; u < H / 64; u++) {
-                const int8_t *cur = w_acquire(ws);
-                if (u + 1 < H / 64) w_prefetch2<4, H>(ws, o_unit(u + 1), H); else w_prefetch2<PR, 64>(ws, up_unit(0), H);
-                mfma_unit2<2, NT>(acc, aop + 2 * u, cur, lane);
+                for (int u = 0; u < M::OU; u++) {
+                    const int8_t *cur = w_acquire(ws);
+                    if (u + 1 < M::OU) pf_o(u + 1); else pf_up(0, 0);
+                    mfma_cols<M::PRO / 2, NTS>(acc, aop + u * (M::PRO / 2), cur, H, col0, lane);
+                }
             }
-            add_perturb<NT>(acc, sbo, ex0, 0, c.sigma, g);
+            add_perturb8<NTS>(acc, sbo, oA, col0, c.sigma, g);
 #pragma unroll
-            for (int nt = 0; nt < NT; nt++) {
-                v4i xr = load_op(p.x + row, nt, g);
+            for (int nt = 0; nt < NTS; nt++) {
+                v4i xr = load_op(xrow, nt, g);
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[nt][r] = sx8(xr[r >> 2], r & 3) + (acc[nt][r] >> c.shift_out);
             }
-            adaptive_norm<NT>(acc, xcur);
+            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red, tm, lane);
+            adaptive_scale<NTS>(acc, mx, xs);
             if (p.x_mid && valid)
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) store_op(p.x_mid + row, ks, g, xcur[ks]);
+                for (int nt = 0; nt < NTS; nt++) store_op(p.x_mid + row + col0, nt, g, xs[nt]);
         }
-        // park the residual (this wave owns the row; invalid padding waves only recompute)
+        // park the residual (this wave owns the slice; invalid padding waves only recompute)
         if (valid)
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) store_op(p.x + row, ks, g, xcur[ks]);
+            for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, g, xs[nt]);
 
         // MLP (mgpu.cu:708-759)
         v4i nrm[KS];
-        standard_norm<KS>(xcur, nrm, lnw, lnb, g);
-        const int sbu = dot_noise<KS, false>(nrm, upB, 0, g);
-        v16i accd[NT];
-        zero_acc<NT>(accd);
-        int sbd = 0;
-        constexpr int NSUB = 4 * H / 64;
-#pragma unroll 1
-        for (int sidx = 0; sidx < NSUB; sidx++) {
-            v16i au[2];
-            zero_acc<2>(au);
-            {
-                const int8_t *cur = w_acquire(ws);
-                w_prefetch2<4, H>(ws, dn_unit(sidx), H);
-                mfma_unit2<KS, 2>(au, nrm, cur, lane);
+        {
+            int tot = sumabs_groups<NTS>(xs);
+            tot += other_half(tot);
+            tot = xreduce<CS, false>(tot, red + M::SITE, tm, lane);
+            int mn = tot / H; if (!mn) mn = 1;
+            if (CS == 1) standard_scale<NTS>(xs, nrm, mn, lnw, lnb, 0, g);
+            else {
+                v4i mine[NTS];
+                standard_scale<NTS>(xs, mine, mn, lnw, lnb, col0, g);
+#pragma unroll
+                for (int nt = 0; nt < NTS; nt++) xch_put(xch, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
+                __syncthreads();
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(xch, KS, tm.tslot, ks, lane);
             }
-            v4i mid[2];
-            const int *dnb32 = reinterpret_cast<const int *>(dnB + 64 * sidx);
+        }
+        const int sbu = dot_noise<KS, false>(nrm, upB, 0, g);
+        v16i accd[NTS];
+        zero_acc<NTS>(accd);
+        int sbd = 0;
+#pragma unroll 1
+        for (int s = 0; s < M::NSUB; s++) {
+            v16i au[NTU];
+            zero_acc<NTU>(au);
 #pragma unroll
-            for (int nt = 0; nt < 2; nt++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    int n0 = 64 * sidx + 32 * nt + 8 * q + 4 * g;
-                    v4i a4 = *reinterpret_cast<const v4i *>(upA + n0);
-                    v4i b4 = *reinterpret_cast<const v4i *>(bup + n0);
-                    int o[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        int a = au[nt][4 * q + e] + (mul24(sbu, a4[e]) >> c.sigma);
-                        int v = clip127((a >> c.shift_mlp_up) + b4[e]);
-                        o[e] = act[(uint8_t)v];
-                    }
-                    mid[nt][q] = pack4(o[0], o[1], o[2], o[3]);
-                    sbd = dot4(mid[nt][q], dnb32[8 * nt + 2 * q + g], sbd);
-                }
-            {
+            for (int ku = 0; ku < M::UPU; ku++) {
                 const int8_t *cur = w_acquire(ws);
-                const int8_t *nx = (sidx + 1 < NSUB) ? up_unit(sidx + 1) : nullptr;
-                if (nx) w_prefetch2<PR, 64>(ws, nx, H);
-                else if (pass + 1 < tm.passes) { if (FIRST) w_prefetch2<PR, 64>(ws, pass_first, H); else w_prefetch2<4, H>(ws, pass_first, H); }
-                mfma_unit2<2, NT>(accd, mid, cur, lane);
+                if (ku + 1 < M::UPU) pf_up(s, ku + 1); else pf_dn(s, 0);
+                mfma_cols<M::PRUP / 2, NTU>(au, nrm + ku * (M::PRUP / 2), cur, SC, tm.cs * 32 * NTU, lane);
+            }
+            v4i mid[CS * NTU];
+            {
+                const int nb = s * SC + tm.cs * 32 * NTU;            // first intermediate column of this wave
+                const int *dnb32 = reinterpret_cast<const int *>(dnB + nb);
+                v4i mine[NTU];
+#pragma unroll
+                for (int nt = 0; nt < NTU; nt++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        int n0 = nb + 32 * nt + 8 * q + 4 * g;
+                        int a4 = *reinterpret_cast<const int *>(upA + n0);
+                        v4i b4 = *reinterpret_cast<const v4i *>(bup + n0);
+                        int o[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            int a = au[nt][4 * q + e] + (mul24(sbu, sx8(a4, e)) >> c.sigma);
+                            int v = clip127((a >> c.shift_mlp_up) + b4[e]);
+                            o[e] = act[(uint8_t)v];
+                        }
+                        mine[nt][q] = pack4(o[0], o[1], o[2], o[3]);
+                        sbd = dot4(mine[nt][q], dnb32[8 * nt + 2 * q + g], sbd);
+                    }
+                if (CS == 1) {
+#pragma unroll
+                    for (int nt = 0; nt < NTU; nt++) mid[nt] = mine[nt];
+                } else {
+#pragma unroll
+                    for (int nt = 0; nt < NTU; nt++) xch_put(xch, CS * NTU, tm.tslot, tm.cs * NTU + nt, lane, mine[nt]);
+                }
+            }
+#pragma unroll
+            for (int du = 0; du < M::DNU; du++) {
+                const int8_t *cur = w_acquire(ws);        // its barrier also publishes the intermediate slices
+                if (CS > 1 && du == 0)
+#pragma unroll
+                    for (int k = 0; k < CS * NTU; k++) mid[k] = xch_get(xch, CS * NTU, tm.tslot, k, lane);
+                if (du + 1 < M::DNU) pf_dn(s, du + 1);
+                else if (s + 1 < M::NSUB) pf_up(s + 1, 0);
+                else if (pass + 1 < tm.passes) pf_pass_first();
+                mfma_cols<M::PRDN / 2, NTS>(accd, mid + du * (M::PRDN / 2), cur, H, col0, lane);
             }
         }
         sbd += other_half(sbd);
-        add_perturb<NT>(accd, sbd, dnA, 0, c.sigma, g);
+        sbd = xreduce<CS, false>(sbd, red + 2 * M::SITE, tm, lane);
+        add_perturb8<NTS>(accd, sbd, dnA, col0, c.sigma, g);
 #pragma unroll
-        for (int nt = 0; nt < NT; nt++) {
-            v4i xr = load_op(p.x + row, nt, g);          // the parked residual (for a padding wave: someone else's row, unused)
-            if (!valid) xr = xcur[nt];
+        for (int nt = 0; nt < NTS; nt++) {
+            v4i xr = load_op(xrow, nt, g);          // the parked residual (for a padding wave: someone else's row, unused)
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                v4i b4 = *reinterpret_cast<const v4i *>(bdn + 32 * nt + 8 * q + 4 * g);
+                v4i b4 = *reinterpret_cast<const v4i *>(bdn + col0 + 32 * nt + 8 * q + 4 * g);
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                     accd[nt][4 * q + e] = sx8(xr[q], e) + (accd[nt][4 * q + e] >> c.shift_mlp_down) + b4[e];
             }
         }
-        v4i xnew[KS];
-        adaptive_norm<NT>(accd, xnew);
+        const int mx2 = xreduce<CS, true>(absmax_groups<NTS>(accd), red + 3 * M::SITE, tm, lane);
+        v4i xnew[NTS];
+        adaptive_scale<NTS>(accd, mx2, xnew);
         if (valid)
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) store_op(p.x + row, ks, g, xnew[ks]);
+            for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, g, xnew[nt]);
     }
 }
 
 // ============================================================================ QKV
 template <int H>
-struct QkvLds {
-    static constexpr int I32 = 5 * H;   // lnw lnb qA kA vA
-    static constexpr int I8 = 3 * H;    // qB kB vB
-    static constexpr int PER_SET = I32 * 4 + I8 + (16 - (I8 % 16)) % 16;
-    static constexpr int UNIT = 64 * H;
+struct QkvCfg {
+    typedef Shape<H> S;
+    static constexpr int CS = S::CS, TPW = S::TPW, HS = S::HS, NTS = S::NTS, KS = S::KS;
+    static constexpr int PR = (H / 16) < (1024 / H) ? (H / 16) : (1024 / H), NU = (H / 16) / PR;   // p-rows per unit, units per matrix
+    static constexpr int UNIT = 16 * PR * H;
     static constexpr int WBYTES = 2 * UNIT;
-    static int total(int sets) { return WBYTES + sets * PER_SET; }
+    static constexpr int PER_SET = 2 * H * 4 + 6 * H;   // lnw lnb (int32) | qA kA vA (int8, times the sign) qB kB vB (int8)
+    static constexpr int XCHG = CS > 1 ? TPW * 32 * H : 0;
+    static constexpr int SITE = EGG_WAVES * 64;
+    static constexpr int RED = CS > 1 ? 4 * SITE * 4 : 0;
+    static int total(int sets) { return WBYTES + sets * PER_SET + XCHG + RED; }
 };
 
 // apply_rope_integer (mgpu.cu:624-644) on the raw accumulators of one token.  The (cos, sin) pairs repeat every
 // head, so a lane needs only the head_dim/32 * 8 pairs of its own slots; they are loaded once and reused.
+// The NT column groups must start at a head boundary.
 template <int NT>
 __device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row, int head_dim, int bit, int g) {
     const long long half = 1ll << (bit - 1);
@@ -271,34 +358,38 @@ __device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row,
 }
 
 template <int H>
-__global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_qkv(QkvParams p) {
-    constexpr int KS = H / 32, NT = H / 32;
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
+    typedef QkvCfg<H> Q;
+    constexpr int CS = Q::CS, KS = Q::KS, NTS = Q::NTS, HS = Q::HS;
     extern __shared__ __align__(16) int8_t smem[];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const FwdCommon &c = p.c;
     const int T = c.T;
-    const TileMap tm = tile_map(T, wave, blockIdx.x);
-    int8_t *tb = smem + QkvLds<H>::WBYTES + tm.set * QkvLds<H>::PER_SET;
-    int *lnw = reinterpret_cast<int *>(tb), *lnb = lnw + H, *qA = lnb + H, *kA = qA + H, *vA = kA + H;
-    int8_t *qB = reinterpret_cast<int8_t *>(vA + H), *kB = qB + H, *vB = kB + H;
+    const TileMap tm = tile_map<CS>(T, wave, blockIdx.x);
+    const int col0 = tm.cs * HS;
+    int8_t *tb = smem + Q::WBYTES + tm.set * Q::PER_SET;
+    int *lnw = reinterpret_cast<int *>(tb), *lnb = lnw + H;
+    int8_t *qA = reinterpret_cast<int8_t *>(lnb + H), *kA = qA + H, *vA = kA + H, *qB = vA + H, *kB = qB + H, *vB = kB + H;
+    int8_t *xch = smem + Q::WBYTES + tm.sets * Q::PER_SET;
+    int *red = reinterpret_cast<int *>(xch + Q::XCHG);
 
-    WStream ws; wstream_init(ws, smem, QkvLds<H>::UNIT);
-    auto w_unit = [&](const int8_t *W, int u) { return W + (size_t)(4 * u) * H * 16; };     // k rows [64u, 64u+64)
-    w_prefetch2<4, H>(ws, w_unit(p.w_q, 0), H);
+    WStream ws; wstream_init(ws, smem, Q::UNIT);
+    auto pf = [&](const int8_t *W, int u) { w_prefetch2<Q::PR, H>(ws, W + (size_t)u * Q::PR * H * 16, H); };
+    pf(p.w_q, 0);
 
     for (int ss = 0; ss < tm.sets; ss++) {
         int ml = blockIdx.x * tm.sets + ss; if (ml >= c.n_members) ml = c.n_members - 1;
         const int mem = c.pop_offset + ml, nsx = (mem & 1) ? -1 : 1;
         const uint32_t sbx = *c.d_step_seed + (uint32_t)(mem / 2) + (uint32_t)p.seed_base;
-        int8_t *t2 = smem + QkvLds<H>::WBYTES + ss * QkvLds<H>::PER_SET;
-        int *lw = reinterpret_cast<int *>(t2), *lb = lw + H, *a0 = lb + H, *a1 = a0 + H, *a2 = a1 + H;
-        int8_t *b0 = reinterpret_cast<int8_t *>(a2 + H), *b1 = b0 + H, *b2 = b1 + H;
+        int8_t *t2 = smem + Q::WBYTES + ss * Q::PER_SET;
+        int *lw = reinterpret_cast<int *>(t2), *lb = lw + H;
+        int8_t *a0 = reinterpret_cast<int8_t *>(lb + H), *a1 = a0 + H, *a2 = a1 + H, *b0 = a2 + H, *b1 = b0 + H, *b2 = b1 + H;
         const int tid = threadIdx.x;
         fill_vec_i32(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_vec_i32(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
-        fill_noise_i32(a0, sbx + OFF_Q_A, H, c.mask, nsx, tid, EGG_THREADS);
-        fill_noise_i32(a1, sbx + OFF_K_A, H, c.mask, nsx, tid, EGG_THREADS);
-        fill_noise_i32(a2, sbx + OFF_V_A, H, c.mask, nsx, tid, EGG_THREADS);
+        fill_noise_i8(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx);
+        fill_noise_i8(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx);
+        fill_noise_i8(a2, sbx + OFF_V_A, H, c.mask, tid, EGG_THREADS, nsx);
         fill_noise_i8(b0, sbx + OFF_Q_B, H, c.mask, tid, EGG_THREADS);
         fill_noise_i8(b1, sbx + OFF_K_B, H, c.mask, tid, EGG_THREADS);
         fill_noise_i8(b2, sbx + OFF_V_B, H, c.mask, tid, EGG_THREADS);
@@ -310,14 +401,27 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_qkv(QkvParam
     if (!valid) mloc = c.n_members - 1;
 
     for (int pass = 0; pass < tm.passes; pass++) {
-        const int t = (tm.tile0 + 4 * pass) * 32 + j;
+        const int t = (tm.tile0 + Q::TPW * pass) * 32 + j;
         const size_t row = ((size_t)mloc * T + t) * H;
         v4i nrm[KS];
         {
-            v4i x[KS];
+            v4i x[NTS];
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
-            standard_norm<KS>(x, nrm, lnw, lnb, g);
+            for (int nt = 0; nt < NTS; nt++) x[nt] = load_op(p.x + row + col0, nt, g);
+            int tot = sumabs_groups<NTS>(x);
+            tot += other_half(tot);
+            tot = xreduce<CS, false>(tot, red, tm, lane);
+            int mn = tot / H; if (!mn) mn = 1;
+            if (CS == 1) standard_scale<NTS>(x, nrm, mn, lnw, lnb, 0, g);
+            else {
+                v4i mine[NTS];
+                standard_scale<NTS>(x, mine, mn, lnw, lnb, col0, g);
+#pragma unroll
+                for (int nt = 0; nt < NTS; nt++) xch_put(xch, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
+                __syncthreads();
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(xch, KS, tm.tslot, ks, lane);
+            }
         }
         const int32_t *rope_row = c.rope_lut + (size_t)t * c.head_dim;
 #pragma unroll 1
@@ -325,25 +429,26 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_qkv(QkvParam
             const int8_t *W = which == 0 ? p.w_q : (which == 1 ? p.w_k : p.w_v);
             const int8_t *nw = which == 0 ? p.w_k : (which == 1 ? p.w_v : ((pass + 1 < tm.passes) ? p.w_q : nullptr));
             const int8_t *Bn = which == 0 ? qB : (which == 1 ? kB : vB);
-            const int *An = which == 0 ? qA : (which == 1 ? kA : vA);
+            const int8_t *An = which == 0 ? qA : (which == 1 ? kA : vA);
             int8_t *dst = which == 0 ? p.q : (which == 1 ? p.k : p.v);
             const int sb = dot_noise<KS, false>(nrm, Bn, 0, g);
-            v16i acc[NT];
-            zero_acc<NT>(acc);
+            v16i acc[NTS];
+            zero_acc<NTS>(acc);
 #pragma unroll
-            for (int u = 0; u < H / 64; u++) {
+            for (int u = 0; u < Q::NU; u++) {
                 const int8_t *cur = w_acquire(ws);
-                if (u + 1 < H / 64) w_prefetch2<4, H>(ws, w_unit(W, u + 1), H);
-                else if (nw) w_prefetch2<4, H>(ws, w_unit(nw, 0), H);
-                mfma_unit2<2, NT>(acc, nrm + 2 * u, cur, lane);
+                if (u + 1 < Q::NU) pf(W, u + 1);
+                else if (nw) pf(nw, 0);
+                mfma_cols<Q::PR / 2, NTS>(acc, nrm + u * (Q::PR / 2), cur, H, col0, lane);
             }
-            add_perturb<NT>(acc, sb, An, 0, c.sigma, g);
-            if (which < 2) rope_inplace<NT>(acc, rope_row, c.head_dim, c.rope_scale_bit, g);
-            v4i o[KS];
-            adaptive_norm<NT>(acc, o);
+            add_perturb8<NTS>(acc, sb, An, col0, c.sigma, g);
+            if (which < 2) rope_inplace<NTS>(acc, rope_row, c.head_dim, c.rope_scale_bit, g);
+            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red + (1 + which) * Q::SITE, tm, lane);
+            v4i o[NTS];
+            adaptive_scale<NTS>(acc, mx, o);
             if (valid)
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) store_op(dst + row, ks, g, o[ks]);
+                for (int nt = 0; nt < NTS; nt++) store_op(dst + row + col0, nt, g, o[nt]);
         }
     }
 }
@@ -589,9 +694,9 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
 // ============================================================================ host launchers
 template <int H>
 static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
-    const int sets = tile_map_sets(p.c.T);
+    const int sets = tile_map_sets(p.c.T, Shape<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
-    size_t lds = MlpLds<H>::total(sets);
+    size_t lds = MlpCfg<H>::total(sets);
     if (first) hipLaunchKernelGGL((k_mlp<H, true>), grid, block, lds, s, p);
     else hipLaunchKernelGGL((k_mlp<H, false>), grid, block, lds, s, p);
     return hipGetLastError();
@@ -608,9 +713,9 @@ hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s) {
 
 template <int H>
 static hipError_t launch_qkv_h(const QkvParams &p, hipStream_t s) {
-    const int sets = tile_map_sets(p.c.T);
+    const int sets = tile_map_sets(p.c.T, Shape<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
-    size_t lds = QkvLds<H>::total(sets);
+    size_t lds = QkvCfg<H>::total(sets);
     hipLaunchKernelGGL((k_qkv<H>), grid, block, lds, s, p);
     return hipGetLastError();
 }
@@ -673,10 +778,10 @@ hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
 #define SET_LDS(kern, bytes) do { hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)); if (e_ != hipSuccess) return e_; } while (0)
 template <int H>
 static hipError_t prepare_h(int T) {
-    const int sets = tile_map_sets(T);
-    SET_LDS((k_mlp<H, true>), MlpLds<H>::total(sets));
-    SET_LDS((k_mlp<H, false>), MlpLds<H>::total(sets));
-    SET_LDS((k_qkv<H>), QkvLds<H>::total(sets));
+    const int sets = tile_map_sets(T, Shape<H>::CS);
+    SET_LDS((k_mlp<H, true>), MlpCfg<H>::total(sets));
+    SET_LDS((k_mlp<H, false>), MlpCfg<H>::total(sets));
+    SET_LDS((k_qkv<H>), QkvCfg<H>::total(sets));
     SET_LDS((k_head<H>), HeadLds<H>::TOTAL);
     return hipSuccess;
 }
