@@ -321,7 +321,8 @@ struct QkvCfg {
     static constexpr int PER_SET = 2 * H * 4 + 6 * H;   // lnw lnb (int32) | qA kA vA (int8, times the sign) qB kB vB (int8)
     static constexpr int XCHG = CS > 1 ? TPW * 32 * H : 0;
     static constexpr int SITE = EGG_WAVES * 64;
-    static constexpr int RED = CS > 1 ? 4 * SITE * 4 : 0;
+    static constexpr int RED = CS > 1 ? 2 * SITE * 4 : 0;       // two reduction sites used alternately
+    static constexpr int OCC = 2;              // workgroups per CU the kernel is built for
     static int total(int sets) { return WBYTES + sets * PER_SET + XCHG + RED; }
 };
 
@@ -358,7 +359,7 @@ __device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row,
 }
 
 template <int H>
-__global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p) {
     typedef QkvCfg<H> Q;
     constexpr int CS = Q::CS, KS = Q::KS, NTS = Q::NTS, HS = Q::HS;
     extern __shared__ __align__(16) int8_t smem[];
@@ -410,7 +411,7 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
             for (int nt = 0; nt < NTS; nt++) x[nt] = load_op(p.x + row + col0, nt, g);
             int tot = sumabs_groups<NTS>(x);
             tot += other_half(tot);
-            tot = xreduce<CS, false>(tot, red, tm, lane);
+            tot = xreduce<CS, false>(tot, red, tm, lane);        // sites alternate 0,1,0,1 through the pass
             int mn = tot / H; if (!mn) mn = 1;
             if (CS == 1) standard_scale<NTS>(x, nrm, mn, lnw, lnb, 0, g);
             else {
@@ -443,7 +444,7 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
             }
             add_perturb8<NTS>(acc, sb, An, col0, c.sigma, g);
             if (which < 2) rope_inplace<NTS>(acc, rope_row, c.head_dim, c.rope_scale_bit, g);
-            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red + (1 + which) * Q::SITE, tm, lane);
+            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red + ((1 + which) & 1) * Q::SITE, tm, lane);
             v4i o[NTS];
             adaptive_scale<NTS>(acc, mx, o);
             if (valid)
@@ -456,15 +457,42 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_qkv(QkvParams p) {
 // ============================================================================ attention core
 // One wave per (member, head).  S^T = K.Q^T per 32x32 tile (lane = query token), two passes over the
 // causal context (row max, then LUT weights), O^T = V^T.P^T with the 19-bit weights split into three
-// 7-bit planes so the weighted sum stays exact on the int8 MFMA.
+// 7-bit planes so the weighted sum stays exact on the int8 MFMA.  The LDS table holds, per exp-LUT index,
+// the weight and its three planes packed as bytes, so the planes of four context positions are regrouped with
+// byte permutes instead of shifts and masks.  Only the diagonal tile needs the causal mask.
+__device__ __forceinline__ void attn_weights(const v16i &s, const int2 *lut, int mxs, int shift, bool diag, int ct, int t, int g,
+                                             v4i *pw, int &den) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        int pk[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            int idx = mxs - (s[4 * q + e] >> shift);
+            idx = min(255, max(0, idx));
+            int2 wp = lut[idx];
+            if (diag && (32 * ct + 8 * q + 4 * g + e) > t) { wp.x = 0; wp.y = 0; }
+            den += wp.x;
+            pk[e] = wp.y;
+        }
+        // bytes of pk[e]: plane0, plane1, plane2, 0  ->  one dword per plane holding the four positions
+        const int ab_lo = __builtin_amdgcn_perm(pk[1], pk[0], 0x05010400);   // a0 b0 a1 b1
+        const int cd_lo = __builtin_amdgcn_perm(pk[3], pk[2], 0x05010400);
+        const int ab_hi = __builtin_amdgcn_perm(pk[1], pk[0], 0x07030602);   // a2 b2 a3 b3
+        const int cd_hi = __builtin_amdgcn_perm(pk[3], pk[2], 0x07030602);
+        pw[0][q] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100);
+        pw[1][q] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302);
+        pw[2][q] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100);
+    }
+}
+
 template <int HD, int CT>
 __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnParams p) {
     constexpr int KS = HD / 32, DT = HD / 32;
     constexpr int T = CT * 32;
     extern __shared__ __align__(16) int8_t smem[];
-    int *lut = reinterpret_cast<int *>(smem);
+    int2 *lut = reinterpret_cast<int2 *>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    int8_t *vl = smem + 1024 + (size_t)wave * T * HD;
+    int8_t *vl = smem + 2048 + (size_t)wave * T * HD;
 
     const FwdCommon &c = p.c;
     const int H = c.H, NH = H / HD;
@@ -474,7 +502,10 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
     const int mloc = unit / NH, h = unit % NH;
     const size_t base = (size_t)mloc * T * H + (size_t)h * HD;
 
-    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) lut[i] = c.exp_lut[i];
+    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) {
+        const int w = c.exp_lut[i];
+        lut[i] = make_int2(w, (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16));
+    }
     // V tile of this (member, head) -> LDS rows [ctx][HD]
     for (int i = lane; i < T * HD / 16; i += 64) {
         int cx = i / (HD / 16), part = i % (HD / 16);
@@ -518,10 +549,15 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                     v4i kf = load_op(p.k + base + (size_t)(32 * ct + j) * H, ks, g);
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
+                if (ct == qt) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    int cx = 32 * ct + ((r >> 2) << 3) + (g << 2) + (r & 3);
-                    if (cx <= t) mx = max(mx, s[r]);
+                    for (int r = 0; r < 16; r++) {
+                        int cx = 32 * ct + ((r >> 2) << 3) + (g << 2) + (r & 3);
+                        if (cx <= t) mx = max(mx, s[r]);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; r += 2) mx = max(max(mx, s[r]), s[r + 1]);
                 }
             }
         }
@@ -544,23 +580,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
                 v4i pw[3];
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    int w0[4], w1[4], w2[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        int r = 4 * q + e;
-                        int cx = 32 * ct + 8 * q + 4 * g + e;
-                        int idx = mxs - (s[r] >> c.shift_attn);
-                        idx = min(255, max(0, idx));
-                        int w = (cx <= t) ? lut[idx] : 0;
-                        den += w;
-                        w0[e] = w & 127; w1[e] = (w >> 7) & 127; w2[e] = w >> 14;
-                    }
-                    pw[0][q] = pack4(w0[0], w0[1], w0[2], w0[3]);
-                    pw[1][q] = pack4(w1[0], w1[1], w1[2], w1[3]);
-                    pw[2][q] = pack4(w2[0], w2[1], w2[2], w2[3]);
-                }
+                if (ct == qt) attn_weights(s, lut, mxs, c.shift_attn, true, ct, t, g, pw, den);
+                else attn_weights(s, lut, mxs, c.shift_attn, false, ct, t, g, pw, den);
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -569,7 +590,11 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
             }
         }
         den += other_half(den);
-        const double dden = (double)(den ? den : 1);
+        // Truncating quotient num / den with one reciprocal per token.  num and den are integers below 2^53, the
+        // quotient is at most 127 in magnitude, and a non-integer quotient is at least 1/den >= 2^-27 away from
+        // the next integer.  Scaling the reciprocal by (1 + 2^-40) pushes an exactly integer quotient k to
+        // k(1 + 2^-40 +- 2^-51), which truncates to k, and moves any other quotient by less than 2^-32.
+        const double rden = (1.0 + 0x1p-40) / (double)(den ? den : 1);
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
             v4i outp;
@@ -579,11 +604,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     int r = 4 * q + e;
-                    long long num = (long long)o[0][dt][r] + ((long long)o[1][dt][r] << 7) + ((long long)o[2][dt][r] << 14);
-                    // exact truncating quotient: |num/den| <= 127 and a non-integer quotient is at least
-                    // 2^-27 away from an integer, far beyond double rounding
-                    int qv = (int)((double)num / dden);
-                    ov[e] = clip127(qv);
+                    double num = __builtin_fma((double)o[2][dt][r], 16384.0, __builtin_fma((double)o[1][dt][r], 128.0, (double)o[0][dt][r]));
+                    ov[e] = clip127((int)(num * rden));
                 }
                 outp[q] = pack4(ov[0], ov[1], ov[2], ov[3]);
             }
@@ -733,7 +755,7 @@ template <int HD, int CT>
 static hipError_t launch_attn_t(const AttnParams &p, hipStream_t s) {
     int units = p.c.n_members * (p.c.H / HD);
     dim3 grid((units + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
-    size_t lds = 1024 + (size_t)EGG_WAVES * CT * 32 * HD;
+    size_t lds = 2048 + (size_t)EGG_WAVES * CT * 32 * HD;
     hipLaunchKernelGGL((k_attn<HD, CT>), grid, block, lds, s, p);
     return hipGetLastError();
 }
@@ -787,7 +809,7 @@ static hipError_t prepare_h(int T) {
 }
 template <int HD, int CT>
 static hipError_t prepare_attn() {
-    SET_LDS((k_attn<HD, CT>), 1024 + (size_t)EGG_WAVES * CT * 32 * HD);
+    SET_LDS((k_attn<HD, CT>), 2048 + (size_t)EGG_WAVES * CT * 32 * HD);
     return hipSuccess;
 }
 template <int HD>
