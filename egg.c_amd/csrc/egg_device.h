@@ -215,13 +215,24 @@ __device__ __forceinline__ void mfma_unit2(v16i *acc, const v4i *xop, const int8
 template <int KSU, int NTW>
 __device__ __forceinline__ void mfma_cols(v16i *acc, const v4i *xop, const int8_t *lds, int cols, int colbase, int lane) {
     const int i = lane & 31, g = lane >> 5;
+    // all fragment reads of a batch are issued before its first MFMA, so one LDS latency is exposed per batch
+    // instead of one per fragment pair
+    constexpr int BK = (KSU * NTW <= 8) ? KSU : (8 / NTW > 0 ? 8 / NTW : 1);     // k-steps per batch
 #pragma unroll
-    for (int ks = 0; ks < KSU; ks++)
+    for (int k0 = 0; k0 < KSU; k0 += BK) {
+        v4i a[BK * NTW];
 #pragma unroll
-        for (int nt = 0; nt < NTW; nt++) {
-            v4i a = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * cols + colbase + nt * 32 + i) * 16);
-            acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, xop[ks], acc[nt], 0, 0, 0);
-        }
+        for (int ks = 0; ks < BK; ks++)
+#pragma unroll
+            for (int nt = 0; nt < NTW; nt++)
+                a[ks * NTW + nt] = *reinterpret_cast<const v4i *>(lds + ((size_t)((k0 + ks) * 2 + g) * cols + colbase + nt * 32 + i) * 16);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < BK; ks++)
+#pragma unroll
+            for (int nt = 0; nt < NTW; nt++)
+                acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks * NTW + nt], xop[k0 + ks], acc[nt], 0, 0, 0);
+    }
 }
 
 // Column split: for hidden sizes above 128 the H-wide accumulators of one 32-token tile do not fit one wave next to

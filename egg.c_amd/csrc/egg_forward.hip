@@ -79,14 +79,18 @@ struct MlpCfg {
     static constexpr int I32 = 9 * H;        // ex0[H] ex1[H] lnw[H] lnb[H] bup[4H] bdn[H]
     static constexpr int I8 = 11 * H;        // exB[H] upB[H] dnB[4H] upA[4H] dnA[H]   (A noise already times the sign)
     static constexpr int PER_SET = I32 * 4 + I8;
-    static constexpr int XCHG = CS > 1 ? TPW * 32 * H : 0;          // normalised input / intermediate exchange
+    // The normalised input is exchanged through whichever W buffer is idle at that point (TPW*32*H <= UNIT bytes);
+    // the intermediate slices have their own small area because both W buffers are busy inside the sub-chunk loop.
+    static constexpr int XCHG = CS > 1 ? TPW * 32 * SC : 0;
     static constexpr int SITE = EGG_WAVES * 64;                       // ints per reduction site
     static constexpr int RED = CS > 1 ? 4 * SITE * 4 : 0;
+    static constexpr int OCC = H == 256 ? 3 : 2;                      // workgroups per CU the kernel is built for
+    static_assert(CS == 1 || TPW * 32 * H <= UNIT, "the operand exchange must fit one W buffer");
     static int total(int sets) { return WBYTES + 256 + sets * PER_SET + XCHG + RED; }
 };
 
 template <int H, bool FIRST>
-__global__ void __launch_bounds__(EGG_THREADS, 2) k_mlp(MlpParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p) {
     typedef MlpCfg<H> M;
     constexpr int CS = M::CS, KS = M::KS, NTS = M::NTS, HS = M::HS, NTU = M::NTU, SC = M::SC;
     extern __shared__ __align__(16) int8_t smem[];
@@ -222,13 +226,15 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_mlp(MlpParams p) {
             int mn = tot / H; if (!mn) mn = 1;
             if (CS == 1) standard_scale<NTS>(xs, nrm, mn, lnw, lnb, 0, g);
             else {
+                // ws.other holds the unit consumed last; every wave has passed a barrier since reading it, and the
+                // next prefetch into it is issued only after the barrier of the next w_acquire
                 v4i mine[NTS];
                 standard_scale<NTS>(xs, mine, mn, lnw, lnb, col0, g);
 #pragma unroll
-                for (int nt = 0; nt < NTS; nt++) xch_put(xch, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
+                for (int nt = 0; nt < NTS; nt++) xch_put(ws.other, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
                 __syncthreads();
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(xch, KS, tm.tslot, ks, lane);
+                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(ws.other, KS, tm.tslot, ks, lane);
             }
         }
         const int sbu = dot_noise<KS, false>(nrm, upB, 0, g);
@@ -319,21 +325,25 @@ struct QkvCfg {
     static constexpr int UNIT = 16 * PR * H;
     static constexpr int WBYTES = 2 * UNIT;
     static constexpr int PER_SET = 2 * H * 4 + 6 * H;   // lnw lnb (int32) | qA kA vA (int8, times the sign) qB kB vB (int8)
-    static constexpr int XCHG = CS > 1 ? TPW * 32 * H : 0;
+    static constexpr int XCHG = 0;             // the normalised input is exchanged through the idle W buffer
     static constexpr int SITE = EGG_WAVES * 64;
     static constexpr int RED = CS > 1 ? 2 * SITE * 4 : 0;       // two reduction sites used alternately
-    static constexpr int OCC = 2;              // workgroups per CU the kernel is built for
+    static constexpr int OCC = 2;                              // workgroups per CU the kernel is built for
+    static_assert(CS == 1 || TPW * 32 * H <= UNIT, "the operand exchange must fit one W buffer");
     static int total(int sets) { return WBYTES + sets * PER_SET + XCHG + RED; }
 };
 
 // apply_rope_integer (mgpu.cu:624-644) on the raw accumulators of one token.  The (cos, sin) pairs repeat every
-// head, so a lane needs only the head_dim/32 * 8 pairs of its own slots; they are loaded once and reused.
-// The NT column groups must start at a head boundary.
-template <int NT>
-__device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row, int head_dim, int bit, int g) {
-    const long long half = 1ll << (bit - 1);
-    int2 cs[2][4][2];
+// head, so a lane needs only the head_dim/32 * 8 pairs of its own slots; they are loaded once per token tile
+// (RopeTab) and reused for every head of Q and K.
+// The reference evaluates (ve*c -+ vo*s + 2^(bit-1)) >> bit in int64.  Here the same value is formed in double
+// precision, where it is exact: |v| < 2^23 and |c|, |s| <= 2^bit <= 2^20 keep every partial sum below 2^45, and the
+// table is pre-scaled by 2^-bit (a power of two).  Adding 2^24 before the truncating conversion makes the operand
+// positive, so truncation equals the arithmetic shift's floor; 2^24 is subtracted again in integers.
+struct RopeTab { double c[2][4][2], s[2][4][2]; };
+__device__ __forceinline__ void rope_load(RopeTab &rt, const int32_t *rope_row, int head_dim, int bit, int g) {
     const int hdt = head_dim >> 5;                 // column groups per head: 1 or 2
+    const double sc = __builtin_ldexp(1.0, -bit);
 #pragma unroll
     for (int h2 = 0; h2 < 2; h2++)
 #pragma unroll
@@ -341,20 +351,29 @@ __device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row,
 #pragma unroll
             for (int ep = 0; ep < 2; ep++) {
                 int n = 32 * (h2 < hdt ? h2 : 0) + 8 * q + 4 * g + 2 * ep;
-                cs[h2][q][ep] = *reinterpret_cast<const int2 *>(rope_row + 2 * (n >> 1));
+                int2 v = *reinterpret_cast<const int2 *>(rope_row + 2 * (n >> 1));
+                rt.c[h2][q][ep] = (double)v.x * sc;
+                rt.s[h2][q][ep] = (double)v.y * sc;
             }
+}
+// The NT column groups must start at a head boundary.
+template <int NT>
+__device__ __forceinline__ void rope_inplace(v16i *acc, const RopeTab &rt, int head_dim) {
+    const int hdt = head_dim >> 5;
+    const double init = 16777216.5;                // 2^24 + the rounding half, both already divided by 2^bit
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
         for (int q = 0; q < 4; q++)
 #pragma unroll
             for (int ep = 0; ep < 2; ep++) {
-                const int2 c2 = (hdt == 2) ? cs[nt & 1][q][ep] : cs[0][q][ep];
-                long long ve = acc[nt][4 * q + 2 * ep], vo = acc[nt][4 * q + 2 * ep + 1];
-                long long re = (ve * c2.x - vo * c2.y + half) >> bit;
-                long long ro = (ve * c2.y + vo * c2.x + half) >> bit;
-                acc[nt][4 * q + 2 * ep] = (int)re;
-                acc[nt][4 * q + 2 * ep + 1] = (int)ro;
+                const double cc = (hdt == 2) ? rt.c[nt & 1][q][ep] : rt.c[0][q][ep];
+                const double ss = (hdt == 2) ? rt.s[nt & 1][q][ep] : rt.s[0][q][ep];
+                const double ve = (double)acc[nt][4 * q + 2 * ep], vo = (double)acc[nt][4 * q + 2 * ep + 1];
+                const double re = __builtin_fma(-vo, ss, __builtin_fma(ve, cc, init));
+                const double ro = __builtin_fma(vo, cc, __builtin_fma(ve, ss, init));
+                acc[nt][4 * q + 2 * ep] = (int)re - 16777216;
+                acc[nt][4 * q + 2 * ep + 1] = (int)ro - 16777216;
             }
 }
 
@@ -418,13 +437,14 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
                 v4i mine[NTS];
                 standard_scale<NTS>(x, mine, mn, lnw, lnb, col0, g);
 #pragma unroll
-                for (int nt = 0; nt < NTS; nt++) xch_put(xch, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
+                for (int nt = 0; nt < NTS; nt++) xch_put(ws.other, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
                 __syncthreads();
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(xch, KS, tm.tslot, ks, lane);
+                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(ws.other, KS, tm.tslot, ks, lane);
             }
         }
-        const int32_t *rope_row = c.rope_lut + (size_t)t * c.head_dim;
+        RopeTab rt;
+        rope_load(rt, c.rope_lut + (size_t)t * c.head_dim, c.head_dim, c.rope_scale_bit, g);
 #pragma unroll 1
         for (int which = 0; which < 3; which++) {
             const int8_t *W = which == 0 ? p.w_q : (which == 1 ? p.w_k : p.w_v);
@@ -443,7 +463,7 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
                 mfma_cols<Q::PR / 2, NTS>(acc, nrm + u * (Q::PR / 2), cur, H, col0, lane);
             }
             add_perturb8<NTS>(acc, sb, An, col0, c.sigma, g);
-            if (which < 2) rope_inplace<NTS>(acc, rope_row, c.head_dim, c.rope_scale_bit, g);
+            if (which < 2) rope_inplace<NTS>(acc, rt, c.head_dim);
             const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red + ((1 + which) & 1) * Q::SITE, tm, lane);
             v4i o[NTS];
             adaptive_scale<NTS>(acc, mx, o);
