@@ -64,8 +64,9 @@ __device__ __forceinline__ int dot4(int a, int b, int c) {
 #endif
 }
 // sum of |bytes| of 4 signed bytes (none equal to -128)
+// x ^ 0x80 is x + 128 as an unsigned byte, so the byte-wise |(x + 128) - 128| of v_sad_u8 is |x|
 __device__ __forceinline__ int sumabs4(int a, int c) {
-    return c + abs(sx8(a, 0)) + abs(sx8(a, 1)) + abs(sx8(a, 2)) + abs(sx8(a, 3));
+    return (int)__builtin_amdgcn_sad_u8((unsigned)a ^ 0x80808080u, 0x80808080u, (unsigned)c);
 }
 
 // full-rate 24-bit multiply (both operands must fit in 24 signed bits, the product in 32)
@@ -298,12 +299,13 @@ __device__ __forceinline__ void fill_noise_i32(int *dst, uint32_t seed, int n, i
     for (int i = lane; i < n; i += nthr) dst[i] = noise_from_hash(seed, i, mask) * mult;
 }
 // dst[i] = base[i] + ((noise(seed_a,i) * noise(seed_b,i) * ns) >> shift)       (mgpu.cu:666-675, :733-735)
+// (the result is stored shifted left by `lshift` where a kernel folds it into a GEMM accumulator)
 __device__ __forceinline__ void fill_vec_i32(int *dst, const int8_t *base, uint32_t seed_a, uint32_t seed_b,
-                                             int n, int mask, int ns, int shift, int lane, int nthr = 64) {
+                                             int n, int mask, int ns, int shift, int lane, int nthr = 64, int lshift = 0) {
     for (int i = lane; i < n; i += nthr) {
         int v = base[i];
         if (ns != 0) v += (noise_from_hash(seed_a, i, mask) * noise_from_hash(seed_b, i, mask) * ns) >> shift;
-        dst[i] = v;
+        dst[i] = v << lshift;
     }
 }
 __device__ __forceinline__ void wave_lds_fence() {

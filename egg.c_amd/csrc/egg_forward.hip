@@ -143,7 +143,8 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         fill_vec_i32(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_vec_i32(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_noise_i8(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx);
-        fill_vec_i32(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        // the up bias is stored as b << shift_mlp_up and seeds the up accumulator: ((a + (b << s)) >> s) == (a >> s) + b
+        fill_vec_i32(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up);
         fill_noise_i8(dA, sbx + p.off_dn_a, H, c.mask, tid, EGG_THREADS, nsx);
         fill_vec_i32(bd, p.b_dn, sbx + p.off_bdn_a, sbx + p.off_bdn_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_noise_i8(uB, sbx + p.off_up_b, H, c.mask, tid, EGG_THREADS);
@@ -244,7 +245,14 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
 #pragma unroll 1
         for (int s = 0; s < M::NSUB; s++) {
             v16i au[NTU];
-            zero_acc<NTU>(au);
+#pragma unroll
+            for (int nt = 0; nt < NTU; nt++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    v4i b4 = *reinterpret_cast<const v4i *>(bup + s * SC + tm.cs * 32 * NTU + 32 * nt + 8 * q + 4 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) au[nt][4 * q + e] = b4[e];
+                }
 #pragma unroll
             for (int ku = 0; ku < M::UPU; ku++) {
                 const int8_t *cur = w_acquire(ws);
@@ -262,12 +270,11 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                     for (int q = 0; q < 4; q++) {
                         int n0 = nb + 32 * nt + 8 * q + 4 * g;
                         int a4 = *reinterpret_cast<const int *>(upA + n0);
-                        v4i b4 = *reinterpret_cast<const v4i *>(bup + n0);
                         int o[4];
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             int a = au[nt][4 * q + e] + (mul24(sbu, sx8(a4, e)) >> c.sigma);
-                            int v = clip127((a >> c.shift_mlp_up) + b4[e]);
+                            int v = clip127(a >> c.shift_mlp_up);
                             o[e] = act[(uint8_t)v];
                         }
                         mine[nt][q] = pack4(o[0], o[1], o[2], o[3]);
