@@ -29,6 +29,9 @@ def main():
     ap.add_argument("--data-mib", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="skip the hipGraph replay leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch one plain elementwise copy of 256 MiB (reads 256 MiB, writes 256 MiB) so that a "
+                         "counter run can scale FETCH_SIZE / WRITE_SIZE by what they read for known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); no multi-GPU figure is produced", file=sys.stderr)
@@ -93,8 +96,12 @@ def main():
     launches, tot_ms = timing[dom]
     tokens_per_launch = P * T * args.steps * (L if dom in ("mlp", "qkv", "attn") else 1) / max(launches, 1)
     achieved = ops_per_token[dom] * tokens_per_launch / (tot_ms / launches * 1e-3) if launches else 0.0
+    # HBM bytes per launch of k_mlp<256,false> at 2048 members x 256 tokens per launch, from two rocprofv3 --pmc runs
+    # (FETCH_SIZE 260,192 KiB x 2.0, WRITE_SIZE 311,756 KiB x 1.0; the factors are what the same counters read for a
+    # plain 256 MiB elementwise copy in the same run: 131,091 KiB fetched, 262,144 KiB written)
+    traffic = (260192 * 2.0 + 311756 * 1.0) * 1024 if (dom == "mlp" and chunk == 2048 and P >= 2048) else None
     roofline = {"kernel": "k_" + dom, "bound": "mfma", "achieved": achieved / 1e12, "peak": PEAK_INT8_OPS / 1e12,
-                "unit": "TOP/s", "frac": achieved / PEAK_INT8_OPS, "traffic": None,
+                "unit": "TOP/s", "frac": achieved / PEAK_INT8_OPS, "traffic": traffic,
                 "avg_launch_ms": tot_ms / launches if launches else None, "launches": launches}
 
     # ---- the same steps replayed as one captured hipGraph per step
@@ -107,6 +114,13 @@ def main():
         run_steps(args.steps, args.warmup + args.steps + 1, seed, True)
         torch.cuda.synchronize()
         graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    if args.calib_copy:
+        a = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
+        b = torch.empty_like(a)
+        torch.add(a, 1, out=b)
+        torch.cuda.synchronize()
+        del a, b
 
     # ---- perturbed-linear microbenchmark (P=8192, T=128, K=N=512), int32 output
     mb = {}
