@@ -43,7 +43,7 @@ EXPORTS = [
     "egg_noise_fill", "egg_perturbed_linear", "egg_population_forward", "egg_population_forward_dev",
     "egg_fitness", "egg_es_update", "egg_update_tensor", "egg_matrix_votes",
     "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
-    "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses",
+    "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
     "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz",
@@ -102,6 +102,7 @@ def lib():
         L.egg_step_capture.argtypes = [vp, vp, i64]
         L.egg_step_launch.argtypes = [vp, i64, u32, C.c_float]
         L.egg_step_losses.argtypes = [vp, vp, vp]
+        L.egg_generate.argtypes = [vp, vp, i32, i32, u32]
         L.egg_learning_rate.restype = C.c_float
         L.egg_learning_rate.argtypes = [C.c_long]
         L.egg_next_seed.restype = u32
@@ -279,6 +280,10 @@ class Context:
         fit = np.zeros(self.cfg.population // 2, np.int32)
         self._ck(lib().egg_step_losses(self._h, _np_ptr(loss), _np_ptr(fit)), "egg_step_losses")
         return loss, fit
+
+    def generate(self, d_buffer, seed_len, gen_len, seed):
+        """Continue the seed_len prompt bytes at device pointer d_buffer by gen_len sampled bytes (in place)."""
+        self._ck(lib().egg_generate(self._h, C.c_void_p(d_buffer), seed_len, gen_len, seed & 0xFFFFFFFF), "egg_generate")
 
     def enable_taps(self, on=True):
         self._ck(lib().egg_ctx_enable_taps(self._h, 1 if on else 0), "egg_ctx_enable_taps")

@@ -60,6 +60,9 @@ struct egg_ctx {
     struct Span { int cls; hipEvent_t a, b; };
     std::vector<Span> spans; size_t spans_used = 0;
     double t_ms[EGG_KCLASS_COUNT] = {0}; long t_n[EGG_KCLASS_COUNT] = {0};
+    // generation (egg_generate): token buffer [T + 1], logits of one member [T][vocab], a zero start index / seed
+    uint8_t *d_gen_tok = nullptr; int32_t *d_gen_logits = nullptr; Scalars *d_gen_scal = nullptr;
+    int mask_override = -1; int32_t *logits_override = nullptr;
     // graph
     hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr; bool captured = false;
     std::string err;
@@ -150,7 +153,7 @@ static void free_all(egg_ctx *ctx) {
     void *ptrs[] = {ctx->muon.x, ctx->muon.swap, ctx->muon.bterm, ctx->muon.partials, ctx->muon.norm,
                     ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
-                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits};
+                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal};
     for (void *p : ptrs) if (p) (void)hipFree(p);
     for (auto &sp : ctx->spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
     if (ctx->gexec) (void)hipGraphExecDestroy(ctx->gexec);
@@ -385,7 +388,8 @@ static FwdCommon make_common(egg_ctx *ctx, const uint8_t *d_data, int64_t len, c
     f.data = d_data; f.data_len = len; f.d_start_idx = d_start; f.d_step_seed = d_seed;
     f.pop_offset = first_member; f.n_members = nm; f.population = c.population;
     f.T = c.seq_len; f.H = c.hidden; f.head_dim = c.head_dim; f.vocab = c.vocab;
-    f.sigma = c.fixed_point + c.sigma_shift; f.sigma_vec = c.sigma_shift_vector; f.mask = c.noise_mask;
+    f.sigma = c.fixed_point + c.sigma_shift; f.sigma_vec = c.sigma_shift_vector;
+    f.mask = ctx->mask_override >= 0 ? ctx->mask_override : c.noise_mask;
     f.shift_attn = c.shift_attn; f.shift_out = c.shift_out; f.shift_logit = c.shift_logit;
     f.shift_mlp_up = c.shift_mlp_up; f.shift_mlp_down = c.shift_mlp_down;
     f.softmax_scale_bit = c.softmax_scale_bit; f.rope_scale_bit = c.rope_scale_bit;
@@ -453,7 +457,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
     {
         HeadParams p; memset(&p, 0, sizeof(p)); p.c = f;
         p.ln_w = M + L.ln_f; p.ln_b = M + L.ln_f_bias; p.embedding_frag = F + L.embedding; p.x = ctx->d_x;
-        p.loss_acc = ctx->d_loss_acc; p.logits_tap = taps ? ctx->d_tap_logits : nullptr;
+        p.loss_acc = ctx->d_loss_acc; p.logits_tap = ctx->logits_override ? ctx->logits_override : (taps ? ctx->d_tap_logits : nullptr);
         span_begin(ctx, EGG_K_HEAD); HIP_TRY(egg_launch_head(p, s)); span_end(ctx);
     }
     return EGG_OK;
@@ -640,6 +644,42 @@ extern "C" uint32_t egg_next_seed(uint32_t seed, uint64_t step) {
 }
 
 // ------------------------------------------------------------------ taps
+// generate_sequence_kernel (mgpu.cu:1154-1283) and its call site (:1701-1708).  The reference walks the sequence
+// token by token with a KV cache; here every new token re-runs the unperturbed forward of one member over the whole
+// window (noise mask 0 makes every perturbation term vanish, i.e. noise_sign = 0) and samples from the logits of
+// position t.  Causality makes the logits at t independent of the not yet generated tail.
+extern "C" int egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed) {
+    if (!ctx || !d_buffer) return EGG_E_INVALID;
+    const egg_config &c = ctx->cfg; const int T = c.seq_len, total = seed_len + gen_len;
+    if (seed_len < 1 || gen_len < 0 || total > T) return fail(ctx, EGG_E_INVALID, "egg_generate: need 1 <= seed_len and seed_len + gen_len <= seq_len");
+    if (ctx->captured) return fail(ctx, EGG_E_STATE, "egg_generate cannot run on a context whose step is captured");
+    hipStream_t s = ctx->stream;
+    if (!ctx->d_gen_tok) {
+        HIP_TRY(hipMalloc(&ctx->d_gen_tok, (size_t)T + 16));
+        HIP_TRY(hipMalloc(&ctx->d_gen_logits, (size_t)T * c.vocab * 4));
+        HIP_TRY(hipMalloc(&ctx->d_gen_scal, sizeof(Scalars)));
+        HIP_TRY(hipMemset(ctx->d_gen_scal, 0, sizeof(Scalars)));
+    }
+    HIP_TRY(hipMemsetAsync(ctx->d_gen_tok, 0, (size_t)T + 16, s));
+    HIP_TRY(hipMemcpyAsync(ctx->d_gen_tok, d_buffer, (size_t)seed_len, hipMemcpyDeviceToDevice, s));
+    int bt = (c.hidden + 31) & ~31; if (bt > 1024) bt = 1024;          // BLOCK_THREADS (mgpu.cu:74-75)
+    const bool taps = ctx->taps; ctx->taps = false;
+    ctx->mask_override = 0; ctx->logits_override = ctx->d_gen_logits;
+    int rc = EGG_OK;
+    for (int t = seed_len - 1; t < total - 1 && rc == EGG_OK; t++) {
+        // data_len = T + 1 puts the member's stream position at 0 (mgpu.cu:864-870 with len - T == 1)
+        rc = forward_chunk(ctx, ctx->d_gen_tok, (int64_t)T + 1, &ctx->d_gen_scal->start, &ctx->d_gen_scal->seed, 0, 1);
+        if (rc == EGG_OK) {
+            hipError_t e = egg_launch_sample(ctx->d_gen_logits + (size_t)t * c.vocab, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_tok + t + 1, s);
+            if (e != hipSuccess) rc = fail(ctx, EGG_E_HIP, "egg_launch_sample", e);
+        }
+    }
+    ctx->mask_override = -1; ctx->logits_override = nullptr; ctx->taps = taps;
+    if (rc) return rc;
+    HIP_TRY(hipMemcpyAsync(d_buffer, ctx->d_gen_tok, (size_t)total, hipMemcpyDeviceToDevice, s));
+    return EGG_OK;
+}
+
 extern "C" int egg_ctx_enable_taps(egg_ctx *ctx, int enable) {
     if (!ctx) return EGG_E_INVALID;
     if (ctx->captured) return fail(ctx, EGG_E_STATE, "taps cannot change after capture");

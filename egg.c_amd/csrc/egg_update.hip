@@ -204,6 +204,47 @@ hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s) {
     return hipGetLastError();
 }
 
+// Three-pass LUT sampling of generate_sequence_kernel (mgpu.cu:1212-1283) for one position: maximum logit,
+// sum of EXP_LUT[clamp(max - logit)], threshold hash_rng(seed + t*555, 0) % sum, then the first vocabulary entry
+// whose running sum exceeds the threshold.  The reference accumulates in thread order with thread `tid` owning
+// v = tid, tid + bt, ... (bt = its block size = hidden rounded up to 32, at most 1024), so for bt < vocab the scan
+// order is thread-major, not natural; `bt` reproduces that.  One workgroup; vocab <= 1024.
+__global__ void __launch_bounds__(256) k_sample(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt,
+                                                uint32_t seed, int t, uint8_t *out) {
+    __shared__ int ex[1024];
+    __shared__ int red[256];
+    int mx = INT_MIN;
+    for (int v = threadIdx.x; v < vocab; v += 256) mx = max(mx, logits[v]);
+    red[threadIdx.x] = mx; __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) { if ((int)threadIdx.x < o) red[threadIdx.x] = max(red[threadIdx.x], red[threadIdx.x + o]); __syncthreads(); }
+    mx = red[0];
+    for (int v = threadIdx.x; v < vocab; v += 256) {
+        int idx = mx - logits[v];
+        idx = idx < 0 ? 0 : (idx > 255 ? 255 : idx);
+        ex[v] = exp_lut[idx];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        long long sum = 0;
+        for (int v = 0; v < vocab; v++) sum += ex[v];
+        const uint32_t r = hash_rng(seed + (uint32_t)t * 555u, 0);
+        const long long thresh = sum > 0 ? (long long)r % sum : 0;
+        int selected = 0; long long running = 0; bool done = false;
+        for (int tid = 0; tid < bt && !done; tid++)
+            for (int v = tid; v < vocab; v += bt) {
+                running += ex[v];
+                if (running > thresh) { selected = v; done = true; break; }
+            }
+        *out = (uint8_t)selected;
+    }
+}
+hipError_t egg_launch_sample(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
+                             uint8_t *out, hipStream_t s) {
+    if (vocab > 1024 || bt < 1) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_sample, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, out);
+    return hipGetLastError();
+}
+
 // canonical blocked weights -> fragment-major copy consumed by the GEMM kernels (layout in egg_device.h)
 __global__ void k_swizzle(const uint32_t *src, v4i *dst, int K, int N, int B, int nat) {
     int c = blockIdx.x * blockDim.x + threadIdx.x;

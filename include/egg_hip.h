@@ -153,6 +153,11 @@ int  egg_step_losses(egg_ctx *ctx, int32_t *host_loss, int32_t *host_fit);
 float    egg_learning_rate(long step);
 uint32_t egg_next_seed(uint32_t seed, uint64_t step);
 
+/* generate_sequence_kernel + its call site (mgpu.cu:1154-1283, :1701-1708): d_buffer holds seed_len prompt bytes
+ * followed by room for gen_len more (seed_len + gen_len <= seq_len); the unperturbed model continues the prompt with
+ * the reference's three-pass LUT sampling, threshold hash_rng(seed + t*555, 0) % sum.  Enqueued on the stream. */
+int  egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed);
+
 /* debug taps (test hook, no reference counterpart beyond EGG_TRACE_STAT, mgpu.cu:723): when enabled, a
  * forward over at most 64 members keeps every stage's activations; egg_tap_download copies one member's
  * "x_init", "q.L", "k.L", "v.L", "ao.L", "x_attn.L", "x_mlp.L" (L = layer) or "logits" to the host. */

@@ -233,6 +233,43 @@ def forward_member(cfg, model, data, start_idx, step_seed, p_idx, ns_override=2,
     return (loss, bufs) if trace else loss
 
 
+def sample_token(logits_row, exp_lut, seed, t, hidden):
+    """Three-pass LUT sampling of generate_sequence_kernel (mgpu.cu:1212-1283) for position t: the threshold is
+    hash_rng(seed + t*555, 0) % sum, and the running sum is taken in the reference's thread order (thread tid owns
+    v = tid, tid + BLOCK_THREADS, ...; BLOCK_THREADS = hidden rounded up to 32, at most 1024, mgpu.cu:74-75)."""
+    V = len(logits_row)
+    bt = min((hidden + 31) & ~31, 1024)
+    gmax = int(logits_row.max())
+    ex = exp_lut[np.clip(gmax - logits_row.astype(np.int64), 0, 255)].astype(np.int64)
+    total = int(ex.sum())
+    lib().orc_hash_rng.restype = C.c_uint32
+    r = int(lib().orc_hash_rng(C.c_uint32((seed + t * 555) & 0xFFFFFFFF), C.c_uint32(0)))
+    thresh = r % total if total > 0 else 0
+    running = 0
+    for tid in range(bt):
+        for v in range(tid, V, bt):
+            running += int(ex[v])
+            if running > thresh:
+                return v
+    return 0
+
+
+def generate(cfg, model, prompt, gen_len, seed):
+    """generate_sequence_kernel (mgpu.cu:1154-1283): unperturbed forward (noise_sign 0), token t+1 sampled from the
+    logits of position t for t >= seed_len - 1.  The window is re-evaluated from position 0 for every new token,
+    which equals the reference's KV-cache walk because position t only sees positions <= t."""
+    T = cfg.seq_len
+    seed_len = len(prompt)
+    assert 1 <= seed_len and seed_len + gen_len <= T
+    exp_lut = tables(cfg)[0]
+    buf = np.zeros(T + 1, np.uint8)
+    buf[:seed_len] = prompt
+    for t in range(seed_len - 1, seed_len + gen_len - 1):
+        _, tr = forward_member(cfg, model, buf, 0, 0, 0, ns_override=0, trace=True)
+        buf[t + 1] = sample_token(tr["logits"][t], exp_lut, seed, t, cfg.hidden)
+    return buf[:seed_len + gen_len].copy()
+
+
 def population_forward(cfg, model, data, start_idx, step_seed, pop_offset=0, count=None):
     count = cfg.population if count is None else count
     loss = np.zeros(cfg.population, np.int32)

@@ -353,3 +353,42 @@ def test_muon_update(pkg, orc, dev):
         d_seed.copy_(_t(dev, np.array([seed], np.uint32).view(np.int32)))
     assert ctx.last_update_count() >= 0
     ctx.close()
+
+
+@pytest.mark.parametrize("kw,seed_len,gen_len", [(dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4), 5, 27),
+                                                 (dict(hidden=128, head_dim=32, n_layers=2, seq_len=64, population=4), 10, 30),
+                                                 (dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4), 16, 40)],
+                         ids=["h64", "h128", "h256"])
+def test_generate(pkg, orc, dev, kw, seed_len, gen_len):
+    """Sampling continuation of a prompt by the unperturbed model against the oracle's token-by-token restatement."""
+    import torch
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    rng = np.random.default_rng(3)
+    for t in orc.tensor_table(ocfg):
+        if not t["is_matrix"]:
+            sl = slice(t["offset"], t["offset"] + t["cols"])
+            model[sl] = rng.integers(-20, 21, t["cols"]).astype(np.int8) + (16 if t["name"].startswith("ln_") and "bias" not in t["name"] else 0)
+        elif t["name"] == "embedding":      # a small tied head keeps the next-byte distribution broad
+            n = t["rows"] * t["cols"]
+            model[t["offset"]:t["offset"] + n] = rng.integers(-5, 6, n).astype(np.int8)
+    prompt = orc.zipf_bytes(4096)[100:100 + seed_len].copy()
+    ref = orc.generate(ocfg, model, prompt, gen_len, 1041)
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_upload(model)
+    buf = torch.zeros(seed_len + gen_len, dtype=torch.uint8, device=dev)
+    buf[:seed_len] = _t(dev, prompt)
+    ctx.generate(buf.data_ptr(), seed_len, gen_len, 1041)
+    ctx.sync()
+    got = buf.cpu().numpy()
+    assert np.array_equal(got, ref), (got.tolist(), ref.tolist())
+    assert len(set(ref[seed_len:].tolist())) > 3      # the continuation is not degenerate
+    # a population forward afterwards is unaffected by the generation's mask / logits overrides
+    data = orc.zipf_bytes(1 << 14)
+    d_loss = torch.zeros(kw["population"], dtype=torch.int32, device=dev)
+    ctx.population_forward(_t(dev, data).data_ptr(), len(data), 0, 77, 0, kw["population"], d_loss.data_ptr())
+    ctx.sync()
+    assert np.array_equal(d_loss.cpu().numpy(), orc.population_forward(ocfg, model, data, 0, 77))
+    with pytest.raises(pkg.EggError):
+        ctx.generate(buf.data_ptr(), seed_len, kw["seq_len"], 1)
+    ctx.close()

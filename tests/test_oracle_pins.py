@@ -475,3 +475,38 @@ def test_ternary_pack_reference_vectors(orc):
         buf = np.zeros(n, np.uint8); back = np.zeros(len(src), np.int32)
         R.ref_ternary_pack(P(src), len(src), P(buf)); R.ref_ternary_unpack(P(buf), len(src), P(back))
         assert np.array_equal(back, src)
+
+
+def test_sampling_closed_forms(orc):
+    """generate_sequence_kernel's sampling (mgpu.cu:1212-1283).  Uniform logits give every vocabulary entry the
+    weight EXP_LUT[0] = 2^18, so the selected entry is the (thresh >> 18)-th one in the reference's scan order
+    (natural for BLOCK_THREADS >= vocab, thread-major below); a logit that leads all others by >= 75 always wins;
+    the threshold hash is pinned through the reference header."""
+    cfg = orc.config(hidden=256, head_dim=64, n_layers=1, seq_len=32, population=2)
+    exp_lut = orc.tables(cfg)[0]
+    assert exp_lut[0] == 1 << 18
+    r = orc.ref()
+    if r is not None:
+        hash_rng = r.ref_hash_rng
+    else:                       # without the compiled reference header the oracle's hash (pinned by known answers) stands in
+        hash_rng = orc.lib().orc_hash_rng
+        hash_rng.restype = C.c_uint32
+    flat = np.full(256, 37, np.int32)
+    for seed, t in ((1041, 0), (1041, 7), (42, 200), (0xFFFFFFF0, 31)):
+        rr = int(hash_rng(C.c_uint32((seed + t * 555) & 0xFFFFFFFF), C.c_uint32(0)))
+        p = (rr % (256 << 18)) >> 18
+        assert orc.sample_token(flat, exp_lut, seed, t, 256) == p
+        assert orc.sample_token(flat, exp_lut, seed, t, 512) == p
+        # BLOCK_THREADS 64: thread tid scans v = tid, tid + 64, tid + 128, tid + 192
+        assert orc.sample_token(flat, exp_lut, seed, t, 64) == (p // 4) + 64 * (p % 4)
+    peak = np.full(256, -500, np.int32)
+    peak[201] = -425            # 75 above the rest: every other weight is EXP_LUT[75] = 0
+    assert exp_lut[75] == 0 and exp_lut[74] > 0
+    for t in range(20):
+        assert orc.sample_token(peak, exp_lut, 99, t, 256) == 201
+    # two candidates with weights 2^18 and EXP_LUT[6]: the split follows thresh < 2^18
+    two = np.full(256, -1000, np.int32); two[10] = 0; two[20] = -6
+    w0, w1 = int(exp_lut[0]), int(exp_lut[6])
+    for t in range(50):
+        rr = int(hash_rng(C.c_uint32((5 + t * 555) & 0xFFFFFFFF), C.c_uint32(0)))
+        assert orc.sample_token(two, exp_lut, 5, t, 256) == (10 if rr % (w0 + w1) < w0 else 20)
