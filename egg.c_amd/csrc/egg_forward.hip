@@ -48,6 +48,27 @@ __device__ __forceinline__ void add_perturb8(v16i *acc, int sb, const int8_t *At
         }
 }
 
+// (acc + ((sb * a) >> sigma)) >> shift.  With FUSE it is evaluated as ((acc << sigma) + sb * a) >> (sigma + shift):
+// floor(floor(y / 2^sigma + acc) / 2^shift) == floor((y + acc * 2^sigma) / 2^(sigma + shift)) for integers, one
+// instruction less.  The host selects FUSE only when |acc| * 2^sigma + |sb * a| < 2^31 for the GEMM depth in question.
+template <bool FUSE>
+__device__ __forceinline__ int perturb_shift(int acc, int sb, int a, int sigma, int shift) {
+    if (FUSE) return (int)(((unsigned)acc << sigma) + (unsigned)mul24(sb, a)) >> (sigma + shift);
+    return (acc + (mul24(sb, a) >> sigma)) >> shift;
+}
+// acc[nt][r] = perturb_shift(acc[nt][r], sb, At[n], ...) for NT column groups starting at table offset n_off
+template <int NT, bool FUSE>
+__device__ __forceinline__ void perturb_shift_groups(v16i *acc, int sb, const int8_t *At, int n_off, int sigma, int shift, int g) {
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            int a4 = *reinterpret_cast<const int *>(At + n_off + 32 * nt + 8 * q + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[nt][4 * q + e] = perturb_shift<FUSE>(acc[nt][4 * q + e], sb, sx8(a4, e), sigma, shift);
+        }
+}
+
 // exchange of packed 32-column groups between the waves sharing a tile: group k of tile slot ts, 16 bytes per lane
 __device__ __forceinline__ void xch_put(int8_t *xch, int groups, int ts, int k, int lane, v4i v) {
     *reinterpret_cast<v4i *>(xch + ((size_t)(ts * groups + k) * 64 + lane) * 16) = v;
@@ -89,9 +110,13 @@ struct MlpCfg {
     static int total(int sets) { return WBYTES + 256 + sets * PER_SET + XCHG + RED; }
 };
 
-template <int H, bool FIRST>
+// FUSE: the host has checked sigma <= 7 and |noise| <= 15, which bounds |acc| * 2^sigma + |sb * a| below 2^31 for
+// GEMM depths up to 1024 (depth * 127 * 127 * 128 + depth * 127 * 225); the down projection (depth 4H) uses the
+// fused form only for 4H <= 1024.
+template <int H, bool FIRST, bool FUSE>
 __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p) {
     typedef MlpCfg<H> M;
+    constexpr bool FUSE_DN = FUSE && 4 * H <= 1024;
     constexpr int CS = M::CS, KS = M::KS, NTS = M::NTS, HS = M::HS, NTU = M::NTU, SC = M::SC;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *act = smem + M::WBYTES;
@@ -200,12 +225,12 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                     mfma_cols<M::PRO / 2, NTS>(acc, aop + u * (M::PRO / 2), cur, H, col0, lane);
                 }
             }
-            add_perturb8<NTS>(acc, sbo, oA, col0, c.sigma, g);
+            perturb_shift_groups<NTS, FUSE>(acc, sbo, oA, col0, c.sigma, c.shift_out, g);
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++) {
                 v4i xr = load_op(xrow, nt, g);
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc[nt][r] = sx8(xr[r >> 2], r & 3) + (acc[nt][r] >> c.shift_out);
+                for (int r = 0; r < 16; r++) acc[nt][r] += sx8(xr[r >> 2], r & 3);
             }
             const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red, tm, lane);
             adaptive_scale<NTS>(acc, mx, xs);
@@ -273,8 +298,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                         int o[4];
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            int a = au[nt][4 * q + e] + (mul24(sbu, sx8(a4, e)) >> c.sigma);
-                            int v = clip127(a >> c.shift_mlp_up);
+                            int v = clip127(perturb_shift<FUSE>(au[nt][4 * q + e], sbu, sx8(a4, e), c.sigma, c.shift_mlp_up));
                             o[e] = act[(uint8_t)v];
                         }
                         mine[nt][q] = pack4(o[0], o[1], o[2], o[3]);
@@ -302,7 +326,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         }
         sbd += other_half(sbd);
         sbd = xreduce<CS, false>(sbd, red + 2 * M::SITE, tm, lane);
-        add_perturb8<NTS>(accd, sbd, dnA, col0, c.sigma, g);
+        perturb_shift_groups<NTS, FUSE_DN>(accd, sbd, dnA, col0, c.sigma, c.shift_mlp_down, g);
 #pragma unroll
         for (int nt = 0; nt < NTS; nt++) {
             v4i xr = load_op(xrow, nt, g);          // the parked residual (for a padding wave: someone else's row, unused)
@@ -311,7 +335,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 v4i b4 = *reinterpret_cast<const v4i *>(bdn + col0 + 32 * nt + 8 * q + 4 * g);
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    accd[nt][4 * q + e] = sx8(xr[q], e) + (accd[nt][4 * q + e] >> c.shift_mlp_down) + b4[e];
+                    accd[nt][4 * q + e] += sx8(xr[q], e) + b4[e];
             }
         }
         const int mx2 = xreduce<CS, true>(absmax_groups<NTS>(accd), red + 3 * M::SITE, tm, lane);
@@ -746,8 +770,9 @@ static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
     const int sets = tile_map_sets(p.c.T, Shape<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = MlpCfg<H>::total(sets);
-    if (first) hipLaunchKernelGGL((k_mlp<H, true>), grid, block, lds, s, p);
-    else hipLaunchKernelGGL((k_mlp<H, false>), grid, block, lds, s, p);
+    const bool fuse = p.c.sigma <= 7 && p.c.mask <= 15;
+    if (first) { if (fuse) hipLaunchKernelGGL((k_mlp<H, true, true>), grid, block, lds, s, p); else hipLaunchKernelGGL((k_mlp<H, true, false>), grid, block, lds, s, p); }
+    else { if (fuse) hipLaunchKernelGGL((k_mlp<H, false, true>), grid, block, lds, s, p); else hipLaunchKernelGGL((k_mlp<H, false, false>), grid, block, lds, s, p); }
     return hipGetLastError();
 }
 hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s) {
@@ -828,8 +853,10 @@ hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
 template <int H>
 static hipError_t prepare_h(int T) {
     const int sets = tile_map_sets(T, Shape<H>::CS);
-    SET_LDS((k_mlp<H, true>), MlpCfg<H>::total(sets));
-    SET_LDS((k_mlp<H, false>), MlpCfg<H>::total(sets));
+    SET_LDS((k_mlp<H, true, true>), MlpCfg<H>::total(sets));
+    SET_LDS((k_mlp<H, false, true>), MlpCfg<H>::total(sets));
+    SET_LDS((k_mlp<H, true, false>), MlpCfg<H>::total(sets));
+    SET_LDS((k_mlp<H, false, false>), MlpCfg<H>::total(sets));
     SET_LDS((k_qkv<H>), QkvCfg<H>::total(sets));
     SET_LDS((k_head<H>), HeadLds<H>::TOTAL);
     return hipSuccess;
