@@ -108,6 +108,20 @@ struct WStream {
 };
 __device__ __forceinline__ void wstream_init(WStream &s, int8_t *lds, int unit_bytes) { s.fill = lds; s.other = lds + unit_bytes; }
 
+// One wave instruction of the global -> LDS copy: lane l moves the 16 bytes at ubase + 16*l to lds_dst + 16*l.
+// Written as inline assembly on purpose: for the compiler's own LDS-DMA intrinsic every later LDS read may alias the
+// destination, so it waits for the copy (s_waitcnt vmcnt(0)) before the next table or fragment read and the copy no
+// longer overlaps anything.  Here the ordering is explicit instead: w_acquire waits for vmcnt(0) and then barriers
+// before anyone reads a unit, and a buffer is only overwritten after the barrier that follows its last reader.
+// Both ubase and lds_dst must be wave-uniform.
+__device__ __forceinline__ void lds_dma16(const int8_t *ubase, uint32_t lane16, const int8_t *lds_dst) {
+    const uint32_t m0v = __builtin_amdgcn_readfirstlane((uint32_t)(size_t)(const __attribute__((address_space(3))) int8_t *)lds_dst);
+    const uint64_t b = (uint64_t)ubase;
+    const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b), bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    const uint64_t sb = ((uint64_t)bhi << 32) | blo;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0v), "v"(lane16), "s"(sb) : "memory", "m0");
+}
+
 template <int B>
 __device__ __forceinline__ void w_prefetch(WStream &s, const int8_t *unit) {
     if (unit == nullptr) return;
@@ -122,15 +136,16 @@ __device__ __forceinline__ void w_prefetch(WStream &s, const int8_t *unit) {
     for (int i = 0; i < PER; i++) {
         const int c0 = (i * EGG_WAVES + wave) * 64;
         if (CHUNKS / 64 % EGG_WAVES == 0 || c0 < CHUNKS) {
-            const int8_t *ubase = unit + (size_t)c0 * 16;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ubase + lane16),
-                                             (__attribute__((address_space(3))) void *)(dst + (size_t)c0 * 16), 16, 0, 0);
+            lds_dma16(unit + (size_t)c0 * 16, lane16, dst + (size_t)c0 * 16);
         }
     }
 }
 // wait for the unit prefetched last, make it visible to the workgroup, and hand it out
 __device__ __forceinline__ const int8_t *w_acquire(WStream &s) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // s_waitcnt vmcnt(0) through the builtin (0x0F70 = vmcnt 0, expcnt/lgkmcnt untouched on gfx9) so that the compiler's
+    // own counter bookkeeping sees it: it then knows none of its loads or stores is pending and does not add
+    // vmcnt waits inside the phase, which would also wait for the copy issued right after this call
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     int8_t *p = s.fill;
     s.fill = s.other; s.other = p;
@@ -192,9 +207,7 @@ __device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, int s
         const int id = i * EGG_WAVES + wave;
         if (INSTR % EGG_WAVES == 0 || id < INSTR) {
             const int pr = id / SEG, seg = id % SEG;
-            const int8_t *ubase = src + ((size_t)pr * src_cols + seg * 64) * 16;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(ubase + lane16),
-                                             (__attribute__((address_space(3))) void *)(dst + ((size_t)pr * COLS + seg * 64) * 16), 16, 0, 0);
+            lds_dma16(src + ((size_t)pr * src_cols + seg * 64) * 16, lane16, dst + ((size_t)pr * COLS + seg * 64) * 16);
         }
     }
 }
