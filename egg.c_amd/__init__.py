@@ -44,6 +44,8 @@ EXPORTS = [
     "egg_fitness", "egg_es_update", "egg_update_tensor", "egg_matrix_votes",
     "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
     "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate",
+    "egg_shape_fitness", "egg_ternary_pack_size", "egg_ternary_pack", "egg_ternary_unpack",
+    "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
     "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz",
@@ -103,6 +105,15 @@ def lib():
         L.egg_step_launch.argtypes = [vp, i64, u32, C.c_float]
         L.egg_step_losses.argtypes = [vp, vp, vp]
         L.egg_generate.argtypes = [vp, vp, i32, i32, u32]
+        L.egg_shape_fitness.argtypes = [vp, i32, i32, C.c_double, i32, C.c_double, vp, vp]
+        L.egg_ternary_pack_size.restype = C.c_size_t
+        L.egg_ternary_pack_size.argtypes = [C.c_size_t]
+        L.egg_ternary_pack.argtypes = [vp, C.c_size_t, vp]
+        L.egg_ternary_unpack.argtypes = [vp, C.c_size_t, vp]
+        L.egg_checkpoint_save.argtypes = [vp, C.c_char_p, C.c_long]
+        L.egg_checkpoint_load.argtypes = [vp, C.c_char_p, C.c_char_p]
+        L.egg_eggc_save.argtypes = [C.c_char_p, C.c_uint64, C.c_uint64, vp, C.c_uint64]
+        L.egg_eggc_load_latest.argtypes = [C.c_char_p, vp, vp, vp, C.c_uint64, vp]
         L.egg_learning_rate.restype = C.c_float
         L.egg_learning_rate.argtypes = [C.c_long]
         L.egg_next_seed.restype = u32
@@ -281,6 +292,12 @@ class Context:
         self._ck(lib().egg_step_losses(self._h, _np_ptr(loss), _np_ptr(fit)), "egg_step_losses")
         return loss, fit
 
+    def checkpoint_save(self, directory, step):
+        self._ck(lib().egg_checkpoint_save(self._h, directory.encode() if directory else None, step), "egg_checkpoint_save")
+
+    def checkpoint_load(self, model_path, state_path=None):
+        self._ck(lib().egg_checkpoint_load(self._h, model_path.encode(), state_path.encode() if state_path else None), "egg_checkpoint_load")
+
     def generate(self, d_buffer, seed_len, gen_len, seed):
         """Continue the seed_len prompt bytes at device pointer d_buffer by gen_len sampled bytes (in place)."""
         self._ck(lib().egg_generate(self._h, C.c_void_p(d_buffer), seed_len, gen_len, seed & 0xFFFFFFFF), "egg_generate")
@@ -317,6 +334,61 @@ def _timing(self):
 Context.enable_timing = _enable_timing
 Context.timing_reset = _timing_reset
 Context.timing = _timing
+
+
+# ---- host-side companions (no GPU needed)
+def shape_fitness(loss, chunk_mean_filter=True, mean_exponent=1.2, adaptive_threshold=True, alpha=None):
+    """d-eggs worker shaping of one chunk's losses -> (fit[count/2] in {-1,0,1}, sum of losses)."""
+    import numpy as np
+    loss = np.ascontiguousarray(loss, np.int32)
+    if alpha is None:
+        alpha = float(np.float32(0.1))          # ADAPTIVE_THRESHOLD_ALPHA is the float literal 0.1f
+    fit = np.zeros(len(loss) // 2, np.int32)
+    total = C.c_int64(0)
+    rc = lib().egg_shape_fitness(_np_ptr(loss), len(loss), int(chunk_mean_filter), mean_exponent,
+                                 int(adaptive_threshold), alpha, _np_ptr(fit), C.byref(total))
+    if rc:
+        raise EggError(f"egg_shape_fitness failed ({rc})")
+    return fit, total.value
+
+
+def ternary_pack(fit):
+    import numpy as np
+    fit = np.ascontiguousarray(fit, np.int32)
+    out = np.zeros(lib().egg_ternary_pack_size(len(fit)), np.uint8)
+    if lib().egg_ternary_pack(_np_ptr(fit), len(fit), _np_ptr(out)):
+        raise EggError("egg_ternary_pack: values must be -1, 0 or 1")
+    return out
+
+
+def ternary_unpack(packed, count):
+    import numpy as np
+    packed = np.ascontiguousarray(packed, np.uint8)
+    out = np.zeros(count, np.int32)
+    if lib().egg_ternary_unpack(_np_ptr(packed), count, _np_ptr(out)):
+        raise EggError("egg_ternary_unpack failed")
+    return out
+
+
+def eggc_save(directory, step, seed, data):
+    import numpy as np
+    data = np.ascontiguousarray(data, np.uint8)
+    if lib().egg_eggc_save(directory.encode(), step, seed, _np_ptr(data), len(data)):
+        raise EggError("egg_eggc_save failed")
+
+
+def eggc_load_latest(directory):
+    """-> (step, seed, data) of the checkpoint with the highest step in `directory`, or None."""
+    import numpy as np
+    step, seed, n = C.c_uint64(0), C.c_uint64(0), C.c_uint64(0)
+    buf = np.zeros(1 << 16, np.uint8)
+    rc = lib().egg_eggc_load_latest(directory.encode(), C.byref(step), C.byref(seed), _np_ptr(buf), len(buf), C.byref(n))
+    if rc == -4 or (rc and n.value > len(buf)):          # EGG_E_STATE: payload larger than the buffer
+        buf = np.zeros(n.value, np.uint8)
+        rc = lib().egg_eggc_load_latest(directory.encode(), C.byref(step), C.byref(seed), _np_ptr(buf), len(buf), C.byref(n))
+    if rc:
+        return None
+    return step.value, seed.value, buf[:n.value].copy()
 
 
 def learning_rate(step):

@@ -158,6 +158,28 @@ uint32_t egg_next_seed(uint32_t seed, uint64_t step);
  * the reference's three-pass LUT sampling, threshold hash_rng(seed + t*555, 0) % sum.  Enqueued on the stream. */
 int  egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed);
 
+/* ---- host-side companions of the GPU path (host code in the reference as well) ---- */
+/* d-eggs worker result shaping (de/src/worker.cu:636-687): loss[count] of `count/2` antithetic pairs -> diff = n - p,
+ * optional chunk-mean shift (int)(sign(m) * |m|^mean_exponent) (CHUNK_MEAN_FILTER / CHUNK_MEAN_EXPONENT), optional
+ * threshold alpha * mean|diff| below which the vote is 0 (USE_ADAPTIVE_THRESHOLD / ADAPTIVE_THRESHOLD_ALPHA; the
+ * reference's alpha is the float literal 0.1f widened to double), else the sign.  sum_loss_out may be NULL. */
+int  egg_shape_fitness(const int32_t *loss, int count, int chunk_mean_filter, double mean_exponent,
+                       int adaptive_threshold, double alpha, int32_t *fit_out, int64_t *sum_loss_out);
+/* base-3 wire packing of ternary votes, five per byte (de/include/utils/ternary_pack.h:11-104) */
+size_t egg_ternary_pack_size(size_t count);
+int  egg_ternary_pack(const int32_t *src, size_t count, uint8_t *dst);
+int  egg_ternary_unpack(const uint8_t *src, size_t count, int32_t *dst);
+/* save_checkpoint / load_model (egg_disk_utils.h:46-82): <dir>/egg_step-%08ld.model.bin and .adam.bin hold the raw
+ * model blob and optimizer state, "egg_transformer_last.*" symlinks point at the newest; dir NULL = "models".
+ * Loading checks the file size against this context's shapes; state_path may be NULL.  Both synchronise. */
+int  egg_checkpoint_save(egg_ctx *ctx, const char *dir, long step);
+int  egg_checkpoint_load(egg_ctx *ctx, const char *model_path, const char *state_path);
+/* d-eggs replay checkpoints (de/include/utils/checkpoint.h:17-128): "checkpoint_%08llu.bin" = {magic "EGGC", version 1,
+ * step, seed, data_size} + data (the packed fitness history).  load_latest picks the highest step in dir; when the
+ * payload exceeds `capacity` it returns EGG_E_STATE with *n set to the size needed. */
+int  egg_eggc_save(const char *dir, uint64_t step, uint64_t seed, const uint8_t *data, uint64_t n);
+int  egg_eggc_load_latest(const char *dir, uint64_t *step, uint64_t *seed, uint8_t *data, uint64_t capacity, uint64_t *n);
+
 /* debug taps (test hook, no reference counterpart beyond EGG_TRACE_STAT, mgpu.cu:723): when enabled, a
  * forward over at most 64 members keeps every stage's activations; egg_tap_download copies one member's
  * "x_init", "q.L", "k.L", "v.L", "ao.L", "x_attn.L", "x_mlp.L" (L = layer) or "logits" to the host. */

@@ -1,6 +1,7 @@
 """GPU parity tests: every call goes through the C ABI of libegg_hip.so and is compared bit-for-bit with the
 CPU oracle on the same seeded inputs."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -392,3 +393,39 @@ def test_generate(pkg, orc, dev, kw, seed_len, gen_len):
     with pytest.raises(pkg.EggError):
         ctx.generate(buf.data_ptr(), seed_len, kw["seq_len"], 1)
     ctx.close()
+
+
+def test_checkpoint_files_round_trip(pkg, orc, dev, tmp_path):
+    """save_checkpoint / load_model (egg_disk_utils.h:46-82): raw model and optimizer-state files, "last" symlinks,
+    byte-identical to what the oracle holds after the same steps; a file of another shape is refused."""
+    import torch
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=40)
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    state = np.zeros(model.size, orc.ADAM_DTYPE)
+    rng = np.random.default_rng(4)
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_upload(model)
+    d_seed = _t(dev, np.array([9], np.uint32).view(np.int32)); d_lr = _t(dev, np.array([5.0], np.float32))
+    for step in range(2):
+        fit = rng.integers(-1, 2, 20).astype(np.int32)
+        ctx.es_update(_t(dev, fit).data_ptr(), d_seed.data_ptr(), d_lr.data_ptr())
+        orc.es_update_adam(ocfg, model, state, fit, 9, 5.0)
+    d = str(tmp_path / "models")
+    ctx.checkpoint_save(d, 7)
+    ctx.checkpoint_save(d, 12)
+    names = sorted(os.listdir(d))
+    assert names == ["egg_step-00000007.adam.bin", "egg_step-00000007.model.bin", "egg_step-00000012.adam.bin",
+                     "egg_step-00000012.model.bin", "egg_transformer_last.adam.bin", "egg_transformer_last.model.bin"]
+    assert os.readlink(os.path.join(d, "egg_transformer_last.model.bin")) == "egg_step-00000012.model.bin"
+    assert open(os.path.join(d, "egg_step-00000012.model.bin"), "rb").read() == model.tobytes()
+    assert open(os.path.join(d, "egg_transformer_last.adam.bin"), "rb").read() == state.tobytes()
+    ctx2 = pkg.Context(pkg.default_config(**kw))
+    ctx2.checkpoint_load(os.path.join(d, "egg_transformer_last.model.bin"), os.path.join(d, "egg_transformer_last.adam.bin"))
+    assert np.array_equal(ctx2.model_download(), model)
+    assert ctx2.opt_state_download().tobytes() == state.tobytes()
+    ctx3 = pkg.Context(pkg.default_config(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=40))
+    with pytest.raises(pkg.EggError):
+        ctx3.checkpoint_load(os.path.join(d, "egg_transformer_last.model.bin"))
+    for c in (ctx, ctx2, ctx3):
+        c.close()
