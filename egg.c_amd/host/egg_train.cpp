@@ -5,7 +5,11 @@
 // hash_rng (d-eggs/src/worker.cu:542) instead of time(NULL); no remote logging; errors return instead of exit(1)
 // inside the library.
 //
-// usage: egg_train [--data FILE] [--steps N] [--population P] [--seq T] [--hidden H] [--layers L] [--graph]
+// Every --gen-every steps it prints a sampled continuation of the current window (mgpu.cu:1698-1731) and every
+// --save-every steps it writes models/egg_step-*.bin (mgpu.cu:1733-1736); --load resumes from a model file.
+//
+// usage: egg_train [--data FILE] [--steps N] [--population P] [--seq T] [--hidden H] [--layers L] [--muon] [--graph]
+//                  [--gen-every N] [--save-every N] [--save-dir DIR] [--load MODEL.bin [--load-state ADAM.bin]]
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -44,6 +48,7 @@ int main(int argc, char **argv) {
     egg_config cfg; egg_default_config(&cfg);
     cfg.seq_len = 256; cfg.population = 40960;
     const char *data_file = nullptr; long steps = 10; bool graph = false; size_t synth_bytes = 64u << 20;
+    long gen_every = 5, save_every = 0; const char *save_dir = "models", *load_model = nullptr, *load_state = nullptr;
     for (int i = 1; i < argc; i++) {
         auto next = [&](const char *name) -> const char * { if (i + 1 >= argc) { fprintf(stderr, "%s needs a value\n", name); exit(2); } return argv[++i]; };
         if (!strcmp(argv[i], "--data")) data_file = next("--data");
@@ -54,6 +59,11 @@ int main(int argc, char **argv) {
         else if (!strcmp(argv[i], "--layers")) cfg.n_layers = atoi(next("--layers"));
         else if (!strcmp(argv[i], "--muon")) cfg.use_muon = 1;
         else if (!strcmp(argv[i], "--graph")) graph = true;
+        else if (!strcmp(argv[i], "--gen-every")) gen_every = atol(next("--gen-every"));
+        else if (!strcmp(argv[i], "--save-every")) save_every = atol(next("--save-every"));
+        else if (!strcmp(argv[i], "--save-dir")) save_dir = next("--save-dir");
+        else if (!strcmp(argv[i], "--load")) load_model = next("--load");
+        else if (!strcmp(argv[i], "--load-state")) load_state = next("--load-state");
         else { fprintf(stderr, "unknown argument %s\n", argv[i]); return 2; }
     }
     std::vector<uint8_t> data;
@@ -72,10 +82,21 @@ int main(int argc, char **argv) {
     egg_ctx *ctx = nullptr;
     int rc = egg_ctx_create(&cfg, &ctx);
     if (rc != EGG_OK) { fprintf(stderr, "egg_ctx_create failed (%d): unsupported configuration or no GPU\n", rc); return 1; }
-    CK(egg_model_init(ctx, 42));
+    if (load_model) CK(egg_checkpoint_load(ctx, load_model, load_state));
+    else CK(egg_model_init(ctx, 42));
     uint8_t *d_data = nullptr;
     HK(hipMalloc(&d_data, data.size()));
     HK(hipMemcpy(d_data, data.data(), data.size(), hipMemcpyHostToDevice));
+    // generation runs on a second, uncaptured context (the captured one is tied to its graph)
+    const int gen_seed_len = std::min(32, cfg.seq_len / 2), gen_total = std::min(cfg.seq_len, gen_seed_len + 64);
+    egg_ctx *gen_ctx = nullptr; uint8_t *d_gen = nullptr;
+    std::vector<uint8_t> h_model;
+    if (gen_every > 0) {
+        egg_config gcfg = cfg; gcfg.population = 2; gcfg.chunk_members = 2;
+        if (egg_ctx_create(&gcfg, &gen_ctx) != EGG_OK) { fprintf(stderr, "generation context failed\n"); return 1; }
+        HK(hipMalloc(&d_gen, (size_t)cfg.seq_len));
+        h_model.resize((size_t)egg_model_bytes(ctx));
+    }
     if (graph) CK(egg_step_capture(ctx, d_data, (int64_t)data.size()));
 
     std::vector<int32_t> loss((size_t)cfg.population), fit((size_t)cfg.population / 2);
@@ -95,8 +116,27 @@ int main(int argc, char **argv) {
         double avg = (double)total / ((double)cfg.population * cfg.seq_len * 16.0);
         printf("Step %ld | Loss: %.4f | Time: %.2f ms | Updates: %llu | Speed: %.2f tok/s | LR: %.3f\n", step, avg, ms,
                (unsigned long long)updates, (double)cfg.population * cfg.seq_len / (ms / 1e3), lr);
+        if (gen_every > 0 && step % gen_every == 0) {
+            CK(egg_model_download(ctx, h_model.data(), h_model.size()));
+            if (egg_model_upload(gen_ctx, h_model.data(), h_model.size()) != EGG_OK) return 1;
+            size_t pos = (size_t)(step * cfg.seq_len) % (data.size() - (size_t)cfg.seq_len);
+            HK(hipMemcpy(d_gen, d_data + pos, (size_t)gen_seed_len, hipMemcpyDeviceToDevice));
+            if (egg_generate(gen_ctx, d_gen, gen_seed_len, gen_total - gen_seed_len, seed + 999) != EGG_OK) { fprintf(stderr, "egg_generate: %s\n", egg_last_error(gen_ctx)); return 1; }
+            if (egg_sync(gen_ctx) != EGG_OK) return 1;
+            std::vector<uint8_t> h((size_t)gen_total);
+            HK(hipMemcpy(h.data(), d_gen, h.size(), hipMemcpyDeviceToHost));
+            printf("\n--- GENERATION ---\n\033[32m");
+            for (int i = 0; i < gen_total; i++) {
+                if (i == gen_seed_len) printf("\033[36m");
+                char c = (char)h[(size_t)i]; putchar((c >= 32 && c <= 126) ? c : '.');
+            }
+            printf("\033[0m\n\n");
+        }
+        if (save_every > 0 && step % save_every == 0) CK(egg_checkpoint_save(ctx, save_dir, step));
         seed = egg_next_seed(seed, (uint64_t)(step + 1));
     }
+    if (d_gen) (void)hipFree(d_gen);
+    if (gen_ctx) egg_ctx_destroy(gen_ctx);
     (void)hipFree(d_data);
     egg_ctx_destroy(ctx);
     return 0;
