@@ -192,24 +192,55 @@ __device__ __forceinline__ void gemm_stream(v16i *acc, const v4i *xop, const int
     }
 }
 
-// ---- generic units for the register-lean kernels: NP p-rows (p = 2*kstep + half) x COLS output columns of a
-// fragment-major block whose rows hold src_cols columns.  LDS image: [NP][COLS][16 bytes].
+// ---- units for the forward kernels: NP p-rows (p = 2*kstep + half) x COLS output columns of a fragment-major block
+// whose rows hold src_cols columns.  LDS image: [NP][COLS][16 bytes], so 64-column segment number id (= pr * COLS/64
+// + seg) lands at LDS byte id * 1024.  Wave w copies the PER consecutive segments w*PER .. w*PER + PER - 1 with one
+// M0 / one SGPR base and the instruction offsets 0, 1024, ...; because that offset is added to the global address as
+// well, each segment's per-lane global offset is precomputed once (DmaPlan) with the instruction offset taken out.
+// Per unit this costs a handful of scalar instructions instead of a 64-bit address computation per segment.
 template <int NP, int COLS>
-__device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, int src_cols) {
-    if (src == nullptr) return;
+struct DmaPlan {
     static_assert(COLS % 64 == 0, "a wave instruction copies 64 columns");
-    constexpr int SEG = COLS / 64, INSTR = NP * SEG, PER = (INSTR + EGG_WAVES - 1) / EGG_WAVES;
+    static constexpr int SEG = COLS / 64, INSTR = NP * SEG, PER = INSTR / EGG_WAVES;
+    static_assert(INSTR % EGG_WAVES == 0 && (PER == 1 || PER == 2 || PER == 4), "unit must split evenly over the waves");
+    uint32_t voff[PER];      // lane * 16 + global byte offset of segment k of this wave - k * 1024
+    uint32_t lds_off;        // first LDS byte of this wave inside the unit
+};
+template <int NP, int COLS>
+__device__ __forceinline__ DmaPlan<NP, COLS> dma_plan(int src_cols) {
+    typedef DmaPlan<NP, COLS> P;
+    P pl;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t lane16 = (threadIdx.x & 63u) * 16u;
-    int8_t *dst = s.fill;
 #pragma unroll
-    for (int i = 0; i < PER; i++) {
-        const int id = i * EGG_WAVES + wave;
-        if (INSTR % EGG_WAVES == 0 || id < INSTR) {
-            const int pr = id / SEG, seg = id % SEG;
-            lds_dma16(src + ((size_t)pr * src_cols + seg * 64) * 16, lane16, dst + ((size_t)pr * COLS + seg * 64) * 16);
-        }
+    for (int k = 0; k < P::PER; k++) {
+        const int id = wave * P::PER + k, pr = id / P::SEG, seg = id % P::SEG;
+        pl.voff[k] = lane16 + (uint32_t)(pr * src_cols + seg * 64) * 16u - (uint32_t)k * 1024u;
     }
+    pl.lds_off = (uint32_t)wave * P::PER * 1024u;
+    return pl;
+}
+// Start the copy of one unit into the fill buffer.  Inline assembly for the reason given at lds_dma16; src must be
+// wave-uniform.
+template <int NP, int COLS>
+__device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, const DmaPlan<NP, COLS> &pl) {
+    typedef DmaPlan<NP, COLS> P;
+    const uint32_t m0v = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(size_t)(const __attribute__((address_space(3))) int8_t *)s.fill) + pl.lds_off;
+    const uint64_t b = (uint64_t)src;
+    // readfirstlane returns a signed int: go through uint32_t so the low half is not sign-extended over the high half
+    const uint32_t blo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b), bhi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    const uint64_t sb = ((uint64_t)bhi << 32) | blo;
+    if (P::PER == 1)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     : : "s"(m0v), "v"(pl.voff[0]), "s"(sb) : "memory", "m0");
+    else if (P::PER == 2)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %3\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024"
+                     : : "s"(m0v), "v"(pl.voff[0]), "v"(pl.voff[P::PER > 1 ? 1 : 0]), "s"(sb) : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
+                     : : "s"(m0v), "v"(pl.voff[0]), "v"(pl.voff[P::PER > 1 ? 1 : 0]), "v"(pl.voff[P::PER > 2 ? 2 : 0]),
+                         "v"(pl.voff[P::PER > 3 ? 3 : 0]), "s"(sb) : "memory", "m0");
 }
 // acc[nt] += unit^T . xop for a unit of KSU k-steps x NTU column groups
 template <int KSU, int NTU>

@@ -137,15 +137,18 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
 
     WStream ws; wstream_init(ws, smem, M::UNIT);
     // unit sources inside the fragment-major copies (block size == H)
+    const DmaPlan<M::PRUP, SC> plan_up = dma_plan<M::PRUP, SC>(H);
+    const DmaPlan<M::PRDN, H> plan_dn = dma_plan<M::PRDN, H>(H);
+    const DmaPlan<M::PRO, H> plan_o = dma_plan<M::PRO, H>(H);
     auto pf_up = [&](int s, int ku) {
         const int n = s * SC;
-        w_prefetch2<M::PRUP, SC>(ws, p.w_up + (size_t)(n / H) * H * H + ((size_t)ku * M::PRUP * H + n % H) * 16, H);
+        w_prefetch2<M::PRUP, SC>(ws, p.w_up + (size_t)(n / H) * H * H + ((size_t)ku * M::PRUP * H + n % H) * 16, plan_up);
     };
     auto pf_dn = [&](int s, int du) {
         const int k = s * SC;
-        w_prefetch2<M::PRDN, H>(ws, p.w_dn + (size_t)(k / H) * H * H + (size_t)((k % H) / 16 + du * M::PRDN) * H * 16, H);
+        w_prefetch2<M::PRDN, H>(ws, p.w_dn + (size_t)(k / H) * H * H + (size_t)((k % H) / 16 + du * M::PRDN) * H * 16, plan_dn);
     };
-    auto pf_o = [&](int u) { w_prefetch2<M::PRO, H>(ws, p.w_o + (size_t)u * M::PRO * H * 16, H); };
+    auto pf_o = [&](int u) { w_prefetch2<M::PRO, H>(ws, p.w_o + (size_t)u * M::PRO * H * 16, plan_o); };
     auto pf_pass_first = [&]() { if (FIRST) pf_up(0, 0); else pf_o(0); };
     pf_pass_first();
 
@@ -425,7 +428,8 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
     int *red = reinterpret_cast<int *>(xch + Q::XCHG);
 
     WStream ws; wstream_init(ws, smem, Q::UNIT);
-    auto pf = [&](const int8_t *W, int u) { w_prefetch2<Q::PR, H>(ws, W + (size_t)u * Q::PR * H * 16, H); };
+    const DmaPlan<Q::PR, H> plan = dma_plan<Q::PR, H>(H);
+    auto pf = [&](const int8_t *W, int u) { w_prefetch2<Q::PR, H>(ws, W + (size_t)u * Q::PR * H * 16, plan); };
     pf(p.w_q, 0);
 
     for (int ss = 0; ss < tm.sets; ss++) {
