@@ -108,38 +108,9 @@ struct WStream {
 };
 __device__ __forceinline__ void wstream_init(WStream &s, int8_t *lds, int unit_bytes) { s.fill = lds; s.other = lds + unit_bytes; }
 
-// One wave instruction of the global -> LDS copy: lane l moves the 16 bytes at ubase + 16*l to lds_dst + 16*l.
-// Written as inline assembly on purpose: for the compiler's own LDS-DMA intrinsic every later LDS read may alias the
-// destination, so it waits for the copy (s_waitcnt vmcnt(0)) before the next table or fragment read and the copy no
-// longer overlaps anything.  Here the ordering is explicit instead: w_acquire waits for vmcnt(0) and then barriers
-// before anyone reads a unit, and a buffer is only overwritten after the barrier that follows its last reader.
-// Both ubase and lds_dst must be wave-uniform.
-__device__ __forceinline__ void lds_dma16(const int8_t *ubase, uint32_t lane16, const int8_t *lds_dst) {
-    const uint32_t m0v = __builtin_amdgcn_readfirstlane((uint32_t)(size_t)(const __attribute__((address_space(3))) int8_t *)lds_dst);
-    const uint64_t b = (uint64_t)ubase;
-    const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b), bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
-    const uint64_t sb = ((uint64_t)bhi << 32) | blo;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0v), "v"(lane16), "s"(sb) : "memory", "m0");
-}
-
 template <int B>
-__device__ __forceinline__ void w_prefetch(WStream &s, const int8_t *unit) {
-    if (unit == nullptr) return;
-    constexpr int CHUNKS = WUnit<B>::BYTES / 16;                 // 16-byte chunks, 64 per wave instruction
-    constexpr int PER = (CHUNKS / 64 + EGG_WAVES - 1) / EGG_WAVES;
-    // the wave index is read through readfirstlane so that the compiler keeps every address part that does not
-    // depend on the lane in scalar registers (LDS destination in M0, global base in an SGPR pair)
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t lane16 = (threadIdx.x & 63u) * 16u;
-    int8_t *dst = s.fill;
-#pragma unroll
-    for (int i = 0; i < PER; i++) {
-        const int c0 = (i * EGG_WAVES + wave) * 64;
-        if (CHUNKS / 64 % EGG_WAVES == 0 || c0 < CHUNKS) {
-            lds_dma16(unit + (size_t)c0 * 16, lane16, dst + (size_t)c0 * 16);
-        }
-    }
-}
+__device__ __forceinline__ void w_prefetch(WStream &s, const int8_t *unit);      // defined with the copy plans below
+
 // wait for the unit prefetched last, make it visible to the workgroup, and hand it out
 __device__ __forceinline__ const int8_t *w_acquire(WStream &s) {
     // s_waitcnt vmcnt(0) through the builtin (0x0F70 = vmcnt 0, expcnt/lgkmcnt untouched on gfx9) so that the compiler's
@@ -220,12 +191,16 @@ __device__ __forceinline__ DmaPlan<NP, COLS> dma_plan(int src_cols) {
     pl.lds_off = (uint32_t)wave * P::PER * 1024u;
     return pl;
 }
-// Start the copy of one unit into the fill buffer.  Inline assembly for the reason given at lds_dma16; src must be
-// wave-uniform.
+// Start the copy of one unit to lds_dst (global -> LDS without passing through registers; lane l of segment k moves
+// 16 bytes).  Written as inline assembly on purpose: for the compiler's own LDS-DMA intrinsic every later LDS read may
+// alias the destination, so it waits for the copy (s_waitcnt vmcnt(0)) before the next table or fragment read and the
+// copy no longer overlaps anything.  Here the ordering is explicit instead: w_acquire waits for vmcnt(0) and then
+// barriers before anyone reads a unit, and a buffer is only overwritten after the barrier that follows its last
+// reader.  src and lds_dst must be wave-uniform.
 template <int NP, int COLS>
-__device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, const DmaPlan<NP, COLS> &pl) {
+__device__ __forceinline__ void dma_unit(const int8_t *lds_dst, const int8_t *src, const DmaPlan<NP, COLS> &pl) {
     typedef DmaPlan<NP, COLS> P;
-    const uint32_t m0v = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(size_t)(const __attribute__((address_space(3))) int8_t *)s.fill) + pl.lds_off;
+    const uint32_t m0v = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(size_t)(const __attribute__((address_space(3))) int8_t *)lds_dst) + pl.lds_off;
     const uint64_t b = (uint64_t)src;
     // readfirstlane returns a signed int: go through uint32_t so the low half is not sign-extended over the high half
     const uint32_t blo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)b), bhi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
@@ -241,6 +216,20 @@ __device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, const
                      "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
                      : : "s"(m0v), "v"(pl.voff[0]), "v"(pl.voff[P::PER > 1 ? 1 : 0]), "v"(pl.voff[P::PER > 2 ? 2 : 0]),
                          "v"(pl.voff[P::PER > 3 ? 3 : 0]), "s"(sb) : "memory", "m0");
+}
+template <int NP, int COLS>
+__device__ __forceinline__ void w_prefetch2(WStream &s, const int8_t *src, const DmaPlan<NP, COLS> &pl) {
+    dma_unit<NP, COLS>(s.fill, src, pl);
+}
+// the same for a whole WUnit<B> (a contiguous slice of a block, so source and LDS image coincide); 32 KB units go as
+// two halves
+template <int B>
+__device__ __forceinline__ void w_prefetch(WStream &s, const int8_t *unit) {
+    if (unit == nullptr) return;
+    constexpr int NP = WUnit<B>::UK / 16, HALVES = (NP * B * 16 > 16384) ? 2 : 1, NPH = NP / HALVES;
+    const DmaPlan<NPH, B> pl = dma_plan<NPH, B>(B);
+#pragma unroll
+    for (int h = 0; h < HALVES; h++) dma_unit<NPH, B>(s.fill + h * (NPH * B * 16), unit + (size_t)h * (NPH * B * 16), pl);
 }
 // acc[nt] += unit^T . xop for a unit of KSU k-steps x NTU column groups
 template <int KSU, int NTU>
