@@ -128,17 +128,20 @@ __device__ __forceinline__ const int8_t *w_unit_ptr(const int8_t *Wf, int n_tota
     return Wf + ((size_t)(k_off / B + kb) * (n_total / B) + n_off / B) * (B * B) + (size_t)h * WUnit<B>::BYTES;
 }
 
-// acc[nt] += W_unit^T . xop for one staged unit; xop[ks] is the token operand of k-step ks of the unit
+// acc[nt] += W_unit^T . xop for one staged unit; xop[ks] is the token operand of k-step ks of the unit.  The
+// fragments of one k-step (at most 8) are read before its MFMAs so that one LDS latency is exposed per k-step.
 template <int B>
 __device__ __forceinline__ void mfma_unit(v16i *acc, const v4i *xop, const int8_t *lds, int lane) {
     const int i = lane & 31, g = lane >> 5;
+    constexpr int NT = B / 32;
 #pragma unroll
     for (int ks = 0; ks < WUnit<B>::UK / 32; ks++) {
+        v4i a[NT];
 #pragma unroll
-        for (int nt = 0; nt < B / 32; nt++) {
-            v4i a = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * B + nt * 32 + i) * 16);
-            acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, xop[ks], acc[nt], 0, 0, 0);
-        }
+        for (int nt = 0; nt < NT; nt++) a[nt] = *reinterpret_cast<const v4i *>(lds + ((size_t)(ks * 2 + g) * B + nt * 32 + i) * 16);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[nt], xop[ks], acc[nt], 0, 0, 0);
     }
 }
 
