@@ -163,6 +163,31 @@ def main():
     except Exception as e:
         gru = {"error": str(e)}
 
+    # ---- the d-eggs-style shape (hidden 512, 8 heads, seq 512, 8 layers, Muon) on one chunk of 2048 members
+    c5 = None
+    try:
+        P5 = 2048
+        c5ctx = pkg.Context(pkg.default_config(hidden=512, head_dim=64, n_layers=8, seq_len=512, population=P5, use_muon=1))
+        c5ctx.set_stream(stream.cuda_stream)
+        c5ctx.model_init(42)
+        c5ctx.step(d_data.data_ptr(), n, 0, 42, 0.3)
+        torch.cuda.synchronize()
+        c5ctx.enable_timing(True); c5ctx.timing_reset()
+        t0 = time.perf_counter()
+        c5ctx.step(d_data.data_ptr(), n, 512, 43, 0.3)
+        torch.cuda.synchronize()
+        sec = time.perf_counter() - t0
+        tm = c5ctx.timing()
+        fwd_ms = sum(tm[k][1] for k in ("mlp_first", "qkv", "attn", "mlp", "head"))
+        upd_ms = tm["update_matrix"][1] + tm["update_vector"][1]
+        c5 = {"value": P5 * 512 / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3, "forward_ms": fwd_ms, "update_ms": upd_ms,
+              "k_mlp_frac_mfma": (2 * 9 * 512 * 512 * P5 * 512) / (tm["mlp"][1] / tm["mlp"][0] * 1e-3) / PEAK_INT8_OPS,
+              "workload": f"hidden 512, 8 heads, seq 512, 8 layers, population {P5} (one chunk), forward+fitness+vote+Muon; "
+                          "a 16,384-member step is 8 such forwards plus one update"}
+        c5ctx.close()
+    except Exception as e:
+        c5 = {"error": str(e)}
+
     # ---- CPU baseline: the oracle's restatement of the same forward on a bounded sample of members
     cpu = None
     cpu_ref_path = None
@@ -170,14 +195,14 @@ def main():
         threads = orc.lib().orc_num_threads()
         ocfg = orc.config(**kw)
         model = orc.init_model(ocfg, 42)
-        sample = 8 * threads
+        sample = 16 * threads
         t0 = time.perf_counter()
         orc.population_forward(ocfg, model, data, 0, 42, 0, sample)
         sec = time.perf_counter() - t0
         cpu = {"value": sample * T / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
                "sample": f"forward only of {sample} of {P} members (T={T}) of the same model, scalar C++/OpenMP oracle, {sec:.1f}s"}
         # the reference's CPU program (full_trained_egg.c: GRU LM, H=512, L=4, P=128), scalar/OpenMP restatement
-        g = orc.gru_config(seq_len=1024)
+        g = orc.gru_config(seq_len=2048)
         gm = orc.gru_init_model(g, 42)
         states = np.zeros(g.population * g.n_layers * g.hidden, np.int8)
         npairs = min(64, 2 * threads)
@@ -196,7 +221,7 @@ def main():
                                f"forward+fitness+vote+AdamW, eager launches (chunk {chunk} members)",
                    "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss},
         "roofline": roofline, "kernels": per_class, "microbench_c2": mb,
-        "gru_c1_gpu": gru, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
+        "gru_c1_gpu": gru, "c5_shape_gpu": c5, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }
     print(json.dumps(out))
     ctx.close()
