@@ -585,6 +585,17 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                 }
     }
 
+    // the V rows are no longer needed once their transposed fragments sit in registers: the wave's LDS region now
+    // takes the K rows of this (member, head), which every query tile re-reads twice per context tile
+    wave_lds_fence();
+    for (int i = lane; i < T * HD / 16; i += 64) {
+        int cx = i / (HD / 16), part = i % (HD / 16);
+        *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + part * 16) =
+            *reinterpret_cast<const v4i *>(p.k + base + (size_t)cx * H + part * 16);
+    }
+    wave_lds_fence();
+    const int8_t *kl = vl;
+
 #pragma unroll 1
     for (int qt = 0; qt < CT; qt++) {
         const int t = qt * 32 + j;
@@ -601,7 +612,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                 for (int r = 0; r < 16; r++) s[r] = 0;
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
-                    v4i kf = load_op(p.k + base + (size_t)(32 * ct + j) * H, ks, g);
+                    v4i kf = load_op(kl + (size_t)(32 * ct + j) * HD, ks, g);
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
                 if (ct == qt) {
@@ -631,7 +642,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                 for (int r = 0; r < 16; r++) s[r] = 0;
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
-                    v4i kf = load_op(p.k + base + (size_t)(32 * ct + j) * H, ks, g);
+                    v4i kf = load_op(kl + (size_t)(32 * ct + j) * HD, ks, g);
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
                 v4i pw[3];
