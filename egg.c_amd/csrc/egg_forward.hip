@@ -587,14 +587,22 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
 
     // the V rows are no longer needed once their transposed fragments sit in registers: the wave's LDS region now
     // takes the K rows of this (member, head), which every query tile re-reads twice per context tile
+    // Rows are HD bytes apart, so the 16-byte chunk a lane reads (row = its context position) would hit the same few
+    // banks for every row; chunk c of row r is therefore kept at position c ^ ((r / RPL) % CH), which spreads eight
+    // consecutive rows over all banks.
+    constexpr int CH = HD / 16, RPL = 128 / HD;
     wave_lds_fence();
     for (int i = lane; i < T * HD / 16; i += 64) {
-        int cx = i / (HD / 16), part = i % (HD / 16);
-        *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + part * 16) =
+        int cx = i / CH, part = i % CH;
+        *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) =
             *reinterpret_cast<const v4i *>(p.k + base + (size_t)cx * H + part * 16);
     }
     wave_lds_fence();
     const int8_t *kl = vl;
+    auto k_frag = [&](int ct, int ks) {
+        const int r = 32 * ct + j;
+        return *reinterpret_cast<const v4i *>(kl + (size_t)r * HD + (((ks * 2 + g) ^ ((r / RPL) % CH)) * 16));
+    };
 
 #pragma unroll 1
     for (int qt = 0; qt < CT; qt++) {
@@ -612,7 +620,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                 for (int r = 0; r < 16; r++) s[r] = 0;
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
-                    v4i kf = load_op(kl + (size_t)(32 * ct + j) * HD, ks, g);
+                    v4i kf = k_frag(ct, ks);
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
                 if (ct == qt) {
@@ -642,7 +650,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                 for (int r = 0; r < 16; r++) s[r] = 0;
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
-                    v4i kf = load_op(kl + (size_t)(32 * ct + j) * HD, ks, g);
+                    v4i kf = k_frag(ct, ks);
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
                 v4i pw[3];
@@ -670,7 +678,9 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     int r = 4 * q + e;
-                    double num = __builtin_fma((double)o[2][dt][r], 16384.0, __builtin_fma((double)o[1][dt][r], 128.0, (double)o[0][dt][r]));
+                    // planes 0 and 1 combine in int32 (127*127*T + 127*127*T*128 < 2^31 for T <= 512)
+                    const int lo = o[0][dt][r] + (o[1][dt][r] << 7);
+                    double num = __builtin_fma((double)o[2][dt][r], 16384.0, (double)lo);
                     ov[e] = clip127((int)(num * rden));
                 }
                 outp[q] = pack4(ov[0], ov[1], ov[2], ov[3]);
