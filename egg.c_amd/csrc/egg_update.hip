@@ -89,87 +89,93 @@ __global__ void k_panels(UpdParams p) {
     else p.panel_b[(size_t)(r - p.cols) * p.pairs_pad + pr] = (int8_t)val;
 }
 
-// one wave per 32(k) x 32(n) tile of the vote matrix; reduction over pairs on the MFMA
+// One workgroup per 32(k) x 32(n) tile of the vote matrix.  The reduction over pairs runs on the MFMA, split four
+// ways over the waves (wave w takes the 32-pair steps w, w+4, ...; integer sums do not depend on the order); the
+// partial tiles meet in LDS and wave q finishes the four k-rows 8q+4g+e of the tile (the Adam / Muon / raw-vote
+// epilogue).  The operand loads are issued several steps ahead of the MFMAs that consume them.
 __global__ void __launch_bounds__(EGG_THREADS) k_vote_adam(UpdParams p) {
+    __shared__ int red[EGG_WAVES][16][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int tiles_n = p.cols / 32, tiles = (p.rows / 32) * tiles_n;
-    const int tile = blockIdx.x * EGG_WAVES + wave;
-    if (tile >= tiles) return;
+    const int tiles_n = p.cols / 32;
+    const int tile = blockIdx.x;
     const int k0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
     const int8_t *pb = p.panel_b + (size_t)(k0 + j) * p.pairs_pad + 16 * g;
     const int8_t *pa = p.panel_a + (size_t)(n0 + j) * p.pairs_pad + 16 * g;
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
-    for (int s = 0; s < p.pairs_pad; s += 32) {
+#pragma unroll 8
+    for (int s = wave * 32; s < p.pairs_pad; s += 32 * EGG_WAVES) {
         v4i a = *reinterpret_cast<const v4i *>(pb + s);
         v4i b = *reinterpret_cast<const v4i *>(pa + s);
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
     }
-    // lane (n = n0 + j, half g), register 4q+e -> k = k0 + 8q + 4g + e ; blocked index of (k, n) (mgpu.cu:1085-1089)
+#pragma unroll
+    for (int r = 0; r < 16; r++) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    const int q = wave;
+    int vote[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        int v = 0;
+#pragma unroll
+        for (int w = 0; w < EGG_WAVES; w++) v += red[w][4 * q + e][lane];
+        vote[e] = v;
+    }
+    // lane (n = n0 + j, half g), element e -> k = k0 + 8q + 4g + e ; blocked index of (k, n) (mgpu.cu:1085-1089)
     const int n = n0 + j;
+    const size_t idx0 = ((size_t)((k0 >> 2) + 2 * q + g) * p.cols + n) * 4;
     if (p.muon_x) {
         // muon_momentum_update_kernel + muon_gather_m_kernel (muon_internal.cuh:15-74): m = mu*m + vote
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const size_t idx0 = ((size_t)((k0 >> 2) + 2 * q + g) * p.cols + n) * 4;
-            float4 *sp = reinterpret_cast<float4 *>(p.state + idx0 * 2);
-            float4 s0 = sp[0], s1 = sp[1];
-            float mv[4] = {s0.x, s0.z, s1.x, s1.z};
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                float t = p.muon_momentum * mv[e];
-                mv[e] = t + (float)acc[4 * q + e];
-                p.muon_x[(size_t)(k0 + 8 * q + 4 * g + e) * p.cols + n] = mv[e];
-            }
-            sp[0] = make_float4(mv[0], s0.y, mv[1], s0.w);
-            sp[1] = make_float4(mv[2], s1.y, mv[3], s1.w);
-        }
-        return;
-    }
-    const float lr = p.votes_out ? 0.f : (*p.d_lr) * p.lr_scale;
-    const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd};
-    int changes = 0;
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const size_t idx0 = ((size_t)((k0 >> 2) + 2 * q + g) * p.cols + n) * 4;
-        if (p.votes_out) {
-            v4i o4;
-#pragma unroll
-            for (int e = 0; e < 4; e++) o4[e] = acc[4 * q + e];
-            *reinterpret_cast<v4i *>(p.votes_out + idx0) = o4;
-            continue;
-        }
-        int w4 = *reinterpret_cast<const int *>(p.W + idx0);
-        float st[12];
-        float4 *sp = reinterpret_cast<float4 *>(p.state + idx0 * 3);
-        float4 s0 = sp[0], s1 = sp[1], s2 = sp[2];
-        st[0] = s0.x; st[1] = s0.y; st[2] = s0.z; st[3] = s0.w; st[4] = s1.x; st[5] = s1.y; st[6] = s1.z; st[7] = s1.w;
-        st[8] = s2.x; st[9] = s2.y; st[10] = s2.z; st[11] = s2.w;
-        int wv[4];
+        float4 *sp = reinterpret_cast<float4 *>(p.state + idx0 * 2);
+        float4 s0 = sp[0], s1 = sp[1];
+        float mv[4] = {s0.x, s0.z, s1.x, s1.z};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            wv[e] = sx8(w4, e);
-            changes += adam_apply(st[3 * e], st[3 * e + 1], st[3 * e + 2], wv[e], -(float)acc[4 * q + e], lr, hy);
+            float t = p.muon_momentum * mv[e];
+            mv[e] = t + (float)vote[e];
+            p.muon_x[(size_t)(k0 + 8 * q + 4 * g + e) * p.cols + n] = mv[e];
         }
-        *reinterpret_cast<int *>(p.W + idx0) = pack4(wv[0], wv[1], wv[2], wv[3]);
-        sp[0] = make_float4(st[0], st[1], st[2], st[3]);
-        sp[1] = make_float4(st[4], st[5], st[6], st[7]);
-        sp[2] = make_float4(st[8], st[9], st[10], st[11]);
+        sp[0] = make_float4(mv[0], s0.y, mv[1], s0.w);
+        sp[1] = make_float4(mv[2], s1.y, mv[3], s1.w);
+        return;
     }
-    if (!p.votes_out) {
+    if (p.votes_out) {
+        v4i o4;
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) changes += __shfl_xor(changes, off, 64);
-        if (lane == 0 && changes) atomicAdd(p.counter, (unsigned long long)changes);
+        for (int e = 0; e < 4; e++) o4[e] = vote[e];
+        *reinterpret_cast<v4i *>(p.votes_out + idx0) = o4;
+        return;
     }
+    const float lr = (*p.d_lr) * p.lr_scale;
+    const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd};
+    int changes = 0;
+    int w4 = *reinterpret_cast<const int *>(p.W + idx0);
+    float st[12];
+    float4 *sp = reinterpret_cast<float4 *>(p.state + idx0 * 3);
+    float4 s0 = sp[0], s1 = sp[1], s2 = sp[2];
+    st[0] = s0.x; st[1] = s0.y; st[2] = s0.z; st[3] = s0.w; st[4] = s1.x; st[5] = s1.y; st[6] = s1.z; st[7] = s1.w;
+    st[8] = s2.x; st[9] = s2.y; st[10] = s2.z; st[11] = s2.w;
+    int wv[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        wv[e] = sx8(w4, e);
+        changes += adam_apply(st[3 * e], st[3 * e + 1], st[3 * e + 2], wv[e], -(float)vote[e], lr, hy);
+    }
+    *reinterpret_cast<int *>(p.W + idx0) = pack4(wv[0], wv[1], wv[2], wv[3]);
+    sp[0] = make_float4(st[0], st[1], st[2], st[3]);
+    sp[1] = make_float4(st[4], st[5], st[6], st[7]);
+    sp[2] = make_float4(st[8], st[9], st[10], st[11]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) changes += __shfl_xor(changes, off, 64);
+    if (lane == 0 && changes) atomicAdd(p.counter, (unsigned long long)changes);
 }
-
 hipError_t egg_launch_update_matrix(const UpdParams &p, hipStream_t s) {
     if (p.rows % 32 || p.cols % 32 || p.pairs_pad % 32) return hipErrorInvalidValue;
     int64_t total = (int64_t)(p.rows + p.cols) * p.pairs_pad;
     hipLaunchKernelGGL(k_panels, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, p);
     int tiles = (p.rows / 32) * (p.cols / 32);
-    hipLaunchKernelGGL(k_vote_adam, dim3((tiles + EGG_WAVES - 1) / EGG_WAVES), dim3(EGG_THREADS), 0, s, p);
+    hipLaunchKernelGGL(k_vote_adam, dim3(tiles), dim3(EGG_THREADS), 0, s, p);
     return hipGetLastError();
 }
 
