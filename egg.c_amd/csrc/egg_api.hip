@@ -63,6 +63,7 @@ struct egg_ctx {
     // generation (egg_generate): token buffer [T + 1], logits of one member [T][vocab], a zero start index / seed
     uint8_t *d_gen_tok = nullptr; int32_t *d_gen_logits = nullptr; Scalars *d_gen_scal = nullptr;
     int mask_override = -1; int32_t *logits_override = nullptr;
+    VecDesc *d_vec_desc = nullptr; int n_vec = 0, vec_total = 0;       // all vector tensors, for the one-launch update
     // graph
     hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr; bool captured = false;
     std::string err;
@@ -153,7 +154,7 @@ static void free_all(egg_ctx *ctx) {
     void *ptrs[] = {ctx->muon.x, ctx->muon.swap, ctx->muon.bterm, ctx->muon.partials, ctx->muon.norm,
                     ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
-                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal};
+                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal, ctx->d_vec_desc};
     for (void *p : ptrs) if (p) (void)hipFree(p);
     for (auto &sp : ctx->spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
     if (ctx->gexec) (void)hipGraphExecDestroy(ctx->gexec);
@@ -215,6 +216,20 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
         ctx->state_bytes = so;
     }
     CR(hipMalloc(&ctx->d_state, ctx->state_bytes)); CR(hipMemset(ctx->d_state, 0, ctx->state_bytes));
+    {
+        std::vector<VecDesc> vd;
+        int first = 0;
+        for (size_t id = 0; id < ctx->tensors.size(); id++) {
+            const egg_tensor_info &t = ctx->tensors[id];
+            if (t.is_matrix) continue;
+            VecDesc d; d.W = ctx->d_model + t.offset; d.state = reinterpret_cast<float *>(ctx->d_state + ctx->t_state_off[id]);
+            d.n = t.cols; d.first = first; d.off_a = t.off_a; d.off_b = t.off_b; d.seed_base = t.seed_base; d.lr_scale = t.lr_scale;
+            vd.push_back(d); first += t.cols;
+        }
+        ctx->n_vec = (int)vd.size(); ctx->vec_total = first;
+        CR(hipMalloc(&ctx->d_vec_desc, vd.size() * sizeof(VecDesc)));
+        CR(hipMemcpy(ctx->d_vec_desc, vd.data(), vd.size() * sizeof(VecDesc), hipMemcpyHostToDevice));
+    }
     if (c.use_muon) {
         size_t mx = (size_t)4 * c.hidden * c.hidden;
         CR(hipMalloc(&ctx->muon.x, mx * 4)); CR(hipMalloc(&ctx->muon.swap, mx * 4));
@@ -547,10 +562,17 @@ extern "C" int egg_matrix_votes(egg_ctx *ctx, int id, const int32_t *d_fit, cons
 extern "C" int egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
     if (!ctx || !d_fit || !d_seed || !d_lr) return fail(ctx, EGG_E_INVALID, "egg_es_update arguments");
     HIP_TRY(egg_launch_zero_u64(ctx->d_counter, 1, ctx->stream));
+    // matrices one by one (each needs the panel workspace), then every vector tensor in one launch; tensors are
+    // independent, so the reference's launch order (mgpu.cu:1603-1643) does not matter
     for (int id = 0; id < (int)ctx->tensors.size(); id++) {
+        if (!ctx->tensors[id].is_matrix) continue;
         int rc = update_one(ctx, id, d_fit, d_seed, d_lr);
         if (rc) return rc;
     }
+    UpdParams common = make_upd(ctx, 0, d_fit, d_seed, d_lr);
+    span_begin(ctx, EGG_K_UPDATE_VECTOR);
+    HIP_TRY(egg_launch_update_vectors(common, ctx->d_vec_desc, ctx->n_vec, ctx->vec_total, ctx->stream));
+    span_end(ctx);
     return EGG_OK;
 }
 extern "C" int64_t egg_opt_state_bytes(const egg_ctx *ctx) { return ctx ? ctx->state_bytes : 0; }

@@ -46,6 +46,9 @@ struct UpdParams {
 };
 hipError_t egg_launch_update_matrix(const UpdParams &p, hipStream_t s);
 hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s);
+// every vector tensor of the model in one launch: descriptors live on the device, `first` is the running element count
+struct VecDesc { int8_t *W; float *state; int n, first, off_a, off_b, seed_base; float lr_scale; };
+hipError_t egg_launch_update_vectors(const UpdParams &common, const VecDesc *d_desc, int n_desc, int total, hipStream_t s);
 
 // Muon chain (muon_internal.cuh:15-342): momentum + gather (vote GEMM epilogue), Frobenius normalisation,
 // 5 Newton-Schulz iterations on fp32 MFMA, quantised apply.

@@ -205,6 +205,42 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vector_adam(UpdParams p) {
         if (ch) atomicAdd(p.counter, 1ull);
     }
 }
+// the same for all vector tensors at once (one wave per element of any of them), so that the small per-tensor
+// launches do not leave most of the GPU idle
+__global__ void __launch_bounds__(EGG_THREADS) k_vectors_adam(UpdParams p, const VecDesc *desc, int n_desc, int total) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int gi = blockIdx.x * EGG_WAVES + wave;
+    if (gi >= total) return;
+    int d = 0;
+    while (d + 1 < n_desc && desc[d + 1].first <= gi) d++;
+    const VecDesc t = desc[d];
+    const int idx = gi - t.first;
+    const uint32_t base = *p.d_seed + (uint32_t)t.seed_base;
+    int vote = 0;
+    for (int pr = lane; pr < p.pairs; pr += 64) {
+        int f = p.fit[pr];
+        if (f == 0) continue;
+        uint32_t s = base + (uint32_t)pr;
+        vote += f * noise_from_hash(s + t.off_a, idx, p.mask) * noise_from_hash(s + t.off_b, idx, p.mask);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) vote += __shfl_xor(vote, off, 64);
+    if (lane == 0) {
+        const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd};
+        const float lr = (*p.d_lr) * t.lr_scale;
+        float *st = t.state + (size_t)idx * 3;
+        float m = st[0], v = st[1], acc = st[2];
+        int w = t.W[idx];
+        int ch = adam_apply(m, v, acc, w, -(float)vote, lr, hy);
+        t.W[idx] = (int8_t)w; st[0] = m; st[1] = v; st[2] = acc;
+        if (ch) atomicAdd(p.counter, 1ull);
+    }
+}
+hipError_t egg_launch_update_vectors(const UpdParams &common, const VecDesc *d_desc, int n_desc, int total, hipStream_t s) {
+    if (total <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_vectors_adam, dim3((total + EGG_WAVES - 1) / EGG_WAVES), dim3(EGG_THREADS), 0, s, common, d_desc, n_desc, total);
+    return hipGetLastError();
+}
 hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s) {
     hipLaunchKernelGGL(k_vector_adam, dim3((p.cols + EGG_WAVES - 1) / EGG_WAVES), dim3(EGG_THREADS), 0, s, p);
     return hipGetLastError();
