@@ -272,6 +272,34 @@ def test_full_step_eager_and_graph(pkg, orc, dev):
         ctx.close()
 
 
+def test_fifty_graph_steps_follow_the_oracle_trajectory(pkg, orc, dev):
+    """50 replays of the captured step graph with the reference's learning-rate schedule and the d-eggs seed chain:
+    int8 weights, float optimizer state and update counts stay bit-identical to the oracle's trajectory."""
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=64)
+    data = orc.zipf_bytes(1 << 16)
+    ocfg = orc.config(**kw)
+    d_data = _t(dev, data)
+    model = orc.init_model(ocfg, 42)
+    state = np.zeros(model.size, orc.ADAM_DTYPE)
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_init(42)
+    ctx.step_capture(d_data.data_ptr(), len(data))
+    seed = 42
+    changed = 0
+    for step in range(50):
+        lr = pkg.learning_rate(step) * 10.0          # a larger rate so that weights actually move within 50 steps
+        start = step * kw["seq_len"]
+        ctx.step_launch(start, seed, lr)
+        ref_fit = orc.fitness(orc.population_forward(ocfg, model, data, start, seed))
+        changed += orc.es_update_adam(ocfg, model, state, ref_fit, seed, np.float32(lr))
+        if step in (0, 9, 24, 49):
+            assert np.array_equal(ctx.model_download(), model), f"weights differ at step {step}"
+            assert ctx.opt_state_download().tobytes() == state.tobytes(), f"optimizer state differs at step {step}"
+        seed = pkg.next_seed(seed, step + 1)
+    assert changed > 100
+    ctx.close()
+
+
 def test_error_paths(pkg, dev):
     with pytest.raises(pkg.EggError):
         pkg.Context(pkg.default_config(hidden=100))
