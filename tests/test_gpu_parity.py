@@ -150,15 +150,18 @@ def test_forward_stages_and_loss(pkg, orc, dev, kw):
     assert not problems, "\n".join(problems[:12])
 
 
-def test_forward_chunked_and_offsets(pkg, orc, dev):
-    """Chunked evaluation (chunk smaller than the population, odd tail) and a sub-range give the same losses."""
+@pytest.mark.parametrize("hidden,head_dim,seq_len", [(64, 32, 32), (256, 64, 32), (128, 32, 64), (512, 64, 32)],
+                         ids=["h64", "h256_t32", "h128_t64", "h512_t32"])
+def test_forward_chunked_and_offsets(pkg, orc, dev, hidden, head_dim, seq_len):
+    """Chunked evaluation (chunk smaller than the population, odd tail that leaves padding waves in the last
+    workgroup) and a sub-range give the same losses."""
     import torch
-    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=22)
+    kw = dict(hidden=hidden, head_dim=head_dim, n_layers=1, seq_len=seq_len, population=22)
     data = orc.zipf_bytes(1 << 14)
     ocfg = orc.config(**kw)
     model = orc.init_model(ocfg, 7)
     ref = orc.population_forward(ocfg, model, data, 64, 555)
-    ctx = pkg.Context(pkg.default_config(chunk_members=6, **kw))
+    ctx = pkg.Context(pkg.default_config(chunk_members=5, **kw))
     ctx.model_upload(model)
     d_data = _t(dev, data)
     d_loss = torch.full((22,), -1, dtype=torch.int32, device=dev)
@@ -166,10 +169,10 @@ def test_forward_chunked_and_offsets(pkg, orc, dev):
     ctx.sync()
     assert np.array_equal(d_loss.cpu().numpy(), ref)
     d_loss.fill_(-1)
-    ctx.population_forward(d_data.data_ptr(), len(data), 64, 555, 4, 10, d_loss.data_ptr())
+    ctx.population_forward(d_data.data_ptr(), len(data), 64, 555, 3, 9, d_loss.data_ptr())
     ctx.sync()
     got = d_loss.cpu().numpy()
-    assert np.array_equal(got[4:14], ref[4:14]) and (got[:4] == -1).all() and (got[14:] == -1).all()
+    assert np.array_equal(got[3:12], ref[3:12]) and (got[:3] == -1).all() and (got[12:] == -1).all()
     ctx.close()
 
 
