@@ -77,6 +77,25 @@ __device__ __forceinline__ v4i xch_get(const int8_t *xch, int groups, int ts, in
     return *reinterpret_cast<const v4i *>(xch + ((size_t)(ts * groups + k) * 64 + lane) * 16);
 }
 
+// Hand the packed groups of the normalised operand from the wave that computed them to every wave of the tile through
+// the idle W buffer `buf` (`unit` bytes).  When the TPW tiles' operands exceed the buffer, the column slices take
+// turns (ROUNDS rounds of SPR slices each).  Every wave of the workgroup must call it.
+template <int CS, int NTS, int KS, int TPW, int UNIT_BYTES>
+__device__ __forceinline__ void exchange_operand(int8_t *buf, const TileMap &tm, int lane, const v4i *mine, v4i *full) {
+    constexpr int ROUNDS = (TPW * KS * 1024 + UNIT_BYTES - 1) / UNIT_BYTES, SPR = CS / ROUNDS, GR = SPR * NTS;
+    static_assert(CS % ROUNDS == 0 && TPW * GR * 1024 <= UNIT_BYTES, "operand exchange does not fit the W buffer");
+#pragma unroll
+    for (int r = 0; r < ROUNDS; r++) {
+        if (tm.cs / SPR == r)
+#pragma unroll
+            for (int nt = 0; nt < NTS; nt++) xch_put(buf, GR, tm.tslot, (tm.cs % SPR) * NTS + nt, lane, mine[nt]);
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < GR; k++) full[r * GR + k] = xch_get(buf, GR, tm.tslot, k, lane);
+        if (r + 1 < ROUNDS) __syncthreads();
+    }
+}
+
 // ============================================================================ MLP block
 // The 4H-wide intermediate is produced SC columns at a time (up GEMM, GELU epilogue, immediately consumed as k-steps
 // of the down GEMM), so only the down accumulator of the wave's column slice, the normalised input and one
@@ -85,7 +104,10 @@ __device__ __forceinline__ v4i xch_get(const int8_t *xch, int groups, int ts, in
 template <int H>
 struct MlpCfg {
     typedef Shape<H> S;
-    static constexpr int CS = S::CS, TPW = S::TPW, HS = S::HS, NTS = S::NTS, KS = S::KS;
+    // hidden 512 runs the MLP with two column slices (not four): twice the MFMAs per staged unit and half the
+    // exchanges outweigh the register spills of the 256-column accumulator
+    static constexpr int CS = H == 512 ? 2 : S::CS;
+    static constexpr int TPW = EGG_WAVES / CS, HS = H / CS, NTS = HS / 32, KS = H / 32;
     static constexpr int NTU = CS == 1 ? 2 : 1;          // up-GEMM column groups per wave and sub-chunk
     static constexpr int SC = 32 * CS * NTU;             // intermediate columns per sub-chunk
     static constexpr int NSUB = 4 * H / SC;
@@ -106,7 +128,6 @@ struct MlpCfg {
     static constexpr int SITE = EGG_WAVES * 64;                       // ints per reduction site
     static constexpr int RED = CS > 1 ? 4 * SITE * 4 : 0;
     static constexpr int OCC = H == 256 ? 3 : 2;                      // workgroups per CU the kernel is built for
-    static_assert(CS == 1 || TPW * 32 * H <= UNIT, "the operand exchange must fit one W buffer");
     static int total(int sets) { return WBYTES + 256 + sets * PER_SET + XCHG + RED; }
 };
 
@@ -253,17 +274,13 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             tot += other_half(tot);
             tot = xreduce<CS, false>(tot, red + M::SITE, tm, lane);
             int mn = tot / H; if (!mn) mn = 1;
-            if (CS == 1) standard_scale<NTS>(xs, nrm, mn, lnw, lnb, 0, g);
+            if constexpr (CS == 1) standard_scale<NTS>(xs, nrm, mn, lnw, lnb, 0, g);
             else {
                 // ws.other holds the unit consumed last; every wave has passed a barrier since reading it, and the
                 // next prefetch into it is issued only after the barrier of the next w_acquire
                 v4i mine[NTS];
                 standard_scale<NTS>(xs, mine, mn, lnw, lnb, col0, g);
-#pragma unroll
-                for (int nt = 0; nt < NTS; nt++) xch_put(ws.other, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
-                __syncthreads();
-#pragma unroll
-                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(ws.other, KS, tm.tslot, ks, lane);
+                exchange_operand<CS, NTS, KS, M::TPW, M::UNIT>(ws.other, tm, lane, mine, nrm);
             }
         }
         const int sbu = dot_noise<KS, false>(nrm, upB, 0, g);
@@ -363,7 +380,6 @@ struct QkvCfg {
     static constexpr int SITE = EGG_WAVES * 64;
     static constexpr int RED = CS > 1 ? 2 * SITE * 4 : 0;       // two reduction sites used alternately
     static constexpr int OCC = 2;                              // workgroups per CU the kernel is built for
-    static_assert(CS == 1 || TPW * 32 * H <= UNIT, "the operand exchange must fit one W buffer");
     static int total(int sets) { return WBYTES + sets * PER_SET + XCHG + RED; }
 };
 
@@ -467,15 +483,11 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
             tot += other_half(tot);
             tot = xreduce<CS, false>(tot, red, tm, lane);        // sites alternate 0,1,0,1 through the pass
             int mn = tot / H; if (!mn) mn = 1;
-            if (CS == 1) standard_scale<NTS>(x, nrm, mn, lnw, lnb, 0, g);
+            if constexpr (CS == 1) standard_scale<NTS>(x, nrm, mn, lnw, lnb, 0, g);
             else {
                 v4i mine[NTS];
                 standard_scale<NTS>(x, mine, mn, lnw, lnb, col0, g);
-#pragma unroll
-                for (int nt = 0; nt < NTS; nt++) xch_put(ws.other, KS, tm.tslot, tm.cs * NTS + nt, lane, mine[nt]);
-                __syncthreads();
-#pragma unroll
-                for (int ks = 0; ks < KS; ks++) nrm[ks] = xch_get(ws.other, KS, tm.tslot, ks, lane);
+                exchange_operand<CS, NTS, KS, Q::TPW, Q::UNIT>(ws.other, tm, lane, mine, nrm);
             }
         }
         RopeTab rt;
@@ -792,7 +804,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
 // ============================================================================ host launchers
 template <int H>
 static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
-    const int sets = tile_map_sets(p.c.T, Shape<H>::CS);
+    const int sets = tile_map_sets(p.c.T, MlpCfg<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = MlpCfg<H>::total(sets);
     const bool fuse = p.c.sigma <= 7 && p.c.mask <= 15;
@@ -878,10 +890,11 @@ hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
 template <int H>
 static hipError_t prepare_h(int T) {
     const int sets = tile_map_sets(T, Shape<H>::CS);
-    SET_LDS((k_mlp<H, true, true>), MlpCfg<H>::total(sets));
-    SET_LDS((k_mlp<H, false, true>), MlpCfg<H>::total(sets));
-    SET_LDS((k_mlp<H, true, false>), MlpCfg<H>::total(sets));
-    SET_LDS((k_mlp<H, false, false>), MlpCfg<H>::total(sets));
+    const int msets = tile_map_sets(T, MlpCfg<H>::CS);
+    SET_LDS((k_mlp<H, true, true>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, false, true>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, true, false>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, false, false>), MlpCfg<H>::total(msets));
     SET_LDS((k_qkv<H>), QkvCfg<H>::total(sets));
     SET_LDS((k_head<H>), HeadLds<H>::TOTAL);
     return hipSuccess;
