@@ -341,34 +341,44 @@ __global__ void k_scale_by_norm(float *x, const float *norm, int n) {
     if (i < n) { float nv = *norm; if (nv > 1e-6f) x[i] /= nv; }
 }
 
-// C[M][N] (row-major, ldc = N) = epilogue(sum_k A(i,k) B(k,j)), generic strides, one wave per 32x32 tile on
-// v_mfma_f32_32x32x2_f32.  mode 0: C = alpha * acc.  mode 1: C = (i == j ? 3 : 0) - acc  (3I - G, muon_internal.cuh:91-109).
+// C[M][N] (row-major, ldc = N) = epilogue(sum_k A(i,k) B(k,j)), generic strides, one workgroup per 32x32 tile on
+// v_mfma_f32_32x32x2_f32.  The k range is dealt to the four waves in steps of two (wave w takes k = 2w, 2w + 8, ...),
+// the partial tiles are added in wave order in LDS (a fixed summation order, so results are reproducible), and wave q
+// writes rows 8q + 4g + e of the tile.  mode 0: C = alpha * acc.  mode 1: C = (i == j ? 3 : 0) - acc  (3I - G,
+// muon_internal.cuh:91-109).
 __global__ void __launch_bounds__(EGG_THREADS) k_sgemm(const float *A, long sa_i, long sa_k, const float *B, long sb_k, long sb_j,
                                                       float *C, int M, int N, int K, float alpha, int mode) {
+    __shared__ float red[EGG_WAVES][16][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int tiles_n = N / 32, tile = blockIdx.x * EGG_WAVES + wave;
-    if (tile >= (M / 32) * tiles_n) return;
+    const int tiles_n = N / 32, tile = blockIdx.x;
     const int i0 = (tile / tiles_n) * 32, j0 = (tile % tiles_n) * 32;
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
     const float *ap = A + (long)(i0 + j) * sa_i + (long)g * sa_k;
     const float *bp = B + (long)g * sb_k + (long)(j0 + j) * sb_j;
-    for (int k = 0; k < K; k += 2) {
+#pragma unroll 8
+    for (int k = 2 * wave; k < K; k += 2 * EGG_WAVES) {
         float a = ap[(long)k * sa_k], b = bp[(long)k * sb_k];
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
     }
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        int i = i0 + ((r >> 2) << 3) + (g << 2) + (r & 3), jj = j0 + j;
-        float v = (mode == 1) ? ((i == jj ? 3.0f : 0.0f) - acc[r]) : alpha * acc[r];
-        C[(size_t)i * N + jj] = v;
+    for (int r = 0; r < 16; r++) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    const int q = wave;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float v = red[0][4 * q + e][lane];
+#pragma unroll
+        for (int w = 1; w < EGG_WAVES; w++) v += red[w][4 * q + e][lane];
+        const int i = i0 + 8 * q + 4 * g + e, jj = j0 + j;
+        C[(size_t)i * N + jj] = (mode == 1) ? ((i == jj ? 3.0f : 0.0f) - v) : alpha * v;
     }
 }
 static void sgemm(const float *A, long sa_i, long sa_k, const float *B, long sb_k, long sb_j, float *C, int M, int N, int K,
                   float alpha, int mode, hipStream_t s) {
     int tiles = (M / 32) * (N / 32);
-    hipLaunchKernelGGL(k_sgemm, dim3((tiles + EGG_WAVES - 1) / EGG_WAVES), dim3(EGG_THREADS), 0, s, A, sa_i, sa_k, B, sb_k, sb_j, C, M, N, K, alpha, mode);
+    hipLaunchKernelGGL(k_sgemm, dim3(tiles), dim3(EGG_THREADS), 0, s, A, sa_i, sa_k, B, sb_k, sb_j, C, M, N, K, alpha, mode);
 }
 __global__ void k_copy_f32(float *dst, const float *src, int n) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -383,18 +393,20 @@ hipError_t egg_launch_newton_schulz(const MuonWork &w, int rows, int cols, int i
     hipLaunchKernelGGL(k_sumsq_partial, dim3(256), dim3(256), 0, s, w.x, n, w.partials);
     hipLaunchKernelGGL(k_norm_finish, dim3(1), dim3(256), 0, s, w.partials, 256, w.norm);
     hipLaunchKernelGGL(k_scale_by_norm, dim3((n + 255) / 256), dim3(256), 0, s, w.x, w.norm, n);
+    float *cur = w.x, *nxt = w.swap;          // ping-pong instead of copying back after every iteration
     for (int it = 0; it < iters; it++) {
         if (use_rows) {
             // G = X X^T (rows x rows); X <- 0.5 (3I - G) X
-            sgemm(w.x, cols, 1, w.x, 1, cols, w.bterm, K, K, cols, 1.f, 1, s);
-            sgemm(w.bterm, K, 1, w.x, cols, 1, w.swap, rows, cols, K, 0.5f, 0, s);
+            sgemm(cur, cols, 1, cur, 1, cols, w.bterm, K, K, cols, 1.f, 1, s);
+            sgemm(w.bterm, K, 1, cur, cols, 1, nxt, rows, cols, K, 0.5f, 0, s);
         } else {
             // G = X^T X (cols x cols); X <- 0.5 X (3I - G)
-            sgemm(w.x, 1, cols, w.x, cols, 1, w.bterm, K, K, rows, 1.f, 1, s);
-            sgemm(w.x, cols, 1, w.bterm, K, 1, w.swap, rows, cols, K, 0.5f, 0, s);
+            sgemm(cur, 1, cols, cur, cols, 1, w.bterm, K, K, rows, 1.f, 1, s);
+            sgemm(cur, cols, 1, w.bterm, K, 1, nxt, rows, cols, K, 0.5f, 0, s);
         }
-        hipLaunchKernelGGL(k_copy_f32, dim3((n + 255) / 256), dim3(256), 0, s, w.x, w.swap, n);
+        float *t = cur; cur = nxt; nxt = t;
     }
+    if (cur != w.x) hipLaunchKernelGGL(k_copy_f32, dim3((n + 255) / 256), dim3(256), 0, s, w.x, cur, n);
     return hipGetLastError();
 }
 
