@@ -702,6 +702,146 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
     }
 }
 
+// The same attention for long sequences (at least 8 tiles): one workgroup per (member, head).  The K rows and the
+// transposed V fragments are built once in LDS and shared by the four waves, which split the query tiles so that
+// the causal work is balanced (wave w takes tiles w and 7 - w of every group of eight).  Keeping the V fragments in
+// LDS instead of registers leaves room for more resident waves.
+template <int HD, int CT>
+struct AttnWg {
+    static constexpr int T = CT * 32, ROWS = T * HD;               // bytes of one K or V head tile
+    static constexpr int LDS = 2048 + 2 * ROWS;                    // LUT | rows (V, then K) | V^T fragments
+    static constexpr int OCC = (2 * LDS <= 80 * 1024) ? 2 : 1;
+};
+template <int HD, int CT>
+__global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(AttnParams p) {
+    constexpr int KS = HD / 32, DT = HD / 32, T = CT * 32, CH = HD / 16, RPL = 128 / HD;
+    static_assert(CT % 8 == 0, "query tiles are dealt in groups of eight");
+    extern __shared__ __align__(16) int8_t smem[];
+    int2 *lut = reinterpret_cast<int2 *>(smem);
+    int8_t *rows = smem + 2048;
+    int8_t *vfrag = rows + AttnWg<HD, CT>::ROWS;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const FwdCommon &c = p.c;
+    const int H = c.H, NH = H / HD;
+    const int unit = blockIdx.x;                                   // grid = n_members * heads exactly
+    const int mloc = unit / NH, h = unit % NH;
+    const size_t base = (size_t)mloc * T * H + (size_t)h * HD;
+
+    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) {
+        const int w = c.exp_lut[i];
+        lut[i] = make_int2(w, (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16));
+    }
+    // V rows of this (member, head) -> LDS [ctx][HD]
+    for (int i = threadIdx.x; i < T * CH; i += EGG_THREADS) {
+        int cx = i / CH, part = i % CH;
+        *reinterpret_cast<v4i *>(rows + (size_t)cx * HD + part * 16) =
+            *reinterpret_cast<const v4i *>(p.v + base + (size_t)cx * H + part * 16);
+    }
+    __syncthreads();
+    // V^T fragments: A-operand row i = natural head dim d = 32dt + i, stored at slot position 16g'+4q'+e'
+    {
+        const int pos = ((j >> 2) & 1) * 16 + (j >> 3) * 4 + (j & 3);
+        for (int f = wave; f < CT * DT; f += EGG_WAVES) {
+            const int ct = f / DT, dt = f % DT;
+            v4i frag;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int b[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) b[e] = rows[(size_t)(32 * ct + 8 * q + 4 * g + e) * HD + 32 * dt + pos];
+                frag[q] = pack4(b[0], b[1], b[2], b[3]);
+            }
+            *reinterpret_cast<v4i *>(vfrag + ((size_t)f * 64 + lane) * 16) = frag;
+        }
+    }
+    __syncthreads();
+    // K rows take the place of the V rows; chunk c of row r sits at c ^ ((r / RPL) % CH) to spread the banks
+    for (int i = threadIdx.x; i < T * CH; i += EGG_THREADS) {
+        int cx = i / CH, part = i % CH;
+        *reinterpret_cast<v4i *>(rows + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) =
+            *reinterpret_cast<const v4i *>(p.k + base + (size_t)cx * H + part * 16);
+    }
+    __syncthreads();
+    auto score_tile = [&](int ct, const v4i *qop) {
+        v16i s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0;
+        const int r = 32 * ct + j;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            v4i kf = *reinterpret_cast<const v4i *>(rows + (size_t)r * HD + (((ks * 2 + g) ^ ((r / RPL) % CH)) * 16));
+            s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
+        }
+        return s;
+    };
+
+#pragma unroll 1
+    for (int qi = 0; qi < CT / 4; qi++) {
+        const int qt = (qi >> 1) * 8 + ((qi & 1) ? 7 - wave : wave);
+        const int t = qt * 32 + j;
+        v4i qop[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) qop[ks] = load_op(p.q + base + (size_t)t * H, ks, g);
+        // pass 1: per-head maximum score over ctx <= t (mgpu.cu:795-802)
+        int mx = INT_MIN;
+#pragma unroll 2
+        for (int ct = 0; ct < qt; ct++) {
+            const v16i s = score_tile(ct, qop);
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) mx = max(max(mx, s[r]), s[r + 1]);
+        }
+        {
+            const v16i s = score_tile(qt, qop);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                int cx = 32 * qt + ((r >> 2) << 3) + (g << 2) + (r & 3);
+                if (cx <= t) mx = max(mx, s[r]);
+            }
+        }
+        mx = max(mx, other_half(mx));
+        const int mxs = mx >> c.shift_attn;
+        // pass 2: weights and weighted V sum (mgpu.cu:810-824)
+        v16i o[3][DT];
+#pragma unroll
+        for (int pl = 0; pl < 3; pl++) zero_acc<DT>(o[pl]);
+        int den = 0;
+        auto weigh_tile = [&](int ct, bool diag) {
+            const v16i s = score_tile(ct, qop);
+            v4i pw[3];
+            attn_weights(s, lut, mxs, c.shift_attn, diag, ct, t, g, pw, den);
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+                const v4i vt = *reinterpret_cast<const v4i *>(vfrag + ((size_t)(ct * DT + dt) * 64 + lane) * 16);
+#pragma unroll
+                for (int pl = 0; pl < 3; pl++) o[pl][dt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vt, pw[pl], o[pl][dt], 0, 0, 0);
+            }
+        };
+#pragma unroll 2
+        for (int ct = 0; ct < qt; ct++) weigh_tile(ct, false);
+        weigh_tile(qt, true);
+        den += other_half(den);
+        // truncating quotient with one reciprocal per token, see k_attn
+        const double rden = (1.0 + 0x1p-40) / (double)(den ? den : 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+            v4i outp;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int ov[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int r = 4 * q + e;
+                    const int lo = o[0][dt][r] + (o[1][dt][r] << 7);
+                    double num = __builtin_fma((double)o[2][dt][r], 16384.0, (double)lo);
+                    ov[e] = clip127((int)(num * rden));
+                }
+                outp[q] = pack4(ov[0], ov[1], ov[2], ov[3]);
+            }
+            store_op(p.ao + base + (size_t)t * H, dt, g, outp);
+        }
+    }
+}
+
 // ============================================================================ head + loss
 template <int H>
 struct HeadLds {
@@ -843,6 +983,11 @@ hipError_t egg_launch_qkv(const QkvParams &p, hipStream_t s) {
 template <int HD, int CT>
 static hipError_t launch_attn_t(const AttnParams &p, hipStream_t s) {
     int units = p.c.n_members * (p.c.H / HD);
+    if constexpr (CT % 8 == 0) {
+        const size_t lds_wg = AttnWg<HD, CT>::LDS;
+        hipLaunchKernelGGL((k_attn_wg<HD, CT>), dim3(units), dim3(EGG_THREADS), lds_wg, s, p);
+        return hipGetLastError();
+    }
     dim3 grid((units + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
     size_t lds = 2048 + (size_t)EGG_WAVES * CT * 32 * HD;
     hipLaunchKernelGGL((k_attn<HD, CT>), grid, block, lds, s, p);
@@ -901,6 +1046,7 @@ static hipError_t prepare_h(int T) {
 }
 template <int HD, int CT>
 static hipError_t prepare_attn() {
+    if constexpr (CT % 8 == 0) SET_LDS((k_attn_wg<HD, CT>), (AttnWg<HD, CT>::LDS));
     SET_LDS((k_attn<HD, CT>), 2048 + (size_t)EGG_WAVES * CT * 32 * HD);
     return hipSuccess;
 }
