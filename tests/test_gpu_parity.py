@@ -94,6 +94,8 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
                                 dict(hidden=128, head_dim=32, n_layers=1, seq_len=64, population=6),
                                 dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4),
                                 dict(hidden=256, head_dim=64, n_layers=1, seq_len=32, population=6),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=256, population=4),
+                                dict(hidden=256, head_dim=64, n_layers=1, seq_len=256, population=2),
                                 dict(hidden=512, head_dim=64, n_layers=1, seq_len=32, population=4),
                                 dict(hidden=512, head_dim=64, n_layers=1, seq_len=128, population=4),
                                 dict(hidden=512, head_dim=64, n_layers=2, seq_len=512, population=2),
@@ -101,7 +103,7 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
                                 dict(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=4, sigma_shift=5, noise_mask=31),
                                 dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4, sigma_shift=1, noise_mask=7,
                                      shift_out=8, shift_mlp_up=7, shift_mlp_down=9)],
-                         ids=["h64", "h128", "h256", "h256_t32", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts"])
+                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts"])
 def test_forward_stages_and_loss(pkg, orc, dev, kw):
     """Every stage tap of every member against the oracle's trace, then the per-member losses."""
     data = orc.zipf_bytes(1 << 15)
