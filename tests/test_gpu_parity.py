@@ -57,13 +57,17 @@ def test_noise_fill(pkg, orc, dev):
     ctx.close()
 
 
-@pytest.mark.parametrize("K,N,members,T", [(64, 64, 4, 32), (256, 256, 6, 64), (512, 512, 8, 32), (256, 1024, 3, 32),
-                                           (1024, 256, 2, 32)])
-def test_perturbed_linear(pkg, orc, dev, K, N, members, T):
+# the last two cases use a wider noise (mask 31, sigma 9): the kernel's fused perturb-and-shift form would overflow
+# there, so they take its two-shift form
+@pytest.mark.parametrize("K,N,members,T,extra", [(64, 64, 4, 32, {}), (256, 256, 6, 64, {}), (512, 512, 8, 32, {}),
+                                                 (256, 1024, 3, 32, {}), (1024, 256, 2, 32, {}),
+                                                 (512, 512, 3, 64, dict(sigma_shift=5, noise_mask=31)),
+                                                 (1024, 256, 2, 32, dict(sigma_shift=5, noise_mask=31))])
+def test_perturbed_linear(pkg, orc, dev, K, N, members, T, extra):
     import torch
     rng = np.random.default_rng(K * 7 + N)
-    ctx = pkg.Context(pkg.default_config(**SMALL))
-    ocfg = orc.config(**SMALL)
+    ctx = pkg.Context(pkg.default_config(**SMALL, **extra))
+    ocfg = orc.config(**SMALL, **extra)
     X = rng.integers(-127, 128, size=(members * T, K), dtype=np.int8)
     W = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
     Wb = np.zeros(K * N, np.int8)
