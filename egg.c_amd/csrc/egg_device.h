@@ -20,6 +20,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// The float steps of the normalisations are single IEEE operations in the reference; a fused multiply-add in
+// round_half_away(val * scale) changes results at exact .5 ties (e.g. max 6, value 3).  The build also passes
+// -ffp-contract=off; this keeps the header right under any flags.
+#pragma clang fp contract(off)
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 

@@ -1,0 +1,146 @@
+"""Checks at the sizes the headline numbers are quoted on (4 layers, hidden 256, 4 heads, sequence 256; populations
+8192 and 40,960).  The CPU oracle needs about 0.75 s per member at this shape, so whole populations are checked
+through properties that do not depend on the size (determinism, independence of the chunking, sub-range evaluation,
+antithetic pairs that coincide when the noise is zero, linearity of the votes) and a sample of members / tensors is
+compared bit-for-bit with the oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = dict(hidden=256, head_dim=64, n_layers=4, seq_len=256)
+
+
+def _t(dev, arr):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+
+
+def _forward(pkg, dev, cfg_kw, model, d_data, data_len, start, seed, offset=0, count=None, repeat=1):
+    import torch
+    pop = cfg_kw["population"]
+    count = pop if count is None else count
+    ctx = pkg.Context(pkg.default_config(**cfg_kw))
+    ctx.model_upload(model)
+    out = []
+    for _ in range(repeat):
+        d_loss = torch.full((pop,), -1, dtype=torch.int32, device=dev)
+        ctx.population_forward(d_data.data_ptr(), data_len, start, seed, offset, count, d_loss.data_ptr())
+        ctx.sync()
+        out.append(d_loss.cpu().numpy())
+    ctx.close()
+    return out
+
+
+def test_population_8192_forward(pkg, orc, dev):
+    pop = 8192
+    kw = dict(population=pop, **SHAPE)
+    data = orc.zipf_bytes(1 << 22)
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    d_data = _t(dev, data)
+    start, seed = 3 * 256, 0xC0FFEE
+
+    a, b = _forward(pkg, dev, dict(chunk_members=2048, **kw), model, d_data, len(data), start, seed, repeat=2)
+    assert np.array_equal(a, b), "two evaluations of the same step differ"
+    assert (a > 0).all()
+    # a chunk size that is neither a divisor of the population nor a multiple of the workgroup's member count
+    (c,) = _forward(pkg, dev, dict(chunk_members=1001, **kw), model, d_data, len(data), start, seed)
+    assert np.array_equal(a, c), f"{np.count_nonzero(a != c)} losses depend on the chunking"
+    # a sub-range leaves the rest of the output alone
+    (d,) = _forward(pkg, dev, dict(chunk_members=2048, **kw), model, d_data, len(data), start, seed, offset=4094, count=6)
+    assert np.array_equal(d[4094:4100], a[4094:4100]) and (d[:4094] == -1).all() and (d[4100:] == -1).all()
+
+    # sampled members against the oracle: first pair, members around both chunkings' boundaries, last pair
+    for first, n in ((0, 2), (1000, 2), (2046, 4), (8190, 2)):
+        ref = orc.population_forward(ocfg, model, data, start, seed, first, n)
+        assert np.array_equal(a[first:first + n], ref[first:first + n]), (first, a[first:first + n], ref[first:first + n])
+
+    # zero noise: both members of a pair evaluate the unperturbed model on the same bytes
+    (z,) = _forward(pkg, dev, dict(chunk_members=2048, noise_mask=0, **kw), model, d_data, len(data), start, seed)
+    assert np.array_equal(z[0::2], z[1::2])
+    zcfg = orc.config(noise_mask=0, **kw)
+    ref = orc.population_forward(zcfg, model, data, start, seed, 4094, 2)
+    assert np.array_equal(z[4094:4096], ref[4094:4096])
+
+
+def test_population_40960_step(pkg, orc, dev):
+    import torch
+    pop = 40960
+    pairs = pop // 2
+    kw = dict(population=pop, **SHAPE)
+    data = orc.zipf_bytes(1 << 23)
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    d_data = _t(dev, data)
+    start, seed, lr = 0, 20261, 0.3
+
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_upload(model)
+    d_loss = torch.zeros(pop, dtype=torch.int32, device=dev)
+    d_fit = torch.zeros(pairs, dtype=torch.int32, device=dev)
+    ctx.population_forward(d_data.data_ptr(), len(data), start, seed, 0, pop, d_loss.data_ptr())
+    ctx.fitness(d_loss.data_ptr(), d_fit.data_ptr(), pairs)
+    ctx.sync()
+    loss = d_loss.cpu().numpy()
+    fit = d_fit.cpu().numpy()
+    assert np.array_equal(fit, np.sign(loss[1::2].astype(np.int64) - loss[0::2]).astype(np.int32))
+    assert np.array_equal(fit, orc.fitness(loss))
+    assert np.count_nonzero(fit) > pairs // 2, "degenerate fitness"
+    for first in (0, 20478, 40958):
+        ref = orc.population_forward(ocfg, model, data, start, seed, first, 2)
+        assert np.array_equal(loss[first:first + 2], ref[first:first + 2]), first
+
+    d_seed = _t(dev, np.array([seed], np.uint32).view(np.int32))
+    d_lr = _t(dev, np.array([lr], np.float32))
+    tensors = {t["name"]: t for t in ctx.tensors()}
+    checked = [tensors["w_q.1"], tensors["embedding"], tensors["ln_2.3"]]
+    # votes of two matrices over all 20,480 pairs; negating every fitness negates every vote
+    d_neg = -d_fit
+    for t in checked[:2]:
+        n = t["rows"] * t["cols"]
+        d_votes = torch.zeros(n, dtype=torch.int32, device=dev)
+        d_votes_neg = torch.zeros(n, dtype=torch.int32, device=dev)
+        ctx.matrix_votes(t["id"], d_fit.data_ptr(), d_seed.data_ptr(), d_votes.data_ptr())
+        ctx.matrix_votes(t["id"], d_neg.data_ptr(), d_seed.data_ptr(), d_votes_neg.data_ptr())
+        ctx.sync()
+        ref = np.zeros(n, np.int32)
+        orc.lib().orc_matrix_votes(C.byref(ocfg), t["rows"], t["cols"], t["off_a"], t["off_b"], t["seed_base"],
+                                   fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed), ref.ctypes.data_as(C.c_void_p))
+        assert np.array_equal(d_votes.cpu().numpy(), ref), t["name"]
+        assert torch.equal(d_votes_neg, -d_votes), t["name"]
+
+    # the whole update; the sampled tensors against the oracle's per-tensor update
+    ctx.es_update(d_fit.data_ptr(), d_seed.data_ptr(), d_lr.data_ptr())
+    got_m = ctx.model_download()
+    got_s = ctx.opt_state_download().view(orc.ADAM_DTYPE)
+    assert ctx.last_update_count() == np.count_nonzero(got_m != model)
+    for t in checked:
+        n = t["rows"] * t["cols"]
+        w = model[t["offset"]:t["offset"] + n].copy()
+        st = np.zeros(n, orc.ADAM_DTYPE)
+        if t["is_matrix"]:
+            orc.lib().orc_update_matrix_adam(C.byref(ocfg), w.ctypes.data_as(C.c_void_p), st.ctypes.data_as(C.c_void_p),
+                                             t["rows"], t["cols"], t["off_a"], t["off_b"], t["seed_base"],
+                                             fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed),
+                                             C.c_float(lr * t["lr_scale"]))
+        else:
+            orc.lib().orc_update_vector_adam(C.byref(ocfg), w.ctypes.data_as(C.c_void_p), st.ctypes.data_as(C.c_void_p),
+                                             n, t["off_a"], t["off_b"], t["seed_base"],
+                                             fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed),
+                                             C.c_float(lr * t["lr_scale"]))
+        sl = slice(t["offset"], t["offset"] + n)
+        assert np.array_equal(got_m[sl], w), t["name"]
+        for f in ("m", "v", "acc"):
+            assert np.array_equal(got_s[f][sl].view(np.int32), st[f].view(np.int32)), (t["name"], f)
+    ctx.close()
+
+    # the same step through the one-call entry point on a fresh context ends in the same weights
+    ctx2 = pkg.Context(pkg.default_config(**kw))
+    ctx2.model_upload(model)
+    ctx2.step(d_data.data_ptr(), len(data), start, seed, lr)
+    ctx2.sync()
+    assert np.array_equal(ctx2.model_download(), got_m)
+    ctx2.close()
