@@ -227,19 +227,57 @@ static inline int8_t blk(const int8_t *Wb, int cols, int k, int n) {   /* logica
     return Wb[(((int64_t)(k >> 2) * cols) + n) * 4 + (k & 3)];
 }
 
-/* mgpu.cu:553-572: dp4a accumulation over the packed input, then the rank-1 term */
+/* d-eggs adaptive noise overlay, de/include/model/layers.cuh:12-53 (ADAPTIVE_NOISE_MODE 1, the default of
+ * de/include/config.h:229-231): the int8 overlay value of a row / column / vector element becomes a float factor
+ * that multiplies the noise before it is truncated to an integer.  A null overlay pointer is the reference without
+ * the overlay (factor 1).  The overlay blob has the layout of the model blob: a vector tensor's values sit at the
+ * tensor's offset; a matrix has its `rows` input-dimension values at its offset and its `cols` output-dimension
+ * values right behind them. */
+extern "C" float orc_adaptive_factor(int ov) {
+    if (ov < 0) return 0.0f;
+    if (ov < 64) return (float)ov / 64.0f;
+    return 1.0f;
+}
+static inline float afac(const int8_t *sc, int64_t i) { return sc ? orc_adaptive_factor(sc[i]) : 1.0f; }
+/* the overlay values that belong to the tensor stored at `tensor` inside the blob starting at `model` */
+static inline const int8_t *sc_of(const int8_t *sc, const int8_t *model, const int8_t *tensor) {
+    return sc ? sc + (tensor - model) : NULL;
+}
+
+/* mgpu.cu:553-572: dp4a accumulation over the packed input, then the rank-1 term; with the overlay the noise is
+ * scaled by the output column's factor and truncated, de/include/model/layers.cuh:76-97 */
 static int32_t linear_proj(const orc_config *c, const int8_t *in, const int8_t *Wb, int K, int N, int n,
-                           int32_t sb, uint32_t noise_seed, int ns) {
+                           int32_t sb, uint32_t noise_seed, int ns, const int8_t *sc_col = NULL) {
     int32_t acc = 0;
     for (int k = 0; k < K; k++) acc += (int32_t)in[k] * (int32_t)blk(Wb, N, k, n);
-    if (ns != 0) acc += ((sb * (int32_t)orc_noise(noise_seed, (uint32_t)n, c->noise_mask)) * ns) >> (c->fixed_point + c->sigma_shift);
+    if (ns != 0) {
+        int8_t nz = orc_noise(noise_seed, (uint32_t)n, c->noise_mask);
+        int32_t a = sc_col ? (int32_t)(nz * afac(sc_col, n)) : (int32_t)nz;
+        acc += ((sb * a) * ns) >> (c->fixed_point + c->sigma_shift);
+    }
     return acc;
+}
+/* x . B with the input-dimension factors: each term is converted to int after the float multiply, as the argument
+ * of the reference's block reduction is (de/include/model/layers.cuh:240, :340-342, :436) */
+static int32_t noise_dot(const orc_config *c, const int8_t *in, int K, uint32_t seed, const int8_t *sc_row) {
+    int32_t sb = 0;
+    for (int k = 0; k < K; k++) {
+        int32_t t = (int32_t)in[k] * orc_noise(seed, k, c->noise_mask);
+        sb += sc_row ? (int32_t)(t * afac(sc_row, k)) : t;
+    }
+    return sb;
 }
 
 /* mgpu.cu:646-678 */
-extern "C" void orc_standard_norm(const orc_config *c, const int8_t *x, const int8_t *w, const int8_t *b, int H,
-                                  uint32_t seed_base, int off_w_a, int off_w_b, int off_b_a, int off_b_b,
-                                  int ns, int8_t *out) {
+/* the two input-side sums of an MLP block under the overlay, exported so that tests can pin them in isolation */
+extern "C" int32_t orc_noise_dot_adaptive(const orc_config *c, const int8_t *in, int K, uint32_t seed, const int8_t *overlay_rows) {
+    return noise_dot(c, in, K, seed, overlay_rows);
+}
+extern "C" int32_t orc_scaled_noise(int noise, int overlay_value) { return (int32_t)((int8_t)noise * orc_adaptive_factor(overlay_value)); }
+
+static void standard_norm(const orc_config *c, const int8_t *x, const int8_t *w, const int8_t *b, int H,
+                          uint32_t seed_base, int off_w_a, int off_w_b, int off_b_a, int off_b_b,
+                          int ns, int8_t *out, const int8_t *sc_w, const int8_t *sc_b) {
     int32_t tot = 0;
     for (int i = 0; i < H; i++) tot += abs((int32_t)x[i]);
     int32_t mn = tot / H; if (!mn) mn = 1;
@@ -249,14 +287,22 @@ extern "C" void orc_standard_norm(const orc_config *c, const int8_t *x, const in
         if (ns != 0) {
             int8_t wn1 = orc_noise(seed_base + off_w_a, tid, c->noise_mask);
             int8_t wn2 = orc_noise(seed_base + off_w_b, tid, c->noise_mask);
-            w_mod += ((int32_t)wn1 * wn2 * ns) >> c->sigma_shift_vector;
+            /* with the overlay: (AccumType)(wn1 * wn2 * scale_w), de/include/model/layers.cuh:171-183 */
+            int32_t wp = (int32_t)wn1 * wn2; if (sc_w) wp = (int32_t)(wp * afac(sc_w, tid));
+            w_mod += (wp * ns) >> c->sigma_shift_vector;
             int8_t bn1 = orc_noise(seed_base + off_b_a, tid, c->noise_mask);
             int8_t bn2 = orc_noise(seed_base + off_b_b, tid, c->noise_mask);
-            b_mod += ((int32_t)bn1 * bn2 * ns) >> c->sigma_shift_vector;
+            int32_t bp = (int32_t)bn1 * bn2; if (sc_b) bp = (int32_t)(bp * afac(sc_b, tid));
+            b_mod += (bp * ns) >> c->sigma_shift_vector;
         }
         res[tid] = orc_clip(((int32_t)x[tid] * w_mod) / mn + b_mod);
     }
     memcpy(out, res.data(), H);
+}
+extern "C" void orc_standard_norm(const orc_config *c, const int8_t *x, const int8_t *w, const int8_t *b, int H,
+                                  uint32_t seed_base, int off_w_a, int off_w_b, int off_b_a, int off_b_b,
+                                  int ns, int8_t *out) {
+    standard_norm(c, x, w, b, H, seed_base, off_w_a, off_w_b, off_b_a, off_b_b, ns, out, NULL, NULL);
 }
 
 /* norm.h:10-103 (both templates have the same body) */
@@ -343,28 +389,49 @@ static const MlpCfg CFG_LAYER = { OFF_LN_2_A, OFF_LN_2_B, OFF_LN_2_BIAS_A, OFF_L
     OFF_MLP_UP_A, OFF_MLP_UP_B, OFF_MLP_BIAS_UP_A, OFF_MLP_BIAS_UP_B,
     OFF_MLP_DOWN_A, OFF_MLP_DOWN_B, OFF_MLP_BIAS_DOWN_A, OFF_MLP_BIAS_DOWN_B };                   /* mgpu.cu:698-706 */
 
-/* mgpu.cu:708-759 */
+/* x . B of the down projection (depth 4H).  Under the overlay the reference thread of hidden unit tid adds its four
+ * terms into an int with `pb += int * int8 * float`, i.e. pb = (int)((float)pb + term) each time
+ * (de/include/model/layers.cuh:268-276); the threads' sums are then added as integers. */
+extern "C" int32_t orc_down_dot_adaptive(const orc_config *c, const int8_t *mlp, int H, uint32_t seed, const int8_t *overlay_rows) {
+    if (!overlay_rows) return noise_dot(c, mlp, 4 * H, seed, NULL);
+    int32_t sb = 0;
+    for (int tid = 0; tid < H; tid++) {
+        int32_t pb = 0;
+        for (int sub = 0; sub < 4; sub++) {
+            int k = tid + sub * H;
+            pb += (int32_t)mlp[k] * orc_noise(seed, k, c->noise_mask) * afac(overlay_rows, k);
+        }
+        sb += pb;
+    }
+    return sb;
+}
+
+/* mgpu.cu:708-759; overlay sites de/include/model/layers.cuh:215-296 */
 static void mlp_block(const orc_config *c, const int8_t *act_lut, int8_t *x,
                       const int8_t *ln_w, const int8_t *ln_b, const int8_t *up_w, const int8_t *up_b,
-                      const int8_t *dn_w, const int8_t *dn_b, uint32_t seed_base, int ns, const MlpCfg &cfg) {
+                      const int8_t *dn_w, const int8_t *dn_b, uint32_t seed_base, int ns, const MlpCfg &cfg,
+                      const int8_t *model = NULL, const int8_t *sc = NULL) {
     int H = c->hidden, H4 = 4 * H, M = c->noise_mask;
+    const int8_t *s_lnw = sc_of(sc, model, ln_w), *s_lnb = sc_of(sc, model, ln_b);
+    const int8_t *s_up = sc_of(sc, model, up_w), *s_bup = sc_of(sc, model, up_b);     /* up: rows H then cols 4H */
+    const int8_t *s_dn = sc_of(sc, model, dn_w), *s_bdn = sc_of(sc, model, dn_b);     /* down: rows 4H then cols H */
     std::vector<int8_t> nrm(H), mlp(H4);
-    orc_standard_norm(c, x, ln_w, ln_b, H, seed_base, cfg.ln_a, cfg.ln_b, cfg.lnb_a, cfg.lnb_b, ns, nrm.data());
-    int32_t sb = 0;
-    for (int k = 0; k < H; k++) sb += (int32_t)nrm[k] * orc_noise(seed_base + cfg.up_b, k, M);
+    standard_norm(c, x, ln_w, ln_b, H, seed_base, cfg.ln_a, cfg.ln_b, cfg.lnb_a, cfg.lnb_b, ns, nrm.data(), s_lnw, s_lnb);
+    int32_t sb = noise_dot(c, nrm.data(), H, seed_base + cfg.up_b, s_up);
     for (int o = 0; o < H4; o++) {
-        int32_t a = linear_proj(c, nrm.data(), up_w, H, H4, o, sb, seed_base + cfg.up_a, ns);
+        int32_t a = linear_proj(c, nrm.data(), up_w, H, H4, o, sb, seed_base + cfg.up_a, ns, s_up ? s_up + H : NULL);
         int8_t nb1 = orc_noise(seed_base + cfg.bup_a, o, M), nb2 = orc_noise(seed_base + cfg.bup_b, o, M);
-        int32_t nv = ((int32_t)nb1 * nb2 * ns) >> c->sigma_shift_vector;
+        int32_t np = (int32_t)nb1 * nb2; if (s_bup) np = (int32_t)(np * afac(s_bup, o));
+        int32_t nv = (np * ns) >> c->sigma_shift_vector;
         mlp[o] = act_lut[(uint8_t)orc_clip((a >> c->shift_mlp_up) + up_b[o] + nv)];
     }
-    sb = 0;
-    for (int k = 0; k < H4; k++) sb += (int32_t)mlp[k] * orc_noise(seed_base + cfg.dn_b, k, M);
+    sb = orc_down_dot_adaptive(c, mlp.data(), H, seed_base + cfg.dn_b, s_dn);
     std::vector<int32_t> pre(H);
     for (int tid = 0; tid < H; tid++) {
-        int32_t adn = linear_proj(c, mlp.data(), dn_w, H4, H, tid, sb, seed_base + cfg.dn_a, ns);
+        int32_t adn = linear_proj(c, mlp.data(), dn_w, H4, H, tid, sb, seed_base + cfg.dn_a, ns, s_dn ? s_dn + H4 : NULL);
         int8_t n1 = orc_noise(seed_base + cfg.bdn_a, tid, M), n2 = orc_noise(seed_base + cfg.bdn_b, tid, M);
-        int32_t nv = ((int32_t)n1 * n2 * ns) >> c->sigma_shift_vector;
+        int32_t np = (int32_t)n1 * n2; if (s_bdn) np = (int32_t)(np * afac(s_bdn, tid));
+        int32_t nv = (np * ns) >> c->sigma_shift_vector;
         pre[tid] = (int32_t)x[tid] + (adn >> c->shift_mlp_down) + dn_b[tid] + nv;
     }
     orc_adaptive_normalize(pre.data(), H, x);
@@ -380,7 +447,8 @@ static Tables make_tables(const orc_config *c) {
 /* mgpu.cu:847-1029 (one block == one member) */
 static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_t *model,
                               const uint8_t *data, int64_t data_len, int64_t start_idx,
-                              uint32_t step_seed, int p_idx, int ns_override, orc_trace *tr) {
+                              uint32_t step_seed, int p_idx, int ns_override, orc_trace *tr,
+                              const int8_t *sc = NULL) {
     const int H = c->hidden, V = c->vocab, T = c->seq_len, NL = c->n_layers, M = c->noise_mask;
     Layout L = make_layout(c);
     int64_t pair_idx = p_idx / 2;
@@ -403,16 +471,21 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
             int8_t emb = blk(model + L.embedding, V, tid, tok);
             int8_t ebias = model[L.emb_bias + tid];
             int8_t n1 = orc_noise(pair_seed + OFF_EMB_BIAS_A, tid, M), n2 = orc_noise(pair_seed + OFF_EMB_BIAS_B, tid, M);
-            int32_t chk = ((int32_t)n1 * n2 * ns) >> c->sigma_shift_vector;
+            /* overlay: de/src/kernels.cu:139-158; the embedding is a matrix [H rows][V cols] in the blob, so its
+             * per-hidden values come first and its per-token values follow */
+            int32_t cp = (int32_t)n1 * n2; if (sc) cp = (int32_t)(cp * afac(sc + L.emb_bias, tid));
+            int32_t chk = (cp * ns) >> c->sigma_shift_vector;
             int8_t a_tok = orc_noise(seed_emb, tok, M), b_dim = orc_noise(seed_emb + H, tid, M);
-            int32_t perturb = ((int32_t)a_tok * b_dim * ns) >> sigma;
+            int32_t pp = (int32_t)a_tok * b_dim;
+            if (sc) pp = (int32_t)(pp * afac(sc + L.embedding + H, tok) * afac(sc + L.embedding, tid));
+            int32_t perturb = (pp * ns) >> sigma;
             x[tid] = orc_clip((int32_t)emb + ebias + chk + perturb);
         }
         if (tr && tr->x_emb) memcpy(tr->x_emb + (size_t)t * H, x.data(), H);
 
         mlp_block(c, tb.act.data(), x.data(), model + L.ln_init, model + L.ln_init_bias,
                   model + L.w_emb_mlp_up, model + L.mlp_emb_bias_up, model + L.w_emb_mlp_down,
-                  model + L.mlp_emb_bias_down, pair_seed, ns, CFG_INIT);
+                  model + L.mlp_emb_bias_down, pair_seed, ns, CFG_INIT, model, sc);
         if (tr && tr->x_init) memcpy(tr->x_init + (size_t)t * H, x.data(), H);
 
         /* 2. layer stack, mgpu.cu:937-952 */
@@ -422,18 +495,18 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
             const int8_t *wq = model + L.w_q + (int64_t)l * H * H, *wk = model + L.w_k + (int64_t)l * H * H;
             const int8_t *wv = model + L.w_v + (int64_t)l * H * H, *wo = model + L.w_o + (int64_t)l * H * H;
             /* attention, mgpu.cu:761-833 */
-            orc_standard_norm(c, x.data(), model + L.ln_1 + (int64_t)l * H, model + L.ln_1_bias + (int64_t)l * H, H,
-                              sbase, OFF_LN_1_A, OFF_LN_1_B, OFF_LN_1_BIAS_A, OFF_LN_1_BIAS_B, ns, nrm.data());
-            int32_t sbq = 0, sbk = 0, sbv = 0;
-            for (int k = 0; k < H; k++) {
-                sbq += (int32_t)nrm[k] * orc_noise(sbase + OFF_Q_B, k, M);
-                sbk += (int32_t)nrm[k] * orc_noise(sbase + OFF_K_B, k, M);
-                sbv += (int32_t)nrm[k] * orc_noise(sbase + OFF_V_B, k, M);
-            }
+            /* overlay sites of the attention block: de/include/model/layers.cuh:313-351, :432-438 */
+            const int8_t *s_q = sc_of(sc, model, wq), *s_k = sc_of(sc, model, wk), *s_v = sc_of(sc, model, wv), *s_o = sc_of(sc, model, wo);
+            standard_norm(c, x.data(), model + L.ln_1 + (int64_t)l * H, model + L.ln_1_bias + (int64_t)l * H, H,
+                          sbase, OFF_LN_1_A, OFF_LN_1_B, OFF_LN_1_BIAS_A, OFF_LN_1_BIAS_B, ns, nrm.data(),
+                          sc ? sc + L.ln_1 + (int64_t)l * H : NULL, sc ? sc + L.ln_1_bias + (int64_t)l * H : NULL);
+            int32_t sbq = noise_dot(c, nrm.data(), H, sbase + OFF_Q_B, s_q);
+            int32_t sbk = noise_dot(c, nrm.data(), H, sbase + OFF_K_B, s_k);
+            int32_t sbv = noise_dot(c, nrm.data(), H, sbase + OFF_V_B, s_v);
             for (int tid = 0; tid < H; tid++) {
-                aq[tid] = linear_proj(c, nrm.data(), wq, H, H, tid, sbq, sbase + OFF_Q_A, ns);
-                ak[tid] = linear_proj(c, nrm.data(), wk, H, H, tid, sbk, sbase + OFF_K_A, ns);
-                av[tid] = linear_proj(c, nrm.data(), wv, H, H, tid, sbv, sbase + OFF_V_A, ns);
+                aq[tid] = linear_proj(c, nrm.data(), wq, H, H, tid, sbq, sbase + OFF_Q_A, ns, s_q ? s_q + H : NULL);
+                ak[tid] = linear_proj(c, nrm.data(), wk, H, H, tid, sbk, sbase + OFF_K_A, ns, s_k ? s_k + H : NULL);
+                av[tid] = linear_proj(c, nrm.data(), wv, H, H, tid, sbv, sbase + OFF_V_A, ns, s_v ? s_v + H : NULL);
             }
             orc_rope(c, tb.rope.data(), aq.data(), t, H, tmp.data());
             orc_adaptive_normalize(tmp.data(), H, qv.data());
@@ -447,10 +520,9 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
             orc_attention_core(c, tb.exp_lut.data(), qv.data(), lk, lv, t, H, ao.data());
             if (tr && tr->ao) memcpy(tr->ao + ((size_t)l * T + t) * H, ao.data(), H);
 
-            int32_t sb = 0;
-            for (int k = 0; k < H; k++) sb += (int32_t)ao[k] * orc_noise(sbase + OFF_O_B, k, M);
+            int32_t sb = noise_dot(c, ao.data(), H, sbase + OFF_O_B, s_o);
             for (int tid = 0; tid < H; tid++) {
-                int32_t aco = linear_proj(c, ao.data(), wo, H, H, tid, sb, sbase + OFF_O_A, ns);
+                int32_t aco = linear_proj(c, ao.data(), wo, H, H, tid, sb, sbase + OFF_O_A, ns, s_o ? s_o + H : NULL);
                 tmp[tid] = (int32_t)x[tid] + (aco >> c->shift_out);
             }
             orc_adaptive_normalize(tmp.data(), H, x.data());
@@ -459,18 +531,21 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
             mlp_block(c, tb.act.data(), x.data(), model + L.ln_2 + (int64_t)l * H, model + L.ln_2_bias + (int64_t)l * H,
                       model + L.w_up + (int64_t)l * H * 4 * H, model + L.mlp_bias_up + (int64_t)l * 4 * H,
                       model + L.w_down + (int64_t)l * 4 * H * H, model + L.mlp_bias_down + (int64_t)l * H,
-                      sbase, ns, CFG_LAYER);
+                      sbase, ns, CFG_LAYER, model, sc);
             if (tr && tr->x_mlp) memcpy(tr->x_mlp + ((size_t)l * T + t) * H, x.data(), H);
         }
 
         /* 3. head + loss, mgpu.cu:955-1024 */
-        orc_standard_norm(c, x.data(), model + L.ln_f, model + L.ln_f_bias, H, pair_seed,
-                          OFF_LN_F_A, OFF_LN_F_B, OFF_LN_F_BIAS_A, OFF_LN_F_BIAS_B, ns, nf.data());
+        /* overlay: the tied head takes the embedding's per-hidden values on its input side and the per-token values
+         * on its output side, de/src/kernels.cu:200-240 */
+        standard_norm(c, x.data(), model + L.ln_f, model + L.ln_f_bias, H, pair_seed,
+                      OFF_LN_F_A, OFF_LN_F_B, OFF_LN_F_BIAS_A, OFF_LN_F_BIAS_B, ns, nf.data(),
+                      sc ? sc + L.ln_f : NULL, sc ? sc + L.ln_f_bias : NULL);
         if (tr && tr->nf) memcpy(tr->nf + (size_t)t * H, nf.data(), H);
-        int32_t sbh = 0;
-        for (int k = 0; k < H; k++) sbh += (int32_t)nf[k] * orc_noise(pair_seed + OFF_EMB + H, k, M);
+        int32_t sbh = noise_dot(c, nf.data(), H, pair_seed + OFF_EMB + H, sc ? sc + L.embedding : NULL);
         for (int v = 0; v < V; v++) {
-            int32_t ah = linear_proj(c, nf.data(), model + L.embedding, H, V, v, sbh, pair_seed + OFF_EMB, ns);
+            int32_t ah = linear_proj(c, nf.data(), model + L.embedding, H, V, v, sbh, pair_seed + OFF_EMB, ns,
+                                     sc ? sc + L.embedding + H : NULL);
             logits[v] = ah >> c->shift_logit;
         }
         if (tr && tr->logits) memcpy(tr->logits + (size_t)t * V, logits.data(), sizeof(int32_t) * V);
@@ -486,6 +561,24 @@ extern "C" int32_t orc_forward_member(const orc_config *c, const int8_t *model, 
                                       int64_t start_idx, uint32_t step_seed, int p_idx, int ns_override, orc_trace *trace) {
     Tables tb = make_tables(c);
     return forward_member(c, tb, model, data, data_len, start_idx, step_seed, p_idx, ns_override, trace);
+}
+
+extern "C" int32_t orc_forward_member_adaptive(const orc_config *c, const int8_t *model, const int8_t *overlay,
+                                               const uint8_t *data, int64_t data_len, int64_t start_idx,
+                                               uint32_t step_seed, int p_idx, int ns_override, orc_trace *trace) {
+    Tables tb = make_tables(c);
+    return forward_member(c, tb, model, data, data_len, start_idx, step_seed, p_idx, ns_override, trace, overlay);
+}
+extern "C" void orc_population_forward_adaptive(const orc_config *c, const int8_t *model, const int8_t *overlay,
+                                                const uint8_t *data, int64_t data_len, int64_t start_idx,
+                                                uint32_t step_seed, int pop_offset, int count, int32_t *loss) {
+    Tables tb = make_tables(c);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int i = 0; i < count; i++) {
+        int p = pop_offset + i;
+        if (p >= c->population) continue;
+        loss[p] = forward_member(c, tb, model, data, data_len, start_idx, step_seed, p, 2, NULL, overlay);
+    }
 }
 
 extern "C" void orc_population_forward(const orc_config *c, const int8_t *model, const uint8_t *data, int64_t data_len,
@@ -612,6 +705,44 @@ extern "C" uint64_t orc_es_update_adam(const orc_config *c, int8_t *model, orc_a
                                                          t.seed_base, fit, pairs, step_seed, lr * t.lr_scale);
         else total += orc_update_vector_adam(c, model + t.offset, state + t.offset, t.cols, t.off_a, t.off_b,
                                              t.seed_base, fit, pairs, step_seed, lr * t.lr_scale);
+    }
+    return total;
+}
+
+/* de/src/kernels.cu:61-77: an element whose row / column / vector entry saw at least one weight change this step
+ * gains `inc`, every other one loses `dec`, clamped to [-127, 127] (de/include/config.h:57-58) */
+extern "C" void orc_update_overlay(const int32_t *changes, int8_t *overlay, int count, int inc, int dec) {
+    for (int i = 0; i < count; i++) {
+        int ov = overlay[i];
+        if (changes[i] > 0) { ov += inc; if (ov > 127) ov = 127; }
+        else { ov -= dec; if (ov < -127) ov = -127; }
+        overlay[i] = (int8_t)ov;
+    }
+}
+
+/* The d-eggs optimizer step (de/src/worker.cu:446-523): the AdamW update of every tensor, with the weight changes
+ * counted per input row and per output column of a matrix (de/include/optimizer/adam.cuh:77-83; the embedding's
+ * counts go to its per-hidden and per-token values, de/src/worker.cu:497-516) or per element of a vector
+ * (adam.cuh:130-132), followed by the overlay rule for that tensor.  The votes do not use the overlay
+ * (adam.cuh:60-67).  A weight byte differs from its old value exactly when the reference sets `change`. */
+extern "C" uint64_t orc_es_update_adam_adaptive(const orc_config *c, int8_t *model, orc_adam_param *state, int8_t *overlay,
+                                                const int32_t *fit, uint32_t step_seed, float lr, int inc, int dec) {
+    std::vector<int8_t> before(model, model + make_layout(c).total);
+    uint64_t total = orc_es_update_adam(c, model, state, fit, step_seed, lr);
+    for (const orc_tensor &t : tensor_table(c)) {
+        if (t.is_matrix) {
+            std::vector<int32_t> cnt((size_t)t.rows + t.cols, 0);
+            for (int64_t idx = 0; idx < (int64_t)t.rows * t.cols; idx++) {
+                if (model[t.offset + idx] == before[t.offset + idx]) continue;
+                int byte_off = idx & 3; int64_t word = idx >> 2; int tid = (int)(word % t.cols); int k = (int)(word / t.cols) * 4 + byte_off;
+                cnt[k]++; cnt[t.rows + tid]++;
+            }
+            orc_update_overlay(cnt.data(), overlay + t.offset, t.rows + t.cols, inc, dec);
+        } else {
+            std::vector<int32_t> cnt((size_t)t.cols, 0);
+            for (int i = 0; i < t.cols; i++) cnt[i] = model[t.offset + i] != before[t.offset + i];
+            orc_update_overlay(cnt.data(), overlay + t.offset, t.cols, inc, dec);
+        }
     }
     return total;
 }

@@ -115,6 +115,22 @@ void orc_population_forward(const orc_config *c, const int8_t *model,
                             const uint8_t *data, int64_t data_len, int64_t start_idx,
                             uint32_t step_seed, int pop_offset, int count, int32_t *loss);
 
+/* d-eggs adaptive noise overlay (de/include/model/layers.cuh:12-53, mode 1; sites :94, :177, :240-296, :332-438,
+ * de/src/kernels.cu:139-240).  `overlay` has the layout of the model blob: a vector tensor's values at the tensor's
+ * offset, a matrix's `rows` input-dimension values at its offset followed by its `cols` output-dimension values.
+ * Parity unpinned beyond the special cases in the tests: the reference has no test or fixture for it and its
+ * CUDA sources cannot be built here. */
+float   orc_adaptive_factor(int overlay_value);
+int32_t orc_scaled_noise(int noise, int overlay_value);          /* (int)(noise * factor), layers.cuh:94 */
+int32_t orc_noise_dot_adaptive(const orc_config *c, const int8_t *in, int K, uint32_t seed, const int8_t *overlay_rows);
+int32_t orc_down_dot_adaptive(const orc_config *c, const int8_t *mlp, int H, uint32_t seed, const int8_t *overlay_rows); /* layers.cuh:268-276 */
+int32_t orc_forward_member_adaptive(const orc_config *c, const int8_t *model, const int8_t *overlay,
+                                    const uint8_t *data, int64_t data_len, int64_t start_idx,
+                                    uint32_t step_seed, int p_idx, int ns_override, orc_trace *trace);
+void    orc_population_forward_adaptive(const orc_config *c, const int8_t *model, const int8_t *overlay,
+                                        const uint8_t *data, int64_t data_len, int64_t start_idx,
+                                        uint32_t step_seed, int pop_offset, int count, int32_t *loss);
+
 /* perturbed linear microbench semantics: rows = members*T, member = row / T,
  * pair = member/2, ns = +1 even / -1 odd member;
  * acc = X.W + (((X.B) * A[n]) * ns >> (fixed_point+sigma_shift)); Y = acc >> shift  (mgpu.cu:553-572) */
@@ -154,6 +170,10 @@ uint64_t orc_update_vector_adam(const orc_config *c, int8_t *V, orc_adam_param *
 uint64_t orc_es_update_adam(const orc_config *c, int8_t *model, orc_adam_param *state,
                             const int32_t *fit, uint32_t step_seed, float lr);
 float orc_learning_rate(long step);   /* mgpu.cu:217-227 */
+/* d-eggs overlay rule and the optimizer step that feeds it (de/src/kernels.cu:61-77, de/src/worker.cu:446-523) */
+void     orc_update_overlay(const int32_t *changes, int8_t *overlay, int count, int inc, int dec);
+uint64_t orc_es_update_adam_adaptive(const orc_config *c, int8_t *model, orc_adam_param *state, int8_t *overlay,
+                                     const int32_t *fit, uint32_t step_seed, float lr, int inc, int dec);
 
 /* ---- Muon (muon_i:15-342, launch macro mgpu.cu:1587-1595) ---- */
 /* fp32 restatement with sequential-k summation; X row-major [rows][cols], in place */

@@ -98,6 +98,23 @@ def lib():
                                              C.c_void_p, C.c_int, C.c_uint32, C.c_float]
         L.orc_es_update_adam.restype = C.c_uint64
         L.orc_es_update_adam.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_float]
+        L.orc_scaled_noise.restype = C.c_int32
+        L.orc_scaled_noise.argtypes = [C.c_int, C.c_int]
+        L.orc_noise_dot_adaptive.restype = C.c_int32
+        L.orc_noise_dot_adaptive.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint32, C.c_void_p]
+        L.orc_down_dot_adaptive.restype = C.c_int32
+        L.orc_down_dot_adaptive.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint32, C.c_void_p]
+        L.orc_adaptive_factor.restype = C.c_float
+        L.orc_adaptive_factor.argtypes = [C.c_int]
+        L.orc_forward_member_adaptive.restype = C.c_int32
+        L.orc_forward_member_adaptive.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                                  C.c_uint32, C.c_int, C.c_int, C.c_void_p]
+        L.orc_population_forward_adaptive.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                                      C.c_int64, C.c_uint32, C.c_int, C.c_int, C.c_void_p]
+        L.orc_update_overlay.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int]
+        L.orc_es_update_adam_adaptive.restype = C.c_uint64
+        L.orc_es_update_adam_adaptive.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                  C.c_uint32, C.c_float, C.c_int, C.c_int]
         L.orc_learning_rate.restype = C.c_float
         L.orc_learning_rate.argtypes = [C.c_long]
         L.orc_newton_schulz_f32.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int]
@@ -212,7 +229,7 @@ def noise_vec(seed, n, mask=15, first=0):
     return np.array([L.orc_noise(C.c_uint32(seed & 0xFFFFFFFF), C.c_uint32(first + i), mask) for i in range(n)], np.int8)
 
 
-def forward_member(cfg, model, data, start_idx, step_seed, p_idx, ns_override=2, trace=False):
+def forward_member(cfg, model, data, start_idx, step_seed, p_idx, ns_override=2, trace=False, overlay=None):
     T, H, NL, V = cfg.seq_len, cfg.hidden, cfg.n_layers, cfg.vocab
     tr = None
     bufs = {}
@@ -227,9 +244,13 @@ def forward_member(cfg, model, data, start_idx, step_seed, p_idx, ns_override=2,
         tr.logits = bufs["logits"].ctypes.data
         bufs["loss_t"] = np.zeros(T, np.int64)
         tr.loss_t = bufs["loss_t"].ctypes.data
-    loss = lib().orc_forward_member(C.byref(cfg), _p(model), _p(data), len(data), start_idx,
-                                    C.c_uint32(step_seed & 0xFFFFFFFF), p_idx, ns_override,
-                                    C.byref(tr) if tr is not None else None)
+    trp = C.byref(tr) if tr is not None else None
+    if overlay is None:
+        loss = lib().orc_forward_member(C.byref(cfg), _p(model), _p(data), len(data), start_idx,
+                                        C.c_uint32(step_seed & 0xFFFFFFFF), p_idx, ns_override, trp)
+    else:
+        loss = lib().orc_forward_member_adaptive(C.byref(cfg), _p(model), _p(overlay), _p(data), len(data), start_idx,
+                                                 C.c_uint32(step_seed & 0xFFFFFFFF), p_idx, ns_override, trp)
     return (loss, bufs) if trace else loss
 
 
@@ -270,11 +291,15 @@ def generate(cfg, model, prompt, gen_len, seed):
     return buf[:seed_len + gen_len].copy()
 
 
-def population_forward(cfg, model, data, start_idx, step_seed, pop_offset=0, count=None):
+def population_forward(cfg, model, data, start_idx, step_seed, pop_offset=0, count=None, overlay=None):
     count = cfg.population if count is None else count
     loss = np.zeros(cfg.population, np.int32)
-    lib().orc_population_forward(C.byref(cfg), _p(model), _p(data), len(data), start_idx,
-                                 C.c_uint32(step_seed & 0xFFFFFFFF), pop_offset, count, _p(loss))
+    if overlay is None:
+        lib().orc_population_forward(C.byref(cfg), _p(model), _p(data), len(data), start_idx,
+                                     C.c_uint32(step_seed & 0xFFFFFFFF), pop_offset, count, _p(loss))
+    else:
+        lib().orc_population_forward_adaptive(C.byref(cfg), _p(model), _p(overlay), _p(data), len(data), start_idx,
+                                              C.c_uint32(step_seed & 0xFFFFFFFF), pop_offset, count, _p(loss))
     return loss
 
 
@@ -301,6 +326,12 @@ def es_update_adam(cfg, model, state, fit, step_seed, lr):
     """in place on model (int8) and state (ADAM_DTYPE, one per model byte); returns update count"""
     return int(lib().orc_es_update_adam(C.byref(cfg), _p(model), _p(state), _p(fit),
                                         C.c_uint32(step_seed & 0xFFFFFFFF), C.c_float(lr)))
+
+
+def es_update_adam_adaptive(cfg, model, state, overlay, fit, step_seed, lr, inc=5, dec=1):
+    """d-eggs optimizer step: in place on model, state and the overlay blob (same layout as the model)"""
+    return int(lib().orc_es_update_adam_adaptive(C.byref(cfg), _p(model), _p(state), _p(overlay), _p(fit),
+                                                 C.c_uint32(step_seed & 0xFFFFFFFF), C.c_float(lr), inc, dec))
 
 
 def gru_init_model(gcfg, seed=42):

@@ -510,3 +510,109 @@ def test_sampling_closed_forms(orc):
     for t in range(50):
         rr = int(hash_rng(C.c_uint32((5 + t * 555) & 0xFFFFFFFF), C.c_uint32(0)))
         assert orc.sample_token(two, exp_lut, 5, t, 256) == (10 if rr % (w0 + w1) < w0 else 20)
+
+
+# ------------------------------------------------------------------ d-eggs adaptive noise overlay
+def test_adaptive_overlay_special_cases(orc):
+    """The overlay restatement has no reference fixture (parity unpinned); these are the cases arithmetic fixes:
+    factor values, truncation toward zero, overlay 64 == no overlay, overlay <= 0 == no noise, and the sequential
+    int += float accumulation of the down projection's input-side sum against exact rational arithmetic."""
+    from fractions import Fraction
+    L = orc.lib()
+    assert [L.orc_adaptive_factor(v) for v in (-127, -1, 0, 16, 32, 63, 64, 65, 127)] == \
+        [0.0, 0.0, 0.0, 0.25, 0.5, 63 / 64, 1.0, 1.0, 1.0]
+    # (int)(noise * factor): toward zero on both sides
+    assert [L.orc_scaled_noise(n, ov) for n, ov in ((-7, 32), (7, 32), (15, 63), (-15, 63), (5, 0), (5, -3), (-5, 100), (1, 63), (-1, 63))] == \
+        [-3, 3, 14, -14, 0, 0, -5, 0, 0]
+
+    kw = dict(hidden=64, head_dim=32, n_layers=2, seq_len=16, population=8)
+    cfg = orc.config(**kw)
+    model = orc.init_model(cfg, 42)
+    data = orc.zipf_bytes(1 << 12)
+    base = orc.population_forward(cfg, model, data, 0, 99)
+    assert np.array_equal(orc.population_forward(cfg, model, data, 0, 99, overlay=np.full(model.size, 64, np.int8)), base)
+    assert np.array_equal(orc.population_forward(cfg, model, data, 0, 99, overlay=np.full(model.size, 127, np.int8)), base)
+    quiet = orc.population_forward(cfg, model, data, 0, 99, overlay=np.full(model.size, 0, np.int8))
+    assert np.array_equal(quiet, orc.population_forward(orc.config(noise_mask=0, **kw), model, data, 0, 99))
+    assert np.array_equal(quiet[0::2], quiet[1::2])
+    rng = np.random.default_rng(5)
+    mixed = orc.population_forward(cfg, model, data, 0, 99, overlay=rng.integers(-20, 100, model.size).astype(np.int8))
+    assert not np.array_equal(mixed, base) and not np.array_equal(mixed, quiet)
+
+    # input-side sums: term-wise truncation for one term per reference thread ...
+    K, seed = 64, 777
+    x = rng.integers(-127, 128, K).astype(np.int8)
+    ov = rng.integers(-10, 80, K).astype(np.int8)
+    nz = np_noise(seed, np.arange(K))
+
+    def fac(v):
+        return Fraction(0) if v < 0 else (Fraction(int(v), 64) if v < 64 else Fraction(1))
+
+    def trunc(fr):
+        return int(fr) if fr >= 0 else -int(-fr)
+
+    want = sum(trunc(int(x[k]) * int(nz[k]) * fac(ov[k])) for k in range(K))
+    assert L.orc_noise_dot_adaptive(C.byref(cfg), P(x), K, C.c_uint32(seed), P(ov)) == want
+    assert L.orc_noise_dot_adaptive(C.byref(cfg), P(x), K, C.c_uint32(seed), None) == int((x.astype(np.int64) * nz).sum())
+    # ... and truncation of the running sum where a reference thread adds four terms (depth 4H)
+    H = 16
+    m = rng.integers(-127, 128, 4 * H).astype(np.int8)
+    ov4 = rng.integers(1, 64, 4 * H).astype(np.int8)         # all fractional
+    nz4 = np_noise(seed, np.arange(4 * H))
+    want, termwise = 0, 0
+    for tid in range(H):
+        pb = 0
+        for sub in range(4):
+            k = tid + sub * H
+            term = int(m[k]) * int(nz4[k]) * fac(ov4[k])
+            pb = trunc(pb + term)
+            termwise += trunc(term)
+        want += pb
+    got = L.orc_down_dot_adaptive(C.byref(orc.config(hidden=H, head_dim=16, n_layers=1, seq_len=16, population=2)), P(m), H,
+                                  C.c_uint32(seed), P(ov4))
+    assert got == want
+    assert want != termwise, "the case does not separate the two readings"
+
+
+def test_overlay_rule_and_adaptive_update(orc):
+    L = orc.lib()
+    changes = np.array([0, 1, 7, 0, 0, 3], np.int32)
+    ov = np.array([64, 64, 125, -127, 0, -127], np.int8)
+    L.orc_update_overlay(P(changes), P(ov), 6, 5, 1)
+    assert ov.tolist() == [63, 69, 127, -127, -1, -122]
+    # the optimizer step: same weights and state as the plain step; overlay entries move by +5 where the tensor's row /
+    # column / element changed and by -1 elsewhere
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=16)
+    cfg = orc.config(**kw)
+    rng = np.random.default_rng(3)
+    fit = rng.integers(-1, 2, 8).astype(np.int32)
+    m1 = orc.init_model(cfg, 42); s1 = np.zeros(m1.size, orc.ADAM_DTYPE)
+    m2 = m1.copy(); s2 = s1.copy()
+    for step in range(3):
+        n1 = orc.es_update_adam(cfg, m1, s1, fit, 100 + step, 5.0)
+    overlay = np.full(m2.size, 64, np.int8)
+    expect = overlay.astype(int)
+    for step in range(3):
+        prev = m2.copy()
+        n2 = orc.es_update_adam_adaptive(cfg, m2, s2, overlay, fit, 100 + step, 5.0)
+        changed = prev != m2
+        for t in orc.tensor_table(cfg):
+            o, r, c = t["offset"], t["rows"], t["cols"]
+            if t["is_matrix"]:
+                # blocked element index -> (input row k, output column n), mgpu.cu:1085-1089
+                idx = np.arange(r * c); k = (idx >> 2) // c * 4 + (idx & 3); n = (idx >> 2) % c
+                ch = changed[o:o + r * c]
+                row_hit = np.zeros(r, bool); col_hit = np.zeros(c, bool)
+                row_hit[k[ch]] = True; col_hit[n[ch]] = True
+                hit = np.concatenate([row_hit, col_hit])
+            else:
+                hit = changed[o:o + c]
+            seg = slice(o, o + len(hit))
+            expect[seg] = np.clip(np.where(hit, expect[seg] + 5, expect[seg] - 1), -127, 127)
+    assert n1 == n2 and np.array_equal(m1, m2) and np.array_equal(s1.view(np.uint8), s2.view(np.uint8))
+    used = np.zeros(m2.size, bool)
+    for t in orc.tensor_table(cfg):
+        used[t["offset"]:t["offset"] + (t["rows"] + t["cols"] if t["is_matrix"] else t["cols"])] = True
+    assert np.array_equal(overlay[used].astype(int), expect[used])
+    assert (overlay[~used] == 64).all(), "bytes of the blob that belong to no row / column / element are left alone"
+    assert (overlay[used] > 64).any() and (overlay[used] < 64).any()
