@@ -42,6 +42,7 @@ EXPORTS = [
     "egg_opt_state_upload", "egg_opt_state_download", "egg_opt_state_reset", "egg_tables_download",
     "egg_noise_fill", "egg_perturbed_linear", "egg_population_forward", "egg_population_forward_dev",
     "egg_fitness", "egg_es_update", "egg_update_tensor", "egg_matrix_votes",
+    "egg_adaptive_enable", "egg_overlay_upload", "egg_overlay_download",
     "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
     "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate",
     "egg_shape_fitness", "egg_ternary_pack_size", "egg_ternary_pack", "egg_ternary_unpack",
@@ -85,8 +86,10 @@ def lib():
         L.egg_model_bytes.restype = i64
         L.egg_model_bytes.argtypes = [vp]
         L.egg_model_init.argtypes = [vp, u32]
-        for f in (L.egg_model_upload, L.egg_model_download, L.egg_opt_state_upload, L.egg_opt_state_download):
+        for f in (L.egg_model_upload, L.egg_model_download, L.egg_opt_state_upload, L.egg_opt_state_download,
+                  L.egg_overlay_upload, L.egg_overlay_download):
             f.argtypes = [vp, vp, C.c_size_t]
+        L.egg_adaptive_enable.argtypes = [vp, i32, i32, i32]
         L.egg_opt_state_reset.argtypes = [vp]
         L.egg_tables_download.argtypes = [vp, vp, vp, vp]
         L.egg_noise_fill.argtypes = [vp, u32, u32, i32, vp]
@@ -252,6 +255,19 @@ class Context:
 
     def es_update(self, d_fit, d_seed, d_lr):
         self._ck(lib().egg_es_update(self._h, C.c_void_p(d_fit), C.c_void_p(d_seed), C.c_void_p(d_lr)), "egg_es_update")
+
+    def adaptive_enable(self, init_value=64, inc=5, dec=1):
+        """d-eggs adaptive noise overlay: on from this call (forward scaling and the overlay rule in es_update / step)"""
+        self._ck(lib().egg_adaptive_enable(self._h, init_value, inc, dec), "egg_adaptive_enable")
+
+    def overlay_upload(self, arr):
+        self._ck(lib().egg_overlay_upload(self._h, _np_ptr(arr), arr.nbytes), "egg_overlay_upload")
+
+    def overlay_download(self):
+        import numpy as np
+        out = np.zeros(self.model_bytes(), np.int8)
+        self._ck(lib().egg_overlay_download(self._h, _np_ptr(out), out.nbytes), "egg_overlay_download")
+        return out
 
     def update_tensor(self, tid, d_fit, d_seed, d_lr):
         self._ck(lib().egg_update_tensor(self._h, tid, C.c_void_p(d_fit), C.c_void_p(d_seed), C.c_void_p(d_lr)),

@@ -64,6 +64,11 @@ struct egg_ctx {
     uint8_t *d_gen_tok = nullptr; int32_t *d_gen_logits = nullptr; Scalars *d_gen_scal = nullptr;
     int mask_override = -1; int32_t *logits_override = nullptr;
     VecDesc *d_vec_desc = nullptr; int n_vec = 0, vec_total = 0;       // all vector tensors, for the one-launch update
+    // adaptive noise overlay (egg_adaptive_enable): raw overlay values, q = clamp(overlay, 0, 64) and change flags, all
+    // laid out like the model blob; one segment (rows + cols, or len) per tensor
+    bool adaptive = false; int ov_inc = 5, ov_dec = 1;
+    int8_t *d_overlay = nullptr, *d_overlay_q = nullptr, *d_flags = nullptr;
+    OvSeg *d_ov_segs = nullptr; int n_ov_segs = 0, ov_max_count = 0;
     // graph
     hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr; bool captured = false;
     std::string err;
@@ -154,7 +159,8 @@ static void free_all(egg_ctx *ctx) {
     void *ptrs[] = {ctx->muon.x, ctx->muon.swap, ctx->muon.bterm, ctx->muon.partials, ctx->muon.norm,
                     ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
-                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal, ctx->d_vec_desc};
+                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal, ctx->d_vec_desc,
+                    ctx->d_overlay, ctx->d_overlay_q, ctx->d_flags, ctx->d_ov_segs};
     for (void *p : ptrs) if (p) (void)hipFree(p);
     for (auto &sp : ctx->spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
     if (ctx->gexec) (void)hipGraphExecDestroy(ctx->gexec);
@@ -224,6 +230,7 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
             if (t.is_matrix) continue;
             VecDesc d; d.W = ctx->d_model + t.offset; d.state = reinterpret_cast<float *>(ctx->d_state + ctx->t_state_off[id]);
             d.n = t.cols; d.first = first; d.off_a = t.off_a; d.off_b = t.off_b; d.seed_base = t.seed_base; d.lr_scale = t.lr_scale;
+            d.flags = nullptr;
             vd.push_back(d); first += t.cols;
         }
         ctx->n_vec = (int)vd.size(); ctx->vec_total = first;
@@ -421,6 +428,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
                          int first_member, int nm) {
     const egg_config &c = ctx->cfg; const Layout &L = ctx->L; const int8_t *M = ctx->d_model; const int H = c.hidden;
     const int8_t *F = ctx->d_wfrag;
+    const int8_t *Q = ctx->adaptive ? ctx->d_overlay_q : nullptr;      // same offsets as the model blob
     hipStream_t s = ctx->stream;
     const bool taps = ctx->taps && nm <= ctx->tap_members;
     const size_t act_bytes = (size_t)nm * c.seq_len * H;
@@ -433,6 +441,10 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = F + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
         p.w_dn = F + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
         p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
+        if (Q) {
+            p.q_ln_w = Q + L.ln_init; p.q_ln_b = Q + L.ln_init_bias; p.q_b_up = Q + L.mlp_emb_bias_up; p.q_b_dn = Q + L.mlp_emb_bias_down;
+            p.q_up = Q + L.w_emb_mlp_up; p.q_dn = Q + L.w_emb_mlp_down; p.q_emb = Q + L.embedding; p.q_emb_bias = Q + L.emb_bias;
+        }
         span_begin(ctx, EGG_K_MLP_FIRST); HIP_TRY(egg_launch_mlp(p, true, s)); span_end(ctx);
         if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 0), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
     }
@@ -443,6 +455,10 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
             p.ln_w = M + L.ln_1 + (int64_t)l * H; p.ln_b = M + L.ln_1_bias + (int64_t)l * H;
             p.w_q = F + L.w_q + l * hh; p.w_k = F + L.w_k + l * hh; p.w_v = F + L.w_v + l * hh;
             p.x = ctx->d_x; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v;
+            if (Q) {
+                p.q_ln_w = Q + L.ln_1 + (int64_t)l * H; p.q_ln_b = Q + L.ln_1_bias + (int64_t)l * H;
+                p.q_wq = Q + L.w_q + l * hh; p.q_wk = Q + L.w_k + l * hh; p.q_wv = Q + L.w_v + l * hh;
+            }
             span_begin(ctx, EGG_K_QKV); HIP_TRY(egg_launch_qkv(p, s)); span_end(ctx);
             if (taps) {
                 HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 0), ctx->d_q, act_bytes, hipMemcpyDeviceToDevice, s));
@@ -465,6 +481,11 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
             p.w_dn = F + L.w_down + l * h4; p.b_dn = M + L.mlp_bias_down + (int64_t)l * H;
             p.w_o = F + L.w_o + l * hh; p.ao = ctx->d_ao; p.x = ctx->d_x;
             p.x_mid = taps ? tap_ptr(ctx, 1 + 6 * l + 4) : nullptr;
+            if (Q) {
+                p.q_ln_w = Q + L.ln_2 + (int64_t)l * H; p.q_ln_b = Q + L.ln_2_bias + (int64_t)l * H;
+                p.q_b_up = Q + L.mlp_bias_up + (int64_t)l * 4 * H; p.q_b_dn = Q + L.mlp_bias_down + (int64_t)l * H;
+                p.q_up = Q + L.w_up + l * h4; p.q_dn = Q + L.w_down + l * h4; p.q_o = Q + L.w_o + l * hh;
+            }
             span_begin(ctx, EGG_K_MLP); HIP_TRY(egg_launch_mlp(p, false, s)); span_end(ctx);
             if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 5), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
         }
@@ -473,6 +494,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         HeadParams p; memset(&p, 0, sizeof(p)); p.c = f;
         p.ln_w = M + L.ln_f; p.ln_b = M + L.ln_f_bias; p.embedding_frag = F + L.embedding; p.x = ctx->d_x;
         p.loss_acc = ctx->d_loss_acc; p.logits_tap = ctx->logits_override ? ctx->logits_override : (taps ? ctx->d_tap_logits : nullptr);
+        if (Q) { p.q_ln_w = Q + L.ln_f; p.q_ln_b = Q + L.ln_f_bias; p.q_emb = Q + L.embedding; }
         span_begin(ctx, EGG_K_HEAD); HIP_TRY(egg_launch_head(p, s)); span_end(ctx);
     }
     return EGG_OK;
@@ -525,9 +547,10 @@ static UpdParams make_upd(egg_ctx *ctx, int id, const int32_t *d_fit, const uint
     p.panel_a = ctx->d_panel_a; p.panel_b = ctx->d_panel_b; p.pairs_pad = ctx->pairs_pad; p.counter = ctx->d_counter;
     return p;
 }
-static int update_one(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
+static int update_one(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr, bool record_flags = false) {
     const egg_tensor_info &t = ctx->tensors[id];
     UpdParams p = make_upd(ctx, id, d_fit, d_seed, d_lr);
+    if (record_flags) p.flags = ctx->d_flags + t.offset;
     if (t.is_matrix && t.muon && ctx->cfg.use_muon) {
         // LAUNCH_ADAM_MATRIX under USE_MUON (mgpu.cu:1587-1595)
         span_begin(ctx, EGG_K_UPDATE_MATRIX);
@@ -566,13 +589,73 @@ extern "C" int egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t 
     // independent, so the reference's launch order (mgpu.cu:1603-1643) does not matter
     for (int id = 0; id < (int)ctx->tensors.size(); id++) {
         if (!ctx->tensors[id].is_matrix) continue;
-        int rc = update_one(ctx, id, d_fit, d_seed, d_lr);
+        int rc = update_one(ctx, id, d_fit, d_seed, d_lr, ctx->adaptive);
         if (rc) return rc;
     }
     UpdParams common = make_upd(ctx, 0, d_fit, d_seed, d_lr);
     span_begin(ctx, EGG_K_UPDATE_VECTOR);
     HIP_TRY(egg_launch_update_vectors(common, ctx->d_vec_desc, ctx->n_vec, ctx->vec_total, ctx->stream));
     span_end(ctx);
+    // d-eggs runs the overlay rule after each tensor's update (de/src/worker.cu:446-523); tensors and their overlay
+    // entries are independent, so one launch over every tensor's segment at the end gives the same values
+    if (ctx->adaptive)
+        HIP_TRY(egg_launch_overlay_update(ctx->d_overlay, ctx->d_overlay_q, ctx->d_flags, ctx->d_ov_segs, ctx->n_ov_segs,
+                                          ctx->ov_max_count, ctx->ov_inc, ctx->ov_dec, ctx->stream));
+    return EGG_OK;
+}
+
+// ------------------------------------------------------------------ adaptive noise overlay (d-eggs)
+// de/src/worker.cu:333 (every overlay value starts at ADAPTIVE_NOISE_INIT), de/include/config.h:229-242 (mode 1,
+// +5 / -1 / 64).  From this call on the forward scales every noise term by its overlay factor
+// (de/include/model/layers.cuh:12-53) and egg_es_update applies the overlay rule after the AdamW update.
+extern "C" int egg_adaptive_enable(egg_ctx *ctx, int init_value, int inc, int dec) {
+    if (!ctx || init_value < -127 || init_value > 127 || inc < 0 || dec < 0) return fail(ctx, EGG_E_INVALID, "egg_adaptive_enable arguments");
+    if (ctx->cfg.use_muon) return fail(ctx, EGG_E_INVALID, "the adaptive noise overlay is defined for the AdamW update only");
+    if (ctx->captured) return fail(ctx, EGG_E_STATE, "enable the overlay before capturing the step");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    const size_t n = (size_t)ctx->L.total;
+    if (!ctx->d_overlay) {
+        HIP_TRY(hipMalloc(&ctx->d_overlay, n)); HIP_TRY(hipMalloc(&ctx->d_overlay_q, n)); HIP_TRY(hipMalloc(&ctx->d_flags, n));
+        std::vector<OvSeg> segs; std::vector<VecDesc> vd; int first = 0;
+        for (size_t id = 0; id < ctx->tensors.size(); id++) {
+            const egg_tensor_info &t = ctx->tensors[id];
+            OvSeg sg; sg.offset = (int)t.offset; sg.count = t.is_matrix ? t.rows + t.cols : t.cols;
+            segs.push_back(sg);
+            if (sg.count > ctx->ov_max_count) ctx->ov_max_count = sg.count;
+            if (t.is_matrix) continue;
+            VecDesc d; d.W = ctx->d_model + t.offset; d.state = reinterpret_cast<float *>(ctx->d_state + ctx->t_state_off[id]);
+            d.n = t.cols; d.first = first; d.off_a = t.off_a; d.off_b = t.off_b; d.seed_base = t.seed_base; d.lr_scale = t.lr_scale;
+            d.flags = ctx->d_flags + t.offset;
+            vd.push_back(d); first += t.cols;
+        }
+        ctx->n_ov_segs = (int)segs.size();
+        HIP_TRY(hipMalloc(&ctx->d_ov_segs, segs.size() * sizeof(OvSeg)));
+        HIP_TRY(hipMemcpy(ctx->d_ov_segs, segs.data(), segs.size() * sizeof(OvSeg), hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(ctx->d_vec_desc, vd.data(), vd.size() * sizeof(VecDesc), hipMemcpyHostToDevice));
+    }
+    HIP_TRY(hipMemset(ctx->d_overlay, init_value & 0xff, n));
+    HIP_TRY(hipMemset(ctx->d_flags, 0, n));
+    HIP_TRY(egg_launch_overlay_q(ctx->d_overlay, ctx->d_overlay_q, (int64_t)n, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    ctx->ov_inc = inc; ctx->ov_dec = dec; ctx->adaptive = true;
+    return EGG_OK;
+}
+// The overlay blob has the layout of the model blob: a vector tensor's values at the tensor's offset; a matrix's
+// input-row values at its offset and its output-column values right behind them.  Other bytes are not used.
+extern "C" int egg_overlay_upload(egg_ctx *ctx, const void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != ctx->L.total) return fail(ctx, EGG_E_INVALID, "overlay size mismatch");
+    if (!ctx->adaptive) return fail(ctx, EGG_E_STATE, "egg_adaptive_enable has not been called");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemcpy(ctx->d_overlay, h, bytes, hipMemcpyHostToDevice));
+    HIP_TRY(egg_launch_overlay_q(ctx->d_overlay, ctx->d_overlay_q, (int64_t)bytes, ctx->stream));
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return EGG_OK;
+}
+extern "C" int egg_overlay_download(egg_ctx *ctx, void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != ctx->L.total) return fail(ctx, EGG_E_INVALID, "overlay size mismatch");
+    if (!ctx->adaptive) return fail(ctx, EGG_E_STATE, "egg_adaptive_enable has not been called");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    HIP_TRY(hipMemcpy(h, ctx->d_overlay, bytes, hipMemcpyDeviceToHost));
     return EGG_OK;
 }
 extern "C" int64_t egg_opt_state_bytes(const egg_ctx *ctx) { return ctx ? ctx->state_bytes : 0; }

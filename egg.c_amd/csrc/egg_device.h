@@ -355,6 +355,32 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// ---------------------------------------------------------------- adaptive noise overlay (d-eggs)
+// de/include/model/layers.cuh:12-53 (mode 1): an int8 overlay value ov scales a noise term by 0 (ov < 0), ov/64
+// (ov < 64) or 1, in float, and the product is converted to int (toward zero).  All operands here are small enough
+// for the float product to be exact, so the same value comes out of integer arithmetic: trunc(v * q / 64) with
+// q = clamp(ov, 0, 64).  The kernels read q from a device blob laid out like the model blob (a vector tensor's values at
+// the tensor's offset; a matrix's input-row values at its offset, its output-column values right behind them).
+__device__ __forceinline__ int overlay_q(int ov) { return ov < 0 ? 0 : (ov > 64 ? 64 : ov); }
+template <int BITS>
+__device__ __forceinline__ int div_pow2_trunc(int t) { return (t + ((t >> 31) & ((1 << BITS) - 1))) >> BITS; }
+__device__ __forceinline__ int overlay_scaled(int v, int q) { return div_pow2_trunc<6>(v * q); }
+// the table fills above with the q values of the tensor's columns / elements applied
+__device__ __forceinline__ void fill_noise_i8_ov(int8_t *dst, uint32_t seed, int n, int mask, int lane, int nthr, int mult, const int8_t *q) {
+    for (int i = lane; i < n; i += nthr) dst[i] = (int8_t)(overlay_scaled(noise_from_hash(seed, i, mask), q[i]) * mult);
+}
+__device__ __forceinline__ void fill_noise_i32_ov(int *dst, uint32_t seed, int n, int mask, int mult, int lane, int nthr, const int8_t *q) {
+    for (int i = lane; i < n; i += nthr) dst[i] = overlay_scaled(noise_from_hash(seed, i, mask), q[i]) * mult;
+}
+__device__ __forceinline__ void fill_vec_i32_ov(int *dst, const int8_t *base, uint32_t seed_a, uint32_t seed_b,
+                                                int n, int mask, int ns, int shift, int lane, int nthr, int lshift, const int8_t *q) {
+    for (int i = lane; i < n; i += nthr) {
+        int v = base[i];
+        if (ns != 0) v += (overlay_scaled(noise_from_hash(seed_a, i, mask) * noise_from_hash(seed_b, i, mask), q[i]) * ns) >> shift;
+        dst[i] = v << lshift;
+    }
+}
+
 // x . B over the operand's k-steps; btab is the int8 noise table in natural order.
 // slot order: dword q of k-step ks covers k = 32ks + 8q + 4g + (0..3); natural: 32ks + 16g + 4q + (0..3)
 template <int KS, bool NAT>
@@ -367,6 +393,26 @@ __device__ __forceinline__ int dot_noise(const v4i *xop, const int8_t *btab, int
         for (int q = 0; q < 4; q++) {
             int kd = NAT ? (8 * ks + 4 * g + q) : (8 * ks + 2 * q + g);
             s = dot4(xop[ks][q], b32[kd], s);
+        }
+    return s + other_half(s);
+}
+
+// x . B under the overlay: every term x[k] * B[k] is scaled by the input row's factor and truncated before it is added
+// (the reference converts each thread's term to int, de/include/model/layers.cuh:240).  qtab holds the rows' q values
+// in the order of btab.
+template <int KS, bool NAT>
+__device__ __forceinline__ int dot_noise_ov(const v4i *xop, const int8_t *btab, const int8_t *qtab, int k_off, int g) {
+    const int *b32 = reinterpret_cast<const int *>(btab + k_off);
+    const int *q32 = reinterpret_cast<const int *>(qtab + k_off);
+    int s = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            int kd = NAT ? (8 * ks + 4 * g + q) : (8 * ks + 2 * q + g);
+            const int xb = xop[ks][q], nb = b32[kd], qb = q32[kd];
+#pragma unroll
+            for (int e = 0; e < 4; e++) s += div_pow2_trunc<6>(mul24(mul24(sx8(xb, e), sx8(nb, e)), sx8(qb, e)));
         }
     return s + other_half(s);
 }

@@ -5,7 +5,7 @@
 // serially over tokens.  Here tokens are the GEMM's free dimension: a wave owns a tile of 32 tokens of
 // one member, four waves share each W block staged in LDS, and a launch covers a chunk of members.
 //   k_mlp<H,true>   embedding stage + initial MLP          (mgpu.cu:901-934, :708-759)
-//   k_qkv<H>        LN1 + Q/K/V projections + RoPE + norms (mgpu.cu:769-784)
+//   k_qkv<H,..>     LN1 + Q/K/V projections + RoPE + norms (mgpu.cu:769-784)
 //   k_attn<HD,CT>   causal exp-LUT attention core          (mgpu.cu:787-825)
 //   k_mlp<H,false>  O-projection + residual norm + MLP     (mgpu.cu:827-831, :708-759)
 //   k_head<H>       final norm + tied head + loss          (mgpu.cu:955-1028)
@@ -134,7 +134,11 @@ struct MlpCfg {
 // FUSE: the host has checked sigma <= 7 and |noise| <= 15, which bounds |acc| * 2^sigma + |sb * a| below 2^31 for
 // GEMM depths up to 1024 (depth * 127 * 127 * 128 + depth * 127 * 225); the down projection (depth 4H) uses the
 // fused form only for 4H <= 1024.
-template <int H, bool FIRST, bool FUSE>
+// ADAPT: the d-eggs adaptive noise overlay is on (de/include/model/layers.cuh:215-296, :432-438,
+// de/src/kernels.cu:139-158); see k_qkv.  The down projection's input-side sum follows the reference thread of a
+// hidden unit, which adds its four terms (k = unit, unit + H, ...) into an int one float addition at a time; the
+// sub-chunks are therefore visited so that those four are consecutive.
+template <int H, bool FIRST, bool FUSE, bool ADAPT>
 __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p) {
     typedef MlpCfg<H> M;
     constexpr bool FUSE_DN = FUSE && 4 * H <= 1024;
@@ -182,6 +186,25 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         int *e0 = reinterpret_cast<int *>(t2), *e1 = e0 + H, *lw = e1 + H, *lb = lw + H, *bu = lb + H, *bd = bu + 4 * H;
         int8_t *eB = reinterpret_cast<int8_t *>(bd + H), *uB = eB + H, *dB = uB + H, *uA = dB + 4 * H, *dA = uA + 4 * H;
         const int tid = threadIdx.x;
+        if (ADAPT) {
+            if (FIRST) {
+                fill_vec_i32_ov(e0, p.emb_bias, pseed + OFF_EMB_BIAS_A, pseed + OFF_EMB_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_emb_bias);
+                // b_dim * q(hidden) * ns, not yet divided: the token's factor joins before the truncation
+                for (int i = tid; i < H; i += EGG_THREADS) e1[i] = noise_from_hash(pseed + OFF_EMB + H, i, c.mask) * p.q_emb[i] * nsx;
+            } else {
+                fill_noise_i8_ov(reinterpret_cast<int8_t *>(e0), sbx + OFF_O_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_o + H);
+                fill_noise_i8(eB, sbx + OFF_O_B, H, c.mask, tid, EGG_THREADS);
+            }
+            fill_vec_i32_ov(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_w);
+            fill_vec_i32_ov(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_b);
+            fill_noise_i8_ov(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx, p.q_up + H);
+            fill_vec_i32_ov(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up, p.q_b_up);
+            fill_noise_i8_ov(dA, sbx + p.off_dn_a, H, c.mask, tid, EGG_THREADS, nsx, p.q_dn + 4 * H);
+            fill_vec_i32_ov(bd, p.b_dn, sbx + p.off_bdn_a, sbx + p.off_bdn_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_b_dn);
+            fill_noise_i8(uB, sbx + p.off_up_b, H, c.mask, tid, EGG_THREADS);
+            fill_noise_i8(dB, sbx + p.off_dn_b, 4 * H, c.mask, tid, EGG_THREADS);
+            continue;
+        }
         if (FIRST) {
             fill_vec_i32(e0, p.emb_bias, pseed + OFF_EMB_BIAS_A, pseed + OFF_EMB_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
             fill_noise_i32(e1, pseed + OFF_EMB + H, H, c.mask, nsx, tid, EGG_THREADS);
@@ -217,7 +240,8 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         if (FIRST) {
             // embedding stage (mgpu.cu:901-931)
             const int tok = c.data[spos + t];
-            const int a_tok = noise_from_hash(pair_seed + OFF_EMB, (uint32_t)tok, c.mask);
+            int a_tok = noise_from_hash(pair_seed + OFF_EMB, (uint32_t)tok, c.mask);
+            if (ADAPT) a_tok *= p.q_emb[H + tok];        // a_tok * q(token); the table holds b_dim * q(hidden) * ns
             const uint32_t *E32 = reinterpret_cast<const uint32_t *>(p.embedding);
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++)
@@ -229,7 +253,11 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                     v4i d4 = *reinterpret_cast<const v4i *>(ex1 + n0);
                     int o[4];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = clip127(sx8(e4, e) + b4[e] + (mul24(a_tok, d4[e]) >> c.sigma));
+                    for (int e = 0; e < 4; e++) {
+                        int pp = mul24(a_tok, d4[e]);
+                        if (ADAPT) pp = div_pow2_trunc<12>(pp);      // (int)(a * b * f(token) * f(hidden)), both factors x/64
+                        o[e] = clip127(sx8(e4, e) + b4[e] + (pp >> c.sigma));
+                    }
                     xs[nt][q] = pack4(o[0], o[1], o[2], o[3]);
                 }
         } else {
@@ -241,7 +269,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 v4i aop[KS];
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) aop[ks] = load_op(p.ao + row, ks, g);
-                sbo = dot_noise<KS, false>(aop, exB, 0, g);
+                sbo = ADAPT ? dot_noise_ov<KS, false>(aop, exB, p.q_o, 0, g) : dot_noise<KS, false>(aop, exB, 0, g);
 #pragma unroll
                 for (int u = 0; u < M::OU; u++) {
                     const int8_t *cur = w_acquire(ws);
@@ -283,12 +311,17 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 exchange_operand<CS, NTS, KS, M::TPW, M::UNIT>(ws.other, tm, lane, mine, nrm);
             }
         }
-        const int sbu = dot_noise<KS, false>(nrm, upB, 0, g);
+        const int sbu = ADAPT ? dot_noise_ov<KS, false>(nrm, upB, p.q_up, 0, g) : dot_noise<KS, false>(nrm, upB, 0, g);
         v16i accd[NTS];
         zero_acc<NTS>(accd);
         int sbd = 0;
+        int pb[ADAPT ? NTU * 16 : 1];           // ADAPT: running sums of the reference threads this lane stands in for
+        // ADAPT: iteration it visits sub-chunk (it % 4) * NSUB/4 + it / 4, so four consecutive iterations cover the
+        // intermediate columns unit, unit + H, unit + 2H, unit + 3H of the same hidden units
+        auto sub_chunk = [](int it) { return ADAPT ? (it & 3) * (M::NSUB / 4) + (it >> 2) : it; };
 #pragma unroll 1
-        for (int s = 0; s < M::NSUB; s++) {
+        for (int it = 0; it < M::NSUB; it++) {
+            const int s = sub_chunk(it);
             v16i au[NTU];
 #pragma unroll
             for (int nt = 0; nt < NTU; nt++)
@@ -322,8 +355,22 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                             o[e] = act[(uint8_t)v];
                         }
                         mine[nt][q] = pack4(o[0], o[1], o[2], o[3]);
-                        sbd = dot4(mine[nt][q], dnb32[8 * nt + 2 * q + g], sbd);
+                        if (!ADAPT) sbd = dot4(mine[nt][q], dnb32[8 * nt + 2 * q + g], sbd);
+                        else {
+                            const int nz4 = dnb32[8 * nt + 2 * q + g], q4 = *reinterpret_cast<const int *>(p.q_dn + n0);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const int idx = ADAPT ? (nt * 4 + q) * 4 + e : 0;
+                                const int prev = (it & 3) ? pb[idx] : 0;
+                                // (int)((float)pb + x * n * q / 64): every value is a multiple of 1/64 below 2^24
+                                pb[idx] = div_pow2_trunc<6>((prev << 6) + mul24(mul24(o[e], sx8(nz4, e)), sx8(q4, e)));
+                            }
+                        }
                     }
+                if (ADAPT && (it & 3) == 3) {
+#pragma unroll
+                    for (int i2 = 0; i2 < (ADAPT ? NTU * 16 : 1); i2++) sbd += pb[i2];
+                }
                 if (CS == 1) {
 #pragma unroll
                     for (int nt = 0; nt < NTU; nt++) mid[nt] = mine[nt];
@@ -339,7 +386,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
 #pragma unroll
                     for (int k = 0; k < CS * NTU; k++) mid[k] = xch_get(xch, CS * NTU, tm.tslot, k, lane);
                 if (du + 1 < M::DNU) pf_dn(s, du + 1);
-                else if (s + 1 < M::NSUB) pf_up(s + 1, 0);
+                else if (it + 1 < M::NSUB) pf_up(sub_chunk(it + 1), 0);
                 else if (pass + 1 < tm.passes) pf_pass_first();
                 mfma_cols<M::PRDN / 2, NTS>(accd, mid + du * (M::PRDN / 2), cur, H, col0, lane);
             }
@@ -427,7 +474,9 @@ __device__ __forceinline__ void rope_inplace(v16i *acc, const RopeTab &rt, int h
             }
 }
 
-template <int H>
+// ADAPT: the d-eggs adaptive noise overlay is on (de/include/model/layers.cuh:313-351): output-side noise and vector
+// noise are scaled when the per-member tables are filled, the input-side sums take the slow term-by-term form.
+template <int H, bool ADAPT>
 __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p) {
     typedef QkvCfg<H> Q;
     constexpr int CS = Q::CS, KS = Q::KS, NTS = Q::NTS, HS = Q::HS;
@@ -456,11 +505,19 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
         int *lw = reinterpret_cast<int *>(t2), *lb = lw + H;
         int8_t *a0 = reinterpret_cast<int8_t *>(lb + H), *a1 = a0 + H, *a2 = a1 + H, *b0 = a2 + H, *b1 = b0 + H, *b2 = b1 + H;
         const int tid = threadIdx.x;
-        fill_vec_i32(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
-        fill_vec_i32(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
-        fill_noise_i8(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx);
-        fill_noise_i8(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx);
-        fill_noise_i8(a2, sbx + OFF_V_A, H, c.mask, tid, EGG_THREADS, nsx);
+        if (ADAPT) {
+            fill_vec_i32_ov(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_w);
+            fill_vec_i32_ov(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_b);
+            fill_noise_i8_ov(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wq + H);
+            fill_noise_i8_ov(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wk + H);
+            fill_noise_i8_ov(a2, sbx + OFF_V_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wv + H);
+        } else {
+            fill_vec_i32(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+            fill_vec_i32(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+            fill_noise_i8(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx);
+            fill_noise_i8(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx);
+            fill_noise_i8(a2, sbx + OFF_V_A, H, c.mask, tid, EGG_THREADS, nsx);
+        }
         fill_noise_i8(b0, sbx + OFF_Q_B, H, c.mask, tid, EGG_THREADS);
         fill_noise_i8(b1, sbx + OFF_K_B, H, c.mask, tid, EGG_THREADS);
         fill_noise_i8(b2, sbx + OFF_V_B, H, c.mask, tid, EGG_THREADS);
@@ -499,7 +556,8 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
             const int8_t *Bn = which == 0 ? qB : (which == 1 ? kB : vB);
             const int8_t *An = which == 0 ? qA : (which == 1 ? kA : vA);
             int8_t *dst = which == 0 ? p.q : (which == 1 ? p.k : p.v);
-            const int sb = dot_noise<KS, false>(nrm, Bn, 0, g);
+            const int sb = ADAPT ? dot_noise_ov<KS, false>(nrm, Bn, which == 0 ? p.q_wq : (which == 1 ? p.q_wk : p.q_wv), 0, g)
+                                 : dot_noise<KS, false>(nrm, Bn, 0, g);
             v16i acc[NTS];
             zero_acc<NTS>(acc);
 #pragma unroll
@@ -850,7 +908,9 @@ struct HeadLds {
     static constexpr int TOTAL = WBLOCK + 1024 + EGG_WAVES * PER_WAVE;
 };
 
-template <int H>
+// ADAPT: adaptive noise overlay; the tied head takes the embedding's per-hidden q values on its input side and the
+// per-token values on its output side (de/src/kernels.cu:200-240)
+template <int H, bool ADAPT>
 __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadParams p) {
     constexpr int KS = H / 32, NV = 256 / 32, BLK = H < 256 ? H : 256;
     extern __shared__ __align__(16) int8_t smem[];
@@ -873,9 +933,15 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
     WStream ws; wstream_init(ws, wlds, WUnit<BLK>::BYTES);
     w_prefetch<BLK>(ws, w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0));
     for (int i = threadIdx.x; i < 256; i += EGG_THREADS) lut[i] = c.exp_lut[i];
-    fill_vec_i32(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane);
-    fill_vec_i32(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
-    fill_noise_i32(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane);
+    if (ADAPT) {
+        fill_vec_i32_ov(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane, 64, 0, p.q_ln_w);
+        fill_vec_i32_ov(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane, 64, 0, p.q_ln_b);
+        fill_noise_i32_ov(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane, 64, p.q_emb + H);
+    } else {
+        fill_vec_i32(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane);
+        fill_vec_i32(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
+        fill_noise_i32(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane);
+    }
     fill_noise_i8(hB, pair_seed + OFF_EMB + H, H, c.mask, lane);
     __syncthreads();
 
@@ -888,7 +954,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
         standard_norm<KS>(x, nf, lnw, lnb, g);
-        const int sbh = dot_noise<KS, false>(nf, hB, 0, g);
+        const int sbh = ADAPT ? dot_noise_ov<KS, false>(nf, hB, p.q_emb, 0, g) : dot_noise<KS, false>(nf, hB, 0, g);
         v16i acc[NV];
         zero_acc<NV>(acc);
         gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, ws, (pass + 1 < T / 32) ? w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0) : nullptr, lane);
@@ -948,8 +1014,13 @@ static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = MlpCfg<H>::total(sets);
     const bool fuse = p.c.sigma <= 7 && p.c.mask <= 15;
-    if (first) { if (fuse) hipLaunchKernelGGL((k_mlp<H, true, true>), grid, block, lds, s, p); else hipLaunchKernelGGL((k_mlp<H, true, false>), grid, block, lds, s, p); }
-    else { if (fuse) hipLaunchKernelGGL((k_mlp<H, false, true>), grid, block, lds, s, p); else hipLaunchKernelGGL((k_mlp<H, false, false>), grid, block, lds, s, p); }
+    if (p.q_ln_w) {      // adaptive noise overlay: one (unfused) variant
+        if (first) hipLaunchKernelGGL((k_mlp<H, true, false, true>), grid, block, lds, s, p);
+        else hipLaunchKernelGGL((k_mlp<H, false, false, true>), grid, block, lds, s, p);
+        return hipGetLastError();
+    }
+    if (first) { if (fuse) hipLaunchKernelGGL((k_mlp<H, true, true, false>), grid, block, lds, s, p); else hipLaunchKernelGGL((k_mlp<H, true, false, false>), grid, block, lds, s, p); }
+    else { if (fuse) hipLaunchKernelGGL((k_mlp<H, false, true, false>), grid, block, lds, s, p); else hipLaunchKernelGGL((k_mlp<H, false, false, false>), grid, block, lds, s, p); }
     return hipGetLastError();
 }
 hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s) {
@@ -967,7 +1038,8 @@ static hipError_t launch_qkv_h(const QkvParams &p, hipStream_t s) {
     const int sets = tile_map_sets(p.c.T, Shape<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = QkvCfg<H>::total(sets);
-    hipLaunchKernelGGL((k_qkv<H>), grid, block, lds, s, p);
+    if (p.q_ln_w) hipLaunchKernelGGL((k_qkv<H, true>), grid, block, lds, s, p);
+    else hipLaunchKernelGGL((k_qkv<H, false>), grid, block, lds, s, p);
     return hipGetLastError();
 }
 hipError_t egg_launch_qkv(const QkvParams &p, hipStream_t s) {
@@ -1016,7 +1088,8 @@ template <int H>
 static hipError_t launch_head_h(const HeadParams &p, hipStream_t s) {
     dim3 grid((p.c.n_members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
     size_t lds = HeadLds<H>::TOTAL;
-    hipLaunchKernelGGL((k_head<H>), grid, block, lds, s, p);
+    if (p.q_ln_w) hipLaunchKernelGGL((k_head<H, true>), grid, block, lds, s, p);
+    else hipLaunchKernelGGL((k_head<H, false>), grid, block, lds, s, p);
     return hipGetLastError();
 }
 hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
@@ -1036,12 +1109,16 @@ template <int H>
 static hipError_t prepare_h(int T) {
     const int sets = tile_map_sets(T, Shape<H>::CS);
     const int msets = tile_map_sets(T, MlpCfg<H>::CS);
-    SET_LDS((k_mlp<H, true, true>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, false, true>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, true, false>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, false, false>), MlpCfg<H>::total(msets));
-    SET_LDS((k_qkv<H>), QkvCfg<H>::total(sets));
-    SET_LDS((k_head<H>), HeadLds<H>::TOTAL);
+    SET_LDS((k_mlp<H, true, true, false>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, false, true, false>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, true, false, false>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, false, false, false>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, true, false, true>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, false, false, true>), MlpCfg<H>::total(msets));
+    SET_LDS((k_qkv<H, false>), QkvCfg<H>::total(sets));
+    SET_LDS((k_qkv<H, true>), QkvCfg<H>::total(sets));
+    SET_LDS((k_head<H, false>), HeadLds<H>::TOTAL);
+    SET_LDS((k_head<H, true>), HeadLds<H>::TOTAL);
     return hipSuccess;
 }
 template <int HD, int CT>

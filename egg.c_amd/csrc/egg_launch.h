@@ -41,14 +41,23 @@ struct UpdParams {
     int8_t *panel_a, *panel_b; int pairs_pad;   // workspace: [cols][pairs_pad], [rows][pairs_pad]
     unsigned long long *counter;
     int32_t *votes_out;                // optional: only compute votes (blocked order), no update
+    int8_t *flags;                     // optional (adaptive noise overlay): [rows] then [cols], set to 1 where a weight of
+                                       // that input row / output column changed (de/include/optimizer/adam.cuh:77-83)
     // Muon (state is {m, acc} per element): momentum pass writes m and the row-major gather buffer
     float muon_momentum; float *muon_x; // [rows][cols] row-major
 };
 hipError_t egg_launch_update_matrix(const UpdParams &p, hipStream_t s);
 hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s);
 // every vector tensor of the model in one launch: descriptors live on the device, `first` is the running element count
-struct VecDesc { int8_t *W; float *state; int n, first, off_a, off_b, seed_base; float lr_scale; };
+struct VecDesc { int8_t *W; float *state; int n, first, off_a, off_b, seed_base; float lr_scale; int8_t *flags; };   // flags: as above, per element, or null
 hipError_t egg_launch_update_vectors(const UpdParams &common, const VecDesc *d_desc, int n_desc, int total, hipStream_t s);
+
+// adaptive noise overlay (de/src/kernels.cu:61-77): for every entry of every segment, +inc where the flag is set, -dec
+// elsewhere, clamped to [-127, 127]; also writes q = clamp(overlay, 0, 64) and clears the flag
+struct OvSeg { int offset, count; };
+hipError_t egg_launch_overlay_update(int8_t *overlay, int8_t *q, int8_t *flags, const OvSeg *d_segs, int n_segs, int max_count,
+                                     int inc, int dec, hipStream_t s);
+hipError_t egg_launch_overlay_q(const int8_t *overlay, int8_t *q, int64_t n, hipStream_t s);
 
 // Muon chain (muon_internal.cuh:15-342): momentum + gather (vote GEMM epilogue), Frobenius normalisation,
 // 5 Newton-Schulz iterations on fp32 MFMA, quantised apply.

@@ -54,6 +54,9 @@ struct MlpParams {
     const int8_t *ao;            // [n_members][T][H] slot order
     int8_t *x;                   // [n_members][T][H] slot order, read (if !FIRST) and written
     int8_t *x_mid;               // optional tap: residual stream after attention (may be null)
+    // adaptive noise overlay (all null when it is off): q values (0..64) of the tensors above; a matrix has its
+    // input-row values first and its output-column values right behind them
+    const int8_t *q_ln_w, *q_ln_b, *q_b_up, *q_b_dn, *q_up, *q_dn, *q_o, *q_emb, *q_emb_bias;
 };
 
 struct QkvParams {
@@ -63,6 +66,7 @@ struct QkvParams {
     const int8_t *w_q, *w_k, *w_v;   // fragment-major copies
     const int8_t *x;
     int8_t *q, *k, *v;           // [n_members][T][H] slot order
+    const int8_t *q_ln_w, *q_ln_b, *q_wq, *q_wk, *q_wv;   // adaptive noise overlay q values, or null
 };
 
 struct AttnParams {
@@ -78,4 +82,5 @@ struct HeadParams {
     const int8_t *x;
     unsigned long long *loss_acc; // [population] two's-complement int64 accumulators
     int32_t *logits_tap;          // optional [n_members][T][vocab] natural order (may be null)
+    const int8_t *q_ln_w, *q_ln_b, *q_emb;   // adaptive noise overlay q values (embedding: H per-hidden, then vocab per-token), or null
 };

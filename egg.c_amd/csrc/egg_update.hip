@@ -160,7 +160,10 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vote_adam(UpdParams p) {
 #pragma unroll
     for (int e = 0; e < 4; e++) {
         wv[e] = sx8(w4, e);
-        changes += adam_apply(st[3 * e], st[3 * e + 1], st[3 * e + 2], wv[e], -(float)vote[e], lr, hy);
+        const int ch = adam_apply(st[3 * e], st[3 * e + 1], st[3 * e + 2], wv[e], -(float)vote[e], lr, hy);
+        changes += ch;
+        // every writer stores the same value, so plain stores do (the overlay rule only asks "any change?")
+        if (ch && p.flags) { p.flags[k0 + 8 * q + 4 * g + e] = 1; p.flags[p.rows + n] = 1; }
     }
     *reinterpret_cast<int *>(p.W + idx0) = pack4(wv[0], wv[1], wv[2], wv[3]);
     sp[0] = make_float4(st[0], st[1], st[2], st[3]);
@@ -234,8 +237,37 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vectors_adam(UpdParams p, const
         int ch = adam_apply(m, v, acc, w, -(float)vote, lr, hy);
         t.W[idx] = (int8_t)w; st[0] = m; st[1] = v; st[2] = acc;
         if (ch) atomicAdd(p.counter, 1ull);
+        if (ch && t.flags) t.flags[idx] = 1;
     }
 }
+// update_overlay_kernel (de/src/kernels.cu:61-77) over a list of segments of the overlay blob
+__global__ void k_overlay_update(int8_t *overlay, int8_t *q, int8_t *flags, const OvSeg *segs, int inc, int dec) {
+    const OvSeg sg = segs[blockIdx.y];
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= sg.count) return;
+    const int at = sg.offset + i;
+    int ov = overlay[at];
+    if (flags[at]) { ov += inc; if (ov > 127) ov = 127; }
+    else { ov -= dec; if (ov < -127) ov = -127; }
+    flags[at] = 0;
+    overlay[at] = (int8_t)ov;
+    q[at] = (int8_t)overlay_q(ov);
+}
+hipError_t egg_launch_overlay_update(int8_t *overlay, int8_t *q, int8_t *flags, const OvSeg *d_segs, int n_segs, int max_count,
+                                     int inc, int dec, hipStream_t s) {
+    if (n_segs <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_overlay_update, dim3((max_count + 255) / 256, n_segs), dim3(256), 0, s, overlay, q, flags, d_segs, inc, dec);
+    return hipGetLastError();
+}
+__global__ void k_overlay_q(const int8_t *overlay, int8_t *q, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) q[i] = (int8_t)overlay_q(overlay[i]);
+}
+hipError_t egg_launch_overlay_q(const int8_t *overlay, int8_t *q, int64_t n, hipStream_t s) {
+    hipLaunchKernelGGL(k_overlay_q, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, overlay, q, n);
+    return hipGetLastError();
+}
+
 hipError_t egg_launch_update_vectors(const UpdParams &common, const VecDesc *d_desc, int n_desc, int total, hipStream_t s) {
     if (total <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_vectors_adam, dim3((total + EGG_WAVES - 1) / EGG_WAVES), dim3(EGG_THREADS), 0, s, common, d_desc, n_desc, total);

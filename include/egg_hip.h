@@ -114,6 +114,21 @@ int  egg_fitness(egg_ctx *ctx, const int32_t *d_loss, int32_t *d_fit, int pairs)
  * rate by device pointer (de/include/optimizer/adam.cuh:38-39); resets then accumulates the update
  * counter (mgpu.cu:1574, :1107-1110) */
 int  egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr);
+/* d-eggs adaptive noise overlay.  egg_adaptive_enable: every overlay value starts at init_value
+ * (de/src/worker.cu:333, ADAPTIVE_NOISE_INIT 64); from then on the forward scales each noise term by its overlay
+ * factor before truncating it (mode 1 of de/include/model/layers.cuh:12-53; sites layers.cuh:94, :177, :240-296,
+ * :332-438, de/src/kernels.cu:139-240) and egg_es_update / egg_step apply update_overlay_kernel
+ * (de/src/kernels.cu:61-77, +inc where a weight of the row / column / element changed, -dec elsewhere; the
+ * reference's ADAPTIVE_NOISE_INC 5, ADAPTIVE_NOISE_DEC 1, de/include/config.h:234-239) after the AdamW update, fed by
+ * the change counters of de/include/optimizer/adam.cuh:77-83, :130-132.  AdamW only (EGG_E_INVALID with use_muon).
+ * The overlay blob (egg_overlay_upload / _download, egg_model_bytes() bytes) has the layout of the model blob: a vector
+ * tensor's values at the tensor's offset, a matrix's `rows` input-dimension values at its offset followed by its
+ * `cols` output-dimension values (AdaptiveScales, de/include/model/definitions.h:92-142, keeps them as separate
+ * *_row / *_col arrays; the embedding's per-hidden values are its rows here, its per-token values its cols). */
+int  egg_adaptive_enable(egg_ctx *ctx, int init_value, int inc, int dec);
+int  egg_overlay_upload(egg_ctx *ctx, const void *host_overlay, size_t bytes);
+int  egg_overlay_download(egg_ctx *ctx, void *host_overlay, size_t bytes);
+
 /* one tensor of the table returned by egg_tensor_info (test hook for update_matrix_adam_kernel,
  * update_vector_adam_kernel mgpu.cu:1067-1152 and the Muon chain mgpu.cu:1587-1595) */
 int  egg_update_tensor(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr);
