@@ -188,6 +188,27 @@ def main():
     except Exception as e:
         c5 = {"error": str(e)}
 
+    # ---- the headline model with the d-eggs adaptive noise overlay on (fractional factors everywhere), one chunk
+    adaptive = None
+    try:
+        PA = min(P, 2048)
+        actx = pkg.Context(pkg.default_config(**dict(kw, population=PA)))
+        actx.set_stream(stream.cuda_stream)
+        actx.model_init(42)
+        actx.adaptive_enable(40, 5, 1)
+        actx.step(d_data.data_ptr(), n, 0, 42, 0.3)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(3):
+            actx.step(d_data.data_ptr(), n, (i + 1) * T, 43 + i, 0.3)
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t0) / 3
+        adaptive = {"value": PA * T / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3,
+                    "workload": f"same model, population {PA} (one chunk), adaptive noise overlay on, forward+fitness+vote+AdamW+overlay rule"}
+        actx.close()
+    except Exception as e:
+        adaptive = {"error": str(e)}
+
     # ---- CPU baseline: the oracle's restatement of the same forward on a bounded sample of members
     cpu = None
     cpu_ref_path = None
@@ -221,7 +242,7 @@ def main():
                                f"forward+fitness+vote+AdamW, eager launches (chunk {chunk} members)",
                    "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss},
         "roofline": roofline, "kernels": per_class, "microbench_c2": mb,
-        "gru_c1_gpu": gru, "c5_shape_gpu": c5, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
+        "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }
     print(json.dumps(out))
     ctx.close()
