@@ -10,6 +10,7 @@
 //
 // usage: egg_train [--data FILE] [--steps N] [--population P] [--seq T] [--hidden H] [--layers L] [--muon] [--graph]
 //                  [--gen-every N] [--save-every N] [--save-dir DIR] [--load MODEL.bin [--load-state ADAM.bin]]
+//                  [--adaptive]   (the d-eggs worker's adaptive noise overlay, d-eggs/src/worker.cu:331-333, :446-523)
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -48,6 +49,7 @@ int main(int argc, char **argv) {
     egg_config cfg; egg_default_config(&cfg);
     cfg.seq_len = 256; cfg.population = 40960;
     const char *data_file = nullptr; long steps = 10; bool graph = false; size_t synth_bytes = 64u << 20;
+    bool adaptive = false;
     long gen_every = 5, save_every = 0; const char *save_dir = "models", *load_model = nullptr, *load_state = nullptr;
     for (int i = 1; i < argc; i++) {
         auto next = [&](const char *name) -> const char * { if (i + 1 >= argc) { fprintf(stderr, "%s needs a value\n", name); exit(2); } return argv[++i]; };
@@ -59,6 +61,7 @@ int main(int argc, char **argv) {
         else if (!strcmp(argv[i], "--layers")) cfg.n_layers = atoi(next("--layers"));
         else if (!strcmp(argv[i], "--muon")) cfg.use_muon = 1;
         else if (!strcmp(argv[i], "--graph")) graph = true;
+        else if (!strcmp(argv[i], "--adaptive")) adaptive = true;
         else if (!strcmp(argv[i], "--gen-every")) gen_every = atol(next("--gen-every"));
         else if (!strcmp(argv[i], "--save-every")) save_every = atol(next("--save-every"));
         else if (!strcmp(argv[i], "--save-dir")) save_dir = next("--save-dir");
@@ -84,6 +87,7 @@ int main(int argc, char **argv) {
     if (rc != EGG_OK) { fprintf(stderr, "egg_ctx_create failed (%d): unsupported configuration or no GPU\n", rc); return 1; }
     if (load_model) CK(egg_checkpoint_load(ctx, load_model, load_state));
     else CK(egg_model_init(ctx, 42));
+    if (adaptive) CK(egg_adaptive_enable(ctx, 64, 5, 1));      // ADAPTIVE_NOISE_INIT / _INC / _DEC, d-eggs/include/config.h:234-242
     uint8_t *d_data = nullptr;
     HK(hipMalloc(&d_data, data.size()));
     HK(hipMemcpy(d_data, data.data(), data.size(), hipMemcpyHostToDevice));
