@@ -176,6 +176,12 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return EGG_E_INVALID;
     if (!(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256 || c.seq_len == 512)) return EGG_E_INVALID;
     if (c.vocab != 256 || c.n_layers < 1 || c.population < 2 || (c.population & 1)) return EGG_E_INVALID;
+    // shift amounts and table scales the kernels can state in 32-bit shifts / 64-bit multiply-adds
+    auto in_range = [](int v, int lo, int hi) { return v >= lo && v <= hi; };
+    if (!in_range(c.rope_scale_bit, 1, 30) || !in_range(c.softmax_scale_bit, 1, 30) || !in_range(c.noise_mask, 0, 127) ||
+        !in_range(c.fixed_point + c.sigma_shift, 0, 24) || !in_range(c.sigma_shift_vector, 0, 24) || !in_range(c.shift_attn, 0, 24) ||
+        !in_range(c.shift_out, 0, 24) || !in_range(c.shift_logit, 0, 24) || !in_range(c.shift_mlp_up, 0, 24) ||
+        !in_range(c.shift_mlp_down, 0, 24)) return EGG_E_INVALID;
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
     ctx->L = make_layout(c);

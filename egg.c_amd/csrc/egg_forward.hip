@@ -433,14 +433,10 @@ struct QkvCfg {
 // apply_rope_integer (mgpu.cu:624-644) on the raw accumulators of one token.  The (cos, sin) pairs repeat every
 // head, so a lane needs only the head_dim/32 * 8 pairs of its own slots; they are loaded once per token tile
 // (RopeTab) and reused for every head of Q and K.
-// The reference evaluates (ve*c -+ vo*s + 2^(bit-1)) >> bit in int64.  Here the same value is formed in double
-// precision, where it is exact: |v| < 2^23 and |c|, |s| <= 2^bit <= 2^20 keep every partial sum below 2^45, and the
-// table is pre-scaled by 2^-bit (a power of two).  Adding 2^24 before the truncating conversion makes the operand
-// positive, so truncation equals the arithmetic shift's floor; 2^24 is subtracted again in integers.
-struct RopeTab { double c[2][4][2], s[2][4][2]; };
-__device__ __forceinline__ void rope_load(RopeTab &rt, const int32_t *rope_row, int head_dim, int bit, int g) {
+// The reference evaluates (ve*c -+ vo*s + 2^(bit-1)) >> bit in int64, and so does this code.
+struct RopeTab { int c[2][4][2], s[2][4][2]; };
+__device__ __forceinline__ void rope_load(RopeTab &rt, const int32_t *rope_row, int head_dim, int g) {
     const int hdt = head_dim >> 5;                 // column groups per head: 1 or 2
-    const double sc = __builtin_ldexp(1.0, -bit);
 #pragma unroll
     for (int h2 = 0; h2 < 2; h2++)
 #pragma unroll
@@ -449,28 +445,30 @@ __device__ __forceinline__ void rope_load(RopeTab &rt, const int32_t *rope_row, 
             for (int ep = 0; ep < 2; ep++) {
                 int n = 32 * (h2 < hdt ? h2 : 0) + 8 * q + 4 * g + 2 * ep;
                 int2 v = *reinterpret_cast<const int2 *>(rope_row + 2 * (n >> 1));
-                rt.c[h2][q][ep] = (double)v.x * sc;
-                rt.s[h2][q][ep] = (double)v.y * sc;
+                rt.c[h2][q][ep] = v.x;
+                rt.s[h2][q][ep] = v.y;
             }
 }
-// The NT column groups must start at a head boundary.
+// The NT column groups must start at a head boundary.  64-bit multiply-adds (v_mad_i64_i32, full rate on gfx950) state
+// the reference's int64 expression directly; the shifted result fits 32 bits like the reference's AccumType.
 template <int NT>
-__device__ __forceinline__ void rope_inplace(v16i *acc, const RopeTab &rt, int head_dim) {
+__device__ __forceinline__ void rope_inplace(v16i *acc, const RopeTab &rt, int head_dim, int bit) {
     const int hdt = head_dim >> 5;
-    const double init = 16777216.5;                // 2^24 + the rounding half, both already divided by 2^bit
+    const long long half = 1ll << (bit - 1);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
         for (int q = 0; q < 4; q++)
 #pragma unroll
             for (int ep = 0; ep < 2; ep++) {
-                const double cc = (hdt == 2) ? rt.c[nt & 1][q][ep] : rt.c[0][q][ep];
-                const double ss = (hdt == 2) ? rt.s[nt & 1][q][ep] : rt.s[0][q][ep];
-                const double ve = (double)acc[nt][4 * q + 2 * ep], vo = (double)acc[nt][4 * q + 2 * ep + 1];
-                const double re = __builtin_fma(-vo, ss, __builtin_fma(ve, cc, init));
-                const double ro = __builtin_fma(vo, cc, __builtin_fma(ve, ss, init));
-                acc[nt][4 * q + 2 * ep] = (int)re - 16777216;
-                acc[nt][4 * q + 2 * ep + 1] = (int)ro - 16777216;
+                const int cc = (hdt == 2) ? rt.c[nt & 1][q][ep] : rt.c[0][q][ep];
+                const int ss = (hdt == 2) ? rt.s[nt & 1][q][ep] : rt.s[0][q][ep];
+                const int ve = acc[nt][4 * q + 2 * ep], vo = acc[nt][4 * q + 2 * ep + 1], nvo = -vo;
+                const long long re = (long long)nvo * ss + ((long long)ve * cc + half);
+                const long long ro = (long long)vo * cc + ((long long)ve * ss + half);
+                // bits [bit+31 : bit] of the 64-bit sums (0 < bit < 32): the arithmetic shift, truncated to 32 bits
+                acc[nt][4 * q + 2 * ep] = (int)__builtin_amdgcn_alignbit((unsigned)(re >> 32), (unsigned)re, (unsigned)bit);
+                acc[nt][4 * q + 2 * ep + 1] = (int)__builtin_amdgcn_alignbit((unsigned)(ro >> 32), (unsigned)ro, (unsigned)bit);
             }
 }
 
@@ -548,7 +546,7 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
             }
         }
         RopeTab rt;
-        rope_load(rt, c.rope_lut + (size_t)t * c.head_dim, c.head_dim, c.rope_scale_bit, g);
+        rope_load(rt, c.rope_lut + (size_t)t * c.head_dim, c.head_dim, g);
 #pragma unroll 1
         for (int which = 0; which < 3; which++) {
             const int8_t *W = which == 0 ? p.w_q : (which == 1 ? p.w_k : p.w_v);
@@ -568,7 +566,7 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
                 mfma_cols<Q::PR / 2, NTS>(acc, nrm + u * (Q::PR / 2), cur, H, col0, lane);
             }
             add_perturb8<NTS>(acc, sb, An, col0, c.sigma, g);
-            if (which < 2) rope_inplace<NTS>(acc, rt, c.head_dim);
+            if (which < 2) rope_inplace<NTS>(acc, rt, c.head_dim, c.rope_scale_bit);
             const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red + ((1 + which) & 1) * Q::SITE, tm, lane);
             v4i o[NTS];
             adaptive_scale<NTS>(acc, mx, o);
