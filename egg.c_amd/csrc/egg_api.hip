@@ -182,6 +182,8 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
         !in_range(c.fixed_point + c.sigma_shift, 0, 24) || !in_range(c.sigma_shift_vector, 0, 24) || !in_range(c.shift_attn, 0, 24) ||
         !in_range(c.shift_out, 0, 24) || !in_range(c.shift_logit, 0, 24) || !in_range(c.shift_mlp_up, 0, 24) ||
         !in_range(c.shift_mlp_down, 0, 24)) return EGG_E_INVALID;
+    // the standard norm divides x * (gain + noise) by the row mean with a 32-bit multiply-high that is exact up to 2^17
+    if (127 * (127 + ((c.noise_mask * c.noise_mask) >> c.sigma_shift_vector)) > (1 << 17)) return EGG_E_INVALID;
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
     ctx->L = make_layout(c);

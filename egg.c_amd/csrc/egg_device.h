@@ -430,9 +430,12 @@ __device__ __forceinline__ int sumabs_groups(const v4i *x) {
         for (int q = 0; q < 4; q++) tot = sumabs4(x[ks][q], tot);
     return tot;
 }
+// wt holds 4 * (w + noise).  trunc(a / mn) for |a| <= 2^17 and 1 <= mn <= 127 is the high word of
+// (4a) * (floor(2^30 / mn) + 1), plus one when a is negative (checked exhaustively on the CPU); the context refuses
+// configurations whose gains could leave that range.
 template <int N>
 __device__ __forceinline__ void standard_scale(const v4i *x, v4i *out, int mn, const int *wt, const int *bt, int col0, int g) {
-    const float md = 1.0f / (float)mn;
+    const int M = (int)(1073741824.0 / (double)mn) + 1;       // exact: the quotient is an integer or at least 1/127 away from one
 #pragma unroll
     for (int ks = 0; ks < N; ks++)
 #pragma unroll
@@ -442,7 +445,10 @@ __device__ __forceinline__ void standard_scale(const v4i *x, v4i *out, int mn, c
             v4i b4 = *reinterpret_cast<const v4i *>(bt + n0);
             int o[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(mul24(sx8(x[ks][q], e), w4[e]), md) + b4[e]);
+            for (int e = 0; e < 4; e++) {
+                const int a4 = mul24(sx8(x[ks][q], e), w4[e]);
+                o[e] = clip127(__mulhi(a4, M) + (int)((unsigned)a4 >> 31) + b4[e]);
+            }
             out[ks][q] = pack4(o[0], o[1], o[2], o[3]);
         }
 }

@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 fill_noise_i8_ov(reinterpret_cast<int8_t *>(e0), sbx + OFF_O_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_o + H);
                 fill_noise_i8(eB, sbx + OFF_O_B, H, c.mask, tid, EGG_THREADS);
             }
-            fill_vec_i32_ov(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_w);
+            fill_vec_i32_ov(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2, p.q_ln_w);
             fill_vec_i32_ov(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_b);
             fill_noise_i8_ov(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx, p.q_up + H);
             fill_vec_i32_ov(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up, p.q_b_up);
@@ -212,7 +212,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             fill_noise_i8(reinterpret_cast<int8_t *>(e0), sbx + OFF_O_A, H, c.mask, tid, EGG_THREADS, nsx);
             fill_noise_i8(eB, sbx + OFF_O_B, H, c.mask, tid, EGG_THREADS);
         }
-        fill_vec_i32(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+        fill_vec_i32(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2);     // 4 * gain, see standard_scale
         fill_vec_i32(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_noise_i8(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx);
         // the up bias is stored as b << shift_mlp_up and seeds the up accumulator: ((a + (b << s)) >> s) == (a >> s) + b
@@ -504,13 +504,13 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
         int8_t *a0 = reinterpret_cast<int8_t *>(lb + H), *a1 = a0 + H, *a2 = a1 + H, *b0 = a2 + H, *b1 = b0 + H, *b2 = b1 + H;
         const int tid = threadIdx.x;
         if (ADAPT) {
-            fill_vec_i32_ov(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_w);
+            fill_vec_i32_ov(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2, p.q_ln_w);
             fill_vec_i32_ov(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_b);
             fill_noise_i8_ov(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wq + H);
             fill_noise_i8_ov(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wk + H);
             fill_noise_i8_ov(a2, sbx + OFF_V_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wv + H);
         } else {
-            fill_vec_i32(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
+            fill_vec_i32(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2);     // 4 * gain, see standard_scale
             fill_vec_i32(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
             fill_noise_i8(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx);
             fill_noise_i8(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx);
@@ -932,11 +932,11 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
     w_prefetch<BLK>(ws, w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0));
     for (int i = threadIdx.x; i < 256; i += EGG_THREADS) lut[i] = c.exp_lut[i];
     if (ADAPT) {
-        fill_vec_i32_ov(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane, 64, 0, p.q_ln_w);
+        fill_vec_i32_ov(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane, 64, 2, p.q_ln_w);
         fill_vec_i32_ov(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane, 64, 0, p.q_ln_b);
         fill_noise_i32_ov(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane, 64, p.q_emb + H);
     } else {
-        fill_vec_i32(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane);
+        fill_vec_i32(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane, 64, 2);   // 4 * gain, see standard_scale
         fill_vec_i32(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
         fill_noise_i32(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane);
     }
