@@ -53,7 +53,13 @@ __device__ __forceinline__ void add_perturb8(v16i *acc, int sb, const int8_t *At
 // instruction less.  The host selects FUSE only when |acc| * 2^sigma + |sb * a| < 2^31 for the GEMM depth in question.
 template <bool FUSE>
 __device__ __forceinline__ int perturb_shift(int acc, int sb, int a, int sigma, int shift) {
-    if (FUSE) return (int)(((unsigned)acc << sigma) + (unsigned)mul24(sb, a)) >> (sigma + shift);
+    if (FUSE) {
+        // keep the product out of a multiply-add: as a plain multiply it takes the noise byte through a sub-dword
+        // operand select, and the shift joins the addition in one v_lshl_add_u32
+        int prod = mul24(sb, a);
+        asm volatile("" : "+v"(prod));
+        return (int)(((unsigned)acc << sigma) + (unsigned)prod) >> (sigma + shift);
+    }
     return (acc + (mul24(sb, a) >> sigma)) >> shift;
 }
 // acc[nt][r] = perturb_shift(acc[nt][r], sb, At[n], ...) for NT column groups starting at table offset n_off
