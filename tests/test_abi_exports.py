@@ -45,3 +45,13 @@ def test_product_sources_do_not_reference_the_oracle():
                 if f == "__init__.py" and re.search(r"import\s+oracle|oracle_py|libegg_oracle", txt):
                     bad.append(f)
     assert not bad, bad
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU per box: asking bench.py for more must end with a message, before anything touches a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
