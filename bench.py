@@ -167,9 +167,24 @@ def main():
     c5 = None
     try:
         P5 = 2048
-        c5ctx = pkg.Context(pkg.default_config(hidden=512, head_dim=64, n_layers=8, seq_len=512, population=P5, use_muon=1))
+        c5ctx = pkg.Context(pkg.default_config(hidden=512, head_dim=64, n_layers=8, seq_len=512, population=P5, use_muon=1,
+                                               weight_limit=1))
         c5ctx.set_stream(stream.cuda_stream)
         c5ctx.model_init(42)
+        # ternary weights: the sign of the reference initialisation where it is large, packed 2 bits per weight on the
+        # host and unpacked by the library on the GPU; the weight limit of 1 keeps the matrices ternary through updates
+        m = c5ctx.model_download()
+        parts = []
+        for t in sorted(c5ctx.tensors(), key=lambda t: t["offset"]):
+            seg = m[t["offset"]:t["offset"] + t["rows"] * t["cols"]]
+            if t["is_matrix"]:
+                tern = (np.sign(seg) * (np.abs(seg) > 5)).astype(np.int8).reshape(-1, 4)
+                f = (tern & 3).astype(np.uint8)
+                parts.append(f[:, 0] | (f[:, 1] << 2) | (f[:, 2] << 4) | (f[:, 3] << 6))
+            else:
+                parts.append(seg.view(np.uint8))
+        c5ctx.model_upload_ternary(np.ascontiguousarray(np.concatenate(parts)))
+        del m, parts
         c5ctx.step(d_data.data_ptr(), n, 0, 42, 0.3)
         torch.cuda.synchronize()
         c5ctx.enable_timing(True); c5ctx.timing_reset()
@@ -182,7 +197,8 @@ def main():
         upd_ms = tm["update_matrix"][1] + tm["update_vector"][1]
         c5 = {"value": P5 * 512 / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3, "forward_ms": fwd_ms, "update_ms": upd_ms,
               "k_mlp_frac_mfma": (2 * 9 * 512 * 512 * P5 * 512) / (tm["mlp"][1] / tm["mlp"][0] * 1e-3) / PEAK_INT8_OPS,
-              "workload": f"hidden 512, 8 heads, seq 512, 8 layers, population {P5} (one chunk), forward+fitness+vote+Muon; "
+              "workload": f"hidden 512, 8 heads, seq 512, 8 layers, ternary-packed weights (unpacked on upload, weight limit 1), "
+                          f"population {P5} (one chunk), forward+fitness+vote+Muon; "
                           "a 16,384-member step is 8 such forwards plus one update"}
         c5ctx.close()
     except Exception as e:

@@ -27,7 +27,7 @@ class EggConfig(C.Structure):
         ("softmax_exp_scale", C.c_double),
         ("adam_beta1", C.c_float), ("adam_beta2", C.c_float), ("adam_eps", C.c_float),
         ("adam_weight_decay", C.c_float), ("muon_momentum", C.c_float), ("muon_lr_scale", C.c_float),
-        ("use_muon", C.c_int), ("chunk_members", C.c_int)]
+        ("use_muon", C.c_int), ("chunk_members", C.c_int), ("weight_limit", C.c_int)]
 
 
 class EggTensorInfo(C.Structure):
@@ -43,6 +43,7 @@ EXPORTS = [
     "egg_noise_fill", "egg_perturbed_linear", "egg_population_forward", "egg_population_forward_dev",
     "egg_fitness", "egg_es_update", "egg_update_tensor", "egg_matrix_votes",
     "egg_adaptive_enable", "egg_overlay_upload", "egg_overlay_download",
+    "egg_ternary_model_bytes", "egg_model_upload_ternary", "egg_model_download_ternary",
     "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
     "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate",
     "egg_shape_fitness", "egg_ternary_pack_size", "egg_ternary_pack", "egg_ternary_unpack",
@@ -90,6 +91,10 @@ def lib():
                   L.egg_overlay_upload, L.egg_overlay_download):
             f.argtypes = [vp, vp, C.c_size_t]
         L.egg_adaptive_enable.argtypes = [vp, i32, i32, i32]
+        L.egg_ternary_model_bytes.restype = i64
+        L.egg_ternary_model_bytes.argtypes = [vp]
+        for f in (L.egg_model_upload_ternary, L.egg_model_download_ternary):
+            f.argtypes = [vp, vp, C.c_size_t]
         L.egg_opt_state_reset.argtypes = [vp]
         L.egg_tables_download.argtypes = [vp, vp, vp, vp]
         L.egg_noise_fill.argtypes = [vp, u32, u32, i32, vp]
@@ -255,6 +260,18 @@ class Context:
 
     def es_update(self, d_fit, d_seed, d_lr):
         self._ck(lib().egg_es_update(self._h, C.c_void_p(d_fit), C.c_void_p(d_seed), C.c_void_p(d_lr)), "egg_es_update")
+
+    def ternary_model_bytes(self):
+        return int(lib().egg_ternary_model_bytes(self._h))
+
+    def model_upload_ternary(self, packed):
+        self._ck(lib().egg_model_upload_ternary(self._h, _np_ptr(packed), packed.nbytes), "egg_model_upload_ternary")
+
+    def model_download_ternary(self):
+        import numpy as np
+        out = np.zeros(self.ternary_model_bytes(), np.uint8)
+        self._ck(lib().egg_model_download_ternary(self._h, _np_ptr(out), out.nbytes), "egg_model_download_ternary")
+        return out
 
     def adaptive_enable(self, init_value=64, inc=5, dec=1):
         """d-eggs adaptive noise overlay: on from this call (forward scaling and the overlay rule in es_update / step)"""

@@ -115,7 +115,7 @@ extern "C" void egg_default_config(egg_config *c) {
     c->softmax_scale_bit = 18; c->rope_scale_bit = 20; c->noise_mask = 15; c->host_mask = 15;
     c->softmax_exp_scale = 6.0;
     c->adam_beta1 = 0.9f; c->adam_beta2 = 0.95f; c->adam_eps = 1e-8f; c->adam_weight_decay = 0.01f;
-    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->use_muon = 0; c->chunk_members = 0;
+    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->use_muon = 0; c->chunk_members = 0; c->weight_limit = 127;
 }
 
 // launch order of mgpu.cu:1603-1643
@@ -184,6 +184,7 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
         !in_range(c.shift_mlp_down, 0, 24)) return EGG_E_INVALID;
     // the standard norm divides x * (gain + noise) by the row mean with a 32-bit multiply-high that is exact up to 2^17
     if (127 * (127 + ((c.noise_mask * c.noise_mask) >> c.sigma_shift_vector)) > (1 << 17)) return EGG_E_INVALID;
+    if (!in_range(c.weight_limit, 1, 127)) return EGG_E_INVALID;
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
     ctx->L = make_layout(c);
@@ -352,6 +353,74 @@ extern "C" int egg_model_download(egg_ctx *ctx, void *h, size_t bytes) {
     HIP_TRY(hipMemcpy(h, ctx->d_model, bytes, hipMemcpyDeviceToHost));
     return EGG_OK;
 }
+// ------------------------------------------------------------------ ternary-packed model (no reference counterpart)
+// The packed blob is the model blob with every matrix tensor stored at 2 bits per weight (see k_ternary_unpack) and
+// every vector tensor left as int8, tensors in the order of their offsets in the model blob.
+static std::vector<int> tensors_by_offset(const egg_ctx *ctx) {
+    std::vector<int> ids(ctx->tensors.size());
+    for (size_t i = 0; i < ids.size(); i++) ids[i] = (int)i;
+    std::sort(ids.begin(), ids.end(), [&](int a, int b) { return ctx->tensors[a].offset < ctx->tensors[b].offset; });
+    return ids;
+}
+extern "C" int64_t egg_ternary_model_bytes(const egg_ctx *ctx) {
+    if (!ctx) return 0;
+    int64_t n = 0;
+    for (const egg_tensor_info &t : ctx->tensors) n += t.is_matrix ? (int64_t)t.rows * t.cols / 4 : t.cols;
+    return n;
+}
+extern "C" int egg_model_upload_ternary(egg_ctx *ctx, const void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != egg_ternary_model_bytes(ctx)) return fail(ctx, EGG_E_INVALID, "ternary model size mismatch");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    uint8_t *d_packed = nullptr;
+    HIP_TRY(hipMalloc(&d_packed, bytes));
+    hipError_t e = hipMemcpy(d_packed, h, bytes, hipMemcpyHostToDevice);
+    int64_t po = 0;
+    for (int id : tensors_by_offset(ctx)) {
+        const egg_tensor_info &t = ctx->tensors[id];
+        if (e != hipSuccess) break;
+        if (t.is_matrix) {
+            e = egg_launch_ternary_unpack(d_packed + po, ctx->d_model + t.offset, t.rows * t.cols, ctx->stream);
+            po += (int64_t)t.rows * t.cols / 4;
+        } else {
+            e = hipMemcpyAsync(ctx->d_model + t.offset, d_packed + po, (size_t)t.cols, hipMemcpyDeviceToDevice, ctx->stream);
+            po += t.cols;
+        }
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(d_packed);
+    if (e != hipSuccess) return fail(ctx, EGG_E_HIP, "egg_model_upload_ternary", e);
+    return refresh_frag(ctx, -1);
+}
+extern "C" int egg_model_download_ternary(egg_ctx *ctx, void *h, size_t bytes) {
+    if (!ctx || !h || (int64_t)bytes != egg_ternary_model_bytes(ctx)) return fail(ctx, EGG_E_INVALID, "ternary model size mismatch");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    uint8_t *d_packed = nullptr;
+    const size_t flag_off = (bytes + 3) & ~(size_t)3;          // the out-of-range flag sits behind the packed bytes
+    HIP_TRY(hipMalloc(&d_packed, flag_off + 4));
+    int *d_bad = reinterpret_cast<int *>(d_packed + flag_off);
+    hipError_t e = hipMemsetAsync(d_bad, 0, 4, ctx->stream);
+    int64_t po = 0;
+    for (int id : tensors_by_offset(ctx)) {
+        const egg_tensor_info &t = ctx->tensors[id];
+        if (e != hipSuccess) break;
+        if (t.is_matrix) {
+            e = egg_launch_ternary_pack(ctx->d_model + t.offset, d_packed + po, t.rows * t.cols, d_bad, ctx->stream);
+            po += (int64_t)t.rows * t.cols / 4;
+        } else {
+            e = hipMemcpyAsync(d_packed + po, ctx->d_model + t.offset, (size_t)t.cols, hipMemcpyDeviceToDevice, ctx->stream);
+            po += t.cols;
+        }
+    }
+    int bad = 0;
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) e = hipMemcpy(&bad, d_bad, 4, hipMemcpyDeviceToHost);
+    if (e == hipSuccess && !bad) e = hipMemcpy(h, d_packed, bytes, hipMemcpyDeviceToHost);
+    (void)hipFree(d_packed);
+    if (e != hipSuccess) return fail(ctx, EGG_E_HIP, "egg_model_download_ternary", e);
+    if (bad) return fail(ctx, EGG_E_INVALID, "a matrix weight is outside {-1, 0, 1}: the model is not ternary");
+    return EGG_OK;
+}
+
 extern "C" int egg_opt_state_upload(egg_ctx *ctx, const void *h, size_t bytes) {
     if (!ctx || !h || (int64_t)bytes != ctx->state_bytes) return fail(ctx, EGG_E_INVALID, "state size mismatch");
     HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -551,6 +620,7 @@ static UpdParams make_upd(egg_ctx *ctx, int id, const int32_t *d_fit, const uint
     p.W = ctx->d_model + t.offset; p.state = reinterpret_cast<float *>(ctx->d_state + ctx->t_state_off[id]);
     p.rows = t.rows; p.cols = t.cols; p.off_a = t.off_a; p.off_b = t.off_b; p.seed_base = t.seed_base;
     p.fit = d_fit; p.pairs = c.population / 2; p.d_seed = d_seed; p.d_lr = d_lr; p.lr_scale = t.lr_scale;
+    p.limit = t.is_matrix ? c.weight_limit : 127;
     p.mask = c.noise_mask; p.beta1 = c.adam_beta1; p.beta2 = c.adam_beta2; p.eps = c.adam_eps; p.wd = c.adam_weight_decay;
     p.panel_a = ctx->d_panel_a; p.panel_b = ctx->d_panel_b; p.pairs_pad = ctx->pairs_pad; p.counter = ctx->d_counter;
     return p;

@@ -38,6 +38,7 @@ struct UpdParams {
     const int32_t *fit; int pairs;
     const uint32_t *d_seed; const float *d_lr; float lr_scale;
     int mask; float beta1, beta2, eps, wd;
+    int limit;                         // weights saturate at +-limit: 127 (mgpu.cu:1056-1062), or the configured limit for matrices
     int8_t *panel_a, *panel_b; int pairs_pad;   // workspace: [cols][pairs_pad], [rows][pairs_pad]
     unsigned long long *counter;
     int32_t *votes_out;                // optional: only compute votes (blocked order), no update
@@ -58,6 +59,10 @@ struct OvSeg { int offset, count; };
 hipError_t egg_launch_overlay_update(int8_t *overlay, int8_t *q, int8_t *flags, const OvSeg *d_segs, int n_segs, int max_count,
                                      int inc, int dec, hipStream_t s);
 hipError_t egg_launch_overlay_q(const int8_t *overlay, int8_t *q, int64_t n, hipStream_t s);
+
+// ternary-packed matrix weights <-> canonical int8 (n_elems a multiple of 4); *d_bad is set when a weight is not in {-1,0,1}
+hipError_t egg_launch_ternary_unpack(const uint8_t *packed, int8_t *dst, int n_elems, hipStream_t s);
+hipError_t egg_launch_ternary_pack(const int8_t *src, uint8_t *packed, int n_elems, int *d_bad, hipStream_t s);
 
 // Muon chain (muon_internal.cuh:15-342): momentum + gather (vote GEMM epilogue), Frobenius normalisation,
 // 5 Newton-Schulz iterations on fp32 MFMA, quantised apply.

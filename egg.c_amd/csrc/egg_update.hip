@@ -55,7 +55,7 @@ hipError_t egg_launch_fitness(const int32_t *loss, int32_t *fit, int pairs, hipS
 }
 
 // apply_adam_update (mgpu.cu:1040-1064); every float operation is a single IEEE-754 operation
-struct AdamHyper { float b1, b2, eps, wd; };
+struct AdamHyper { float b1, b2, eps, wd; int limit; };     // limit: the weight saturates at +-limit (127 in the reference)
 __device__ __forceinline__ int adam_apply(float &m, float &v, float &acc, int &w, float gr, float lr, const AdamHyper &h) {
     float t1 = h.b1 * m; float t2 = (1.0f - h.b1) * gr; m = t1 + t2;
     float t3 = h.b2 * v; float gg = gr * gr; float t4 = (1.0f - h.b2) * gg; v = t3 + t4;
@@ -66,9 +66,9 @@ __device__ __forceinline__ int adam_apply(float &m, float &v, float &acc, int &w
     acc += step;
     int change = 0;
     if (acc >= 1.0f) {
-        if (w < 127) { w++; change = 1; acc -= 1.0f; } else acc = 1.0f;
+        if (w < h.limit) { w++; change = 1; acc -= 1.0f; } else acc = 1.0f;
     } else if (acc <= -1.0f) {
-        if (w > -127) { w--; change = 1; acc += 1.0f; } else acc = -1.0f;
+        if (w > -h.limit) { w--; change = 1; acc += 1.0f; } else acc = -1.0f;
     }
     return change;
 }
@@ -148,7 +148,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vote_adam(UpdParams p) {
         return;
     }
     const float lr = (*p.d_lr) * p.lr_scale;
-    const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd};
+    const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd, p.limit};
     int changes = 0;
     int w4 = *reinterpret_cast<const int *>(p.W + idx0);
     float st[12];
@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vector_adam(UpdParams p) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) vote += __shfl_xor(vote, off, 64);
     if (lane == 0) {
-        const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd};
+        const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd, 127};     // vector tensors keep the reference's +-127
         const float lr = (*p.d_lr) * p.lr_scale;
         float *st = p.state + (size_t)idx * 3;
         float m = st[0], v = st[1], acc = st[2];
@@ -229,7 +229,7 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vectors_adam(UpdParams p, const
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) vote += __shfl_xor(vote, off, 64);
     if (lane == 0) {
-        const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd};
+        const AdamHyper hy = {p.beta1, p.beta2, p.eps, p.wd, 127};     // vector tensors keep the reference's +-127
         const float lr = (*p.d_lr) * t.lr_scale;
         float *st = t.state + (size_t)idx * 3;
         float m = st[0], v = st[1], acc = st[2];
@@ -240,6 +240,47 @@ __global__ void __launch_bounds__(EGG_THREADS) k_vectors_adam(UpdParams p, const
         if (ch && t.flags) t.flags[idx] = 1;
     }
 }
+// Ternary-packed matrix weights (no counterpart in the reference, whose weights are plain int8): four consecutive
+// elements of the blocked matrix -- the four input rows that share one dword -- per byte, element e in bits 2e+1..2e
+// as a 2-bit two's complement number (00 = 0, 01 = +1, 11 = -1).  Unpacking writes the canonical int8 blob, from which
+// the fragment-major copy the MFMAs read is rebuilt.
+__global__ void k_ternary_unpack(const uint8_t *packed, int *words, int n_words) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_words) return;
+    const int b = packed[i];
+    int w = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int v = ((b >> (2 * e)) & 3) << 30 >> 30;       // sign-extend the 2-bit field
+        w |= (v & 0xff) << (8 * e);
+    }
+    words[i] = w;
+}
+__global__ void k_ternary_pack(const int *words, uint8_t *packed, int n_words, int *bad) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_words) return;
+    const int w = words[i];
+    int b = 0, out_of_range = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int v = sx8(w, e);
+        out_of_range |= (v < -1) | (v > 1);
+        b |= (v & 3) << (2 * e);
+    }
+    packed[i] = (uint8_t)b;
+    if (out_of_range) *bad = 1;      // every writer stores the same value
+}
+hipError_t egg_launch_ternary_unpack(const uint8_t *packed, int8_t *dst, int n_elems, hipStream_t s) {
+    const int n = n_elems / 4;
+    hipLaunchKernelGGL(k_ternary_unpack, dim3((n + 255) / 256), dim3(256), 0, s, packed, reinterpret_cast<int *>(dst), n);
+    return hipGetLastError();
+}
+hipError_t egg_launch_ternary_pack(const int8_t *src, uint8_t *packed, int n_elems, int *d_bad, hipStream_t s) {
+    const int n = n_elems / 4;
+    hipLaunchKernelGGL(k_ternary_pack, dim3((n + 255) / 256), dim3(256), 0, s, reinterpret_cast<const int *>(src), packed, n, d_bad);
+    return hipGetLastError();
+}
+
 // update_overlay_kernel (de/src/kernels.cu:61-77) over a list of segments of the overlay blob
 __global__ void k_overlay_update(int8_t *overlay, int8_t *q, int8_t *flags, const OvSeg *segs, int inc, int dec) {
     const OvSeg sg = segs[blockIdx.y];
@@ -456,8 +497,8 @@ __global__ void __launch_bounds__(256) k_muon_apply(UpdParams p, float wd) {
         float wdw = wd * (float)w;
         float step = (-lr) * (u + wdw);
         acc += step;
-        if (acc >= 1.0f) { if (w < 127) { w++; change = 1; acc -= 1.0f; } else acc = 1.0f; }
-        else if (acc <= -1.0f) { if (w > -127) { w--; change = 1; acc += 1.0f; } else acc = -1.0f; }
+        if (acc >= 1.0f) { if (w < p.limit) { w++; change = 1; acc -= 1.0f; } else acc = 1.0f; }
+        else if (acc <= -1.0f) { if (w > -p.limit) { w--; change = 1; acc += 1.0f; } else acc = -1.0f; }
         p.W[idx] = (int8_t)w; st[1] = acc;
     }
     unsigned long long m = __ballot(change);

@@ -55,6 +55,8 @@ typedef struct egg_config {
     float muon_momentum, muon_lr_scale;                          /* .85 1.0          */
     int use_muon;            /* USE_MUON: 2-D hidden matrices use Muon instead of AdamW */
     int chunk_members;       /* members evaluated per forward pass over the layers; 0 = auto */
+    int weight_limit;        /* matrix weights saturate at +-weight_limit in the update rule: 127 as in the reference
+                              * (mgpu.cu:1056-1062); 1 keeps them ternary (no reference counterpart)     */
 } egg_config;
 
 void egg_default_config(egg_config *cfg);
@@ -114,6 +116,16 @@ int  egg_fitness(egg_ctx *ctx, const int32_t *d_loss, int32_t *d_fit, int pairs)
  * rate by device pointer (de/include/optimizer/adam.cuh:38-39); resets then accumulates the update
  * counter (mgpu.cu:1574, :1107-1110) */
 int  egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr);
+/* Ternary-packed matrix weights: no counterpart in the reference (its weights are plain int8; what d-eggs packs in
+ * base 3 is the fitness vector, de/include/utils/ternary_pack.h).  The packed blob is the model blob with every matrix
+ * tensor at 2 bits per weight -- the four bytes of one blocked dword per byte, element e in bits 2e+1..2e as a 2-bit
+ * two's complement number -- and every vector tensor unchanged, tensors in the order of their offsets.  Upload unpacks
+ * on the GPU into the canonical int8 blob that every other call uses; download fails with EGG_E_INVALID when a matrix
+ * weight is outside {-1, 0, 1} (egg_config.weight_limit = 1 keeps a trained model there). */
+int64_t egg_ternary_model_bytes(const egg_ctx *ctx);
+int  egg_model_upload_ternary(egg_ctx *ctx, const void *host_packed, size_t bytes);
+int  egg_model_download_ternary(egg_ctx *ctx, void *host_packed, size_t bytes);
+
 /* d-eggs adaptive noise overlay.  egg_adaptive_enable: every overlay value starts at init_value
  * (de/src/worker.cu:333, ADAPTIVE_NOISE_INIT 64); from then on the forward scales each noise term by its overlay
  * factor before truncating it (mode 1 of de/include/model/layers.cuh:12-53; sites layers.cuh:94, :177, :240-296,

@@ -46,7 +46,7 @@ extern "C" void orc_default_config(orc_config *c) {
     c->softmax_scale_bit = 18; c->rope_scale_bit = 20; c->noise_mask = 15; c->host_mask = 15;
     c->softmax_exp_scale = 6.0;
     c->adam_beta1 = 0.9f; c->adam_beta2 = 0.95f; c->adam_eps = 1e-8f; c->adam_weight_decay = 0.01f;
-    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f;
+    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->weight_limit = 127;
 }
 
 /* ------------------------------------------------------------------ RNG */
@@ -184,6 +184,50 @@ extern "C" int orc_tensor_table(const orc_config *c, orc_tensor *out, int max_ou
     int n = (int)v.size();
     for (int i = 0; i < n && i < max_out; i++) out[i] = v[i];
     return n;
+}
+
+/* Ternary-packed matrix weights (no reference counterpart; the self-consistent statement the GPU path is checked
+ * against): tensors in the order of their offsets in the model blob; a vector tensor is copied; a matrix tensor takes
+ * one byte per four consecutive blob elements, element e in bits 2e+1..2e as a 2-bit two's complement number. */
+static std::vector<orc_tensor> tensors_by_offset(const orc_config *c) {
+    std::vector<orc_tensor> v = tensor_table(c);
+    for (size_t i = 1; i < v.size(); i++)
+        for (size_t j = i; j > 0 && v[j - 1].offset > v[j].offset; j--) { orc_tensor t = v[j]; v[j] = v[j - 1]; v[j - 1] = t; }
+    return v;
+}
+extern "C" int64_t orc_ternary_model_bytes(const orc_config *c) {
+    int64_t n = 0;
+    for (const orc_tensor &t : tensor_table(c)) n += t.is_matrix ? (int64_t)t.rows * t.cols / 4 : t.cols;
+    return n;
+}
+extern "C" int orc_ternary_model_pack(const orc_config *c, const int8_t *model, uint8_t *packed) {
+    int64_t po = 0; int bad = 0;
+    for (const orc_tensor &t : tensors_by_offset(c)) {
+        if (!t.is_matrix) { memcpy(packed + po, model + t.offset, t.cols); po += t.cols; continue; }
+        for (int64_t i = 0; i < (int64_t)t.rows * t.cols; i += 4) {
+            int b = 0;
+            for (int e = 0; e < 4; e++) {
+                int v = model[t.offset + i + e];
+                if (v < -1 || v > 1) bad = 1;
+                b |= (v & 3) << (2 * e);
+            }
+            packed[po++] = (uint8_t)b;
+        }
+    }
+    return bad ? -1 : 0;
+}
+extern "C" void orc_ternary_model_unpack(const orc_config *c, const uint8_t *packed, int8_t *model) {
+    int64_t po = 0;
+    for (const orc_tensor &t : tensors_by_offset(c)) {
+        if (!t.is_matrix) { memcpy(model + t.offset, packed + po, t.cols); po += t.cols; continue; }
+        for (int64_t i = 0; i < (int64_t)t.rows * t.cols; i += 4) {
+            int b = packed[po++];
+            for (int e = 0; e < 4; e++) {
+                int f = (b >> (2 * e)) & 3;
+                model[t.offset + i + e] = (int8_t)(f >= 2 ? f - 4 : f);
+            }
+        }
+    }
 }
 
 /* mgpu.cu:443-459: src is [In=rows][Out=cols]; dst word (k/4)*cols + n holds bytes k..k+3 */
@@ -620,7 +664,11 @@ extern "C" void orc_fitness(const int32_t *loss, int32_t *fit, int pairs) {
 
 /* ------------------------------------------------------------------ AdamW + votes */
 /* mgpu.cu:1040-1064 */
+static void adam_apply_limit(const orc_config *c, orc_adam_param *p, int8_t *w, float g, float lr, int *change, int limit);
 extern "C" void orc_adam_apply(const orc_config *c, orc_adam_param *p, int8_t *w, float g, float lr, int *change) {
+    adam_apply_limit(c, p, w, g, lr, change, 127);
+}
+static void adam_apply_limit(const orc_config *c, orc_adam_param *p, int8_t *w, float g, float lr, int *change, int limit) {
     float b1 = c->adam_beta1, b2 = c->adam_beta2;
     float t1 = b1 * p->m; float t2 = (1.0f - b1) * g; p->m = t1 + t2;
     float t3 = b2 * p->v; float gg = g * g; float t4 = (1.0f - b2) * gg; p->v = t3 + t4;
@@ -630,9 +678,9 @@ extern "C" void orc_adam_apply(const orc_config *c, orc_adam_param *p, int8_t *w
     float step = (-lr) * (q + wdw);
     p->acc += step;
     if (p->acc >= 1.0f) {
-        if (*w < 127) { (*w)++; *change = 1; p->acc -= 1.0f; } else p->acc = 1.0f;
+        if (*w < limit) { (*w)++; *change = 1; p->acc -= 1.0f; } else p->acc = 1.0f;
     } else if (p->acc <= -1.0f) {
-        if (*w > -127) { (*w)--; *change = 1; p->acc += 1.0f; } else p->acc = -1.0f;
+        if (*w > -limit) { (*w)--; *change = 1; p->acc += 1.0f; } else p->acc = -1.0f;
     }
 }
 
@@ -670,7 +718,7 @@ extern "C" uint64_t orc_update_matrix_adam(const orc_config *c, int8_t *W, orc_a
     uint64_t changes = 0;
     for (int64_t idx = 0; idx < n; idx++) {
         int change = 0;
-        orc_adam_apply(c, &st[idx], &W[idx], -(float)votes[idx], lr, &change);
+        adam_apply_limit(c, &st[idx], &W[idx], -(float)votes[idx], lr, &change, c->weight_limit);
         changes += change;
     }
     return changes;
@@ -812,8 +860,9 @@ extern "C" uint64_t orc_update_matrix_muon(const orc_config *c, int8_t *W, orc_m
         float wdw = c->adam_weight_decay * (float)W[idx];
         float step = (-lrs) * (u + wdw);
         st[idx].acc += step;
-        if (st[idx].acc >= 1.0f) { if (W[idx] < 127) { W[idx]++; changes++; st[idx].acc -= 1.0f; } else st[idx].acc = 1.0f; }
-        else if (st[idx].acc <= -1.0f) { if (W[idx] > -127) { W[idx]--; changes++; st[idx].acc += 1.0f; } else st[idx].acc = -1.0f; }
+        const int lim = c->weight_limit;
+        if (st[idx].acc >= 1.0f) { if (W[idx] < lim) { W[idx]++; changes++; st[idx].acc -= 1.0f; } else st[idx].acc = 1.0f; }
+        else if (st[idx].acc <= -1.0f) { if (W[idx] > -lim) { W[idx]--; changes++; st[idx].acc += 1.0f; } else st[idx].acc = -1.0f; }
     }
     return changes;
 }

@@ -58,6 +58,8 @@ typedef struct orc_config {
     float adam_beta1, adam_beta2, adam_eps, adam_weight_decay; /* mgpu.cu:246-257 */
     float muon_momentum;     /* 0.85                  mgpu.cu:264 */
     float muon_lr_scale;     /* 1.0                   mgpu.cu:267 */
+    int weight_limit;        /* matrix weights saturate at +-this in the update rule: 127, mgpu.cu:1056-1062;
+                              * other values have no counterpart in the reference (ternary weights: 1) */
 } orc_config;
 
 void orc_default_config(orc_config *c);
@@ -90,6 +92,11 @@ int     orc_tensor_table(const orc_config *c, orc_tensor *out, int max_out); /* 
 void    orc_repack(int8_t *dst, const int8_t *src, int rows, int cols);      /* mgpu.cu:443 */
 void    orc_unpack(int8_t *dst, const int8_t *src_blocked, int rows, int cols);
 void    orc_init_model(const orc_config *c, int8_t *model, uint32_t seed);  /* mgpu.cu:461 */
+
+/* ternary-packed matrix weights: no reference counterpart (parity unpinned by construction); see egg_oracle.cpp */
+int64_t orc_ternary_model_bytes(const orc_config *c);
+int     orc_ternary_model_pack(const orc_config *c, const int8_t *model, uint8_t *packed);   /* -1: a weight outside {-1,0,1} */
+void    orc_ternary_model_unpack(const orc_config *c, const uint8_t *packed, int8_t *model);
 
 /* ---- forward (mgpu.cu:553-1029, norm.h) ---- */
 typedef struct orc_trace {   /* any pointer may be NULL */

@@ -22,7 +22,8 @@ class OrcConfig(C.Structure):
         "softmax_scale_bit", "rope_scale_bit", "noise_mask", "host_mask")] + [
         ("softmax_exp_scale", C.c_double),
         ("adam_beta1", C.c_float), ("adam_beta2", C.c_float), ("adam_eps", C.c_float),
-        ("adam_weight_decay", C.c_float), ("muon_momentum", C.c_float), ("muon_lr_scale", C.c_float)]
+        ("adam_weight_decay", C.c_float), ("muon_momentum", C.c_float), ("muon_lr_scale", C.c_float),
+        ("weight_limit", C.c_int)]
 
 
 class OrcTensor(C.Structure):
@@ -104,6 +105,10 @@ def lib():
         L.orc_noise_dot_adaptive.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint32, C.c_void_p]
         L.orc_down_dot_adaptive.restype = C.c_int32
         L.orc_down_dot_adaptive.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint32, C.c_void_p]
+        L.orc_ternary_model_bytes.restype = C.c_int64
+        L.orc_ternary_model_bytes.argtypes = [C.c_void_p]
+        L.orc_ternary_model_pack.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
+        L.orc_ternary_model_unpack.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_adaptive_factor.restype = C.c_float
         L.orc_adaptive_factor.argtypes = [C.c_int]
         L.orc_forward_member_adaptive.restype = C.c_int32
@@ -332,6 +337,20 @@ def es_update_adam_adaptive(cfg, model, state, overlay, fit, step_seed, lr, inc=
     """d-eggs optimizer step: in place on model, state and the overlay blob (same layout as the model)"""
     return int(lib().orc_es_update_adam_adaptive(C.byref(cfg), _p(model), _p(state), _p(overlay), _p(fit),
                                                  C.c_uint32(step_seed & 0xFFFFFFFF), C.c_float(lr), inc, dec))
+
+
+def ternary_model_pack(cfg, model):
+    """2-bit packing of the matrix tensors (vectors stay int8); raises when a matrix weight is outside {-1, 0, 1}"""
+    out = np.zeros(int(lib().orc_ternary_model_bytes(C.byref(cfg))), np.uint8)
+    if lib().orc_ternary_model_pack(C.byref(cfg), _p(model), _p(out)) != 0:
+        raise ValueError("matrix weight outside {-1, 0, 1}")
+    return out
+
+
+def ternary_model_unpack(cfg, packed):
+    out = np.zeros(model_bytes(cfg), np.int8)
+    lib().orc_ternary_model_unpack(C.byref(cfg), _p(packed), _p(out))
+    return out
 
 
 def gru_init_model(gcfg, seed=42):

@@ -616,3 +616,40 @@ def test_overlay_rule_and_adaptive_update(orc):
     assert np.array_equal(overlay[used].astype(int), expect[used])
     assert (overlay[~used] == 64).all(), "bytes of the blob that belong to no row / column / element are left alone"
     assert (overlay[used] > 64).any() and (overlay[used] < 64).any()
+
+
+# ------------------------------------------------------------------ ternary-packed weights, weight limit (extensions)
+def test_ternary_model_packing_and_weight_limit(orc):
+    """No reference counterpart: hand-computed bytes, a round trip, and the update rule's saturation at the limit."""
+    cfg = orc.config(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=8, weight_limit=1)
+    tt = sorted(orc.tensor_table(cfg), key=lambda t: t["offset"])
+    assert tt[0]["name"] == "embedding" and tt[0]["is_matrix"] and tt[1]["name"] == "emb_bias"
+    rng = np.random.default_rng(9)
+    model = np.zeros(orc.model_bytes(cfg), np.int8)
+    for t in tt:
+        n = t["rows"] * t["cols"]
+        sl = slice(t["offset"], t["offset"] + n)
+        model[sl] = rng.integers(-1, 2, n) if t["is_matrix"] else rng.integers(-127, 128, n)
+    model[0:8] = [1, 0, -1, 1, -1, -1, 0, 0]
+    packed = orc.ternary_model_pack(cfg, model)
+    n_mat = sum(t["rows"] * t["cols"] for t in tt if t["is_matrix"])
+    n_vec = sum(t["cols"] for t in tt if not t["is_matrix"])
+    assert packed.size == n_mat // 4 + n_vec
+    # 01 | 00<<2 | 11<<4 | 01<<6 = 0x71 ;  11 | 11<<2 | 00 | 00 = 0x0f
+    assert packed[0] == 0x71 and packed[1] == 0x0F
+    e0 = tt[0]["rows"] * tt[0]["cols"] // 4
+    assert np.array_equal(packed[e0:e0 + 64].view(np.int8), model[tt[1]["offset"]:tt[1]["offset"] + 64])   # vectors are copied
+    assert np.array_equal(orc.ternary_model_unpack(cfg, packed), model)
+    bad = model.copy(); bad[5] = 2
+    with pytest.raises(ValueError):
+        orc.ternary_model_pack(cfg, bad)
+    # weight_limit 1: matrices stay in {-1, 0, 1} through large-rate updates, vectors still move beyond
+    state = np.zeros(model.size, orc.ADAM_DTYPE)
+    fit = rng.integers(-1, 2, 4).astype(np.int32)
+    for step in range(6):
+        orc.es_update_adam(cfg, model, state, fit, 50 + step, 8.0)
+    mats = np.concatenate([model[t["offset"]:t["offset"] + t["rows"] * t["cols"]] for t in tt if t["is_matrix"]])
+    assert mats.min() == -1 and mats.max() == 1
+    orc.ternary_model_pack(cfg, model)              # still packable
+    sat = state["acc"][:tt[0]["rows"] * tt[0]["cols"]]
+    assert ((sat == 1.0) | (sat == -1.0)).any(), "no accumulator hit the clamp at the limit"
