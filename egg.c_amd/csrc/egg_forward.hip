@@ -53,13 +53,9 @@ __device__ __forceinline__ void add_perturb8(v16i *acc, int sb, const int8_t *At
 // instruction less.  The host selects FUSE only when |acc| * 2^sigma + |sb * a| < 2^31 for the GEMM depth in question.
 template <bool FUSE>
 __device__ __forceinline__ int perturb_shift(int acc, int sb, int a, int sigma, int shift) {
-    if (FUSE) {
-        // keep the product out of a multiply-add: as a plain multiply it takes the noise byte through a sub-dword
-        // operand select, and the shift joins the addition in one v_lshl_add_u32
-        int prod = mul24(sb, a);
-        asm volatile("" : "+v"(prod));
-        return (int)(((unsigned)acc << sigma) + (unsigned)prod) >> (sigma + shift);
-    }
+    // (measured: forcing the multiply apart from the add -- v_mul_i32_i24 with a byte operand select plus
+    // v_lshl_add_u32, one instruction less per element -- runs 2 % slower than the multiply-add the compiler picks)
+    if (FUSE) return (int)(((unsigned)acc << sigma) + (unsigned)mul24(sb, a)) >> (sigma + shift);
     return (acc + (mul24(sb, a) >> sigma)) >> shift;
 }
 // acc[nt][r] = perturb_shift(acc[nt][r], sb, At[n], ...) for NT column groups starting at table offset n_off
