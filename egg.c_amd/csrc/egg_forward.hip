@@ -825,11 +825,13 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0;
         const int r = 32 * ct + j;
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             v4i kf = *reinterpret_cast<const v4i *>(rows + (size_t)r * HD + (((ks * 2 + g) ^ ((r / RPL) % CH)) * 16));
             s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
         }
+        __builtin_amdgcn_s_setprio(0);
         return s;
     };
 
@@ -867,12 +869,14 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
             const v16i s = score_tile(ct, qop);
             v4i pw[3];
             attn_weights(s, lut, mxs, c.shift_attn, diag, ct, t, g, pw, den);
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
                 const v4i vt = *reinterpret_cast<const v4i *>(vfrag + ((size_t)(ct * DT + dt) * 64 + lane) * 16);
 #pragma unroll
                 for (int pl = 0; pl < 3; pl++) o[pl][dt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vt, pw[pl], o[pl][dt], 0, 0, 0);
             }
+            __builtin_amdgcn_s_setprio(0);
         };
 #pragma unroll 2
         for (int ct = 0; ct < qt; ct++) weigh_tile(ct, false);
