@@ -90,16 +90,18 @@ def main():
     # ---- dominant kernel: O-projection + MLP block (k_mlp), MFMA-bound
     per_class = {k: {"launches": v[0], "avg_ms": (v[1] / v[0] if v[0] else None), "total_ms": v[1]} for k, v in timing.items()}
     dom = max(("mlp", "qkv", "attn", "mlp_first", "head"), key=lambda k: timing[k][1])
-    chunk = min(P, args.chunk if args.chunk > 0 else 2048)
+    chunk = min(P, args.chunk if args.chunk > 0 else 8192)
     ops_per_token = {"mlp": 2 * (H * H + 2 * H * 4 * H), "mlp_first": 2 * (2 * H * 4 * H), "qkv": 2 * 3 * H * H,
                      "head": 2 * H * 256, "attn": 2 * 2 * H * (T + 1) // 2}
     launches, tot_ms = timing[dom]
     tokens_per_launch = P * T * args.steps * (L if dom in ("mlp", "qkv", "attn") else 1) / max(launches, 1)
     achieved = ops_per_token[dom] * tokens_per_launch / (tot_ms / launches * 1e-3) if launches else 0.0
-    # HBM bytes per launch of k_mlp<256,false> at 2048 members x 256 tokens per launch, from two rocprofv3 --pmc runs
-    # (FETCH_SIZE 260,192 KiB x 2.0, WRITE_SIZE 311,756 KiB x 1.0; the factors are what the same counters read for a
-    # plain 256 MiB elementwise copy in the same run: 131,091 KiB fetched, 262,144 KiB written)
-    traffic = (260192 * 2.0 + 311756 * 1.0) * 1024 if (dom == "mlp" and chunk == 2048 and P >= 2048) else None
+    # HBM bytes per token of k_mlp<256,false>, from two rocprofv3 --pmc runs at 2048 members x 256 tokens per launch
+    # (FETCH_SIZE 260,192 KiB x 2.0, WRITE_SIZE 311,756 KiB x 1.0 per launch; the factors are what the same counters read
+    # for a plain 256 MiB elementwise copy in the same run: 131,091 KiB fetched, 262,144 KiB written); the kernel's
+    # traffic is per token, so a launch moves that figure times its tokens
+    traffic_per_token = (260192 * 2.0 + 311756 * 1.0) * 1024 / (2048 * 256)
+    traffic = traffic_per_token * tokens_per_launch if (dom == "mlp" and H == 256) else None
     roofline = {"kernel": "k_" + dom, "bound": "mfma", "achieved": achieved / 1e12, "peak": PEAK_INT8_OPS / 1e12,
                 "unit": "TOP/s", "frac": achieved / PEAK_INT8_OPS, "traffic": traffic,
                 "avg_launch_ms": tot_ms / launches if launches else None, "launches": launches}
