@@ -107,9 +107,12 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
                                 dict(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=4, sigma_shift=5, noise_mask=31),
                                 dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4, sigma_shift=1, noise_mask=7,
                                      shift_out=8, shift_mlp_up=7, shift_mlp_down=9),
+                                # the longest sequence with 32-wide heads, and with hidden 128
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=512, population=2),
+                                dict(hidden=128, head_dim=64, n_layers=1, seq_len=512, population=2),
                                 # a RoPE table scale of 2^30, the largest an int32 table holds (products then need all 64 bits)
                                 dict(hidden=128, head_dim=64, n_layers=1, seq_len=64, population=2, rope_scale_bit=30)],
-                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "rope_2_30"])
+                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30"])
 def test_forward_stages_and_loss(pkg, orc, dev, kw):
     """Every stage tap of every member against the oracle's trace, then the per-member losses."""
     data = orc.zipf_bytes(1 << 15)
