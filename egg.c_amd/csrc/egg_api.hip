@@ -844,7 +844,7 @@ extern "C" int egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int g
         HIP_TRY(hipMalloc(&ctx->d_gen_scal, sizeof(Scalars)));
         HIP_TRY(hipMemset(ctx->d_gen_scal, 0, sizeof(Scalars)));
     }
-    HIP_TRY(hipMemsetAsync(ctx->d_gen_tok, 0, (size_t)T + 16, s));
+    HIP_TRY(egg_launch_zero_u64(reinterpret_cast<unsigned long long *>(ctx->d_gen_tok), (T + 16) / 8, s));   // a fill kernel, not a memset node: a caller may be capturing this stream
     HIP_TRY(hipMemcpyAsync(ctx->d_gen_tok, d_buffer, (size_t)seed_len, hipMemcpyDeviceToDevice, s));
     int bt = (c.hidden + 31) & ~31; if (bt > 1024) bt = 1024;          // BLOCK_THREADS (mgpu.cu:74-75)
     const bool taps = ctx->taps; ctx->taps = false;
