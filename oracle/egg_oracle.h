@@ -22,8 +22,12 @@
  *       force and special cases in tests/test_oracle_*.py.
  *   Muon Newton-Schulz : fp64 restatement + orthogonality invariants; the
  *       reference's cuBLAS summation order is unspecified => tolerance only.
- *   whole forward / whole step : restatement only ("parity unpinned" beyond
- *       the per-stage checks above; no reference golden vectors exist).
+ *   whole forward : no reference golden vectors exist, so its composition is
+ *       stated a second time, independently and in a different shape (numpy, all
+ *       tokens of the window at once: oracle/forward_numpy.py), and the two must
+ *       agree on every residual-stream tap, logit and loss.  Beyond the
+ *       per-stage checks above and that agreement it is "parity unpinned", and so
+ *       is the whole step (forward + fitness + update), which only this file states.
  */
 #ifndef EGG_ORACLE_H
 #define EGG_ORACLE_H

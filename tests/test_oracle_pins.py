@@ -653,3 +653,38 @@ def test_ternary_model_packing_and_weight_limit(orc):
     orc.ternary_model_pack(cfg, model)              # still packable
     sat = state["acc"][:tt[0]["rows"] * tt[0]["cols"]]
     assert ((sat == 1.0) | (sat == -1.0)).any(), "no accumulator hit the clamp at the limit"
+
+
+# ------------------------------------------------------------------ the whole forward, stated twice
+@pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=2, seq_len=16, population=6),
+                                dict(hidden=128, head_dim=64, n_layers=1, seq_len=24, population=4),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=40, population=4, sigma_shift=1, noise_mask=31,
+                                     shift_out=8, shift_mlp_up=7, shift_mlp_down=9, sigma_shift_vector=3),
+                                dict(hidden=256, head_dim=64, n_layers=4, seq_len=8, population=2)],
+                         ids=["h64", "h128", "other_shifts", "h256_l4"])
+def test_two_restatements_of_the_forward_agree(orc, kw):
+    """Nothing external pins the composition of the whole forward (the reference ships no golden vectors), so it is
+    stated twice: the C++ oracle walks token by token with a K/V cache as the reference kernel does, the numpy
+    restatement evaluates every stage for the whole window as matrix products.  They share only the lookup tables
+    and tensor offsets, and must agree on every residual-stream tap, every logit and the loss."""
+    from oracle import forward_numpy as fn
+    cfg = orc.config(**kw)
+    data = orc.zipf_bytes(1 << 13)
+    model = orc.init_model(cfg, 42)
+    rng = np.random.default_rng(21)
+    for t in orc.tensor_table(cfg):          # non-trivial gains and biases
+        if not t["is_matrix"]:
+            sl = slice(t["offset"], t["offset"] + t["cols"])
+            model[sl] = rng.integers(-20, 21, t["cols"]).astype(np.int8) + (16 if t["name"].startswith("ln_") and "bias" not in t["name"] else 0)
+    tables = orc.tables(cfg)
+    tt = orc.tensor_table(cfg)
+    start, seed = 3 * kw["seq_len"], 0xABCDEF01
+    for m in range(kw["population"]):
+        ref_loss, tr = orc.forward_member(cfg, model, data, start, seed, m, trace=True)
+        loss, st = fn.forward_member(cfg, model, tt, tables, data, start, seed, m)
+        assert np.array_equal(st["x_init"], tr["x_init"]), m
+        for l in range(kw["n_layers"]):
+            assert np.array_equal(st["x_attn"][l], tr["x_attn"][l]), (m, l)
+            assert np.array_equal(st["x_mlp"][l], tr["x_mlp"][l]), (m, l)
+        assert np.array_equal(st["logits"], tr["logits"]), m
+        assert loss == ref_loss, m
