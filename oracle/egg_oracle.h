@@ -25,9 +25,9 @@
  *   whole forward : no reference golden vectors exist, so its composition is
  *       stated a second time, independently and in a different shape (numpy, all
  *       tokens of the window at once: oracle/forward_numpy.py), and the two must
- *       agree on every residual-stream tap, logit and loss.  Beyond the
- *       per-stage checks above and that agreement it is "parity unpinned", and so
- *       is the whole step (forward + fitness + update), which only this file states.
+ *       agree on every residual-stream tap, logit and loss; the same file states
+ *       the whole AdamW update a second time.  Beyond the per-stage checks above
+ *       and that agreement the whole forward and the whole step are "parity unpinned".
  */
 #ifndef EGG_ORACLE_H
 #define EGG_ORACLE_H

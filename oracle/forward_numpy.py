@@ -185,3 +185,47 @@ def forward_member(cfg, model, tensor_table, tables, data, start_idx, step_seed,
     total = int(loss_t.sum())
     stages["logits"] = logits
     return ((total + 2 ** 31) % 2 ** 32) - 2 ** 31, stages                                   # (int32) my_loss
+
+
+def es_update_adam(cfg, model, state, tensor_table, fit, step_seed, lr):
+    """The AdamW ES update of every tensor, mgpu.cu:1040-1152 and the launch list :1603-1643, with numpy: votes as
+    integer matrix products over the pairs, AdamW in float32 array arithmetic (one rounding per operation).  `state` is a
+    structured array with float32 fields m, v, acc per model byte.  In place; returns the number of changed weights."""
+    f32 = np.float32
+    pairs = cfg.population // 2
+    fit = np.asarray(fit, np.int64)
+    p = np.arange(pairs)
+    changed = 0
+    for e in tensor_table:
+        n = e["rows"] * e["cols"]
+        sl = slice(e["offset"], e["offset"] + n)
+        seeds = (step_seed + p + e["seed_base"]) & 0xFFFFFFFF
+        if e["is_matrix"]:
+            # A[p, n_out], B[p, k_in]; vote[k, n] = sum_p fit_p * A[p, n] * B[p, k]   (mgpu.cu:1092-1098)
+            A = np.stack([noise(int(s) + e["off_a"], np.arange(e["cols"]), cfg.noise_mask) for s in seeds])
+            B = np.stack([noise(int(s) + e["off_b"], np.arange(e["rows"]), cfg.noise_mask) for s in seeds])
+            vote_kn = (B * fit[:, None]).T @ A
+            # blocked element index -> (k, n), mgpu.cu:1085-1089
+            idx = np.arange(n)
+            vote = vote_kn[(idx >> 2) // e["cols"] * 4 + (idx & 3), (idx >> 2) % e["cols"]]
+        else:
+            i = np.arange(n)
+            n1 = np.stack([noise(int(s) + e["off_a"], i, cfg.noise_mask) for s in seeds])
+            n2 = np.stack([noise(int(s) + e["off_b"], i, cfg.noise_mask) for s in seeds])
+            vote = (fit[:, None] * n1 * n2).sum(axis=0)
+        # apply_adam_update, mgpu.cu:1040-1064 (no bias correction; fractional accumulator moves the int8 weight)
+        g = -(vote.astype(f32))
+        w = model[sl].astype(np.int64)
+        m, v, acc = state["m"][sl], state["v"][sl], state["acc"][sl]
+        b1, b2 = f32(cfg.adam_beta1), f32(cfg.adam_beta2)
+        m = b1 * m + (f32(1.0) - b1) * g
+        v = b2 * v + (f32(1.0) - b2) * (g * g)
+        step = (-f32(lr * e["lr_scale"])) * (m / (np.sqrt(v) + f32(cfg.adam_eps)) + f32(cfg.adam_weight_decay) * w.astype(f32))
+        acc = acc + step
+        up, dn = acc >= f32(1.0), acc <= f32(-1.0)
+        w_new = np.where(up & (w < 127), w + 1, np.where(dn & (w > -127), w - 1, w))
+        acc = np.where(up, np.where(w < 127, acc - f32(1.0), f32(1.0)), np.where(dn, np.where(w > -127, acc + f32(1.0), f32(-1.0)), acc)).astype(f32)
+        changed += int(np.count_nonzero(w_new != w))
+        model[sl] = w_new.astype(np.int8)
+        state["m"][sl], state["v"][sl], state["acc"][sl] = m, v, acc
+    return changed

@@ -688,3 +688,30 @@ def test_two_restatements_of_the_forward_agree(orc, kw):
             assert np.array_equal(st["x_mlp"][l], tr["x_mlp"][l]), (m, l)
         assert np.array_equal(st["logits"], tr["logits"]), m
         assert loss == ref_loss, m
+
+
+def test_two_restatements_of_the_update_agree(orc):
+    """The whole AdamW ES update (votes of every tensor, float32 optimizer state, int8 weights, change count) in numpy
+    array arithmetic against the C++ oracle's element-by-element loops, over several steps that cross the +-1 thresholds."""
+    from oracle import forward_numpy as fn
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=24)
+    cfg = orc.config(**kw)
+    tt = orc.tensor_table(cfg)
+    rng = np.random.default_rng(8)
+    m1 = orc.init_model(cfg, 42)
+    m1[rng.integers(0, m1.size, 40)] = 127
+    m1[rng.integers(0, m1.size, 40)] = -127
+    m2 = m1.copy()
+    s1 = np.zeros(m1.size, orc.ADAM_DTYPE); s2 = s1.copy()
+    total = 0
+    for step in range(5):
+        fit = rng.integers(-1, 2, 12).astype(np.int32)
+        lr = np.float32(0.3 if step < 2 else 6.0)
+        n1 = orc.es_update_adam(cfg, m1, s1, fit, 900 + step, lr)
+        n2 = fn.es_update_adam(cfg, m2, s2, tt, fit, 900 + step, lr)
+        assert n1 == n2, step
+        assert np.array_equal(m1, m2), step
+        for f in ("m", "v", "acc"):
+            assert np.array_equal(s1[f].view(np.int32), s2[f].view(np.int32)), (step, f)
+        total += n1
+    assert total > 50
