@@ -26,7 +26,8 @@
  *       stated a second time, independently and in a different shape (numpy, all
  *       tokens of the window at once: oracle/forward_numpy.py), and the two must
  *       agree on every residual-stream tap, logit and loss; the same file states
- *       the whole AdamW update a second time.  Beyond the per-stage checks above
+ *       the whole AdamW update a second time, and oracle/gru_numpy.py does so for
+ *       the CPU program (egg_gru_oracle.cpp).  Beyond the per-stage checks above
  *       and that agreement the whole forward and the whole step are "parity unpinned".
  */
 #ifndef EGG_ORACLE_H

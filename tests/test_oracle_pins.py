@@ -715,3 +715,63 @@ def test_two_restatements_of_the_update_agree(orc):
             assert np.array_equal(s1[f].view(np.int32), s2[f].view(np.int32)), (step, f)
         total += n1
     assert total > 50
+
+
+def test_two_restatements_of_the_gru_program_agree(orc):
+    """oracle/gru_numpy.py restates full_trained_egg.c independently of egg_gru_oracle.cpp (named arrays and whole
+    matrix products instead of a blob and scalar loops); the two must agree on every value: noise vectors at counts
+    around the 16-wide blocks, perturbed products at both shifts and signs, the norm, the loss, two ES steps of
+    losses, fitness, recurrent state carried across the steps, and the updated weights."""
+    from oracle import gru_numpy as gn
+    L = orc.lib()
+    for count in (1, 15, 16, 17, 40):
+        st = C.c_uint32(987654321); out = np.zeros(count, np.int8)
+        L.orc_gru_noise_vector(C.byref(st), P(out), count)
+        ref, st2 = gn.noise_vector(987654321, count)
+        assert np.array_equal(out, ref) and st.value == st2, count
+
+    g = orc.gru_config(hidden=32, n_layers=2, seq_len=5, population=8, update_threshold=12)
+    rng = np.random.default_rng(77)
+    for rows, cols, shift in ((32, 32, 8), (128, 32, 8), (32, 128, 9), (256, 32, 8)):
+        x = rng.integers(-127, 128, cols).astype(np.int8)
+        W = rng.integers(-127, 128, rows * cols).astype(np.int8)
+        for sign in (1, -1, 0):
+            out = np.zeros(rows, np.int8)
+            L.orc_gru_matmul_perturbed(C.byref(g), P(x), P(W), P(out), rows, cols, C.c_uint32(31337 + rows), sign, shift)
+            assert np.array_equal(out, gn.matmul_perturbed(g, x, W, rows, cols, 31337 + rows, sign, shift)), (rows, cols, sign)
+    for scale in (0, 1, 3, 127):
+        x = rng.integers(-scale, scale + 1, 32).astype(np.int8)
+        w = rng.integers(-127, 128, 32).astype(np.int8)
+        out = np.zeros(32, np.int8)
+        L.orc_gru_ln(P(x), P(w), P(out), 32)
+        assert np.array_equal(out, gn.ln(x, w)), scale
+    tab = gn.exp2_table(4)
+    for _ in range(8):
+        lg = rng.integers(-127, 128, 256).astype(np.int8)
+        tgt = int(rng.integers(0, 256))
+        assert L.orc_gru_compute_loss(P(lg), 256, tgt, 4) == gn.compute_loss(tab, lg.astype(np.int64), tgt)
+
+    data = orc.zipf_bytes(4096)
+    m_c = orc.gru_init_model(g, 42)
+    # biases are zero after initialisation; give them values so the gate's clipped adds are exercised
+    views = gn.model_views(g, m_c)
+    views["gru_biases"][...] = rng.integers(-20, 21, views["gru_biases"].shape)
+    m_n = m_c.copy()
+    model_n = gn.model_views(g, m_n)
+    pairs = g.population // 2
+    s_c = np.zeros(g.population * g.n_layers * g.hidden, np.int8)
+    s_n = np.zeros((g.population, g.n_layers, g.hidden), np.int8)
+    moved = 0
+    for step in range(2):
+        seed = 5000 + 17 * step
+        loss_c, fit_c = orc.gru_population(g, m_c, data, step * g.seq_len, seed, 0, pairs, s_c)
+        loss_n, fit_n = gn.population(g, model_n, data, step * g.seq_len, seed, s_n)
+        assert np.array_equal(loss_c, loss_n), step
+        assert np.array_equal(fit_c, fit_n), step
+        assert np.array_equal(s_c.reshape(s_n.shape), s_n), step
+        before = m_c.copy()
+        L.orc_gru_update_all(C.byref(g), P(m_c), C.c_uint32(seed), P(fit_c))
+        gn.update_all(g, model_n, seed, fit_n)
+        assert np.array_equal(m_c, m_n), step
+        moved += np.count_nonzero(m_c != before)
+    assert s_n.any() and moved > 0
