@@ -519,6 +519,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = F + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
         p.w_dn = F + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
         p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
+        p.tab = ctx->d_q;            // free until the first layer's QKV projection writes it
         if (Q) {
             p.q_ln_w = Q + L.ln_init; p.q_ln_b = Q + L.ln_init_bias; p.q_b_up = Q + L.mlp_emb_bias_up; p.q_b_dn = Q + L.mlp_emb_bias_down;
             p.q_up = Q + L.w_emb_mlp_up; p.q_dn = Q + L.w_emb_mlp_down; p.q_emb = Q + L.embedding; p.q_emb_bias = Q + L.emb_bias;

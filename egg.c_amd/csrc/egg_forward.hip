@@ -130,7 +130,11 @@ struct MlpCfg {
     static constexpr int SITE = EGG_WAVES * 64;                       // ints per reduction site
     static constexpr int RED = CS > 1 ? 4 * SITE * 4 : 0;
     static constexpr int OCC = H == 256 ? 3 : 2;                      // workgroups per CU the kernel is built for
-    static int total(int sets) { return WBYTES + 256 + sets * PER_SET + XCHG + RED; }
+    // first block only: rank of every byte value among the values present in the member's window [256], wave counts
+    // [4 ints], and below hidden 256 the list of present values [256] (from hidden 256 on it lives in the table slot
+    // of the O projection's noise, which the first block does not use)
+    static constexpr int DEDUP = 256 + 16 + (H < 256 ? 256 : 0);
+    static int total(int sets, bool first) { return WBYTES + 256 + sets * PER_SET + XCHG + RED + (first ? DEDUP : 0); }
 };
 
 // FUSE: the host has checked sigma <= 7 and |noise| <= 15, which bounds |acc| * 2^sigma + |sb * a| below 2^31 for
@@ -233,15 +237,44 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
     const uint32_t pair_seed = *c.d_step_seed + (uint32_t)(member / 2);
     const int64_t spos = FIRST ? stream_pos_of(c, member) : 0;
 
-    for (int pass = 0; pass < tm.passes; pass++) {
-        const int t = (tm.tile0 + M::TPW * pass) * 32 + j;
+    // The first block (embedding, norm, MLP, residual, adaptive norm) has no attention in front of it: its result is a
+    // function of the member and the byte value alone.  It is therefore evaluated once per distinct byte value of the
+    // member's window -- row r of `p.tab` belongs to the r-th smallest value present -- and copied to every position
+    // that holds the value at the end.  (A workgroup that serves several members keeps the per-position form.)
+    const bool dedup = FIRST && p.tab != nullptr && tm.sets == 1;
+    uint8_t *rnk = reinterpret_cast<uint8_t *>(red) + M::RED;
+    int *wcnt = reinterpret_cast<int *>(rnk + 256);
+    uint8_t *uniq = H < 256 ? rnk + 272 : reinterpret_cast<uint8_t *>(exB);
+    int npass = tm.passes, nrows = T;
+    if (FIRST && dedup) {
+        static_assert(EGG_THREADS == 256, "one thread per byte value");
+        rnk[threadIdx.x] = 0;
+        __syncthreads();
+        for (int t = threadIdx.x; t < T; t += EGG_THREADS) rnk[c.data[spos + t]] = 1;
+        __syncthreads();
+        const bool present = rnk[threadIdx.x] != 0;
+        const unsigned long long bal = __ballot(present);
+        if (lane == 0) wcnt[wave] = __popcll(bal);
+        __syncthreads();
+        int below = 0;
+        nrows = 0;
+#pragma unroll
+        for (int w = 0; w < EGG_WAVES; w++) { const int n = wcnt[w]; if (w < wave) below += n; nrows += n; }
+        const int r = below + __popcll(bal & ((1ull << lane) - 1ull));
+        if (present) { rnk[threadIdx.x] = (uint8_t)r; uniq[r] = (uint8_t)threadIdx.x; }
+        __syncthreads();
+        npass = (nrows + 32 * M::TPW - 1) / (32 * M::TPW);
+    }
+
+    for (int pass = 0; pass < npass; pass++) {
+        const int t = (tm.tile0 + M::TPW * pass) * 32 + j;     // token position; with dedup, row of the table
         const size_t row = ((size_t)mloc * T + t) * H;
-        int8_t *xrow = p.x + row + col0;                 // this wave's slice of the residual row
+        int8_t *xrow = (FIRST && dedup ? p.tab : p.x) + row + col0;   // this wave's slice of the residual row
         v4i xs[NTS];
 
         if (FIRST) {
             // embedding stage (mgpu.cu:901-931)
-            const int tok = c.data[spos + t];
+            const int tok = dedup ? uniq[min(t, nrows - 1)] : c.data[spos + t];
             int a_tok = noise_from_hash(pair_seed + OFF_EMB, (uint32_t)tok, c.mask);
             if (ADAPT) a_tok *= p.q_emb[H + tok];        // a_tok * q(token); the table holds b_dim * q(hidden) * ns
             const uint32_t *E32 = reinterpret_cast<const uint32_t *>(p.embedding);
@@ -389,7 +422,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                     for (int k = 0; k < CS * NTU; k++) mid[k] = xch_get(xch, CS * NTU, tm.tslot, k, lane);
                 if (du + 1 < M::DNU) pf_dn(s, du + 1);
                 else if (it + 1 < M::NSUB) pf_up(sub_chunk(it + 1), 0);
-                else if (pass + 1 < tm.passes) pf_pass_first();
+                else if (pass + 1 < npass) pf_pass_first();
                 mfma_cols<M::PRDN / 2, NTS>(accd, mid + du * (M::PRDN / 2), cur, H, col0, lane);
             }
         }
@@ -413,6 +446,17 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         if (valid)
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, g, xnew[nt]);
+    }
+    if (FIRST && dedup) {
+        // every position takes the row of its byte value (16 bytes per thread and step)
+        __syncthreads();
+        constexpr int PARTS = H / 16;
+        for (int i = threadIdx.x; i < T * PARTS; i += EGG_THREADS) {
+            const int t = i / PARTS, part = i % PARTS;
+            const int r = rnk[c.data[spos + t]];
+            const v4i v = *reinterpret_cast<const v4i *>(p.tab + ((size_t)mloc * T + r) * H + part * 16);
+            *reinterpret_cast<v4i *>(p.x + ((size_t)mloc * T + t) * H + part * 16) = v;
+        }
     }
 }
 
@@ -1016,7 +1060,7 @@ template <int H>
 static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
     const int sets = tile_map_sets(p.c.T, MlpCfg<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
-    size_t lds = MlpCfg<H>::total(sets);
+    size_t lds = MlpCfg<H>::total(sets, first);
     const bool fuse = p.c.sigma <= 7 && p.c.mask <= 15;
     if (p.q_ln_w) {      // adaptive noise overlay: one (unfused) variant
         if (first) hipLaunchKernelGGL((k_mlp<H, true, false, true>), grid, block, lds, s, p);
@@ -1113,12 +1157,12 @@ template <int H>
 static hipError_t prepare_h(int T) {
     const int sets = tile_map_sets(T, Shape<H>::CS);
     const int msets = tile_map_sets(T, MlpCfg<H>::CS);
-    SET_LDS((k_mlp<H, true, true, false>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, false, true, false>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, true, false, false>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, false, false, false>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, true, false, true>), MlpCfg<H>::total(msets));
-    SET_LDS((k_mlp<H, false, false, true>), MlpCfg<H>::total(msets));
+    SET_LDS((k_mlp<H, true, true, false>), MlpCfg<H>::total(msets, true));
+    SET_LDS((k_mlp<H, false, true, false>), MlpCfg<H>::total(msets, false));
+    SET_LDS((k_mlp<H, true, false, false>), MlpCfg<H>::total(msets, true));
+    SET_LDS((k_mlp<H, false, false, false>), MlpCfg<H>::total(msets, false));
+    SET_LDS((k_mlp<H, true, false, true>), MlpCfg<H>::total(msets, true));
+    SET_LDS((k_mlp<H, false, false, true>), MlpCfg<H>::total(msets, false));
     SET_LDS((k_qkv<H, false>), QkvCfg<H>::total(sets));
     SET_LDS((k_qkv<H, true>), QkvCfg<H>::total(sets));
     SET_LDS((k_head<H, false>), HeadLds<H>::TOTAL);

@@ -54,6 +54,7 @@ struct MlpParams {
     const int8_t *ao;            // [n_members][T][H] slot order
     int8_t *x;                   // [n_members][T][H] slot order, read (if !FIRST) and written
     int8_t *x_mid;               // optional tap: residual stream after attention (may be null)
+    int8_t *tab;                 // FIRST: [n_members][T][H] scratch rows, one per distinct byte value of a member's window (null: one row per position)
     // adaptive noise overlay (all null when it is off): q values (0..64) of the tensors above; a matrix has its
     // input-row values first and its output-column values right behind them
     const int8_t *q_ln_w, *q_ln_b, *q_b_up, *q_b_dn, *q_up, *q_dn, *q_o, *q_emb, *q_emb_bias;

@@ -187,6 +187,40 @@ def test_forward_chunked_and_offsets(pkg, orc, dev, hidden, head_dim, seq_len):
     ctx.close()
 
 
+@pytest.mark.parametrize("hidden,head_dim,distinct", [(256, 64, (1, 2, 64, 65, 128, 129, 256)), (64, 32, (1, 128, 129, 256)),
+                                                      (512, 64, (33, 200))], ids=["h256", "h64", "h512"])
+def test_first_block_with_repeated_bytes(pkg, orc, dev, hidden, head_dim, distinct):
+    """The block in front of the first attention layer is evaluated once per distinct byte value of a member's window:
+    windows with 1 ... 256 distinct values (around the multiples of the tokens a workgroup handles per pass), in
+    scrambled order, give the oracle's residual stream and losses."""
+    import torch
+    T = 256
+    kw = dict(hidden=hidden, head_dim=head_dim, n_layers=1, seq_len=T, population=2)
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 11)
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_upload(model)
+    ctx.enable_taps(True)
+    rng = np.random.default_rng(31)
+    for U in distinct:
+        values = rng.permutation(256)[:U]
+        window = rng.permutation(np.concatenate([values, values[rng.integers(0, U, T - U)]]))
+        data = np.zeros(4 * T, np.uint8)
+        start = 17
+        data[start:start + T] = window.astype(np.uint8)
+        data[start + T] = values[0]                      # the last position's target
+        assert len(set(data[start:start + T].tolist())) == U
+        d_data = _t(dev, data)
+        d_loss = torch.zeros(2, dtype=torch.int32, device=dev)
+        ctx.population_forward(d_data.data_ptr(), len(data), start, 4242 + U, 0, 2, d_loss.data_ptr())
+        ctx.sync()
+        for m in range(2):
+            ref_loss, tr = orc.forward_member(ocfg, model, data, start, 4242 + U, m, trace=True)
+            assert np.array_equal(ctx.tap("x_init", m), tr["x_init"]), (U, m)
+            assert int(d_loss[m].item()) == ref_loss, (U, m)
+    ctx.close()
+
+
 def test_fitness(pkg, orc, dev):
     import torch
     ctx = pkg.Context(pkg.default_config(**SMALL))
