@@ -58,6 +58,9 @@ def main():
     data = orc.zipf_bytes(args.data_mib << 20, seed=1234)
     d_data = torch.from_numpy(data).to(dev)
     n = len(data)
+    # the block in front of the first attention layer is evaluated once per distinct byte value of a member's window
+    # (exact: it does not depend on the position); report how many values the synthetic stream's windows hold
+    distinct = float(np.mean([len(np.unique(data[i:i + T])) for i in range(0, n - T, max(1, (n - T) // 512))]))
 
     def run_steps(k, first_step, seed, graph):
         for i in range(k):
@@ -258,7 +261,8 @@ def main():
         "dtype": "int8 (int32 accumulate), f32 optimizer state", "data": "synthetic Zipf(1.1) bytes, seed 1234",
         "config": {"workload": f"full ES step: Int8NativeFormer L={L} H={H} heads={H // HD} T={T}, population {P}, "
                                f"forward+fitness+vote+AdamW, eager launches (chunk {chunk} members)",
-                   "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss},
+                   "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss,
+                   "distinct_bytes_per_window": round(distinct, 1)},
         "roofline": roofline, "kernels": per_class, "microbench_c2": mb,
         "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }
