@@ -472,56 +472,43 @@ struct QkvCfg {
     static constexpr int XCHG = 0;             // the normalised input is exchanged through the idle W buffer
     static constexpr int SITE = EGG_WAVES * 64;
     static constexpr int RED = CS > 1 ? 2 * SITE * 4 : 0;       // two reduction sites used alternately
-    static constexpr int OCC = 2;                              // workgroups per CU the kernel is built for
+    static constexpr int OCC = H == 256 ? 3 : 2;               // workgroups per CU the kernel is built for
     static int total(int sets) { return WBYTES + sets * PER_SET + XCHG + RED; }
 };
 
 // apply_rope_integer (mgpu.cu:624-644) on the raw accumulators of one token.  The (cos, sin) pairs repeat every
-// head, so a lane needs only the head_dim/32 * 8 pairs of its own slots; they are loaded once per token tile
-// (RopeTab) and reused for every head of Q and K.
-// The reference evaluates (ve*c -+ vo*s + 2^(bit-1)) >> bit in int64, and so does this code.
-struct RopeTab { int c[2][4][2], s[2][4][2]; };
-__device__ __forceinline__ void rope_load(RopeTab &rt, const int32_t *rope_row, int head_dim, int g) {
-    const int hdt = head_dim >> 5;                 // column groups per head: 1 or 2
-#pragma unroll
-    for (int h2 = 0; h2 < 2; h2++)
-#pragma unroll
-        for (int q = 0; q < 4; q++)
-#pragma unroll
-            for (int ep = 0; ep < 2; ep++) {
-                int n = 32 * (h2 < hdt ? h2 : 0) + 8 * q + 4 * g + 2 * ep;
-                int2 v = *reinterpret_cast<const int2 *>(rope_row + 2 * (n >> 1));
-                rt.c[h2][q][ep] = v.x;
-                rt.s[h2][q][ep] = v.y;
-            }
-}
-// The NT column groups must start at a head boundary.  64-bit multiply-adds (v_mad_i64_i32, full rate on gfx950) state
-// the reference's int64 expression directly; the shifted result fits 32 bits like the reference's AccumType.
+// head, so a lane needs only the head_dim/32 * 8 pairs of its own slots.
+// The reference evaluates (ve*c -+ vo*s + 2^(bit-1)) >> bit in int64, and so does this code: 64-bit multiply-adds
+// (v_mad_i64_i32, full rate on gfx950); the shifted result fits 32 bits like the reference's AccumType.
+// The NT column groups must start at a head boundary.  The
+// pairs are read where they are used (one 16-byte load per two pairs, cache hits): holding a token's 16 pairs in
+// registers across the three projections costs the 32 registers that separate two from three workgroups per CU.
 template <int NT>
-__device__ __forceinline__ void rope_inplace(v16i *acc, const RopeTab &rt, int head_dim, int bit) {
+__device__ __forceinline__ void rope_inplace(v16i *acc, const int32_t *rope_row, int head_dim, int g, int bit) {
     const int hdt = head_dim >> 5;
     const long long half = 1ll << (bit - 1);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++)
 #pragma unroll
-        for (int q = 0; q < 4; q++)
+        for (int q = 0; q < 4; q++) {
+            const int n = 32 * (hdt == 2 ? (nt & 1) : 0) + 8 * q + 4 * g;
+            const v4i cs = *reinterpret_cast<const v4i *>(rope_row + n);        // c0 s0 c1 s1
 #pragma unroll
             for (int ep = 0; ep < 2; ep++) {
-                const int cc = (hdt == 2) ? rt.c[nt & 1][q][ep] : rt.c[0][q][ep];
-                const int ss = (hdt == 2) ? rt.s[nt & 1][q][ep] : rt.s[0][q][ep];
+                const int cc = cs[2 * ep], ss = cs[2 * ep + 1];
                 const int ve = acc[nt][4 * q + 2 * ep], vo = acc[nt][4 * q + 2 * ep + 1], nvo = -vo;
                 const long long re = (long long)nvo * ss + ((long long)ve * cc + half);
                 const long long ro = (long long)vo * cc + ((long long)ve * ss + half);
-                // bits [bit+31 : bit] of the 64-bit sums (0 < bit < 32): the arithmetic shift, truncated to 32 bits
                 acc[nt][4 * q + 2 * ep] = (int)__builtin_amdgcn_alignbit((unsigned)(re >> 32), (unsigned)re, (unsigned)bit);
                 acc[nt][4 * q + 2 * ep + 1] = (int)__builtin_amdgcn_alignbit((unsigned)(ro >> 32), (unsigned)ro, (unsigned)bit);
             }
+        }
 }
 
 // ADAPT: the d-eggs adaptive noise overlay is on (de/include/model/layers.cuh:313-351): output-side noise and vector
 // noise are scaled when the per-member tables are filled, the input-side sums take the slow term-by-term form.
 template <int H, bool ADAPT>
-__global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p) {
+__global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv(QkvParams p) {
     typedef QkvCfg<H> Q;
     constexpr int CS = Q::CS, KS = Q::KS, NTS = Q::NTS, HS = Q::HS;
     extern __shared__ __align__(16) int8_t smem[];
@@ -591,8 +578,6 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
                 exchange_operand<CS, NTS, KS, Q::TPW, Q::UNIT>(ws.other, tm, lane, mine, nrm);
             }
         }
-        RopeTab rt;
-        rope_load(rt, c.rope_lut + (size_t)t * c.head_dim, c.head_dim, g);
 #pragma unroll 1
         for (int which = 0; which < 3; which++) {
             const int8_t *W = which == 0 ? p.w_q : (which == 1 ? p.w_k : p.w_v);
@@ -612,7 +597,7 @@ __global__ void __launch_bounds__(EGG_THREADS, QkvCfg<H>::OCC) k_qkv(QkvParams p
                 mfma_cols<Q::PR / 2, NTS>(acc, nrm + u * (Q::PR / 2), cur, H, col0, lane);
             }
             add_perturb8<NTS>(acc, sb, An, col0, c.sigma, g);
-            if (which < 2) rope_inplace<NTS>(acc, rt, c.head_dim, c.rope_scale_bit);
+            if (which < 2) rope_inplace<NTS>(acc, c.rope_lut + (size_t)t * c.head_dim, c.head_dim, g, c.rope_scale_bit);
             const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red + ((1 + which) & 1) * Q::SITE, tm, lane);
             v4i o[NTS];
             adaptive_scale<NTS>(acc, mx, o);
