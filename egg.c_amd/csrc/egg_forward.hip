@@ -612,10 +612,12 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
 // One wave per (member, head).  S^T = K.Q^T per 32x32 tile (lane = query token), two passes over the
 // causal context (row max, then LUT weights), O^T = V^T.P^T with the 19-bit weights split into three
 // 7-bit planes so the weighted sum stays exact on the int8 MFMA.  The LDS table holds, per exp-LUT index,
-// the weight and its three planes packed as bytes, so the planes of four context positions are regrouped with
-// byte permutes instead of shifts and masks.  Only the diagonal tile needs the causal mask.
-__device__ __forceinline__ void attn_weights(const v16i &s, const int2 *lut, int mxs, int shift, bool diag, int ct, int t, int g,
-                                             v4i *pw, int &den) {
+// the three planes packed as bytes (4-byte entries: the gathers are what loads the LDS pipe), so the planes of four
+// context positions are regrouped with byte permutes instead of shifts and masks; the sum of the weights is rebuilt
+// from per-plane byte sums.  Only the diagonal tile needs the causal mask.
+// den[pl] accumulates the plane sums; the sum of the weights is den[0] + 128 den[1] + 16384 den[2] (attn_den).
+__device__ __forceinline__ void attn_weights(const v16i &s, const int *lut, int mxs, int shift, bool diag, int ct, int t, int g,
+                                             v4i *pw, int *den) {
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         int pk[4];
@@ -623,10 +625,8 @@ __device__ __forceinline__ void attn_weights(const v16i &s, const int2 *lut, int
         for (int e = 0; e < 4; e++) {
             int idx = mxs - (s[4 * q + e] >> shift);
             idx = min(255, max(0, idx));
-            int2 wp = lut[idx];
-            if (diag && (32 * ct + 8 * q + 4 * g + e) > t) { wp.x = 0; wp.y = 0; }
-            den += wp.x;
-            pk[e] = wp.y;
+            pk[e] = lut[idx];
+            if (diag && (32 * ct + 8 * q + 4 * g + e) > t) pk[e] = 0;
         }
         // bytes of pk[e]: plane0, plane1, plane2, 0  ->  one dword per plane holding the four positions
         const int ab_lo = __builtin_amdgcn_perm(pk[1], pk[0], 0x05010400);   // a0 b0 a1 b1
@@ -636,15 +636,18 @@ __device__ __forceinline__ void attn_weights(const v16i &s, const int2 *lut, int
         pw[0][q] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100);
         pw[1][q] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302);
         pw[2][q] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100);
+#pragma unroll
+        for (int pl = 0; pl < 3; pl++) den[pl] = dot4(pw[pl][q], 0x01010101, den[pl]);
     }
 }
+__device__ __forceinline__ int attn_den(const int *den) { return den[0] + (den[1] << 7) + (den[2] << 14); }
 
 template <int HD, int CT>
 __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnParams p) {
     constexpr int KS = HD / 32, DT = HD / 32;
     constexpr int T = CT * 32;
     extern __shared__ __align__(16) int8_t smem[];
-    int2 *lut = reinterpret_cast<int2 *>(smem);
+    int *lut = reinterpret_cast<int *>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     int8_t *vl = smem + 2048 + (size_t)wave * T * HD;
 
@@ -658,7 +661,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
 
     for (int i = threadIdx.x; i < 256; i += EGG_THREADS) {
         const int w = c.exp_lut[i];
-        lut[i] = make_int2(w, (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16));
+        lut[i] = (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16);
     }
     // V tile of this (member, head) -> LDS rows [ctx][HD]
     for (int i = lane; i < T * HD / 16; i += 64) {
@@ -740,7 +743,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
         v16i o[3][DT];
 #pragma unroll
         for (int pl = 0; pl < 3; pl++) zero_acc<DT>(o[pl]);
-        int den = 0;
+        int dpl[3] = {0, 0, 0};
 #pragma unroll
         for (int ct = 0; ct < CT; ct++) {
             if (ct <= qt) {
@@ -753,8 +756,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
                 v4i pw[3];
-                if (ct == qt) attn_weights(s, lut, mxs, c.shift_attn, true, ct, t, g, pw, den);
-                else attn_weights(s, lut, mxs, c.shift_attn, false, ct, t, g, pw, den);
+                if (ct == qt) attn_weights(s, lut, mxs, c.shift_attn, true, ct, t, g, pw, dpl);
+                else attn_weights(s, lut, mxs, c.shift_attn, false, ct, t, g, pw, dpl);
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -762,6 +765,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                         o[pl][dt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vt[ct][dt], pw[pl], o[pl][dt], 0, 0, 0);
             }
         }
+        int den = attn_den(dpl);
         den += other_half(den);
         // Truncating quotient num / den with one reciprocal per token.  num and den are integers below 2^53, the
         // quotient is at most 127 in magnitude, and a non-integer quotient is at least 1/den >= 2^-27 away from
@@ -796,17 +800,18 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
 template <int HD, int CT>
 struct AttnWg {
     static constexpr int T = CT * 32, ROWS = T * HD;               // bytes of one K or V head tile
-    static constexpr int LDS = 2048 + 2 * ROWS;                    // LUT | rows (V, then K) | V^T fragments
-    static constexpr int OCC = (2 * LDS <= 80 * 1024) ? 2 : 1;
+    static constexpr int LDS = 2048 + 3 * ROWS;                    // LUT | rows (V, then K) | V^T fragments | Q rows
+    static constexpr int OCC = (3 * LDS <= 160 * 1024) ? 3 : 1;    // workgroups per CU the kernel is built for
 };
 template <int HD, int CT>
 __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(AttnParams p) {
     constexpr int KS = HD / 32, DT = HD / 32, T = CT * 32, CH = HD / 16, RPL = 128 / HD;
     static_assert(CT % 8 == 0, "query tiles are dealt in groups of eight");
     extern __shared__ __align__(16) int8_t smem[];
-    int2 *lut = reinterpret_cast<int2 *>(smem);
+    int *lut = reinterpret_cast<int *>(smem);
     int8_t *rows = smem + 2048;
     int8_t *vfrag = rows + AttnWg<HD, CT>::ROWS;
+    int8_t *qrows = vfrag + AttnWg<HD, CT>::ROWS;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const FwdCommon &c = p.c;
     const int H = c.H, NH = H / HD;
@@ -816,13 +821,34 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
 
     for (int i = threadIdx.x; i < 256; i += EGG_THREADS) {
         const int w = c.exp_lut[i];
-        lut[i] = make_int2(w, (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16));
+        lut[i] = (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16);
     }
-    // V rows of this (member, head) -> LDS [ctx][HD]
-    for (int i = threadIdx.x; i < T * CH; i += EGG_THREADS) {
-        int cx = i / CH, part = i % CH;
-        *reinterpret_cast<v4i *>(rows + (size_t)cx * HD + part * 16) =
-            *reinterpret_cast<const v4i *>(p.v + base + (size_t)cx * H + part * 16);
+    // the K rows are requested now and held in registers until the V rows have left the shared row area, so that their
+    // latency overlaps the V stage instead of following it
+    constexpr int PER = T * CH / EGG_THREADS;
+    static_assert(T * CH % EGG_THREADS == 0, "row chunks are dealt evenly to the threads");
+    v4i kreg[PER];
+#pragma unroll
+    for (int n = 0; n < PER; n++) {
+        const int i = threadIdx.x + n * EGG_THREADS, cx = i / CH, part = i % CH;
+        kreg[n] = *reinterpret_cast<const v4i *>(p.k + base + (size_t)cx * H + part * 16);
+    }
+    // Q rows -> LDS in the K rows' layout (every wave reads its query tiles from there: one round of global latency
+    // for the whole workgroup instead of one per query tile), V rows of this (member, head) -> LDS [ctx][HD]
+    {
+        v4i qreg[PER], vreg[PER];
+#pragma unroll
+        for (int n = 0; n < PER; n++) {
+            const int i = threadIdx.x + n * EGG_THREADS, cx = i / CH, part = i % CH;
+            qreg[n] = *reinterpret_cast<const v4i *>(p.q + base + (size_t)cx * H + part * 16);
+            vreg[n] = *reinterpret_cast<const v4i *>(p.v + base + (size_t)cx * H + part * 16);
+        }
+#pragma unroll
+        for (int n = 0; n < PER; n++) {
+            const int i = threadIdx.x + n * EGG_THREADS, cx = i / CH, part = i % CH;
+            *reinterpret_cast<v4i *>(rows + (size_t)cx * HD + part * 16) = vreg[n];
+            *reinterpret_cast<v4i *>(qrows + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) = qreg[n];
+        }
     }
     __syncthreads();
     // V^T fragments: A-operand row i = natural head dim d = 32dt + i, stored at slot position 16g'+4q'+e'
@@ -843,10 +869,10 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
     }
     __syncthreads();
     // K rows take the place of the V rows; chunk c of row r sits at c ^ ((r / RPL) % CH) to spread the banks
-    for (int i = threadIdx.x; i < T * CH; i += EGG_THREADS) {
-        int cx = i / CH, part = i % CH;
-        *reinterpret_cast<v4i *>(rows + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) =
-            *reinterpret_cast<const v4i *>(p.k + base + (size_t)cx * H + part * 16);
+#pragma unroll
+    for (int n = 0; n < PER; n++) {
+        const int i = threadIdx.x + n * EGG_THREADS, cx = i / CH, part = i % CH;
+        *reinterpret_cast<v4i *>(rows + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) = kreg[n];
     }
     __syncthreads();
     auto score_tile = [&](int ct, const v4i *qop) {
@@ -870,17 +896,20 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
         const int t = qt * 32 + j;
         v4i qop[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) qop[ks] = load_op(p.q + base + (size_t)t * H, ks, g);
+        for (int ks = 0; ks < KS; ks++)
+            qop[ks] = *reinterpret_cast<const v4i *>(qrows + (size_t)t * HD + (((ks * 2 + g) ^ ((t / RPL) % CH)) * 16));
         // pass 1: per-head maximum score over ctx <= t (mgpu.cu:795-802)
+        // (both passes issue the score MFMAs of the next context tile before they work on the current one)
         int mx = INT_MIN;
-#pragma unroll 2
-        for (int ct = 0; ct < qt; ct++) {
-            const v16i s = score_tile(ct, qop);
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) mx = max(max(mx, s[r]), s[r + 1]);
-        }
         {
-            const v16i s = score_tile(qt, qop);
+            v16i s = score_tile(0, qop);
+#pragma unroll 2
+            for (int ct = 0; ct < qt; ct++) {
+                const v16i sn = score_tile(ct + 1, qop);
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) mx = max(max(mx, s[r]), s[r + 1]);
+                s = sn;
+            }
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 int cx = 32 * qt + ((r >> 2) << 3) + (g << 2) + (r & 3);
@@ -893,11 +922,10 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
         v16i o[3][DT];
 #pragma unroll
         for (int pl = 0; pl < 3; pl++) zero_acc<DT>(o[pl]);
-        int den = 0;
-        auto weigh_tile = [&](int ct, bool diag) {
-            const v16i s = score_tile(ct, qop);
+        int dpl[3] = {0, 0, 0};
+        auto weigh_tile = [&](const v16i &s, int ct, bool diag) {
             v4i pw[3];
-            attn_weights(s, lut, mxs, c.shift_attn, diag, ct, t, g, pw, den);
+            attn_weights(s, lut, mxs, c.shift_attn, diag, ct, t, g, pw, dpl);
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
@@ -907,9 +935,17 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
             }
             __builtin_amdgcn_s_setprio(0);
         };
+        {
+            v16i s = score_tile(0, qop);
 #pragma unroll 2
-        for (int ct = 0; ct < qt; ct++) weigh_tile(ct, false);
-        weigh_tile(qt, true);
+            for (int ct = 0; ct < qt; ct++) {
+                const v16i sn = score_tile(ct + 1, qop);
+                weigh_tile(s, ct, false);
+                s = sn;
+            }
+            weigh_tile(s, qt, true);
+        }
+        int den = attn_den(dpl);
         den += other_half(den);
         // truncating quotient with one reciprocal per token, see k_attn
         const double rden = (1.0 + 0x1p-40) / (double)(den ? den : 1);
