@@ -201,6 +201,7 @@ def main():
         fwd_ms = sum(tm[k][1] for k in ("mlp_first", "qkv", "attn", "mlp", "head"))
         upd_ms = tm["update_matrix"][1] + tm["update_vector"][1]
         c5 = {"value": P5 * 512 / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3, "forward_ms": fwd_ms, "update_ms": upd_ms,
+              "kernel_avg_ms": {k: round(tm[k][1] / tm[k][0], 4) for k in ("mlp_first", "qkv", "attn", "mlp", "head") if tm[k][0]},
               "k_mlp_frac_mfma": (2 * 9 * 512 * 512 * P5 * 512) / (tm["mlp"][1] / tm["mlp"][0] * 1e-3) / PEAK_INT8_OPS,
               "workload": f"hidden 512, 8 heads, seq 512, 8 layers, ternary-packed weights (unpacked on upload, weight limit 1), "
                           f"population {P5} (one chunk), forward+fitness+vote+Muon; "

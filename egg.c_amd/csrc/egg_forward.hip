@@ -800,8 +800,11 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
 template <int HD, int CT>
 struct AttnWg {
     static constexpr int T = CT * 32, ROWS = T * HD;               // bytes of one K or V head tile
-    static constexpr int LDS = 2048 + 3 * ROWS;                    // LUT | rows (V, then K) | V^T fragments | Q rows
-    static constexpr int OCC = (3 * LDS <= 160 * 1024) ? 3 : 1;    // workgroups per CU the kernel is built for
+    // The Q rows of all query tiles go through LDS as well when three workgroups per CU still fit; otherwise (sequence
+    // 512) every query tile loads its operand from global memory and two workgroups share a CU.
+    static constexpr bool QLDS = 3 * (2048 + 3 * ROWS) <= 160 * 1024;
+    static constexpr int LDS = 2048 + (QLDS ? 3 : 2) * ROWS;       // LUT | rows (V, then K) | V^T fragments | Q rows
+    static constexpr int OCC = QLDS ? 3 : (2 * LDS <= 160 * 1024 ? 2 : 1);    // workgroups per CU the kernel is built for
 };
 template <int HD, int CT>
 __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(AttnParams p) {
@@ -836,18 +839,19 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
     // Q rows -> LDS in the K rows' layout (every wave reads its query tiles from there: one round of global latency
     // for the whole workgroup instead of one per query tile), V rows of this (member, head) -> LDS [ctx][HD]
     {
-        v4i qreg[PER], vreg[PER];
+        constexpr bool QLDS = AttnWg<HD, CT>::QLDS;
+        v4i qreg[QLDS ? PER : 1], vreg[PER];
 #pragma unroll
         for (int n = 0; n < PER; n++) {
             const int i = threadIdx.x + n * EGG_THREADS, cx = i / CH, part = i % CH;
-            qreg[n] = *reinterpret_cast<const v4i *>(p.q + base + (size_t)cx * H + part * 16);
+            if constexpr (QLDS) qreg[n] = *reinterpret_cast<const v4i *>(p.q + base + (size_t)cx * H + part * 16);
             vreg[n] = *reinterpret_cast<const v4i *>(p.v + base + (size_t)cx * H + part * 16);
         }
 #pragma unroll
         for (int n = 0; n < PER; n++) {
             const int i = threadIdx.x + n * EGG_THREADS, cx = i / CH, part = i % CH;
             *reinterpret_cast<v4i *>(rows + (size_t)cx * HD + part * 16) = vreg[n];
-            *reinterpret_cast<v4i *>(qrows + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) = qreg[n];
+            if constexpr (QLDS) *reinterpret_cast<v4i *>(qrows + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) = qreg[n];
         }
     }
     __syncthreads();
@@ -896,8 +900,11 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
         const int t = qt * 32 + j;
         v4i qop[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++)
-            qop[ks] = *reinterpret_cast<const v4i *>(qrows + (size_t)t * HD + (((ks * 2 + g) ^ ((t / RPL) % CH)) * 16));
+        for (int ks = 0; ks < KS; ks++) {
+            if constexpr (AttnWg<HD, CT>::QLDS)
+                qop[ks] = *reinterpret_cast<const v4i *>(qrows + (size_t)t * HD + (((ks * 2 + g) ^ ((t / RPL) % CH)) * 16));
+            else qop[ks] = load_op(p.q + base + (size_t)t * H, ks, g);
+        }
         // pass 1: per-head maximum score over ctx <= t (mgpu.cu:795-802)
         // (both passes issue the score MFMAs of the next context tile before they work on the current one)
         int mx = INT_MIN;
