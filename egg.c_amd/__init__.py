@@ -178,7 +178,7 @@ class Context:
         self._h = C.c_void_p()
         rc = lib().egg_ctx_create(C.byref(cfg), C.byref(self._h))
         if rc != 0:
-            raise EggError(f"egg_ctx_create failed with {rc} (unsupported configuration or HIP error)")
+            raise EggError(f"egg_ctx_create failed with {rc}: {lib().egg_last_error(None).decode()}")
 
     def close(self):
         if self._h:

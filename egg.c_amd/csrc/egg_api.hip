@@ -168,28 +168,39 @@ static void free_all(egg_ctx *ctx) {
     if (ctx->own_stream && ctx->stream) (void)hipStreamDestroy(ctx->stream);
 }
 
+// why the last egg_ctx_create of this thread failed (there is no context to hold the message yet)
+static thread_local std::string g_create_err;
+static int refuse(const char *why) { g_create_err = why; return EGG_E_INVALID; }
+
 extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
-    if (!cfg || !out) return EGG_E_INVALID;
+    if (!cfg || !out) return refuse("egg_ctx_create: null argument");
     *out = nullptr;
     const egg_config &c = *cfg;
-    if (!(c.hidden == 64 || c.hidden == 128 || c.hidden == 256 || c.hidden == 512)) return EGG_E_INVALID;
-    if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return EGG_E_INVALID;
-    if (!(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256 || c.seq_len == 512)) return EGG_E_INVALID;
-    if (c.vocab != 256 || c.n_layers < 1 || c.population < 2 || (c.population & 1)) return EGG_E_INVALID;
+    if (!(c.hidden == 64 || c.hidden == 128 || c.hidden == 256 || c.hidden == 512)) return refuse("hidden must be 64, 128, 256 or 512");
+    if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return refuse("head_dim must be 32 or 64 and divide hidden");
+    if (!(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256 || c.seq_len == 512))
+        return refuse("seq_len must be 32, 64, 128, 256 or 512");
+    if (c.vocab != 256) return refuse("vocab must be 256 (byte-level model)");
+    if (c.n_layers < 1 || c.population < 2 || (c.population & 1)) return refuse("n_layers >= 1 and an even population >= 2 are required");
     // shift amounts and table scales the kernels can state in 32-bit shifts / 64-bit multiply-adds
     auto in_range = [](int v, int lo, int hi) { return v >= lo && v <= hi; };
-    if (!in_range(c.rope_scale_bit, 1, 30) || !in_range(c.softmax_scale_bit, 1, 30) || !in_range(c.noise_mask, 0, 127) ||
-        !in_range(c.fixed_point + c.sigma_shift, 0, 24) || !in_range(c.sigma_shift_vector, 0, 24) || !in_range(c.shift_attn, 0, 24) ||
+    if (!in_range(c.rope_scale_bit, 1, 30) || !in_range(c.softmax_scale_bit, 1, 30)) return refuse("rope_scale_bit and softmax_scale_bit must be 1..30");
+    if (!in_range(c.noise_mask, 0, 127)) return refuse("noise_mask must be 0..127");
+    if (!in_range(c.fixed_point + c.sigma_shift, 0, 24) || !in_range(c.sigma_shift_vector, 0, 24) || !in_range(c.shift_attn, 0, 24) ||
         !in_range(c.shift_out, 0, 24) || !in_range(c.shift_logit, 0, 24) || !in_range(c.shift_mlp_up, 0, 24) ||
-        !in_range(c.shift_mlp_down, 0, 24)) return EGG_E_INVALID;
+        !in_range(c.shift_mlp_down, 0, 24)) return refuse("shift amounts must be 0..24");
     // the standard norm divides x * (gain + noise) by the row mean with a 32-bit multiply-high that is exact up to 2^17
-    if (127 * (127 + ((c.noise_mask * c.noise_mask) >> c.sigma_shift_vector)) > (1 << 17)) return EGG_E_INVALID;
-    if (!in_range(c.weight_limit, 1, 127)) return EGG_E_INVALID;
+    if (127 * (127 + ((c.noise_mask * c.noise_mask) >> c.sigma_shift_vector)) > (1 << 17))
+        return refuse("noise_mask^2 >> sigma_shift_vector is too large for the norm's exact division");
+    if (!in_range(c.weight_limit, 1, 127)) return refuse("weight_limit must be 1..127");
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
     ctx->L = make_layout(c);
     build_tensor_table(ctx);
-    auto bail = [&](int code, const char *what, hipError_t e) { fprintf(stderr, "egg_ctx_create: %s: %s\n", what, hipGetErrorString(e)); free_all(ctx); delete ctx; return code; };
+    auto bail = [&](int code, const char *what, hipError_t e) {
+        g_create_err = std::string(what) + ": " + hipGetErrorString(e);
+        free_all(ctx); delete ctx; return code;
+    };
 #define CR(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return bail(EGG_E_HIP, #call, e_); } while (0)
     CR(hipStreamCreate(&ctx->stream)); ctx->own_stream = true;
     CR(egg_prepare_forward(c.hidden, c.head_dim, c.seq_len));
@@ -290,7 +301,7 @@ extern "C" void egg_ctx_destroy(egg_ctx *ctx) {
     free_all(ctx);
     delete ctx;
 }
-extern "C" const char *egg_last_error(const egg_ctx *ctx) { return ctx ? ctx->err.c_str() : "null context"; }
+extern "C" const char *egg_last_error(const egg_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_err.c_str(); }
 extern "C" int egg_ctx_set_stream(egg_ctx *ctx, void *s) {
     if (!ctx) return EGG_E_INVALID;
     if (ctx->captured) return fail(ctx, EGG_E_STATE, "stream cannot change after egg_step_capture");

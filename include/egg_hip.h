@@ -64,6 +64,7 @@ void egg_default_config(egg_config *cfg);
 /* init_tables + cudaMemcpyToSymbol + per-GPU allocation (mgpu.cu:394-426, :1442-1489) */
 int  egg_ctx_create(const egg_config *cfg, egg_ctx **out);
 void egg_ctx_destroy(egg_ctx *ctx);
+/* message of the last failed call on ctx; with ctx == NULL, why this thread's last egg_ctx_create failed */
 const char *egg_last_error(const egg_ctx *ctx);
 /* run on a caller-provided hipStream_t instead of the context's own (d-eggs update_stream, de/src/worker.cu:352-357) */
 int  egg_ctx_set_stream(egg_ctx *ctx, void *hip_stream);

@@ -55,3 +55,18 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "one GPU" in (r.stdout + r.stderr)
+
+
+def test_unsupported_configurations_are_refused_with_a_reason(pkg):
+    """egg_ctx_create validates the configuration before it touches the device, so the refusals (and the reason
+    egg_last_error(NULL) keeps for them) can be checked without a GPU."""
+    lib = pkg.lib()
+    for kw, word in ((dict(hidden=100), "hidden"), (dict(head_dim=48), "head_dim"), (dict(seq_len=48), "seq_len"),
+                     (dict(population=7), "population"), (dict(rope_scale_bit=31), "rope_scale_bit"),
+                     (dict(noise_mask=127, sigma_shift_vector=0), "noise_mask"), (dict(weight_limit=0), "weight_limit"),
+                     (dict(shift_mlp_up=40), "shift")):
+        cfg = pkg.default_config(**kw)
+        h = ctypes.c_void_p()
+        rc = lib.egg_ctx_create(ctypes.byref(cfg), ctypes.byref(h))
+        assert rc == -1 and not h.value, kw
+        assert word in lib.egg_last_error(None).decode(), (kw, lib.egg_last_error(None))
