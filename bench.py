@@ -109,6 +109,17 @@ def main():
                 "unit": "TOP/s", "frac": achieved / PEAK_INT8_OPS, "traffic": traffic,
                 "avg_launch_ms": tot_ms / launches if launches else None, "launches": launches}
 
+    # ---- for comparison: the same eager steps with the block in front of the first attention layer evaluated at every
+    # position instead of once per distinct byte value of a window (identical results, more work on repetitive data)
+    ctx.first_block_dedup(False)
+    s2 = run_steps(1, 1000, seed, False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_steps(args.steps, 1001, s2, False)
+    torch.cuda.synchronize()
+    per_position_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ctx.first_block_dedup(True)
+
     # ---- the same steps replayed as one captured hipGraph per step
     graph_ms = None
     if not args.no_graph:
@@ -263,7 +274,8 @@ def main():
         "config": {"workload": f"full ES step: Int8NativeFormer L={L} H={H} heads={H // HD} T={T}, population {P}, "
                                f"forward+fitness+vote+AdamW, eager launches (chunk {chunk} members)",
                    "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss,
-                   "distinct_bytes_per_window": round(distinct, 1)},
+                   "distinct_bytes_per_window": round(distinct, 1),
+                   "ms_per_step_first_block_at_every_position": per_position_ms},
         "roofline": roofline, "kernels": per_class, "microbench_c2": mb,
         "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }

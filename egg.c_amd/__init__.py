@@ -48,7 +48,7 @@ EXPORTS = [
     "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate",
     "egg_shape_fitness", "egg_ternary_pack_size", "egg_ternary_pack", "egg_ternary_unpack",
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
-    "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_tap_download",
+    "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
     "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
@@ -127,6 +127,7 @@ def lib():
         L.egg_next_seed.restype = u32
         L.egg_next_seed.argtypes = [u32, C.c_uint64]
         L.egg_ctx_enable_taps.argtypes = [vp, i32]
+        L.egg_ctx_first_block_dedup.argtypes = [vp, i32]
         L.egg_tap_download.argtypes = [vp, C.c_char_p, i32, vp]
         L.egg_ctx_enable_timing.argtypes = [vp, i32]
         L.egg_timing_reset.argtypes = [vp]
@@ -337,6 +338,9 @@ class Context:
 
     def enable_taps(self, on=True):
         self._ck(lib().egg_ctx_enable_taps(self._h, 1 if on else 0), "egg_ctx_enable_taps")
+
+    def first_block_dedup(self, on=True):
+        self._ck(lib().egg_ctx_first_block_dedup(self._h, 1 if on else 0), "egg_ctx_first_block_dedup")
 
     def tap(self, name, member):
         import numpy as np

@@ -63,6 +63,7 @@ struct egg_ctx {
     // generation (egg_generate): token buffer [T + 1], logits of one member [T][vocab], a zero start index / seed
     uint8_t *d_gen_tok = nullptr; int32_t *d_gen_logits = nullptr; Scalars *d_gen_scal = nullptr;
     int mask_override = -1; int32_t *logits_override = nullptr;
+    bool first_dedup = true;        // first block once per distinct byte value of a member's window (egg_ctx_first_block_dedup)
     VecDesc *d_vec_desc = nullptr; int n_vec = 0, vec_total = 0;       // all vector tensors, for the one-launch update
     // adaptive noise overlay (egg_adaptive_enable): raw overlay values, q = clamp(overlay, 0, 64) and change flags, all
     // laid out like the model blob; one segment (rows + cols, or len) per tensor
@@ -530,7 +531,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = F + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
         p.w_dn = F + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
         p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
-        p.tab = ctx->d_q;            // free until the first layer's QKV projection writes it
+        p.tab = ctx->first_dedup ? ctx->d_q : nullptr;     // the q buffer is free until the first layer's QKV projection writes it
         if (Q) {
             p.q_ln_w = Q + L.ln_init; p.q_ln_b = Q + L.ln_init_bias; p.q_b_up = Q + L.mlp_emb_bias_up; p.q_b_dn = Q + L.mlp_emb_bias_down;
             p.q_up = Q + L.w_emb_mlp_up; p.q_dn = Q + L.w_emb_mlp_down; p.q_emb = Q + L.embedding; p.q_emb_bias = Q + L.emb_bias;
@@ -888,6 +889,12 @@ extern "C" int egg_ctx_enable_taps(egg_ctx *ctx, int enable) {
         HIP_TRY(hipMalloc(&ctx->d_tap_logits, (size_t)ctx->tap_members * c.seq_len * 256 * 4));
     }
     ctx->taps = enable != 0;
+    return EGG_OK;
+}
+extern "C" int egg_ctx_first_block_dedup(egg_ctx *ctx, int enable) {
+    if (!ctx) return EGG_E_INVALID;
+    if (ctx->captured) return fail(ctx, EGG_E_STATE, "the first block's form cannot change after capture");
+    ctx->first_dedup = enable != 0;
     return EGG_OK;
 }
 extern "C" int egg_tap_download(egg_ctx *ctx, const char *name, int member, void *host_out) {

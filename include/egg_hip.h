@@ -212,6 +212,12 @@ int  egg_eggc_load_latest(const char *dir, uint64_t *step, uint64_t *seed, uint8
  * forward over at most 64 members keeps every stage's activations; egg_tap_download copies one member's
  * "x_init", "q.L", "k.L", "v.L", "ao.L", "x_attn.L", "x_mlp.L" (L = layer) or "logits" to the host. */
 int  egg_ctx_enable_taps(egg_ctx *ctx, int enable);
+/* No counterpart in the reference (train_sequence_kernel walks every position, mgpu.cu:901-934).  The block in front of
+   the first attention layer depends on the member and the byte value only, so by default it is evaluated once per
+   distinct byte value of a member's window and copied to the positions that hold the value; enable = 0 evaluates it
+   at every position instead.  The results are identical; the switch exists so that both can be measured and compared.
+   Not after egg_step_capture. */
+int  egg_ctx_first_block_dedup(egg_ctx *ctx, int enable);
 int  egg_tap_download(egg_ctx *ctx, const char *name, int member, void *host_out /* int8 [T][H] natural order; "logits": int32 [T][256] */);
 
 /* ---- the reference's CPU program on the GPU (full_trained_egg.c: GRU-style recurrent byte LM, sequential

@@ -18,12 +18,13 @@ def _t(dev, arr):
     return torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
 
 
-def _forward(pkg, dev, cfg_kw, model, d_data, data_len, start, seed, offset=0, count=None, repeat=1):
+def _forward(pkg, dev, cfg_kw, model, d_data, data_len, start, seed, offset=0, count=None, repeat=1, dedup=True):
     import torch
     pop = cfg_kw["population"]
     count = pop if count is None else count
     ctx = pkg.Context(pkg.default_config(**cfg_kw))
     ctx.model_upload(model)
+    ctx.first_block_dedup(dedup)
     out = []
     for _ in range(repeat):
         d_loss = torch.full((pop,), -1, dtype=torch.int32, device=dev)
@@ -49,6 +50,9 @@ def test_population_8192_forward(pkg, orc, dev):
     # a chunk size that is neither a divisor of the population nor a multiple of the workgroup's member count
     (c,) = _forward(pkg, dev, dict(chunk_members=1001, **kw), model, d_data, len(data), start, seed)
     assert np.array_equal(a, c), f"{np.count_nonzero(a != c)} losses depend on the chunking"
+    # the first block evaluated at every position instead of once per distinct byte value of a window
+    (e,) = _forward(pkg, dev, dict(chunk_members=2048, **kw), model, d_data, len(data), start, seed, dedup=False)
+    assert np.array_equal(a, e), f"{np.count_nonzero(a != e)} losses depend on the form of the first block"
     # a sub-range leaves the rest of the output alone
     (d,) = _forward(pkg, dev, dict(chunk_members=2048, **kw), model, d_data, len(data), start, seed, offset=4094, count=6)
     assert np.array_equal(d[4094:4100], a[4094:4100]) and (d[:4094] == -1).all() and (d[4100:] == -1).all()
