@@ -649,7 +649,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
     extern __shared__ __align__(16) int8_t smem[];
     int *lut = reinterpret_cast<int *>(smem);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    int8_t *vl = smem + 2048 + (size_t)wave * T * HD;
+    int8_t *vl = smem + 2048 + (size_t)wave * 2 * T * HD;      // per wave: rows (V, then K) | Q rows
+    int8_t *ql = vl + T * HD;
 
     const FwdCommon &c = p.c;
     const int H = c.H, NH = H / HD;
@@ -663,11 +664,26 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
         const int w = c.exp_lut[i];
         lut[i] = (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16);
     }
-    // V tile of this (member, head) -> LDS rows [ctx][HD]
-    for (int i = lane; i < T * HD / 16; i += 64) {
-        int cx = i / (HD / 16), part = i % (HD / 16);
-        *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + part * 16) =
-            *reinterpret_cast<const v4i *>(p.v + base + (size_t)cx * H + part * 16);
+    // All three row sets of this (member, head) are requested at once, so the wave waits for global memory once: the K
+    // rows stay in registers until the V rows have left the row area, the Q rows go to LDS in the K rows' layout
+    // (chunk c of row r at c ^ ((r / RPL) % CH), see below), the V rows to LDS rows [ctx][HD].
+    constexpr int CH = HD / 16, RPL = 128 / HD, PER = T * CH / 64;
+    v4i kreg[PER];
+    {
+        v4i qreg[PER], vreg[PER];
+#pragma unroll
+        for (int n = 0; n < PER; n++) {
+            const int i = lane + n * 64, cx = i / CH, part = i % CH;
+            kreg[n] = *reinterpret_cast<const v4i *>(p.k + base + (size_t)cx * H + part * 16);
+            qreg[n] = *reinterpret_cast<const v4i *>(p.q + base + (size_t)cx * H + part * 16);
+            vreg[n] = *reinterpret_cast<const v4i *>(p.v + base + (size_t)cx * H + part * 16);
+        }
+#pragma unroll
+        for (int n = 0; n < PER; n++) {
+            const int i = lane + n * 64, cx = i / CH, part = i % CH;
+            *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + part * 16) = vreg[n];
+            *reinterpret_cast<v4i *>(ql + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) = qreg[n];
+        }
     }
     __syncthreads();
     // V^T fragments: A-operand row i = natural head dim d = 32dt + i, stored at slot position 16g'+4q'+e'
@@ -692,12 +708,11 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
     // Rows are HD bytes apart, so the 16-byte chunk a lane reads (row = its context position) would hit the same few
     // banks for every row; chunk c of row r is therefore kept at position c ^ ((r / RPL) % CH), which spreads eight
     // consecutive rows over all banks.
-    constexpr int CH = HD / 16, RPL = 128 / HD;
     wave_lds_fence();
-    for (int i = lane; i < T * HD / 16; i += 64) {
-        int cx = i / CH, part = i % CH;
-        *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) =
-            *reinterpret_cast<const v4i *>(p.k + base + (size_t)cx * H + part * 16);
+#pragma unroll
+    for (int n = 0; n < PER; n++) {
+        const int i = lane + n * 64, cx = i / CH, part = i % CH;
+        *reinterpret_cast<v4i *>(vl + (size_t)cx * HD + ((part ^ ((cx / RPL) % CH)) * 16)) = kreg[n];
     }
     wave_lds_fence();
     const int8_t *kl = vl;
@@ -711,7 +726,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
         const int t = qt * 32 + j;
         v4i qop[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) qop[ks] = load_op(p.q + base + (size_t)t * H, ks, g);
+        for (int ks = 0; ks < KS; ks++)
+            qop[ks] = *reinterpret_cast<const v4i *>(ql + (size_t)t * HD + (((ks * 2 + g) ^ ((t / RPL) % CH)) * 16));
         // pass 1: per-head maximum score over ctx <= t (mgpu.cu:795-802)
         int mx = INT_MIN;
 #pragma unroll
@@ -1134,11 +1150,11 @@ static hipError_t launch_attn_t(const AttnParams &p, hipStream_t s) {
     if constexpr (CT % 8 == 0) {
         const size_t lds_wg = AttnWg<HD, CT>::LDS;
         hipLaunchKernelGGL((k_attn_wg<HD, CT>), dim3(units), dim3(EGG_THREADS), lds_wg, s, p);
-        return hipGetLastError();
+    } else {
+        dim3 grid((units + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
+        size_t lds = 2048 + (size_t)EGG_WAVES * 2 * CT * 32 * HD;
+        hipLaunchKernelGGL((k_attn<HD, CT>), grid, block, lds, s, p);
     }
-    dim3 grid((units + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
-    size_t lds = 2048 + (size_t)EGG_WAVES * CT * 32 * HD;
-    hipLaunchKernelGGL((k_attn<HD, CT>), grid, block, lds, s, p);
     return hipGetLastError();
 }
 template <int HD>
@@ -1200,7 +1216,7 @@ static hipError_t prepare_h(int T) {
 template <int HD, int CT>
 static hipError_t prepare_attn() {
     if constexpr (CT % 8 == 0) SET_LDS((k_attn_wg<HD, CT>), (AttnWg<HD, CT>::LDS));
-    SET_LDS((k_attn<HD, CT>), 2048 + (size_t)EGG_WAVES * CT * 32 * HD);
+    else SET_LDS((k_attn<HD, CT>), 2048 + (size_t)EGG_WAVES * 2 * CT * 32 * HD);
     return hipSuccess;
 }
 template <int HD>
