@@ -348,9 +348,9 @@ __device__ __forceinline__ void fill_noise_i32(int *dst, uint32_t seed, int n, i
 // dst[i] = base[i] + ((noise(seed_a,i) * noise(seed_b,i) * ns) >> shift)       (mgpu.cu:666-675, :733-735)
 // (the result is stored shifted left by `lshift` where a kernel folds it into a GEMM accumulator)
 __device__ __forceinline__ void fill_vec_i32(int *dst, const int8_t *base, uint32_t seed_a, uint32_t seed_b,
-                                             int n, int mask, int ns, int shift, int lane, int nthr = 64, int lshift = 0) {
+                                             int n, int mask, int ns, int shift, int lane, int nthr = 64, int lshift = 0, int add = 0) {
     for (int i = lane; i < n; i += nthr) {
-        int v = base[i];
+        int v = base[i] + add;
         if (ns != 0) v += (noise_from_hash(seed_a, i, mask) * noise_from_hash(seed_b, i, mask) * ns) >> shift;
         dst[i] = v << lshift;
     }
@@ -379,9 +379,9 @@ __device__ __forceinline__ void fill_noise_i32_ov(int *dst, uint32_t seed, int n
     for (int i = lane; i < n; i += nthr) dst[i] = overlay_scaled(noise_from_hash(seed, i, mask), q[i]) * mult;
 }
 __device__ __forceinline__ void fill_vec_i32_ov(int *dst, const int8_t *base, uint32_t seed_a, uint32_t seed_b,
-                                                int n, int mask, int ns, int shift, int lane, int nthr, int lshift, const int8_t *q) {
+                                                int n, int mask, int ns, int shift, int lane, int nthr, int lshift, const int8_t *q, int add = 0) {
     for (int i = lane; i < n; i += nthr) {
-        int v = base[i];
+        int v = base[i] + add;
         if (ns != 0) v += (overlay_scaled(noise_from_hash(seed_a, i, mask) * noise_from_hash(seed_b, i, mask), q[i]) * ns) >> shift;
         dst[i] = v << lshift;
     }

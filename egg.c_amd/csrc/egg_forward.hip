@@ -134,7 +134,8 @@ struct MlpCfg {
     // [4 ints], and below hidden 256 the list of present values [256] (from hidden 256 on it lives in the table slot
     // of the O projection's noise, which the first block does not use)
     static constexpr int DEDUP = 256 + 16 + (H < 256 ? 256 : 0);
-    static int total(int sets, bool first) { return WBYTES + 256 + sets * PER_SET + XCHG + RED + (first ? DEDUP : 0); }
+    static constexpr int ACT = 256;          // GELU table: entry v + 128 holds the activation of the int8 value v
+    static int total(int sets, bool first) { return WBYTES + ACT + sets * PER_SET + XCHG + RED + (first ? DEDUP : 0); }
 };
 
 // FUSE: the host has checked sigma <= 7 and |noise| <= 15, which bounds |acc| * 2^sigma + |sb * a| below 2^31 for
@@ -151,19 +152,23 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
     constexpr int CS = M::CS, KS = M::KS, NTS = M::NTS, HS = M::HS, NTU = M::NTU, SC = M::SC;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *act = smem + M::WBYTES;
+    // The GELU table is read through an LDS address formed from the index itself plus a constant offset, which assumes
+    // that the dynamic LDS block starts at LDS address 0 (the kernel declares no static LDS); built from the `act`
+    // pointer instead, every read carries an extra add of that (zero) base.
+    typedef const __attribute__((address_space(3))) uint8_t *lds_u8_ptr;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const FwdCommon &c = p.c;
     const int T = c.T;
     const TileMap tm = tile_map<CS>(T, wave, blockIdx.x);
     const int col0 = tm.cs * HS;                      // first output column of this wave's slice
-    int8_t *tb = act + 256 + tm.set * M::PER_SET;
+    int8_t *tb = act + M::ACT + tm.set * M::PER_SET;
     int *ex0 = reinterpret_cast<int *>(tb);           // FIRST: emb_bias + noise   | else: O-proj A noise * ns as int8
     int *ex1 = ex0 + H;                               // FIRST: b_dim noise * ns    | else: unused
     int *lnw = ex1 + H, *lnb = lnw + H, *bup = lnb + H, *bdn = bup + 4 * H;
     int8_t *exB = reinterpret_cast<int8_t *>(bdn + H);   // O-proj B noise
     int8_t *upB = exB + H, *dnB = upB + H, *upA = dnB + 4 * H, *dnA = upA + 4 * H;
     const int8_t *oA = reinterpret_cast<const int8_t *>(ex0);
-    int8_t *xch = act + 256 + tm.sets * M::PER_SET;
+    int8_t *xch = act + M::ACT + tm.sets * M::PER_SET;
     int *red = reinterpret_cast<int *>(xch + M::XCHG);
 
     WStream ws; wstream_init(ws, smem, M::UNIT);
@@ -183,12 +188,13 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
     auto pf_pass_first = [&]() { if (FIRST) pf_up(0, 0); else pf_o(0); };
     pf_pass_first();
 
-    for (int i = threadIdx.x; i < 256; i += EGG_THREADS) act[i] = c.act_lut[i];
+    for (int i = threadIdx.x; i < 256; i += EGG_THREADS)      // act_lut is indexed by the value's two's-complement byte
+        act[(i + 128) & 255] = c.act_lut[i];
     for (int ss = 0; ss < tm.sets; ss++) {
         int ml = blockIdx.x * tm.sets + ss; if (ml >= c.n_members) ml = c.n_members - 1;
         const int mem = c.pop_offset + ml, nsx = (mem & 1) ? -1 : 1;
         const uint32_t pseed = *c.d_step_seed + (uint32_t)(mem / 2), sbx = pseed + (uint32_t)p.seed_base;
-        int8_t *t2 = act + 256 + ss * M::PER_SET;
+        int8_t *t2 = act + M::ACT + ss * M::PER_SET;
         int *e0 = reinterpret_cast<int *>(t2), *e1 = e0 + H, *lw = e1 + H, *lb = lw + H, *bu = lb + H, *bd = bu + 4 * H;
         int8_t *eB = reinterpret_cast<int8_t *>(bd + H), *uB = eB + H, *dB = uB + H, *uA = dB + 4 * H, *dA = uA + 4 * H;
         const int tid = threadIdx.x;
@@ -204,7 +210,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             fill_vec_i32_ov(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2, p.q_ln_w);
             fill_vec_i32_ov(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_b);
             fill_noise_i8_ov(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx, p.q_up + H);
-            fill_vec_i32_ov(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up, p.q_b_up);
+            fill_vec_i32_ov(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up, p.q_b_up, 128);
             fill_noise_i8_ov(dA, sbx + p.off_dn_a, H, c.mask, tid, EGG_THREADS, nsx, p.q_dn + 4 * H);
             fill_vec_i32_ov(bd, p.b_dn, sbx + p.off_bdn_a, sbx + p.off_bdn_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_b_dn);
             fill_noise_i8(uB, sbx + p.off_up_b, H, c.mask, tid, EGG_THREADS);
@@ -221,8 +227,9 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         fill_vec_i32(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2);     // 4 * gain, see standard_scale
         fill_vec_i32(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_noise_i8(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx);
-        // the up bias is stored as b << shift_mlp_up and seeds the up accumulator: ((a + (b << s)) >> s) == (a >> s) + b
-        fill_vec_i32(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up);
+        // the up bias is stored as (b + 128) << shift_mlp_up and seeds the up accumulator: ((a + (b << s)) >> s) == (a >> s) + b;
+        // the 128 makes the clamped result (1..255) the GELU table's index
+        fill_vec_i32(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up, 128);
         fill_noise_i8(dA, sbx + p.off_dn_a, H, c.mask, tid, EGG_THREADS, nsx);
         fill_vec_i32(bd, p.b_dn, sbx + p.off_bdn_a, sbx + p.off_bdn_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
         fill_noise_i8(uB, sbx + p.off_up_b, H, c.mask, tid, EGG_THREADS);
@@ -383,13 +390,16 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                     for (int q = 0; q < 4; q++) {
                         int n0 = nb + 32 * nt + 8 * q + 4 * g;
                         int a4 = *reinterpret_cast<const int *>(upA + n0);
-                        int o[4];
+                        uint32_t r4[4];          // the activation of element e as an unsigned byte
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            int v = clip127(perturb_shift<FUSE>(au[nt][4 * q + e], sbu, sx8(a4, e), c.sigma, c.shift_mlp_up));
-                            o[e] = act[(uint8_t)v];
+                            // the accumulator carries + 128 (see the bias table): clamping to 1..255 is the clamp to +-127,
+                            // and the result is the table index as it stands
+                            const int idx = min(255, max(1, perturb_shift<FUSE>(au[nt][4 * q + e], sbu, sx8(a4, e), c.sigma, c.shift_mlp_up)));
+                            r4[e] = reinterpret_cast<lds_u8_ptr>((uintptr_t)(uint32_t)idx)[M::WBYTES];
                         }
-                        mine[nt][q] = pack4(o[0], o[1], o[2], o[3]);
+                        // bytes 0 of the four results side by side: two byte permutes and an or
+                        mine[nt][q] = (int)(__builtin_amdgcn_perm(r4[1], r4[0], 0x0c0c0400u) | __builtin_amdgcn_perm(r4[3], r4[2], 0x04000c0cu));
                         if (!ADAPT) sbd = dot4(mine[nt][q], dnb32[8 * nt + 2 * q + g], sbd);
                         else {
                             const int nz4 = dnb32[8 * nt + 2 * q + g], q4 = *reinterpret_cast<const int *>(p.q_dn + n0);
@@ -398,7 +408,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                                 const int idx = ADAPT ? (nt * 4 + q) * 4 + e : 0;
                                 const int prev = (it & 3) ? pb[idx] : 0;
                                 // (int)((float)pb + x * n * q / 64): every value is a multiple of 1/64 below 2^24
-                                pb[idx] = div_pow2_trunc<6>((prev << 6) + mul24(mul24(o[e], sx8(nz4, e)), sx8(q4, e)));
+                                pb[idx] = div_pow2_trunc<6>((prev << 6) + mul24(mul24(sx8((int)r4[e], 0), sx8(nz4, e)), sx8(q4, e)));
                             }
                         }
                     }
