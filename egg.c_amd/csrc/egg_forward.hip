@@ -1207,10 +1207,23 @@ hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
 // ---------------------------------------------------------------- one-time LDS opt-in (not a stream operation,
 // so it is done at context creation and never while a stream is capturing)
 #define SET_LDS(kern, bytes) do { hipError_t e_ = hipFuncSetAttribute(reinterpret_cast<const void *>(&kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)); if (e_ != hipSuccess) return e_; } while (0)
+// k_mlp reads its GELU table through LDS addresses that assume the dynamic LDS block starts at address 0, i.e. that the
+// kernel has no static LDS in front of it; refuse to run if a build ever gives it some
+template <typename K>
+static hipError_t no_static_lds(K kern) {
+    hipFuncAttributes a;
+    hipError_t e = hipFuncGetAttributes(&a, reinterpret_cast<const void *>(kern));
+    if (e != hipSuccess) return e;
+    return a.sharedSizeBytes == 0 ? hipSuccess : hipErrorInvalidConfiguration;
+}
 template <int H>
 static hipError_t prepare_h(int T) {
     const int sets = tile_map_sets(T, Shape<H>::CS);
     const int msets = tile_map_sets(T, MlpCfg<H>::CS);
+    for (hipError_t e : {no_static_lds(&k_mlp<H, true, true, false>), no_static_lds(&k_mlp<H, false, true, false>),
+                         no_static_lds(&k_mlp<H, true, false, false>), no_static_lds(&k_mlp<H, false, false, false>),
+                         no_static_lds(&k_mlp<H, true, false, true>), no_static_lds(&k_mlp<H, false, false, true>)})
+        if (e != hipSuccess) return e;
     SET_LDS((k_mlp<H, true, true, false>), MlpCfg<H>::total(msets, true));
     SET_LDS((k_mlp<H, false, true, false>), MlpCfg<H>::total(msets, false));
     SET_LDS((k_mlp<H, true, false, false>), MlpCfg<H>::total(msets, true));
