@@ -7,6 +7,7 @@
 // copy in L2, B operand = the 32 members' input vectors in LDS), output rows are split over the waves and the
 // int8 results go back to LDS as the next matmul's input.  Noise vectors of all (pair, matrix) are generated once
 // per step by replaying the reference's xorshift stream (4 discarded draws per block of 16, egg.c:87-105).
+#include <type_traits>
 #include "egg_device.h"
 #include "egg_launch.h"
 #include "../../include/egg_hip.h"
@@ -81,25 +82,59 @@ __global__ void k_gru_swizzle(const int8_t *W, int8_t *F, int rows, int cols) {
     reinterpret_cast<v4i *>(F)[c] = v;
 }
 
-// one 32-row strip: acc += W[32nt.., :] . in, in = LDS [32 members][K (+16 pad)] in slot order
-template <int DUMMY = 0>
-__device__ __forceinline__ void gru_strip(v16i &acc, const int8_t *ftile, const int8_t *ldsB, int K, int lane) {
-    const int i = lane & 31, g = lane >> 5, stride = K + 16;
-    for (int ks = 0; ks < K / 32; ks++) {
-        v4i a = *reinterpret_cast<const v4i *>(ftile + ((size_t)(2 * ks + g) * 32 + i) * 16);
-        v4i b = *reinterpret_cast<const v4i *>(ldsB + (size_t)i * stride + 32 * ks + 16 * g);
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
-    }
-}
-// xB = sum_c in[c] * B[c] for the lane's member (egg.c:122-140)
-__device__ __forceinline__ int gru_xb(const int8_t *ldsB, const int8_t *bvec, int K, int lane) {
-    const int j = lane & 31, g = lane >> 5, stride = K + 16;
-    int s = 0;
-    for (int ks = 0; ks < K / 32; ks++) {
-        v4i b = *reinterpret_cast<const v4i *>(ldsB + (size_t)j * stride + 32 * ks + 16 * g);
-        v4i n = *reinterpret_cast<const v4i *>(bvec + 32 * ks + 16 * g);
+// one 32-row strip: acc += W[32nt.., :] . in, in = LDS [32 members][K (+16 pad)] in slot order.  The W fragments come
+// straight from global memory (L2); eight k-steps' worth are in flight ahead of the MFMAs that use them, so
+// the strip pays for one memory latency instead of one per k-step.
+template <int KS>
+struct GruStrip {
+    static constexpr int K = KS * 32, stride = K + 16, BATCH = KS < 8 ? KS : 8;
+    static_assert(KS % BATCH == 0, "k-steps come in whole batches");
+    v4i a[BATCH];
+    const int8_t *fa;
+    // request the first batch of fragments (call it as early as the strip is known, before unrelated work)
+    __device__ __forceinline__ void begin(const int8_t *ftile, int lane) {
+        fa = ftile + ((size_t)(lane >> 5) * 32 + (lane & 31)) * 16;          // k-step ks adds ks * 1024
 #pragma unroll
-        for (int q = 0; q < 4; q++) s = dot4(b[q], n[q], s);
+        for (int u = 0; u < BATCH; u++) a[u] = *reinterpret_cast<const v4i *>(fa + (size_t)u * 1024);
+    }
+    __device__ __forceinline__ void run(v16i &acc, const int8_t *ldsB, int lane) {
+        const int8_t *fb = ldsB + (size_t)(lane & 31) * stride + 16 * (lane >> 5);   // k-step ks adds ks * 32
+#pragma unroll 1
+        for (int k0 = 0; k0 < KS; k0 += BATCH) {
+#pragma unroll
+            for (int u = 0; u < BATCH; u++) {
+                const v4i b = *reinterpret_cast<const v4i *>(fb + (k0 + u) * 32);
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u], b, acc, 0, 0, 0);
+                // the register set is refilled for the next batch as soon as its MFMA has been issued
+                if (k0 + BATCH < KS) a[u] = *reinterpret_cast<const v4i *>(fa + (size_t)(k0 + BATCH + u) * 1024);
+            }
+        }
+    }
+};
+template <int KS>
+__device__ __forceinline__ void gru_strip(v16i &acc, const int8_t *ftile, const int8_t *ldsB, int lane) {
+    GruStrip<KS> st;
+    st.begin(ftile, lane);
+    st.run(acc, ldsB, lane);
+}
+// xB = sum_c in[c] * B[c] for the lane's member (egg.c:122-140); the noise rows are requested a batch ahead as well
+template <int KS>
+__device__ __forceinline__ int gru_xb(const int8_t *ldsB, const int8_t *bvec, int lane) {
+    constexpr int K = KS * 32, stride = K + 16, BATCH = KS < 8 ? KS : 8;
+    static_assert(KS % BATCH == 0, "k-steps come in whole batches");
+    const int j = lane & 31, g = lane >> 5;
+    int s = 0;
+#pragma unroll 1
+    for (int k0 = 0; k0 < KS; k0 += BATCH) {
+        v4i n[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; u++) n[u] = *reinterpret_cast<const v4i *>(bvec + 32 * (k0 + u) + 16 * g);
+#pragma unroll
+        for (int u = 0; u < BATCH; u++) {
+            const v4i b = *reinterpret_cast<const v4i *>(ldsB + (size_t)j * stride + 32 * (k0 + u) + 16 * g);
+#pragma unroll
+            for (int q = 0; q < 4; q++) s = dot4(b[q], n[u][q], s);
+        }
     }
     return s + other_half(s);
 }
@@ -127,6 +162,8 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
     constexpr int NT4 = 4 * H / 32;
     constexpr int MAXT4 = (NT4 + GRU_WAVES - 1) / GRU_WAVES;
     constexpr int SH = H + 16, S4 = 4 * H + 16; // padded LDS row strides
+    constexpr std::integral_constant<int, H / 32> KH{};          // k-steps of an H-deep and of a 4H-deep matmul
+    constexpr std::integral_constant<int, 4 * H / 32> K4H{};
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *XN = smem, *HB = XN + 32 * SH, *MB = HB + 32 * SH;
     int *psum = reinterpret_cast<int *>(MB + 32 * S4);          // [GRU_WAVES][32]
@@ -177,15 +214,18 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
         return out;
     };
     // perturbed matmul of an H-wide output: the own strip's packed result
-    auto matmul_h = [&](int mi, const int8_t *in, int K) -> v4i {
+    auto matmul_h = [&](int mi, const int8_t *in, auto ks_tag) -> v4i {
+        constexpr int KS = decltype(ks_tag)::value, K = KS * 32;
         v4i r = {0, 0, 0, 0};
         if (own) {
             const GruMat m = p.mats[mi];
-            const int xb = gru_xb(in, p.noise + m.b_off + (long long)pair * K, K, lane);
+            GruStrip<KS> st;
+            st.begin(p.frag + m.w_off + (size_t)wave * 32 * K, lane);       // on its way while x.B is summed
+            const int xb = gru_xb<KS>(in, p.noise + m.b_off + (long long)pair * K, lane);
             v16i acc;
 #pragma unroll
             for (int t = 0; t < 16; t++) acc[t] = 0;
-            gru_strip(acc, p.frag + m.w_off + (size_t)wave * 32 * K, in, K, lane);
+            st.run(acc, in, lane);
             r = gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, wave, ns, p.sigma, m.shift, g);
         }
         return r;
@@ -211,8 +251,8 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
             v4i xn = layer_norm(x, lnw);
             if (own) { put(XN, SH, wave, xn); put(HB, SH, wave, hcur); }
             __syncthreads();
-            v4i b1 = matmul_h(6 * l + 0, XN, H);
-            v4i b2 = matmul_h(6 * l + 1, HB, H);
+            v4i b1 = matmul_h(6 * l + 0, XN, KH);
+            v4i b2 = matmul_h(6 * l + 1, HB, KH);
             v4i ft = {0, 0, 0, 0}, gated = {0, 0, 0, 0};
             if (own) {
 #pragma unroll
@@ -230,8 +270,8 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
             __syncthreads();                       // every wave has finished reading HB (old state)
             if (own) put(HB, SH, wave, gated);
             __syncthreads();
-            b1 = matmul_h(6 * l + 2, XN, H);
-            b2 = matmul_h(6 * l + 3, HB, H);
+            b1 = matmul_h(6 * l + 2, XN, KH);
+            b2 = matmul_h(6 * l + 3, HB, KH);
             if (own) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
@@ -255,20 +295,20 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
             __syncthreads();
             {
                 const GruMat m = p.mats[6 * l + 4];
-                const int xb = gru_xb(XN, p.noise + m.b_off + (long long)pair * H, H, lane);
+                const int xb = gru_xb<H / 32>(XN, p.noise + m.b_off + (long long)pair * H, lane);
                 for (int ti = 0; ti < MAXT4; ti++) {
                     const int nt = wave + GRU_WAVES * ti;
                     if (nt < NT4) {
                         v16i acc;
 #pragma unroll
                         for (int r = 0; r < 16; r++) acc[r] = 0;
-                        gru_strip(acc, p.frag + m.w_off + (size_t)nt * 32 * H, XN, H, lane);
+                        gru_strip<H / 32>(acc, p.frag + m.w_off + (size_t)nt * 32 * H, XN, lane);
                         put(MB, S4, nt, gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g));
                     }
                 }
             }
             __syncthreads();
-            v4i pr = matmul_h(6 * l + 5, MB, 4 * H);
+            v4i pr = matmul_h(6 * l + 5, MB, K4H);
             if (own)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
@@ -286,11 +326,11 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
         int part = 0;
         if (wave < V / 32) {
             const GruMat m = p.mats[6 * L];
-            const int xb = gru_xb(XN, p.noise + m.b_off + (long long)pair * H, H, lane);
+            const int xb = gru_xb<H / 32>(XN, p.noise + m.b_off + (long long)pair * H, lane);
             v16i acc;
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[r] = 0;
-            gru_strip(acc, p.frag + m.w_off + (size_t)wave * 32 * H, XN, H, lane);
+            gru_strip<H / 32>(acc, p.frag + m.w_off + (size_t)wave * 32 * H, XN, lane);
             v4i lg = gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, wave, ns, p.sigma, m.shift, g);
 #pragma unroll
             for (int q = 0; q < 4; q++)
