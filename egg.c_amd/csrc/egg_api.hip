@@ -75,6 +75,9 @@ struct egg_ctx {
     std::string err;
 };
 
+// magnitude mask plus the Gaussian flag, as the kernels take it
+static int noise_word(const egg_config &c) { return c.noise_mask | (c.device_gaussian ? EGG_NOISE_GAUSSIAN : 0); }
+
 static int fail(egg_ctx *ctx, int code, const char *what, hipError_t e = hipSuccess) {
     if (ctx) {
         ctx->err = what;
@@ -117,6 +120,7 @@ extern "C" void egg_default_config(egg_config *c) {
     c->softmax_exp_scale = 6.0;
     c->adam_beta1 = 0.9f; c->adam_beta2 = 0.95f; c->adam_eps = 1e-8f; c->adam_weight_decay = 0.01f;
     c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->use_muon = 0; c->chunk_members = 0; c->weight_limit = 127;
+    c->device_gaussian = 0; c->host_gaussian = 0;
 }
 
 // launch order of mgpu.cu:1603-1643
@@ -186,12 +190,16 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     // shift amounts and table scales the kernels can state in 32-bit shifts / 64-bit multiply-adds
     auto in_range = [](int v, int lo, int hi) { return v >= lo && v <= hi; };
     if (!in_range(c.rope_scale_bit, 1, 30) || !in_range(c.softmax_scale_bit, 1, 30)) return refuse("rope_scale_bit and softmax_scale_bit must be 1..30");
-    if (!in_range(c.noise_mask, 0, 127)) return refuse("noise_mask must be 0..127");
+    if (!in_range(c.noise_mask, 0, 127) || !in_range(c.host_mask, 0, 127)) return refuse("noise_mask and host_mask must be 0..127");
+    const int mag = c.device_gaussian ? 3 * c.noise_mask : c.noise_mask;        // largest |noise|
+    if (mag > 127 || (c.host_gaussian ? 3 : 1) * c.host_mask > 127) return refuse("Gaussian noise needs 3 * mask <= 127");
+    // x.B sums enter 24-bit multiplies: |sum| <= 4 * hidden * 127 * |noise|
+    if ((long long)4 * c.hidden * 127 * mag >= (1LL << 23)) return refuse("noise too wide for this hidden size (4 * hidden * 127 * |noise| must stay below 2^23)");
     if (!in_range(c.fixed_point + c.sigma_shift, 0, 24) || !in_range(c.sigma_shift_vector, 0, 24) || !in_range(c.shift_attn, 0, 24) ||
         !in_range(c.shift_out, 0, 24) || !in_range(c.shift_logit, 0, 24) || !in_range(c.shift_mlp_up, 0, 24) ||
         !in_range(c.shift_mlp_down, 0, 24)) return refuse("shift amounts must be 0..24");
     // the standard norm divides x * (gain + noise) by the row mean with a 32-bit multiply-high that is exact up to 2^17
-    if (127 * (127 + ((c.noise_mask * c.noise_mask) >> c.sigma_shift_vector)) > (1 << 17))
+    if (127 * (127 + ((mag * mag) >> c.sigma_shift_vector)) > (1 << 17))
         return refuse("noise_mask^2 >> sigma_shift_vector is too large for the norm's exact division");
     if (!in_range(c.weight_limit, 1, 127)) return refuse("weight_limit must be 1..127");
     egg_ctx *ctx = new egg_ctx();
@@ -320,9 +328,11 @@ extern "C" int64_t egg_model_bytes(const egg_ctx *ctx) { return ctx ? ctx->L.tot
 
 // ------------------------------------------------------------------ init_model (mgpu.cu:428-519)
 static inline uint32_t xorshift32_host(uint32_t *st) { uint32_t x = *st; x ^= x << 13; x ^= x >> 17; x ^= x << 5; *st = x; return x; }
-static inline int8_t gen_noise_host(uint32_t *rng, int mask) {
+static inline int8_t gen_noise_host(uint32_t *rng, int mask, int gaussian) {
     uint32_t r = xorshift32_host(rng);
-    return (int8_t)((r & 1 ? 1 : -1) * (int)((r >> 1) & (uint32_t)mask));
+    int n = (r & 1 ? 1 : -1) * (int)((r >> 1) & (uint32_t)mask);
+    if (gaussian) n += (r & 32 ? 1 : -1) * (int)((r >> 6) & (uint32_t)mask) + (r & 1024 ? 1 : -1) * (int)((r >> 11) & (uint32_t)mask);
+    return (int8_t)n;
 }
 // [In][Out] row-major -> blocked [In/4][Out][4]
 static void repack_matrix(int8_t *dst, const int8_t *src, int rows, int cols) {
@@ -336,7 +346,7 @@ extern "C" int egg_model_init(egg_ctx *ctx, uint32_t seed) {
     std::vector<int8_t> m((size_t)L.total, 0), tmp((size_t)H * 4 * H > (size_t)V * H ? (size_t)H * 4 * H : (size_t)V * H);
     uint32_t rng = seed;
     auto gen = [&](int8_t *dst, int rows, int cols) {
-        for (size_t i = 0; i < (size_t)rows * cols; i++) tmp[i] = gen_noise_host(&rng, c.host_mask);
+        for (size_t i = 0; i < (size_t)rows * cols; i++) tmp[i] = gen_noise_host(&rng, c.host_mask, c.host_gaussian);
         repack_matrix(dst, tmp.data(), rows, cols);
     };
     gen(&m[L.embedding], H, V);
@@ -463,7 +473,7 @@ extern "C" int egg_tables_download(egg_ctx *ctx, int32_t *ex, int8_t *act, int32
 
 extern "C" int egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first, int n, int8_t *d_out) {
     if (!ctx || !d_out || n < 0) return fail(ctx, EGG_E_INVALID, "egg_noise_fill arguments");
-    HIP_TRY(egg_launch_noise_fill(seed, first, n, ctx->cfg.noise_mask, d_out, ctx->stream));
+    HIP_TRY(egg_launch_noise_fill(seed, first, n, noise_word(ctx->cfg), d_out, ctx->stream));
     return EGG_OK;
 }
 
@@ -480,7 +490,7 @@ extern "C" int egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_
         ctx->plin_frag_bytes = (size_t)K * N;
     }
     PlinParams p = {d_X, ctx->d_plin_frag, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
-                    ctx->cfg.noise_mask, d_Y32, d_Y8};
+                    noise_word(ctx->cfg), d_Y32, d_Y8};
     const int PB = egg_plinear_block(K, N);
     if (K % PB || N % PB) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");
     span_begin(ctx, EGG_K_PLINEAR);
@@ -501,7 +511,7 @@ static FwdCommon make_common(egg_ctx *ctx, const uint8_t *d_data, int64_t len, c
     f.pop_offset = first_member; f.n_members = nm; f.population = c.population;
     f.T = c.seq_len; f.H = c.hidden; f.head_dim = c.head_dim; f.vocab = c.vocab;
     f.sigma = c.fixed_point + c.sigma_shift; f.sigma_vec = c.sigma_shift_vector;
-    f.mask = ctx->mask_override >= 0 ? ctx->mask_override : c.noise_mask;
+    f.mask = ctx->mask_override >= 0 ? ctx->mask_override : noise_word(c);
     f.shift_attn = c.shift_attn; f.shift_out = c.shift_out; f.shift_logit = c.shift_logit;
     f.shift_mlp_up = c.shift_mlp_up; f.shift_mlp_down = c.shift_mlp_down;
     f.softmax_scale_bit = c.softmax_scale_bit; f.rope_scale_bit = c.rope_scale_bit;
@@ -635,7 +645,7 @@ static UpdParams make_upd(egg_ctx *ctx, int id, const int32_t *d_fit, const uint
     p.rows = t.rows; p.cols = t.cols; p.off_a = t.off_a; p.off_b = t.off_b; p.seed_base = t.seed_base;
     p.fit = d_fit; p.pairs = c.population / 2; p.d_seed = d_seed; p.d_lr = d_lr; p.lr_scale = t.lr_scale;
     p.limit = t.is_matrix ? c.weight_limit : 127;
-    p.mask = c.noise_mask; p.beta1 = c.adam_beta1; p.beta2 = c.adam_beta2; p.eps = c.adam_eps; p.wd = c.adam_weight_decay;
+    p.mask = noise_word(c); p.beta1 = c.adam_beta1; p.beta2 = c.adam_beta2; p.eps = c.adam_eps; p.wd = c.adam_weight_decay;
     p.panel_a = ctx->d_panel_a; p.panel_b = ctx->d_panel_b; p.pairs_pad = ctx->pairs_pad; p.counter = ctx->d_counter;
     return p;
 }

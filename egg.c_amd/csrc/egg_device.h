@@ -19,6 +19,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include "egg_params.h"
 
 // The float steps of the normalisations are single IEEE operations in the reference; a fused multiply-add in
 // round_half_away(val * scale) changes results at exact .5 ties (e.g. max 6, value 3).  The build also passes
@@ -37,11 +38,20 @@ __device__ __forceinline__ uint32_t hash_rng(uint32_t s, uint32_t idx) {
     x ^= x >> 16; x *= 0x85ebca6bu; x ^= x >> 13; x *= 0xc2b2ae35u; x ^= x >> 16;
     return x;
 }
+// `mask` is the magnitude mask (DEVICE_MASK) in its low byte; EGG_NOISE_GAUSSIAN (egg_params.h) on top of it selects the reference's
+// DEVICE_GAUSSIAN form, the sum of three such fields taken from bits 0-5, 5-10 and 10-15 of the hash
 __device__ __forceinline__ int noise_from_hash(uint32_t s, uint32_t idx, int mask) {
     uint32_t r = hash_rng(s, idx);
-    int mag = (int)((r >> 1) & (uint32_t)mask);
-    return (r & 1) ? mag : -mag;
+    const uint32_t m = (uint32_t)mask & 0xffu;
+    int mag = (int)((r >> 1) & m);
+    int n = (r & 1) ? mag : -mag;
+    if (mask & EGG_NOISE_GAUSSIAN) {
+        mag = (int)((r >> 6) & m); n += (r & 32) ? mag : -mag;
+        mag = (int)((r >> 11) & m); n += (r & 1024) ? mag : -mag;
+    }
+    return n;
 }
+
 __device__ __forceinline__ int clip127(int a) { return min(127, max(-127, a)); }
 
 // ---------------------------------------------------------------- lane helpers

@@ -1115,7 +1115,7 @@ static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
     const int sets = tile_map_sets(p.c.T, MlpCfg<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = MlpCfg<H>::total(sets, first);
-    const bool fuse = p.c.sigma <= 7 && p.c.mask <= 15;
+    const bool fuse = p.c.sigma <= 7 && egg_noise_magnitude(p.c.mask) <= 15;
     if (p.q_ln_w) {      // adaptive noise overlay: one (unfused) variant
         if (first) hipLaunchKernelGGL((k_mlp<H, true, false, true>), grid, block, lds, s, p);
         else hipLaunchKernelGGL((k_mlp<H, false, false, true>), grid, block, lds, s, p);

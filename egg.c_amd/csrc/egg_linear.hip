@@ -250,7 +250,8 @@ template <int K, int N>
 static hipError_t launch_kn(const PlinParams &p, hipStream_t s) {
     // the fused form needs |acc| * 2^sigma + |sb * a| < 2^31 for any int8 inputs: |acc| <= K * 128 * 128,
     // |sb| <= K * 128 * mask, |a| <= mask
-    const long long bound = ((long long)K * 128 * 128 << p.sigma) + (long long)K * 128 * p.mask * p.mask;
+    const long long mag = egg_noise_magnitude(p.mask);
+    const long long bound = ((long long)K * 128 * 128 << p.sigma) + (long long)K * 128 * mag * mag;
     const bool fuse = p.sigma >= 0 && p.sigma <= 12 && p.sigma + p.shift < 32 && bound < (1LL << 31);
     // both outputs requested: two launches (the test hook asks for one at a time)
     hipError_t e = hipSuccess;

@@ -18,6 +18,12 @@ enum {
     OFF_EMB_MLP_BIAS_DOWN_A = 516, OFF_EMB_MLP_BIAS_DOWN_B = 517
 };
 
+// A noise mask word is the magnitude mask (DEVICE_MASK, mgpu.cu:201) in its low byte, plus this flag for the
+// reference's DEVICE_GAUSSIAN form (mgpu.cu:530-534: the sum of three masked fields of the hash)
+#define EGG_NOISE_GAUSSIAN 0x100
+// largest |noise| a mask word can produce
+static inline int egg_noise_magnitude(int mask) { return (mask & EGG_NOISE_GAUSSIAN) ? 3 * (mask & 0xff) : (mask & 0xff); }
+
 // what every forward kernel needs to know about the run
 struct FwdCommon {
     const uint8_t  *data;        // token stream (device)

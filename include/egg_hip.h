@@ -57,6 +57,8 @@ typedef struct egg_config {
     int chunk_members;       /* members evaluated per forward pass over the layers; 0 = auto */
     int weight_limit;        /* matrix weights saturate at +-weight_limit in the update rule: 127 as in the reference
                               * (mgpu.cu:1056-1062); 1 keeps them ternary (no reference counterpart)     */
+    int device_gaussian;     /* DEVICE_GAUSSIAN (mgpu.cu:195-196, :530-534): perturbation noise = sum of three masked fields */
+    int host_gaussian;       /* HOST_GAUSSIAN (mgpu.cu:192-193, :433-437): the same for the initial weights              */
 } egg_config;
 
 void egg_default_config(egg_config *cfg);

@@ -46,7 +46,7 @@ extern "C" void orc_default_config(orc_config *c) {
     c->softmax_scale_bit = 18; c->rope_scale_bit = 20; c->noise_mask = 15; c->host_mask = 15;
     c->softmax_exp_scale = 6.0;
     c->adam_beta1 = 0.9f; c->adam_beta2 = 0.95f; c->adam_eps = 1e-8f; c->adam_weight_decay = 0.01f;
-    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->weight_limit = 127;
+    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->weight_limit = 127; c->device_gaussian = 0; c->host_gaussian = 0;
 }
 
 /* ------------------------------------------------------------------ RNG */
@@ -56,20 +56,30 @@ extern "C" uint32_t orc_hash_rng(uint32_t s, uint32_t idx) {
     x ^= x >> 16; x *= 0x85ebca6bu; x ^= x >> 13; x *= 0xc2b2ae35u; x ^= x >> 16;
     return x;
 }
-/* mgpu.cu:528-538 (DEVICE_GAUSSIAN false) */
+/* the three fields of the Gaussian forms (mgpu.cu:433-436, :530-533): sign bits 0, 5, 10; magnitudes from bits 1, 6, 11 */
+static inline int noise_fields(uint32_t r, int maskword) {
+    const uint32_t m = (uint32_t)maskword & 0xffu;
+    int n = (r & 1 ? 1 : -1) * (int)((r >> 1) & m);
+    if (maskword & ORC_NOISE_GAUSSIAN) {
+        n += (r & 32 ? 1 : -1) * (int)((r >> 6) & m);
+        n += (r & 1024 ? 1 : -1) * (int)((r >> 11) & m);
+    }
+    return n;
+}
+/* mgpu.cu:528-538; mask is a noise mask word */
 extern "C" int8_t orc_noise(uint32_t s, uint32_t idx, int mask) {
-    uint32_t r = orc_hash_rng(s, idx);
-    return (int8_t)((r & 1 ? 1 : -1) * (int)((r >> 1) & (uint32_t)mask));
+    return (int8_t)noise_fields(orc_hash_rng(s, idx), mask);
 }
 /* mgpu.cu:428-430 */
 extern "C" uint32_t orc_xorshift32(uint32_t *state) {
     uint32_t x = *state; x ^= x << 13; x ^= x >> 17; x ^= x << 5; *state = x; return x;
 }
-/* mgpu.cu:431-441 (HOST_GAUSSIAN false) */
+/* mgpu.cu:431-441; mask is a noise mask word */
 extern "C" int8_t orc_gen_noise_host(uint32_t *state, int mask) {
-    uint32_t r = orc_xorshift32(state);
-    return (int8_t)((r & 1 ? 1 : -1) * (int)((r >> 1) & (uint32_t)mask));
+    return (int8_t)noise_fields(orc_xorshift32(state), mask);
 }
+static inline int dev_mask(const orc_config *c) { return c->noise_mask | (c->device_gaussian ? ORC_NOISE_GAUSSIAN : 0); }
+static inline int host_mask_word(const orc_config *c) { return c->host_mask | (c->host_gaussian ? ORC_NOISE_GAUSSIAN : 0); }
 /* mgpu.cu:539 */
 extern "C" int8_t orc_clip(int32_t a) { return (a > 127) ? 127 : ((a < -127) ? -127 : (int8_t)a); }
 
@@ -248,7 +258,7 @@ extern "C" void orc_init_model(const orc_config *c, int8_t *model, uint32_t seed
     Layout L = make_layout(c); int H = c->hidden, V = c->vocab; uint32_t rng = seed;
     memset(model, 0, (size_t)L.total);
     std::vector<int8_t> tmp((size_t)H * 4 * H > (size_t)V * H ? (size_t)H * 4 * H : (size_t)V * H);
-    auto fill = [&](int64_t n) { for (int64_t i = 0; i < n; i++) tmp[i] = orc_gen_noise_host(&rng, c->host_mask); };
+    auto fill = [&](int64_t n) { for (int64_t i = 0; i < n; i++) tmp[i] = orc_gen_noise_host(&rng, host_mask_word(c)); };
     fill((int64_t)V * H); orc_repack(model + L.embedding, tmp.data(), H, V);
     for (int i = 0; i < H; i++) { model[L.ln_init + i] = 16; }
     fill((int64_t)H * 4 * H); orc_repack(model + L.w_emb_mlp_up, tmp.data(), H, 4 * H);
@@ -295,7 +305,7 @@ static int32_t linear_proj(const orc_config *c, const int8_t *in, const int8_t *
     int32_t acc = 0;
     for (int k = 0; k < K; k++) acc += (int32_t)in[k] * (int32_t)blk(Wb, N, k, n);
     if (ns != 0) {
-        int8_t nz = orc_noise(noise_seed, (uint32_t)n, c->noise_mask);
+        int8_t nz = orc_noise(noise_seed, (uint32_t)n, dev_mask(c));
         int32_t a = sc_col ? (int32_t)(nz * afac(sc_col, n)) : (int32_t)nz;
         acc += ((sb * a) * ns) >> (c->fixed_point + c->sigma_shift);
     }
@@ -306,7 +316,7 @@ static int32_t linear_proj(const orc_config *c, const int8_t *in, const int8_t *
 static int32_t noise_dot(const orc_config *c, const int8_t *in, int K, uint32_t seed, const int8_t *sc_row) {
     int32_t sb = 0;
     for (int k = 0; k < K; k++) {
-        int32_t t = (int32_t)in[k] * orc_noise(seed, k, c->noise_mask);
+        int32_t t = (int32_t)in[k] * orc_noise(seed, k, dev_mask(c));
         sb += sc_row ? (int32_t)(t * afac(sc_row, k)) : t;
     }
     return sb;
@@ -329,13 +339,13 @@ static void standard_norm(const orc_config *c, const int8_t *x, const int8_t *w,
     for (int tid = 0; tid < H; tid++) {
         int32_t w_mod = w[tid], b_mod = b[tid];
         if (ns != 0) {
-            int8_t wn1 = orc_noise(seed_base + off_w_a, tid, c->noise_mask);
-            int8_t wn2 = orc_noise(seed_base + off_w_b, tid, c->noise_mask);
+            int8_t wn1 = orc_noise(seed_base + off_w_a, tid, dev_mask(c));
+            int8_t wn2 = orc_noise(seed_base + off_w_b, tid, dev_mask(c));
             /* with the overlay: (AccumType)(wn1 * wn2 * scale_w), de/include/model/layers.cuh:171-183 */
             int32_t wp = (int32_t)wn1 * wn2; if (sc_w) wp = (int32_t)(wp * afac(sc_w, tid));
             w_mod += (wp * ns) >> c->sigma_shift_vector;
-            int8_t bn1 = orc_noise(seed_base + off_b_a, tid, c->noise_mask);
-            int8_t bn2 = orc_noise(seed_base + off_b_b, tid, c->noise_mask);
+            int8_t bn1 = orc_noise(seed_base + off_b_a, tid, dev_mask(c));
+            int8_t bn2 = orc_noise(seed_base + off_b_b, tid, dev_mask(c));
             int32_t bp = (int32_t)bn1 * bn2; if (sc_b) bp = (int32_t)(bp * afac(sc_b, tid));
             b_mod += (bp * ns) >> c->sigma_shift_vector;
         }
@@ -443,7 +453,7 @@ extern "C" int32_t orc_down_dot_adaptive(const orc_config *c, const int8_t *mlp,
         int32_t pb = 0;
         for (int sub = 0; sub < 4; sub++) {
             int k = tid + sub * H;
-            pb += (int32_t)mlp[k] * orc_noise(seed, k, c->noise_mask) * afac(overlay_rows, k);
+            pb += (int32_t)mlp[k] * orc_noise(seed, k, dev_mask(c)) * afac(overlay_rows, k);
         }
         sb += pb;
     }
@@ -455,7 +465,7 @@ static void mlp_block(const orc_config *c, const int8_t *act_lut, int8_t *x,
                       const int8_t *ln_w, const int8_t *ln_b, const int8_t *up_w, const int8_t *up_b,
                       const int8_t *dn_w, const int8_t *dn_b, uint32_t seed_base, int ns, const MlpCfg &cfg,
                       const int8_t *model = NULL, const int8_t *sc = NULL) {
-    int H = c->hidden, H4 = 4 * H, M = c->noise_mask;
+    int H = c->hidden, H4 = 4 * H, M = dev_mask(c);
     const int8_t *s_lnw = sc_of(sc, model, ln_w), *s_lnb = sc_of(sc, model, ln_b);
     const int8_t *s_up = sc_of(sc, model, up_w), *s_bup = sc_of(sc, model, up_b);     /* up: rows H then cols 4H */
     const int8_t *s_dn = sc_of(sc, model, dn_w), *s_bdn = sc_of(sc, model, dn_b);     /* down: rows 4H then cols H */
@@ -493,7 +503,7 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
                               const uint8_t *data, int64_t data_len, int64_t start_idx,
                               uint32_t step_seed, int p_idx, int ns_override, orc_trace *tr,
                               const int8_t *sc = NULL) {
-    const int H = c->hidden, V = c->vocab, T = c->seq_len, NL = c->n_layers, M = c->noise_mask;
+    const int H = c->hidden, V = c->vocab, T = c->seq_len, NL = c->n_layers, M = dev_mask(c);
     Layout L = make_layout(c);
     int64_t pair_idx = p_idx / 2;
     int64_t stride = data_len / (c->population / 2);
@@ -646,11 +656,11 @@ extern "C" void orc_perturbed_linear(const orc_config *c, const int8_t *X, const
         int64_t member = r / T; uint32_t ps = seed + (uint32_t)(member / 2); int ns = (member % 2 == 0) ? 1 : -1;
         const int8_t *x = X + r * K;
         int32_t sb = 0;
-        for (int k = 0; k < K; k++) sb += (int32_t)x[k] * orc_noise(ps + off_b, k, c->noise_mask);
+        for (int k = 0; k < K; k++) sb += (int32_t)x[k] * orc_noise(ps + off_b, k, dev_mask(c));
         std::vector<int32_t> acc(N, 0);
         for (int k = 0; k < K; k++) { int32_t xv = x[k]; const int8_t *wr = &W[(size_t)k * N]; for (int n = 0; n < N; n++) acc[n] += xv * wr[n]; }
         for (int n = 0; n < N; n++) {
-            int32_t a = acc[n] + (((sb * (int32_t)orc_noise(ps + off_a, n, c->noise_mask)) * ns) >> (c->fixed_point + c->sigma_shift));
+            int32_t a = acc[n] + (((sb * (int32_t)orc_noise(ps + off_a, n, dev_mask(c))) * ns) >> (c->fixed_point + c->sigma_shift));
             Y[r * N + n] = a >> shift;
         }
     }
@@ -693,8 +703,8 @@ extern "C" int64_t orc_matrix_votes(const orc_config *c, int rows, int cols, int
 #pragma omp parallel for schedule(static)
     for (int p = 0; p < pairs; p++) {
         uint32_t s = step_seed + (uint32_t)p + (uint32_t)seed_base;
-        for (int n2 = 0; n2 < cols; n2++) A[(size_t)p * cols + n2] = orc_noise(s + off_a, n2, c->noise_mask);
-        for (int k = 0; k < rows; k++) B[(size_t)p * rows + k] = orc_noise(s + off_b, k, c->noise_mask);
+        for (int n2 = 0; n2 < cols; n2++) A[(size_t)p * cols + n2] = orc_noise(s + off_a, n2, dev_mask(c));
+        for (int k = 0; k < rows; k++) B[(size_t)p * rows + k] = orc_noise(s + off_b, k, dev_mask(c));
     }
 #pragma omp parallel for schedule(static)
     for (int64_t idx = 0; idx < n; idx++) {
@@ -733,8 +743,8 @@ extern "C" uint64_t orc_update_vector_adam(const orc_config *c, int8_t *V, orc_a
         int32_t vote = 0;
         for (int p = 0; p < pairs; p++) {
             int f = fit[p]; if (f == 0) continue;
-            int32_t n1 = orc_noise(step_seed + p + seed_base + off_a, idx, c->noise_mask);
-            int32_t n2 = orc_noise(step_seed + p + seed_base + off_b, idx, c->noise_mask);
+            int32_t n1 = orc_noise(step_seed + p + seed_base + off_a, idx, dev_mask(c));
+            int32_t n2 = orc_noise(step_seed + p + seed_base + off_b, idx, dev_mask(c));
             vote += f * n1 * n2;
         }
         int change = 0;

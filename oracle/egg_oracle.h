@@ -65,7 +65,11 @@ typedef struct orc_config {
     float muon_lr_scale;     /* 1.0                   mgpu.cu:267 */
     int weight_limit;        /* matrix weights saturate at +-this in the update rule: 127, mgpu.cu:1056-1062;
                               * other values have no counterpart in the reference (ternary weights: 1) */
+    int device_gaussian;     /* DEVICE_GAUSSIAN false  mgpu.cu:195-196 */
+    int host_gaussian;       /* HOST_GAUSSIAN false    mgpu.cu:192-193 */
 } orc_config;
+/* a noise mask word: the magnitude mask in the low byte, 0x100 on top for the Gaussian form (three masked fields) */
+#define ORC_NOISE_GAUSSIAN 0x100
 
 void orc_default_config(orc_config *c);
 

@@ -17,14 +17,21 @@ OFF = dict(EMB=0, EMB_BIAS=(50, 51), LN_1=(100, 101), LN_1_BIAS=(110, 111), Q=(2
 M32 = np.uint64(0xFFFFFFFF)
 
 
-def noise(seed, idx, mask):
-    """hash_rng + noise_from_hash, mgpu.cu:525-538: murmur3 fmix32 of seed + idx * 0x9e3779b9; sign from bit 0"""
+def noise(seed, idx, cfg):
+    """hash_rng + noise_from_hash, mgpu.cu:525-538: murmur3 fmix32 of seed + idx * 0x9e3779b9; a field is a sign bit
+    followed by the masked magnitude; DEVICE_GAUSSIAN adds the fields that start at bits 5 and 10 to the one at bit 0.
+    cfg is the configuration, or a plain magnitude mask."""
+    mask, gaussian = (cfg, 0) if isinstance(cfg, int) else (cfg.noise_mask, cfg.device_gaussian)
     x = (np.uint64(int(seed) & 0xFFFFFFFF) + np.asarray(idx, np.uint64) * np.uint64(0x9E3779B9)) & M32
     x ^= x >> np.uint64(16); x = (x * np.uint64(0x85EBCA6B)) & M32
     x ^= x >> np.uint64(13); x = (x * np.uint64(0xC2B2AE35)) & M32
     x ^= x >> np.uint64(16)
-    mag = ((x >> np.uint64(1)) & np.uint64(mask)).astype(np.int64)
-    return np.where((x & np.uint64(1)) != 0, mag, -mag)
+    total = 0
+    for start in ((0, 5, 10) if gaussian else (0,)):
+        f = x >> np.uint64(start)
+        mag = ((f >> np.uint64(1)) & np.uint64(mask)).astype(np.int64)
+        total = total + np.where((f & np.uint64(1)) != 0, mag, -mag)
+    return total
 
 
 def clip(a):
@@ -51,8 +58,8 @@ def standard_norm(cfg, x, w, b, seed, off_w, off_b, ns):
     h = np.arange(H)
     mn = np.abs(x).sum(axis=1) // H
     mn = np.where(mn == 0, 1, mn)[:, None]
-    w_mod = w.astype(np.int64) + ((noise(seed + off_w[0], h, cfg.noise_mask) * noise(seed + off_w[1], h, cfg.noise_mask) * ns) >> cfg.sigma_shift_vector)
-    b_mod = b.astype(np.int64) + ((noise(seed + off_b[0], h, cfg.noise_mask) * noise(seed + off_b[1], h, cfg.noise_mask) * ns) >> cfg.sigma_shift_vector)
+    w_mod = w.astype(np.int64) + ((noise(seed + off_w[0], h, cfg) * noise(seed + off_w[1], h, cfg) * ns) >> cfg.sigma_shift_vector)
+    b_mod = b.astype(np.int64) + ((noise(seed + off_b[0], h, cfg) * noise(seed + off_b[1], h, cfg) * ns) >> cfg.sigma_shift_vector)
     return clip(trunc_div(x * w_mod[None, :], mn) + b_mod[None, :])
 
 
@@ -70,8 +77,8 @@ def linear(cfg, x, W, seed, off, ns):
     K, N = W.shape
     acc = x @ W
     if ns != 0:
-        sb = x @ noise(seed + off[1], np.arange(K), cfg.noise_mask)
-        a = noise(seed + off[0], np.arange(N), cfg.noise_mask)
+        sb = x @ noise(seed + off[1], np.arange(K), cfg)
+        a = noise(seed + off[0], np.arange(N), cfg)
         acc = acc + ((sb[:, None] * a[None, :] * ns) >> (cfg.fixed_point + cfg.sigma_shift))
     return acc
 
@@ -119,12 +126,12 @@ def mlp_block(cfg, x, t, seed, ns, act_lut, names, offs):
     nrm = standard_norm(cfg, x, t[ln_w], t[ln_b], seed, o_ln, o_lnb, ns)
     a = linear(cfg, nrm, t[w_up], seed, o_up, ns)
     o = np.arange(4 * H)
-    nv = (noise(seed + o_bup[0], o, cfg.noise_mask) * noise(seed + o_bup[1], o, cfg.noise_mask) * ns) >> cfg.sigma_shift_vector
+    nv = (noise(seed + o_bup[0], o, cfg) * noise(seed + o_bup[1], o, cfg) * ns) >> cfg.sigma_shift_vector
     pre = clip((a >> cfg.shift_mlp_up) + t[b_up].astype(np.int64)[None, :] + nv[None, :])
     mid = act_lut.astype(np.int64)[pre & 0xFF]                          # ACT_LUT[(uint8_t)clip(...)]
     adn = linear(cfg, mid, t[w_dn], seed, o_dn, ns)
     hh = np.arange(H)
-    nv = (noise(seed + o_bdn[0], hh, cfg.noise_mask) * noise(seed + o_bdn[1], hh, cfg.noise_mask) * ns) >> cfg.sigma_shift_vector
+    nv = (noise(seed + o_bdn[0], hh, cfg) * noise(seed + o_bdn[1], hh, cfg) * ns) >> cfg.sigma_shift_vector
     return adaptive_normalize(x + (adn >> cfg.shift_mlp_down) + t[b_dn].astype(np.int64)[None, :] + nv[None, :])
 
 
@@ -148,9 +155,9 @@ def forward_member(cfg, model, tensor_table, tables, data, start_idx, step_seed,
     hh = np.arange(H)
     # embedding, mgpu.cu:901-931
     E = t["embedding"]                                                                      # [H, V]
-    chk = (noise(pseed + OFF["EMB_BIAS"][0], hh, cfg.noise_mask) * noise(pseed + OFF["EMB_BIAS"][1], hh, cfg.noise_mask) * ns) >> cfg.sigma_shift_vector
-    a_tok = noise(pseed + OFF["EMB"], tok, cfg.noise_mask)
-    b_dim = noise(pseed + OFF["EMB"] + H, hh, cfg.noise_mask)
+    chk = (noise(pseed + OFF["EMB_BIAS"][0], hh, cfg) * noise(pseed + OFF["EMB_BIAS"][1], hh, cfg) * ns) >> cfg.sigma_shift_vector
+    a_tok = noise(pseed + OFF["EMB"], tok, cfg)
+    b_dim = noise(pseed + OFF["EMB"] + H, hh, cfg)
     perturb = (a_tok[:, None] * b_dim[None, :] * ns) >> (cfg.fixed_point + cfg.sigma_shift)
     x = clip(E[:, tok].T + t["emb_bias"][None, :] + chk[None, :] + perturb)
     x = mlp_block(cfg, x, t, pseed, ns, act_lut,
@@ -174,8 +181,8 @@ def forward_member(cfg, model, tensor_table, tables, data, start_idx, step_seed,
     # head and loss, mgpu.cu:955-1024
     nf = standard_norm(cfg, x, t["ln_f"], t["ln_f_bias"], pseed, OFF["LN_F"], OFF["LN_F_BIAS"], ns)
     acc = nf @ E
-    sbh = nf @ noise(pseed + OFF["EMB"] + H, hh, cfg.noise_mask)
-    acc = acc + ((sbh[:, None] * noise(pseed + OFF["EMB"], np.arange(V), cfg.noise_mask)[None, :] * ns) >> (cfg.fixed_point + cfg.sigma_shift))
+    sbh = nf @ noise(pseed + OFF["EMB"] + H, hh, cfg)
+    acc = acc + ((sbh[:, None] * noise(pseed + OFF["EMB"], np.arange(V), cfg)[None, :] * ns) >> (cfg.fixed_point + cfg.sigma_shift))
     logits = acc >> cfg.shift_logit
     G = logits.max(axis=1)
     S = exp_lut.astype(np.int64)[np.clip(G[:, None] - logits, 0, 255)].sum(axis=1)
@@ -202,16 +209,16 @@ def es_update_adam(cfg, model, state, tensor_table, fit, step_seed, lr):
         seeds = (step_seed + p + e["seed_base"]) & 0xFFFFFFFF
         if e["is_matrix"]:
             # A[p, n_out], B[p, k_in]; vote[k, n] = sum_p fit_p * A[p, n] * B[p, k]   (mgpu.cu:1092-1098)
-            A = np.stack([noise(int(s) + e["off_a"], np.arange(e["cols"]), cfg.noise_mask) for s in seeds])
-            B = np.stack([noise(int(s) + e["off_b"], np.arange(e["rows"]), cfg.noise_mask) for s in seeds])
+            A = np.stack([noise(int(s) + e["off_a"], np.arange(e["cols"]), cfg) for s in seeds])
+            B = np.stack([noise(int(s) + e["off_b"], np.arange(e["rows"]), cfg) for s in seeds])
             vote_kn = (B * fit[:, None]).T @ A
             # blocked element index -> (k, n), mgpu.cu:1085-1089
             idx = np.arange(n)
             vote = vote_kn[(idx >> 2) // e["cols"] * 4 + (idx & 3), (idx >> 2) % e["cols"]]
         else:
             i = np.arange(n)
-            n1 = np.stack([noise(int(s) + e["off_a"], i, cfg.noise_mask) for s in seeds])
-            n2 = np.stack([noise(int(s) + e["off_b"], i, cfg.noise_mask) for s in seeds])
+            n1 = np.stack([noise(int(s) + e["off_a"], i, cfg) for s in seeds])
+            n2 = np.stack([noise(int(s) + e["off_b"], i, cfg) for s in seeds])
             vote = (fit[:, None] * n1 * n2).sum(axis=0)
         # apply_adam_update, mgpu.cu:1040-1064 (no bias correction; fractional accumulator moves the int8 weight)
         g = -(vote.astype(f32))

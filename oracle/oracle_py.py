@@ -23,7 +23,7 @@ class OrcConfig(C.Structure):
         ("softmax_exp_scale", C.c_double),
         ("adam_beta1", C.c_float), ("adam_beta2", C.c_float), ("adam_eps", C.c_float),
         ("adam_weight_decay", C.c_float), ("muon_momentum", C.c_float), ("muon_lr_scale", C.c_float),
-        ("weight_limit", C.c_int)]
+        ("weight_limit", C.c_int), ("device_gaussian", C.c_int), ("host_gaussian", C.c_int)]
 
 
 class OrcTensor(C.Structure):
@@ -180,6 +180,25 @@ def ref():
         R.ref_ternary_unpack.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p]
         _ref = R
     return _ref
+
+
+_ref_gaussian = None
+
+
+def ref_gaussian():
+    """oracle/_ref/libegg_ref_gaussian.so: the same reference header compiled with -DDEVICE_GAUSSIAN=true
+    -DHOST_GAUSSIAN=true; None if absent."""
+    global _ref_gaussian
+    path = os.path.join(os.path.dirname(REF_PATH), "libegg_ref_gaussian.so")
+    if _ref_gaussian is None:
+        if not os.path.exists(path):
+            return None
+        R = C.CDLL(path)
+        R.ref_noise_from_hash.restype = C.c_int
+        R.ref_noise_from_hash.argtypes = [C.c_uint32, C.c_uint32]
+        R.ref_gen_noise_host.restype = C.c_int
+        _ref_gaussian = R
+    return _ref_gaussian
 
 
 # ----------------------------------------------------------------------------- helpers

@@ -63,7 +63,9 @@ def test_unsupported_configurations_are_refused_with_a_reason(pkg):
     lib = pkg.lib()
     for kw, word in ((dict(hidden=100), "hidden"), (dict(head_dim=48), "head_dim"), (dict(seq_len=48), "seq_len"),
                      (dict(population=7), "population"), (dict(rope_scale_bit=31), "rope_scale_bit"),
-                     (dict(noise_mask=127, sigma_shift_vector=0), "noise_mask"), (dict(weight_limit=0), "weight_limit"),
+                     (dict(noise_mask=60, sigma_shift_vector=0), "noise_mask"), (dict(weight_limit=0), "weight_limit"),
+                     (dict(noise_mask=127), "noise too wide"), (dict(device_gaussian=1, noise_mask=50), "Gaussian"),
+                     (dict(hidden=512, device_gaussian=1), "noise too wide"),
                      (dict(shift_mlp_up=40), "shift")):
         cfg = pkg.default_config(**kw)
         h = ctypes.c_void_p()

@@ -30,7 +30,8 @@ def _mapping_hint(got, exp):
 
 
 def test_tables_and_model_init(pkg, orc, dev):
-    for kw in (SMALL, dict(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=4)):
+    for kw in (SMALL, dict(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=4),
+               dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4, host_gaussian=1)):
         ctx = pkg.Context(pkg.default_config(**kw))
         ocfg = orc.config(**kw)
         ex, act, rope = ctx.tables()
@@ -54,6 +55,14 @@ def test_noise_fill(pkg, orc, dev):
         ctx.noise_fill(seed, first, n, out.data_ptr())
         ctx.sync()
         assert np.array_equal(out.cpu().numpy(), orc.noise_vec(seed, n, 15, first)), (seed, first)
+    ctx.close()
+    # DEVICE_GAUSSIAN: the sum of three masked fields (mask word 15 | 0x100 in the oracle)
+    ctx = pkg.Context(pkg.default_config(device_gaussian=1, **SMALL))
+    out = torch.zeros(4096, dtype=torch.int8, device=dev)
+    ctx.noise_fill(777, 5, 4096, out.data_ptr())
+    ctx.sync()
+    got = out.cpu().numpy()
+    assert np.array_equal(got, orc.noise_vec(777, 4096, 15 | 0x100, 5)) and got.min() < -30 and got.max() > 30
     ctx.close()
 
 
@@ -111,8 +120,10 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
                                 dict(hidden=64, head_dim=32, n_layers=1, seq_len=512, population=2),
                                 dict(hidden=128, head_dim=64, n_layers=1, seq_len=512, population=2),
                                 # a RoPE table scale of 2^30, the largest an int32 table holds (products then need all 64 bits)
-                                dict(hidden=128, head_dim=64, n_layers=1, seq_len=64, population=2, rope_scale_bit=30)],
-                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30"])
+                                dict(hidden=128, head_dim=64, n_layers=1, seq_len=64, population=2, rope_scale_bit=30),
+                                # DEVICE_GAUSSIAN / HOST_GAUSSIAN: noise up to +-45 (the kernels' unfused shift path)
+                                dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4, device_gaussian=1, host_gaussian=1)],
+                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30", "gaussian"])
 def test_forward_stages_and_loss(pkg, orc, dev, kw):
     """Every stage tap of every member against the oracle's trace, then the per-member losses."""
     data = orc.zipf_bytes(1 << 15)
@@ -235,8 +246,9 @@ def test_fitness(pkg, orc, dev):
 
 @pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=200),
                                 dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=66),
-                                dict(hidden=512, head_dim=64, n_layers=1, seq_len=128, population=40)],
-                         ids=["p200", "p66", "h512"])
+                                dict(hidden=512, head_dim=64, n_layers=1, seq_len=128, population=40),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=200, device_gaussian=1)],
+                         ids=["p200", "p66", "h512", "gaussian"])
 def test_votes_and_adam_update(pkg, orc, dev, kw):
     import torch
     ocfg = orc.config(**kw)

@@ -100,6 +100,37 @@ def test_repack_roundtrip_and_embedding_access(orc):
         assert Wb[((h >> 2) * N + tok) * 4 + (h & 3)] == W[h, tok]
 
 
+def test_gaussian_noise_against_reference_header(orc):
+    """DEVICE_GAUSSIAN / HOST_GAUSSIAN (mgpu.cu:433-437, :530-534): the reference's own header compiled with both macros
+    on, against the oracle's mask word 15 | 0x100; plus the definition on hand-built hash values."""
+    L = orc.lib()
+    G = 15 | 0x100
+    # a draw of 0b_00111_1_01010_0_00011_1: fields +3, -10, +7
+    r = (0b001111 << 10) | (0b010100 << 5) | 0b000111
+    sign = lambda b: 1 if b else -1
+    assert sign(r & 1) * ((r >> 1) & 15) + sign(r & 32) * ((r >> 6) & 15) + sign(r & 1024) * ((r >> 11) & 15) == 3 - 10 + 7
+    vals = [int(L.orc_noise(1234, i, G)) for i in range(4096)]
+    assert min(vals) < -30 and max(vals) > 30 and abs(sum(vals)) < 4096        # three fields: range +-45, centred
+    R = orc.ref_gaussian()
+    if R is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    rng = np.random.default_rng(3)
+    for s, i in rng.integers(0, 2**32, size=(4000, 2), dtype=np.uint64):
+        assert int(L.orc_noise(int(s), int(i), G)) == R.ref_noise_from_hash(int(s), int(i))
+    a, b = C.c_uint32(42), C.c_uint32(42)
+    for _ in range(2000):
+        assert int(L.orc_gen_noise_host(C.byref(a), G)) == R.ref_gen_noise_host(C.byref(b))
+    assert a.value == b.value
+    # the model initialised with HOST_GAUSSIAN is that stream
+    cfg = orc.config(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4, host_gaussian=1)
+    m = orc.init_model(cfg, 42)
+    t = {t["name"]: t for t in orc.tensor_table(cfg)}["embedding"]
+    emb = np.zeros((t["rows"], t["cols"]), np.int8)
+    L.orc_unpack(P(emb), P(np.ascontiguousarray(m[t["offset"]:t["offset"] + t["rows"] * t["cols"]])), t["rows"], t["cols"])
+    st = C.c_uint32(42)
+    assert emb.ravel()[:512].tolist() == [R.ref_gen_noise_host(C.byref(st)) for _ in range(512)]
+
+
 def test_init_model_stream_order(orc):
     cfg = orc.config(hidden=64, head_dim=32, n_layers=2, seq_len=32, population=8)
     m = orc.init_model(cfg, 42)
@@ -660,8 +691,9 @@ def test_ternary_model_packing_and_weight_limit(orc):
                                 dict(hidden=128, head_dim=64, n_layers=1, seq_len=24, population=4),
                                 dict(hidden=64, head_dim=32, n_layers=1, seq_len=40, population=4, sigma_shift=1, noise_mask=31,
                                      shift_out=8, shift_mlp_up=7, shift_mlp_down=9, sigma_shift_vector=3),
-                                dict(hidden=256, head_dim=64, n_layers=4, seq_len=8, population=2)],
-                         ids=["h64", "h128", "other_shifts", "h256_l4"])
+                                dict(hidden=256, head_dim=64, n_layers=4, seq_len=8, population=2),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=4, device_gaussian=1, host_gaussian=1)],
+                         ids=["h64", "h128", "other_shifts", "h256_l4", "gaussian"])
 def test_two_restatements_of_the_forward_agree(orc, kw):
     """Nothing external pins the composition of the whole forward (the reference ships no golden vectors), so it is
     stated twice: the C++ oracle walks token by token with a K/V cache as the reference kernel does, the numpy
@@ -690,11 +722,12 @@ def test_two_restatements_of_the_forward_agree(orc, kw):
         assert loss == ref_loss, m
 
 
-def test_two_restatements_of_the_update_agree(orc):
+@pytest.mark.parametrize("gaussian", [0, 1], ids=["uniform", "gaussian"])
+def test_two_restatements_of_the_update_agree(orc, gaussian):
     """The whole AdamW ES update (votes of every tensor, float32 optimizer state, int8 weights, change count) in numpy
     array arithmetic against the C++ oracle's element-by-element loops, over several steps that cross the +-1 thresholds."""
     from oracle import forward_numpy as fn
-    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=24)
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=24, device_gaussian=gaussian)
     cfg = orc.config(**kw)
     tt = orc.tensor_table(cfg)
     rng = np.random.default_rng(8)
