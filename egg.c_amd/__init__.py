@@ -28,7 +28,7 @@ class EggConfig(C.Structure):
         ("adam_beta1", C.c_float), ("adam_beta2", C.c_float), ("adam_eps", C.c_float),
         ("adam_weight_decay", C.c_float), ("muon_momentum", C.c_float), ("muon_lr_scale", C.c_float),
         ("use_muon", C.c_int), ("chunk_members", C.c_int), ("weight_limit", C.c_int),
-        ("device_gaussian", C.c_int), ("host_gaussian", C.c_int)]
+        ("device_gaussian", C.c_int), ("host_gaussian", C.c_int), ("use_same_data", C.c_int)]
 
 
 class EggTensorInfo(C.Structure):

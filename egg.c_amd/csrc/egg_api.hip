@@ -120,7 +120,7 @@ extern "C" void egg_default_config(egg_config *c) {
     c->softmax_exp_scale = 6.0;
     c->adam_beta1 = 0.9f; c->adam_beta2 = 0.95f; c->adam_eps = 1e-8f; c->adam_weight_decay = 0.01f;
     c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->use_muon = 0; c->chunk_members = 0; c->weight_limit = 127;
-    c->device_gaussian = 0; c->host_gaussian = 0;
+    c->device_gaussian = 0; c->host_gaussian = 0; c->use_same_data = 0;
 }
 
 // launch order of mgpu.cu:1603-1643
@@ -508,7 +508,7 @@ static FwdCommon make_common(egg_ctx *ctx, const uint8_t *d_data, int64_t len, c
     const egg_config &c = ctx->cfg;
     FwdCommon f;
     f.data = d_data; f.data_len = len; f.d_start_idx = d_start; f.d_step_seed = d_seed;
-    f.pop_offset = first_member; f.n_members = nm; f.population = c.population;
+    f.pop_offset = first_member; f.n_members = nm; f.population = c.population; f.same_data = c.use_same_data != 0;
     f.T = c.seq_len; f.H = c.hidden; f.head_dim = c.head_dim; f.vocab = c.vocab;
     f.sigma = c.fixed_point + c.sigma_shift; f.sigma_vec = c.sigma_shift_vector;
     f.mask = ctx->mask_override >= 0 ? ctx->mask_override : noise_word(c);

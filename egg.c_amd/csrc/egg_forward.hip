@@ -17,7 +17,7 @@
 
 // stream position of a member's pair (mgpu.cu:864-870)
 __device__ __forceinline__ int64_t stream_pos_of(const FwdCommon &c, int member) {
-    int64_t pair = member / 2;
+    int64_t pair = c.same_data ? 0 : member / 2;
     int64_t stride = c.data_len / (c.population / 2);
     return (*c.d_start_idx + pair * stride) % (c.data_len - c.T);
 }

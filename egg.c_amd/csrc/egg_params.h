@@ -33,6 +33,7 @@ struct FwdCommon {
     int pop_offset;              // global index of the chunk's first member
     int n_members;               // members in the chunk
     int population;
+    int same_data;               // USE_SAME_DATA: every pair reads the window at the start index
     int T, H, head_dim, vocab;
     int sigma;                   // fixed_point + sigma_shift
     int sigma_vec;               // sigma_shift_vector

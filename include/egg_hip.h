@@ -59,6 +59,7 @@ typedef struct egg_config {
                               * (mgpu.cu:1056-1062); 1 keeps them ternary (no reference counterpart)     */
     int device_gaussian;     /* DEVICE_GAUSSIAN (mgpu.cu:195-196, :530-534): perturbation noise = sum of three masked fields */
     int host_gaussian;       /* HOST_GAUSSIAN (mgpu.cu:192-193, :433-437): the same for the initial weights              */
+    int use_same_data;       /* USE_SAME_DATA (mgpu.cu:212-213, :866-867): every pair reads the window at start_idx      */
 } egg_config;
 
 void egg_default_config(egg_config *cfg);

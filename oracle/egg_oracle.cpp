@@ -46,7 +46,7 @@ extern "C" void orc_default_config(orc_config *c) {
     c->softmax_scale_bit = 18; c->rope_scale_bit = 20; c->noise_mask = 15; c->host_mask = 15;
     c->softmax_exp_scale = 6.0;
     c->adam_beta1 = 0.9f; c->adam_beta2 = 0.95f; c->adam_eps = 1e-8f; c->adam_weight_decay = 0.01f;
-    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->weight_limit = 127; c->device_gaussian = 0; c->host_gaussian = 0;
+    c->muon_momentum = 0.85f; c->muon_lr_scale = 1.0f; c->weight_limit = 127; c->device_gaussian = 0; c->host_gaussian = 0; c->use_same_data = 0;
 }
 
 /* ------------------------------------------------------------------ RNG */
@@ -507,7 +507,7 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
     Layout L = make_layout(c);
     int64_t pair_idx = p_idx / 2;
     int64_t stride = data_len / (c->population / 2);
-    int64_t stream_pos = (start_idx + pair_idx * stride) % (data_len - T);
+    int64_t stream_pos = (c->use_same_data ? start_idx : start_idx + pair_idx * stride) % (data_len - T);   /* mgpu.cu:866-870 */
     int ns = (p_idx % 2 == 0) ? 1 : -1;
     if (ns_override != 2) ns = ns_override;
     uint32_t pair_seed = step_seed + (uint32_t)pair_idx;

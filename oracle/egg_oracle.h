@@ -67,6 +67,7 @@ typedef struct orc_config {
                               * other values have no counterpart in the reference (ternary weights: 1) */
     int device_gaussian;     /* DEVICE_GAUSSIAN false  mgpu.cu:195-196 */
     int host_gaussian;       /* HOST_GAUSSIAN false    mgpu.cu:192-193 */
+    int use_same_data;       /* USE_SAME_DATA 0        mgpu.cu:212-213 */
 } orc_config;
 /* a noise mask word: the magnitude mask in the low byte, 0x100 on top for the Gaussian form (three masked fields) */
 #define ORC_NOISE_GAUSSIAN 0x100

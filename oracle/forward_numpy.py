@@ -148,7 +148,7 @@ def forward_member(cfg, model, tensor_table, tables, data, start_idx, step_seed,
     pair = p_idx // 2
     ns = 1 if p_idx % 2 == 0 else -1
     stride = len(data) // (cfg.population // 2)
-    pos = (start_idx + pair * stride) % (len(data) - T)                                     # mgpu.cu:864-870
+    pos = (start_idx + (0 if cfg.use_same_data else pair * stride)) % (len(data) - T)       # mgpu.cu:864-870
     tok = data[pos:pos + T].astype(np.int64)
     target = data[pos + 1:pos + T + 1].astype(np.int64)
     pseed = (step_seed + pair) & 0xFFFFFFFF

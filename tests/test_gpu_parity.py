@@ -122,8 +122,10 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
                                 # a RoPE table scale of 2^30, the largest an int32 table holds (products then need all 64 bits)
                                 dict(hidden=128, head_dim=64, n_layers=1, seq_len=64, population=2, rope_scale_bit=30),
                                 # DEVICE_GAUSSIAN / HOST_GAUSSIAN: noise up to +-45 (the kernels' unfused shift path)
-                                dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4, device_gaussian=1, host_gaussian=1)],
-                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30", "gaussian"])
+                                dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4, device_gaussian=1, host_gaussian=1),
+                                # USE_SAME_DATA: every pair reads the same window
+                                dict(hidden=128, head_dim=64, n_layers=1, seq_len=128, population=6, use_same_data=1)],
+                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30", "gaussian", "same_data"])
 def test_forward_stages_and_loss(pkg, orc, dev, kw):
     """Every stage tap of every member against the oracle's trace, then the per-member losses."""
     data = orc.zipf_bytes(1 << 15)

@@ -692,8 +692,9 @@ def test_ternary_model_packing_and_weight_limit(orc):
                                 dict(hidden=64, head_dim=32, n_layers=1, seq_len=40, population=4, sigma_shift=1, noise_mask=31,
                                      shift_out=8, shift_mlp_up=7, shift_mlp_down=9, sigma_shift_vector=3),
                                 dict(hidden=256, head_dim=64, n_layers=4, seq_len=8, population=2),
-                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=4, device_gaussian=1, host_gaussian=1)],
-                         ids=["h64", "h128", "other_shifts", "h256_l4", "gaussian"])
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=4, device_gaussian=1, host_gaussian=1),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=6, use_same_data=1)],
+                         ids=["h64", "h128", "other_shifts", "h256_l4", "gaussian", "same_data"])
 def test_two_restatements_of_the_forward_agree(orc, kw):
     """Nothing external pins the composition of the whole forward (the reference ships no golden vectors), so it is
     stated twice: the C++ oracle walks token by token with a K/V cache as the reference kernel does, the numpy
