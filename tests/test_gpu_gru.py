@@ -16,7 +16,9 @@ def _t(dev, arr):
     (dict(hidden=64, n_layers=2, seq_len=6, population=32, update_threshold=12), 3),
     (dict(hidden=128, n_layers=1, seq_len=5, population=64, update_threshold=20), 2),
     (dict(hidden=512, n_layers=4, seq_len=3, population=32, update_threshold=10), 2),
-], ids=["h64", "h128", "h512"])
+    (dict(hidden=256, n_layers=2, seq_len=4, population=96, update_threshold=30), 2),
+    (dict(hidden=64, n_layers=1, seq_len=9, population=32, update_threshold=5, sigma_shift=2), 3),
+], ids=["h64", "h128", "h512", "h256_p96", "sigma_2"])
 def test_gru_steps(pkg, orc, dev, kw, steps):
     import ctypes as C
     g = orc.gru_config(**kw)
