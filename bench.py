@@ -146,11 +146,17 @@ def main():
         W = torch.randint(-127, 128, (K * N,), dtype=torch.int8, device=dev)
         Y = torch.empty((members * Tm, N), dtype=torch.int32, device=dev)
         Y8 = torch.empty((members * Tm, N), dtype=torch.int8, device=dev)
-        for name, y32, y8, bytes_row in (("int32_out", Y.data_ptr(), None, K + 4 * N), ("int8_out", None, Y8.data_ptr(), K + N)):
-            ctx.perturbed_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 3, 200, 201, 8, y32, y8)
+        # the last leg is the shared-weight GEMM alone (no rank-1 term: the reference's ns == 0 case)
+        for name, y32, y8, bytes_row in (("int32_out", Y.data_ptr(), None, K + 4 * N), ("int8_out", None, Y8.data_ptr(), K + N),
+                                         ("int8_out_shared_gemm_only", None, Y8.data_ptr(), K + N)):
+            if name.endswith("only"):
+                run = lambda: ctx.shared_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 8, y32, y8)
+            else:
+                run = lambda: ctx.perturbed_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 3, 200, 201, 8, y32, y8)
+            run()
             ctx.enable_timing(True); ctx.timing_reset()
             for _ in range(5):
-                ctx.perturbed_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 3, 200, 201, 8, y32, y8)
+                run()
             nl, ms = ctx.timing()["plinear"]
             ctx.enable_timing(False)
             sec = ms / nl * 1e-3

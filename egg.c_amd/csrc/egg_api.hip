@@ -477,8 +477,18 @@ extern "C" int egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first, int n
     return EGG_OK;
 }
 
+static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
+                       uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8, int plain);
 extern "C" int egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
                                     uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8) {
+    return linear_impl(ctx, d_X, d_W, members, T, K, N, seed, off_a, off_b, shift, d_Y32, d_Y8, 0);
+}
+extern "C" int egg_shared_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
+                                 int shift, int32_t *d_Y32, int8_t *d_Y8) {
+    return linear_impl(ctx, d_X, d_W, members, T, K, N, 0, 0, 0, shift, d_Y32, d_Y8, 1);
+}
+static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
+                       uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8, int plain) {
     if (!ctx || !d_X || !d_W || members < 1 || T < 32 || T % 32 || (!d_Y32 && !d_Y8) || shift < 0 || shift > 31)
         return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear arguments");
     if (K < 64 || N < 64 || K % 64 || N % 64) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: K and N must be multiples of 64");
@@ -490,7 +500,7 @@ extern "C" int egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_
         ctx->plin_frag_bytes = (size_t)K * N;
     }
     PlinParams p = {d_X, ctx->d_plin_frag, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
-                    noise_word(ctx->cfg), d_Y32, d_Y8};
+                    noise_word(ctx->cfg), d_Y32, d_Y8, plain};
     const int PB = egg_plinear_block(K, N);
     if (K % PB || N % PB) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");
     span_begin(ctx, EGG_K_PLINEAR);

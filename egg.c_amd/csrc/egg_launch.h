@@ -17,6 +17,7 @@ struct PlinParams {
     int members, T, K, N;
     uint32_t seed; int off_a, off_b, shift, sigma, mask;
     int32_t *Y32; int8_t *Y8;
+    int plain;              // the shared-weight product alone: no rank-1 term (the reference's ns == 0 case)
 };
 hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s);
 int egg_plinear_block(int K, int N);

@@ -9,6 +9,7 @@
 // next token tile are loaded while the current one is multiplied, and results leave through a per-wave LDS
 // transpose so that eight lanes write one full 128-byte line of a row (in the MFMA result layout a store
 // instruction would touch 32 rows with 32 bytes each).
+#include <type_traits>
 #include "egg_device.h"
 #include "egg_launch.h"
 
@@ -92,8 +93,10 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
         }
     };
     for (int i = 0; i < P::AHEAD; i++) request();
-    fill_noise_i32(At, ps + p.off_a, N, p.mask, ns, lane);
-    fill_noise_i8(Bt, ps + p.off_b, K, p.mask, lane);
+    if (!p.plain) {
+        fill_noise_i32(At, ps + p.off_a, N, p.mask, ns, lane);
+        fill_noise_i8(Bt, ps + p.off_b, K, p.mask, lane);
+    }
     __syncthreads();
 
     int used = 0;                                  // units consumed so far
@@ -120,7 +123,7 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) xnext[P::PREFETCH_X ? ks : 0] = load_op(p.X + (row + 32) * K, ks, g);
         }
-        const int sb = dot_noise<KS, true>(xop, Bt, 0, g);
+        const int sb = p.plain ? 0 : dot_noise<KS, true>(xop, Bt, 0, g);
 #pragma unroll 1
         for (int nb = 0; nb < P::NBLK; nb++) {
             v16i acc[NTB];
@@ -171,6 +174,10 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
                     acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(frag[slot][nt], xlast, acc[nt], 0, 0, 0);
             }
             const size_t row_base = (size_t)member * p.T + pass * 32;
+            // PLAIN: acc >> shift without the rank-1 term (a wave-uniform choice made once per column block)
+            auto finish_block = [&](auto plain_tag) {
+            constexpr bool PLAIN = decltype(plain_tag)::value;
+            auto fin = [&](int a, int an) { return PLAIN ? (a >> p.shift) : perturbed<FUSE>(a, sb, an, p.sigma, p.shift); };
             if (OUT32) {
                 // one 32 x 32 int32 tile (128 bytes per row) at a time
 #pragma unroll
@@ -178,10 +185,10 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
                         int n0 = nb * B + 32 * nt + 8 * q + 4 * g;
-                        v4i a4 = *reinterpret_cast<const v4i *>(At + n0);
+                        v4i a4 = {0, 0, 0, 0}; if (!PLAIN) a4 = *reinterpret_cast<const v4i *>(At + n0);
                         v4i o4;
 #pragma unroll
-                        for (int e = 0; e < 4; e++) o4[e] = perturbed<FUSE>(acc[nt][4 * q + e], sb, a4[e], p.sigma, p.shift);
+                        for (int e = 0; e < 4; e++) o4[e] = fin(acc[nt][4 * q + e], a4[e]);
                         *reinterpret_cast<v4i *>(stage + j * 128 + (((2 * q + g) ^ (j & 7)) * 16)) = o4;
                     }
                     wave_lds_fence();
@@ -200,10 +207,10 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
                         int n0 = nb * B + 32 * nt + 8 * q + 4 * g;
-                        v4i a4 = *reinterpret_cast<const v4i *>(At + n0);
+                        v4i a4 = {0, 0, 0, 0}; if (!PLAIN) a4 = *reinterpret_cast<const v4i *>(At + n0);
                         int o[4];
 #pragma unroll
-                        for (int e = 0; e < 4; e++) o[e] = clip127(perturbed<FUSE>(acc[nt][4 * q + e], sb, a4[e], p.sigma, p.shift));
+                        for (int e = 0; e < 4; e++) o[e] = clip127(fin(acc[nt][4 * q + e], a4[e]));
                         const int col = 32 * nt + 8 * q + 4 * g;                 // byte column inside the 128-byte row
                         *reinterpret_cast<int *>(stage + j * 128 + (((col >> 4) ^ (j & 7)) * 16) + (col & 15)) = pack4(o[0], o[1], o[2], o[3]);
                     }
@@ -221,13 +228,15 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
                         int n0 = nb * B + 32 * nt + 8 * q + 4 * g;
-                        v4i a4 = *reinterpret_cast<const v4i *>(At + n0);
+                        v4i a4 = {0, 0, 0, 0}; if (!PLAIN) a4 = *reinterpret_cast<const v4i *>(At + n0);
                         int o[4];
 #pragma unroll
-                        for (int e = 0; e < 4; e++) o[e] = clip127(perturbed<FUSE>(acc[nt][4 * q + e], sb, a4[e], p.sigma, p.shift));
+                        for (int e = 0; e < 4; e++) o[e] = clip127(fin(acc[nt][4 * q + e], a4[e]));
                         *reinterpret_cast<int *>(y8 + row * N + n0) = pack4(o[0], o[1], o[2], o[3]);
                     }
             }
+            };
+            if (p.plain) finish_block(std::true_type{}); else finish_block(std::false_type{});
         }
         if (!P::PREFETCH_X && pass + 1 < passes) {
 #pragma unroll

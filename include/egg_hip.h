@@ -101,6 +101,10 @@ int  egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first_idx, int n, int8
 int  egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocked,
                           int members, int T, int K, int N, uint32_t seed, int off_a, int off_b,
                           int shift, int32_t *d_Y32, int8_t *d_Y8);
+/* The same product without the rank-1 term: compute_linear_projection with ns == 0 (mgpu.cu:568, the guard the
+ * reference's generation path takes), Y = (X . W) >> shift.  It is the shared-weight GEMM on its own. */
+int  egg_shared_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocked,
+                       int members, int T, int K, int N, int shift, int32_t *d_Y32, int8_t *d_Y8);
 
 /* train_sequence_kernel<<<batch,...>>> (mgpu.cu:847-1029, launch :1531): evaluates members
  * [pop_offset, pop_offset+pop_count) on tokens d_data[stream_pos + t], writes d_loss[member] (int32).

@@ -97,6 +97,13 @@ def test_perturbed_linear(pkg, orc, dev, K, N, members, T, extra):
                 f"gpu[0,:16]={got[0, :16].tolist()}\nref[0,:16]={ref[0, :16].tolist()}\nplain xW>>s[0,:16]={(plain[0, :16] >> shift).tolist()}\n"
                 + _mapping_hint(got, ref))
         assert np.array_equal(y8.cpu().numpy(), np.clip(ref, -127, 127).astype(np.int8))
+        # the shared-weight product alone (the reference's ns == 0 case): the textbook integer matrix product
+        y32.fill_(7); y8.fill_(7)
+        ctx.shared_linear(dX.data_ptr(), dW.data_ptr(), members, T, K, N, shift, y32.data_ptr(), y8.data_ptr())
+        ctx.sync()
+        plain = (X.astype(np.int64) @ W.astype(np.int64)) >> shift
+        assert np.array_equal(y32.cpu().numpy(), plain), f"shared linear K={K} N={N} shift={shift}"
+        assert np.array_equal(y8.cpu().numpy(), np.clip(plain, -127, 127).astype(np.int8))
     ctx.close()
 
 
