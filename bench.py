@@ -272,6 +272,25 @@ def main():
         cpu_ref_path = {"value": 2 * npairs * g.seq_len / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
                         "sample": f"full_trained_egg.c defaults (GRU H=512 L=4), forward of {npairs} pairs x {g.seq_len} tokens, {sec:.1f}s"}
 
+    # ---- what MFMA rate the GPU sustains on this box (child process: a bare loop of int8 MFMAs on register operands)
+    sustained = None
+    probe = os.path.join(ROOT, "egg.c_amd", "mfma_probe")
+    if os.path.exists(probe):
+        try:
+            import subprocess
+            torch.cuda.synchronize()
+            r = subprocess.run([probe], capture_output=True, text=True, timeout=120)
+            if r.returncode == 0:
+                sustained = json.loads(r.stdout.strip().splitlines()[-1])
+                sustained["note"] = ("a bare loop of independent MFMAs, no memory traffic; with random operand bytes the clock drops under "
+                                     "power, so kernels on real data are bounded by random_operands_TOPs rather than by the published peak")
+                if roofline and sustained.get("random_operands_TOPs"):
+                    roofline["frac_of_measured_sustained_rate"] = roofline["achieved"] / sustained["random_operands_TOPs"]
+            else:
+                sustained = {"error": r.stderr[-200:]}
+        except Exception as e:
+            sustained = {"error": str(e)}
+
     out = {
         "metric": "member-tokens/sec on 1 MI355X (pop 40,960) + % int8 MFMA peak",
         "value": value, "unit": "member-tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -282,7 +301,7 @@ def main():
                    "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss,
                    "distinct_bytes_per_window": round(distinct, 1),
                    "ms_per_step_first_block_at_every_position": per_position_ms},
-        "roofline": roofline, "kernels": per_class, "microbench_c2": mb,
+        "roofline": roofline, "mfma_sustained": sustained, "kernels": per_class, "microbench_c2": mb,
         "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }
     print(json.dumps(out))

@@ -501,10 +501,8 @@ static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int m
     }
     PlinParams p = {d_X, ctx->d_plin_frag, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
                     noise_word(ctx->cfg), d_Y32, d_Y8, plain};
-    const int PB = egg_plinear_block(K, N);
-    if (K % PB || N % PB) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");
     span_begin(ctx, EGG_K_PLINEAR);
-    hipError_t e = egg_launch_swizzle(d_W, ctx->d_plin_frag, K, N, PB, 1, ctx->stream);
+    hipError_t e = egg_launch_plinear_swizzle(d_W, ctx->d_plin_frag, T, K, N, ctx->stream);
     if (e == hipSuccess) e = egg_launch_plinear(p, ctx->stream);
     span_end(ctx);
     if (e == hipErrorInvalidValue) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");

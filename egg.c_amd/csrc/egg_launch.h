@@ -13,7 +13,7 @@ hipError_t egg_prepare_forward(int H, int head_dim, int T);
 
 struct PlinParams {
     const int8_t *X;        // [members*T][K] natural order
-    const int8_t *Wfrag;    // fragment-major copy of W (natural k order), block size egg_plinear_block(K, N)
+    const int8_t *Wfrag;    // fragment-major copy of W (natural k order) as egg_launch_plinear_swizzle lays it out for (T, K, N)
     int members, T, K, N;
     uint32_t seed; int off_a, off_b, shift, sigma, mask;
     int32_t *Y32; int8_t *Y8;
@@ -21,6 +21,8 @@ struct PlinParams {
 };
 hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s);
 int egg_plinear_block(int K, int N);
+// canonical blocked W -> the layout the kernel chosen for (T, K, N) reads
+hipError_t egg_launch_plinear_swizzle(const int8_t *W_blocked, int8_t *W_frag, int T, int K, int N, hipStream_t s);
 // canonical blocked [K/4][N][4] -> fragment-major (see egg_device.h); nat = natural k order inside a k-step
 hipError_t egg_launch_swizzle(const int8_t *W_blocked, int8_t *W_frag, int K, int N, int B, int nat, hipStream_t s);
 
