@@ -148,3 +148,44 @@ def test_population_40960_step(pkg, orc, dev):
     ctx2.sync()
     assert np.array_equal(ctx2.model_download(), got_m)
     ctx2.close()
+
+
+def test_population_40960_fifty_graph_steps_match_eager(pkg, orc, dev):
+    """The headline run shape itself: 50 replays of the captured step graph at population 40,960, with a learning rate
+    large enough that weights change every step.  Eager launches of the same 50 steps from the same start must give
+    the same losses at every step and the same weights and optimizer state at the end; the first step's sampled
+    members are the oracle's (test_population_40960_step covers the update of that step)."""
+    pop = 40960
+    kw = dict(population=pop, **SHAPE)
+    data = orc.zipf_bytes(1 << 23)
+    d_data = _t(dev, data)
+    steps, lr = 50, 8.0
+    trace = {}
+    for mode in ("eager", "graph"):
+        ctx = pkg.Context(pkg.default_config(**kw))
+        ctx.model_init(42)
+        if mode == "graph":
+            ctx.step_capture(d_data.data_ptr(), len(data))
+        seed, losses, updates = 42, [], 0
+        for step in range(steps):
+            start = step * SHAPE["seq_len"]
+            if mode == "graph":
+                ctx.step_launch(start, seed, lr)
+            else:
+                ctx.step(d_data.data_ptr(), len(data), start, seed, lr)
+            if step % 7 == 0 or step == steps - 1:
+                losses.append(ctx.step_losses()[0].copy())
+                updates += ctx.last_update_count()
+            seed = pkg.next_seed(seed, step + 1)
+        trace[mode] = (losses, updates, ctx.model_download().copy(), ctx.opt_state_download().copy())
+        ctx.close()
+    e, g = trace["eager"], trace["graph"]
+    assert e[1] > 0, "no weight changed: the trajectory would not test the update"
+    for i, (a, b) in enumerate(zip(e[0], g[0])):
+        assert np.array_equal(a, b), f"losses differ at checkpoint {i}"
+    assert np.array_equal(e[2], g[2]), "weights after 50 steps"
+    assert np.array_equal(e[3], g[3]), "optimizer state after 50 steps"
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    ref = orc.population_forward(ocfg, model, data, 0, 42, 20478, 2)
+    assert np.array_equal(e[0][0][20478:20480], ref[20478:20480])
