@@ -472,13 +472,20 @@ static hipError_t launch_kn(const PlinParams &p, hipStream_t s) {
 
 int egg_plinear_block(int K, int N) { int m = K < N ? K : N; return m < 128 ? m : 128; }
 
-// the two-tile kernel serves K = 256 / 512 with whole pairs of token tiles, as long as its tables fit next to a second
-// workgroup's on the CU
-static bool two_tile_shape(int T, int K, int N) {
-    if (T % 64 || N % 64 || N < 64) return false;
-    if (K == 256) return 2 * Plin2<256>::total(N) <= 160 * 1024;
-    if (K == 512) return 2 * Plin2<512>::total(N) <= 160 * 1024;
+static bool one_tile_case(int K, int N) {
+#define CASE(K_, N_) if (K == K_ && N == N_) return true;
+    CASE(64, 64) CASE(64, 256) CASE(256, 64) CASE(128, 128) CASE(128, 512) CASE(512, 128)
+    CASE(256, 256) CASE(256, 1024) CASE(1024, 256) CASE(512, 512)
+#undef CASE
     return false;
+}
+
+// the two-tile kernel serves K = 256 / 512 with whole pairs of token tiles: whenever its tables fit next to a second
+// workgroup's on the CU, and alone on the CU for the wide outputs the one-tile kernel has no instance for
+static bool two_tile_shape(int T, int K, int N) {
+    if (T % 64 || N % 64 || N < 64 || (K != 256 && K != 512)) return false;
+    const size_t lds = K == 256 ? Plin2<256>::total(N) : Plin2<512>::total(N);
+    return 2 * lds <= 160 * 1024 || (lds <= 160 * 1024 && !one_tile_case(K, N));
 }
 
 template <int K>

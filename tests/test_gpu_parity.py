@@ -71,7 +71,9 @@ def test_noise_fill(pkg, orc, dev):
 @pytest.mark.parametrize("K,N,members,T,extra", [(64, 64, 4, 32, {}), (256, 256, 6, 64, {}), (512, 512, 8, 32, {}),
                                                  (256, 1024, 3, 32, {}), (1024, 256, 2, 32, {}),
                                                  (512, 512, 5, 128, {}), (256, 1024, 3, 64, {}), (512, 128, 2, 192, {}),
-                                                 (256, 64, 7, 64, {}),
+                                                 (256, 64, 7, 64, {}), (512, 192, 3, 64, {}), (256, 320, 2, 128, {}),
+                                                 (512, 64, 2, 64, {}), (512, 1024, 1, 128, {}),
+                                                 (256, 256, 5, 256, dict(sigma_shift=5, noise_mask=31)),
                                                  (512, 512, 3, 64, dict(sigma_shift=5, noise_mask=31)),
                                                  (1024, 256, 2, 32, dict(sigma_shift=5, noise_mask=31))])
 def test_perturbed_linear(pkg, orc, dev, K, N, members, T, extra):
