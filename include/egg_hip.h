@@ -97,7 +97,10 @@ int  egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first_idx, int n, int8
  *   acc[n] = sum_k X[r][k] W[k][n] + (((sum_k X[r][k] B[k]) * A[n]) * ns >> (fixed_point+sigma_shift))
  *   A[n] = noise(seed + pair + off_a, n), B[k] = noise(seed + pair + off_b, k)
  * d_Y32 receives acc >> shift as int32 [rows][N] (may be NULL); d_Y8 receives clip(acc >> shift) as int8
- * [rows][N] (may be NULL).  K, N multiples of 64; T multiple of 32. */
+ * [rows][N] (may be NULL).  T is a multiple of 32.  Supported shapes: K = 256 or 512 with T a multiple of 64 and any N
+ * that is a multiple of 64 up to 1024; otherwise (K, N) from {64, 128, 256, 512, 1024}^2 pairs the transformer uses
+ * (64x64, 64x256, 256x64, 128x128, 128x512, 512x128, 256x256, 256x1024, 1024x256, 512x512).  Other shapes return
+ * EGG_E_INVALID with the reason in egg_last_error. */
 int  egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocked,
                           int members, int T, int K, int N, uint32_t seed, int off_a, int off_b,
                           int shift, int32_t *d_Y32, int8_t *d_Y8);
