@@ -272,6 +272,28 @@ def main():
         cpu_ref_path = {"value": 2 * npairs * g.seq_len / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
                         "sample": f"full_trained_egg.c defaults (GRU H=512 L=4), forward of {npairs} pairs x {g.seq_len} tokens, {sec:.1f}s"}
 
+    # ---- what HBM rate a plain copy / fill reaches on this box (torch elementwise kernels, 1 GiB each way)
+    hbm = None
+    try:
+        n = 1 << 30
+        a = torch.empty(n, dtype=torch.int8, device=dev); b = torch.empty_like(a)
+        a.fill_(1); b.copy_(a); torch.cuda.synchronize()
+        e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        e0.record()
+        for _ in range(5):
+            b.copy_(a)
+        e1.record()
+        for _ in range(5):
+            b.fill_(3)
+        e2.record(); torch.cuda.synchronize()
+        hbm = {"copy_GBs": 5 * 2 * n / (e0.elapsed_time(e1) * 1e-3) / 1e9, "fill_GBs": 5 * n / (e1.elapsed_time(e2) * 1e-3) / 1e9,
+               "note": "read + write bytes of a 1 GiB device-to-device copy, and bytes of a 1 GiB fill, per second"}
+        del a, b
+        if isinstance(mb, dict) and "int32_out" in mb:
+            mb["int32_out"]["frac_of_measured_copy_rate"] = mb["int32_out"]["GB/s"] / hbm["copy_GBs"]
+    except Exception as e:
+        hbm = {"error": str(e)}
+
     # ---- what MFMA rate the GPU sustains on this box (child process: a bare loop of int8 MFMAs on register operands)
     sustained = None
     probe = os.path.join(ROOT, "egg.c_amd", "mfma_probe")
@@ -301,7 +323,7 @@ def main():
                    "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss,
                    "distinct_bytes_per_window": round(distinct, 1),
                    "ms_per_step_first_block_at_every_position": per_position_ms},
-        "roofline": roofline, "mfma_sustained": sustained, "kernels": per_class, "microbench_c2": mb,
+        "roofline": roofline, "mfma_sustained": sustained, "hbm_sustained": hbm, "kernels": per_class, "microbench_c2": mb,
         "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }
     print(json.dumps(out))
