@@ -109,6 +109,21 @@ def main():
                 "unit": "TOP/s", "frac": achieved / PEAK_INT8_OPS, "traffic": traffic,
                 "avg_launch_ms": tot_ms / launches if launches else None, "launches": launches}
 
+    # ---- every forward kernel against both roofs: algorithmic int8 ops and algorithmic HBM bytes per token (int8
+    # activations in and out; weights and regenerated noise count nothing) over its event-timed launches
+    bytes_per_token = {"mlp": 2 * H + H, "qkv": H + 3 * H, "attn": 3 * H + H, "head": H}
+    kernel_rooflines = {}
+    for k in ("mlp", "qkv", "attn", "head"):
+        nl, ms = timing[k]
+        if not nl:
+            continue
+        tok = P * T * args.steps * (L if k != "head" else 1) / nl
+        sec = ms / nl * 1e-3
+        kernel_rooflines["k_" + k] = {"avg_launch_ms": ms / nl, "TOP/s": ops_per_token[k] * tok / sec / 1e12,
+                                      "frac_mfma": ops_per_token[k] * tok / sec / PEAK_INT8_OPS,
+                                      "GB/s": bytes_per_token[k] * tok / sec / 1e9,
+                                      "frac_hbm": bytes_per_token[k] * tok / sec / PEAK_HBM}
+
     # ---- for comparison: the same eager steps with the block in front of the first attention layer evaluated at every
     # position instead of once per distinct byte value of a window (identical results, more work on repetitive data)
     ctx.first_block_dedup(False)
@@ -323,7 +338,7 @@ def main():
                    "graph_ms_per_step": graph_ms, "updates_last_step": updates, "mean_loss_last_step": mean_loss,
                    "distinct_bytes_per_window": round(distinct, 1),
                    "ms_per_step_first_block_at_every_position": per_position_ms},
-        "roofline": roofline, "mfma_sustained": sustained, "hbm_sustained": hbm, "kernels": per_class, "microbench_c2": mb,
+        "roofline": roofline, "kernel_rooflines": kernel_rooflines, "mfma_sustained": sustained, "hbm_sustained": hbm, "kernels": per_class, "microbench_c2": mb,
         "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
     }
     print(json.dumps(out))
