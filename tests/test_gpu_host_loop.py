@@ -41,3 +41,18 @@ def test_host_loop_eager_graph_adaptive_and_checkpoints(dev, tmp_path):
     assert len(resumed) == 4
     if sum(u for s, _, u in saved if s <= 2) > 0:                 # weights moved before the last checkpoint
         assert resumed[0][1] != eager[0][1], "the resumed run started from the initialisation, not from the checkpoint"
+
+
+def test_mfma_probe_reports_plausible_rates(dev):
+    """The measurement aid bench.py runs as a child process: one JSON line, rates between a fifth of the published int8
+    peak and a little above it, zero operands not slower than random ones."""
+    import json
+    probe = os.path.join(ROOT, "egg.c_amd", "mfma_probe")
+    if not os.path.exists(probe):
+        pytest.fail("egg.c_amd/mfma_probe is not built (run __graft_entry__.build())")
+    r = subprocess.run([probe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-500:]
+    d = json.loads(r.stdout.strip().splitlines()[-1])
+    for k in ("zero_operands_TOPs", "random_operands_TOPs", "random_operands_changing_every_mfma_TOPs"):
+        assert 1000.0 < d[k] < 5500.0, (k, d[k])
+    assert d["zero_operands_TOPs"] >= 0.95 * d["random_operands_TOPs"]
