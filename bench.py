@@ -93,7 +93,8 @@ def main():
     # ---- dominant kernel: O-projection + MLP block (k_mlp), MFMA-bound
     per_class = {k: {"launches": v[0], "avg_ms": (v[1] / v[0] if v[0] else None), "total_ms": v[1]} for k, v in timing.items()}
     dom = max(("mlp", "qkv", "attn", "mlp_first", "head"), key=lambda k: timing[k][1])
-    chunk = min(P, args.chunk if args.chunk > 0 else 8192)
+    # the library's default: the whole population per launch while five activation buffers stay within 32 GiB
+    chunk = min(P, args.chunk if args.chunk > 0 else (P if 5 * P * T * H <= (32 << 30) else 8192))
     ops_per_token = {"mlp": 2 * (H * H + 2 * H * 4 * H), "mlp_first": 2 * (2 * H * 4 * H), "qkv": 2 * 3 * H * H,
                      "head": 2 * H * 256, "attn": 2 * 2 * H * (T + 1) // 2}
     launches, tot_ms = timing[dom]

@@ -54,7 +54,8 @@ typedef struct egg_config {
     float adam_beta1, adam_beta2, adam_eps, adam_weight_decay;   /* .9 .95 1e-8 .01  */
     float muon_momentum, muon_lr_scale;                          /* .85 1.0          */
     int use_muon;            /* USE_MUON: 2-D hidden matrices use Muon instead of AdamW */
-    int chunk_members;       /* members evaluated per forward pass over the layers; 0 = auto */
+    int chunk_members;       /* members evaluated per forward pass over the layers; 0 = auto (the whole population
+                                while its activation buffers stay within 32 GiB, else 8192) */
     int weight_limit;        /* matrix weights saturate at +-weight_limit in the update rule: 127 as in the reference
                               * (mgpu.cu:1056-1062); 1 keeps them ternary (no reference counterpart)     */
     int device_gaussian;     /* DEVICE_GAUSSIAN (mgpu.cu:195-196, :530-534): perturbation noise = sum of three masked fields */

@@ -189,3 +189,25 @@ def test_population_40960_fifty_graph_steps_match_eager(pkg, orc, dev):
     model = orc.init_model(ocfg, 42)
     ref = orc.population_forward(ocfg, model, data, 0, 42, 20478, 2)
     assert np.array_equal(e[0][0][20478:20480], ref[20478:20480])
+
+
+def test_population_40960_one_launch_equals_chunks_of_8192(pkg, orc, dev):
+    """The default evaluates the whole population in one launch per kernel (2.7 GB per activation buffer: row offsets
+    pass 2^31); five launches of 8192 members must give the same per-member losses."""
+    import torch
+    pop = 40960
+    kw = dict(population=pop, **SHAPE)
+    data = orc.zipf_bytes(1 << 23)
+    d_data = _t(dev, data)
+    model = orc.init_model(orc.config(**kw), 42)
+    got = {}
+    for chunk in (0, 8192):
+        ctx = pkg.Context(pkg.default_config(chunk_members=chunk, **kw))
+        ctx.model_upload(model)
+        d_loss = torch.full((pop,), -1, dtype=torch.int32, device=dev)
+        ctx.population_forward(d_data.data_ptr(), len(data), 512, 777, 0, pop, d_loss.data_ptr())
+        ctx.sync()
+        got[chunk] = d_loss.cpu().numpy()
+        ctx.close()
+    assert got[0].min() > 0
+    assert np.array_equal(got[0], got[8192])
