@@ -51,7 +51,7 @@ EXPORTS = [
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
-    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz",
+    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
     "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
     "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
@@ -136,6 +136,7 @@ def lib():
         L.egg_timing_get.argtypes = [vp, i32, vp, vp]
         L.egg_opt_state_bytes.restype = i64
         L.egg_opt_state_bytes.argtypes = [vp]
+        L.egg_describe_layout.argtypes = [vp, i32, vp, vp, vp, vp]
         L.egg_tensor_state_offset.restype = i64
         L.egg_tensor_state_offset.argtypes = [vp, i32]
         L.egg_newton_schulz.argtypes = [vp, vp, i32, i32, i32]
@@ -166,6 +167,23 @@ def default_config(**kw):
             raise KeyError(k)
         setattr(c, k, v)
     return c
+
+
+def describe_layout(cfg):
+    """Host-only: (tensors, model_bytes, state_bytes) of a configuration; each tensor dict also carries its byte
+    offset into the optimizer state.  No GPU is touched."""
+    mb, sb = C.c_int64(), C.c_int64()
+    n = lib().egg_describe_layout(C.byref(cfg), -1, None, None, C.byref(mb), C.byref(sb))
+    if n < 0:
+        raise EggError("egg_describe_layout: invalid configuration")
+    out = []
+    for i in range(n):
+        t, so = EggTensorInfo(), C.c_int64()
+        lib().egg_describe_layout(C.byref(cfg), i, C.byref(t), C.byref(so), None, None)
+        out.append(dict(id=i, name=t.name.decode(), is_matrix=t.is_matrix, rows=t.rows, cols=t.cols, offset=t.offset,
+                        off_a=t.off_a, off_b=t.off_b, seed_base=t.seed_base, lr_scale=t.lr_scale, muon=t.muon,
+                        state_offset=int(so.value)))
+    return out, int(mb.value), int(sb.value)
 
 
 def _np_ptr(a):

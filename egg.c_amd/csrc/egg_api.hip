@@ -124,14 +124,14 @@ extern "C" void egg_default_config(egg_config *c) {
 }
 
 // launch order of mgpu.cu:1603-1643
-static void build_tensor_table(egg_ctx *ctx) {
-    const egg_config &c = ctx->cfg; const Layout &L = ctx->L; int H = c.hidden, V = c.vocab;
+static std::vector<egg_tensor_info> build_tensor_table(const egg_config &c, const Layout &L) {
+    std::vector<egg_tensor_info> tensors; int H = c.hidden, V = c.vocab;
     auto add = [&](const char *name, int l, int is_matrix, int rows, int cols, int64_t off, int oa, int ob, int base, float lrs, int muon) {
         egg_tensor_info t; memset(&t, 0, sizeof(t));
         if (l >= 0) snprintf(t.name, sizeof(t.name), "%s.%d", name, l); else snprintf(t.name, sizeof(t.name), "%s", name);
         t.is_matrix = is_matrix; t.rows = rows; t.cols = cols; t.offset = off; t.off_a = oa; t.off_b = ob;
         t.seed_base = base; t.lr_scale = lrs; t.muon = muon;
-        ctx->tensors.push_back(t);
+        tensors.push_back(t);
     };
     for (int l = 0; l < c.n_layers; l++) {
         int b = l * 1000; int64_t hh = (int64_t)H * H, h4 = (int64_t)H * 4 * H;
@@ -158,6 +158,38 @@ static void build_tensor_table(egg_ctx *ctx) {
     add("mlp_emb_bias_down", -1, 0, 1, H, L.mlp_emb_bias_down, OFF_EMB_MLP_BIAS_DOWN_A, OFF_EMB_MLP_BIAS_DOWN_B, 0, 1.f, 0);
     add("emb_bias", -1, 0, 1, H, L.emb_bias, OFF_EMB_BIAS_A, OFF_EMB_BIAS_B, 0, 0.1f, 0);
     add("embedding", -1, 1, H, V, L.embedding, OFF_EMB, OFF_EMB + H, 0, 1.f, 0);
+    return tensors;
+}
+// optimizer state in the field order of AdamModel (mgpu.cu:337-370): {m,v,acc} per element, or {m,acc} for the
+// matrices that use Muon (HIDDEN_OPT_TYPE, mgpu.cu:327-335); returns the total size
+static int64_t state_offsets(const egg_config &c, const std::vector<egg_tensor_info> &tensors, std::vector<int64_t> &off) {
+    std::vector<int> order(tensors.size());
+    for (size_t i = 0; i < order.size(); i++) order[i] = (int)i;
+    std::sort(order.begin(), order.end(), [&](int a, int b) { return tensors[a].offset < tensors[b].offset; });
+    off.assign(tensors.size(), 0);
+    int64_t so = 0;
+    for (int id : order) {
+        const egg_tensor_info &t = tensors[id];
+        off[id] = so;
+        so += (int64_t)t.rows * t.cols * ((c.use_muon && t.muon) ? 8 : 12);
+    }
+    return so;
+}
+// host-only view of the same tables (no device is touched)
+extern "C" int egg_describe_layout(const egg_config *cfg, int tensor_id, egg_tensor_info *out, int64_t *state_offset,
+                                   int64_t *model_bytes, int64_t *state_bytes) {
+    if (!cfg || cfg->hidden < 4 || cfg->n_layers < 1 || cfg->vocab < 1) return EGG_E_INVALID;
+    const Layout L = make_layout(*cfg);
+    const std::vector<egg_tensor_info> tensors = build_tensor_table(*cfg, L);
+    std::vector<int64_t> off;
+    const int64_t sb = state_offsets(*cfg, tensors, off);
+    if (model_bytes) *model_bytes = L.total;
+    if (state_bytes) *state_bytes = sb;
+    if (tensor_id < 0) return (int)tensors.size();
+    if (tensor_id >= (int)tensors.size()) return EGG_E_INVALID;
+    if (out) *out = tensors[tensor_id];
+    if (state_offset) *state_offset = off[tensor_id];
+    return (int)tensors.size();
 }
 
 static void free_all(egg_ctx *ctx) {
@@ -205,7 +237,7 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
     ctx->L = make_layout(c);
-    build_tensor_table(ctx);
+    ctx->tensors = build_tensor_table(c, ctx->L);
     auto bail = [&](int code, const char *what, hipError_t e) {
         g_create_err = std::string(what) + ": " + hipGetErrorString(e);
         free_all(ctx); delete ctx; return code;
@@ -236,20 +268,7 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     CR(hipMemcpy(ctx->d_rope, rope.data(), rope.size() * 4, hipMemcpyHostToDevice));
     CR(hipMalloc(&ctx->d_model, ctx->L.total)); CR(hipMemset(ctx->d_model, 0, ctx->L.total));
     CR(hipMalloc(&ctx->d_wfrag, ctx->L.total)); CR(hipMemset(ctx->d_wfrag, 0, ctx->L.total));
-    {   // optimizer state in the field order of AdamModel (mgpu.cu:337-370): {m,v,acc} per element, or {m,acc} for
-        // the matrices that use Muon (HIDDEN_OPT_TYPE, mgpu.cu:327-335)
-        std::vector<int> order(ctx->tensors.size());
-        for (size_t i = 0; i < order.size(); i++) order[i] = (int)i;
-        std::sort(order.begin(), order.end(), [&](int a, int b) { return ctx->tensors[a].offset < ctx->tensors[b].offset; });
-        ctx->t_state_off.assign(ctx->tensors.size(), 0);
-        int64_t so = 0;
-        for (int id : order) {
-            const egg_tensor_info &t = ctx->tensors[id];
-            ctx->t_state_off[id] = so;
-            so += (int64_t)t.rows * t.cols * ((c.use_muon && t.muon) ? 8 : 12);
-        }
-        ctx->state_bytes = so;
-    }
+    ctx->state_bytes = state_offsets(c, ctx->tensors, ctx->t_state_off);
     CR(hipMalloc(&ctx->d_state, ctx->state_bytes)); CR(hipMemset(ctx->d_state, 0, ctx->state_bytes));
     {
         std::vector<VecDesc> vd;

@@ -171,6 +171,12 @@ typedef struct egg_tensor_info {
     float   lr_scale;
     int     muon;
 } egg_tensor_info;
+/* The same tables without a context or a GPU (host code only): the tensor table, byte offsets into the model blob
+ * (== offsetof in the reference's TransformerModel, mgpu.cu:284-318 / de/include/model/definitions.h:21-54) and into the
+ * optimizer state (== offsetof in AdamModel, definitions.h:56-90, with MuonParam for the hidden matrices under use_muon)
+ * that a context of this configuration has.  tensor_id < 0 only counts.  Returns the tensor count, or EGG_E_INVALID. */
+int  egg_describe_layout(const egg_config *cfg, int tensor_id, egg_tensor_info *out, int64_t *state_offset,
+                         int64_t *model_bytes, int64_t *state_bytes);
 int  egg_tensor_count(const egg_ctx *ctx);
 int  egg_tensor_info_get(const egg_ctx *ctx, int tensor_id, egg_tensor_info *out);
 

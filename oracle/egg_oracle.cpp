@@ -37,6 +37,26 @@ enum {
     OFF_EMB_MLP_BIAS_DOWN_A = 516, OFF_EMB_MLP_BIAS_DOWN_B = 517
 };
 
+/* the enum above by the reference's macro name ("SEED_OFF_Q_A" -> OFF_Q_A); -1 for an unknown name.  It exists so
+ * that a test can hold this table against the reference's own d-eggs/include/config.h:79-134. */
+extern "C" int orc_seed_offset(const char *name) {
+    static const struct { const char *n; int v; } tab[] = {
+#define SO(x) {"SEED_OFF_" #x, OFF_##x}
+        SO(EMB), SO(EMB_BIAS_A), SO(EMB_BIAS_B), SO(LN_1_A), SO(LN_1_B), SO(LN_1_BIAS_A), SO(LN_1_BIAS_B),
+        SO(Q_A), SO(Q_B), SO(K_A), SO(K_B), SO(V_A), SO(V_B), SO(O_A), SO(O_B),
+        SO(LN_2_A), SO(LN_2_B), SO(LN_2_BIAS_A), SO(LN_2_BIAS_B),
+        SO(MLP_UP_A), SO(MLP_UP_B), SO(MLP_DOWN_A), SO(MLP_DOWN_B),
+        SO(MLP_BIAS_UP_A), SO(MLP_BIAS_UP_B), SO(MLP_BIAS_DOWN_A), SO(MLP_BIAS_DOWN_B),
+        SO(LN_F_A), SO(LN_F_B), SO(LN_F_BIAS_A), SO(LN_F_BIAS_B),
+        SO(LN_INIT_A), SO(LN_INIT_B), SO(LN_INIT_BIAS_A), SO(LN_INIT_BIAS_B),
+        SO(EMB_MLP_UP_A), SO(EMB_MLP_UP_B), SO(EMB_MLP_DOWN_A), SO(EMB_MLP_DOWN_B),
+        SO(EMB_MLP_BIAS_UP_A), SO(EMB_MLP_BIAS_UP_B), SO(EMB_MLP_BIAS_DOWN_A), SO(EMB_MLP_BIAS_DOWN_B),
+#undef SO
+    };
+    for (const auto &e : tab) if (!strcmp(e.n, name)) return e.v;
+    return -1;
+}
+
 extern "C" void orc_default_config(orc_config *c) {
     memset(c, 0, sizeof(*c));
     c->hidden = 256; c->head_dim = 64; c->n_layers = 4; c->seq_len = 32; c->vocab = 256;

@@ -73,6 +73,7 @@ typedef struct orc_config {
 #define ORC_NOISE_GAUSSIAN 0x100
 
 void orc_default_config(orc_config *c);
+int  orc_seed_offset(const char *reference_macro_name);   /* the oracle's seed-offset enum, by reference macro name */
 
 /* ---- RNG (mgpu.cu:428-441, :525-539) ---- */
 uint32_t orc_hash_rng(uint32_t s, uint32_t idx);

@@ -138,6 +138,7 @@ def lib():
         L.orc_repack.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int]
         L.orc_unpack.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int]
         L.orc_xorshift32.argtypes = [C.c_void_p]
+        L.orc_seed_offset.argtypes = [C.c_char_p]
         L.orc_gen_noise_host.argtypes = [C.c_void_p, C.c_int]
         L.orc_default_config.argtypes = [C.c_void_p]
         L.orc_gru_default_config.argtypes = [C.c_void_p]
@@ -181,6 +182,32 @@ def ref():
         _ref = R
     return _ref
 
+
+def ref_layout(tag):
+    """oracle/_ref/libegg_ref_layout_<tag>.so -> (macros, fields): the reference's own config.h / definitions.h /
+    optimizer/base.h compiled for one (HIDDEN_DIM, N_LAYERS, USE_MUON) variant.  macros: name -> value; fields:
+    (struct, field) -> (offset, size), field "" = the struct's size.  None if the library is absent."""
+    path = os.path.join(os.path.dirname(REF_PATH), "libegg_ref_layout_%s.so" % tag)
+    if not os.path.exists(path):
+        return None
+    R = C.CDLL(path)
+    R.ref_macro_name.restype = C.c_char_p
+    R.ref_macro_value.restype = C.c_double
+    R.ref_field_struct.restype = C.c_char_p
+    R.ref_field_name.restype = C.c_char_p
+    R.ref_field_offset.restype = C.c_uint64
+    R.ref_field_size.restype = C.c_uint64
+    R.ref_deggs_learning_rate.restype = C.c_float
+    R.ref_deggs_learning_rate.argtypes = [C.c_long]
+    macros = {R.ref_macro_name(i).decode(): R.ref_macro_value(i) for i in range(R.ref_macro_count())}
+    fields = {(R.ref_field_struct(i).decode(), R.ref_field_name(i).decode()): (int(R.ref_field_offset(i)), int(R.ref_field_size(i)))
+              for i in range(R.ref_field_count())}
+    macros["deggs_learning_rate(0,99,100,199,200,100000)"] = [float(R.ref_deggs_learning_rate(s)) for s in (0, 99, 100, 199, 200, 100000)]
+    return macros, fields
+
+
+REF_LAYOUT_TAGS = {"h256_l4_adam": dict(hidden=256, n_layers=4, use_muon=0), "h512_l8_muon": dict(hidden=512, n_layers=8, use_muon=1),
+                   "h64_l2_adam": dict(hidden=64, n_layers=2, use_muon=0), "h64_l2_muon": dict(hidden=64, n_layers=2, use_muon=1)}
 
 _ref_gaussian = None
 

@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/reference_known_answers.json.
+"""Writes tests/golden/reference_known_answers.json and tests/golden/reference_layout.json.
 
 RNG answers come from the reference's own host-compilable header (d-eggs/include/utils/egg_math.h) compiled into
 oracle/_ref/libegg_ref.so by oracle/Makefile; it therefore runs only where /root/reference is mounted.  Table
@@ -41,4 +41,14 @@ out["gelu_lut"] = {str(i): gelu(i) for i in (-128, -32, -16, -8, -1, 0, 1, 8, 16
 out["exp2_table"] = {str(i): int(2.0 ** (i / 16) * 16) for i in (0, 16, 128, 255)}
 out["ternary_vectors"] = [[-1, 0, 1, -1, 0, 1, 1, 0, -1, 0], [-1, 0, 1, -1, 0, 1, 1]]
 json.dump(out, open(os.path.join(HERE, "reference_known_answers.json"), "w"), indent=1)
+
+# configuration macros and struct layouts of the reference's own host-compilable headers (d-eggs/include/config.h,
+# optimizer/base.h, model/definitions.h, utils/training.h), compiled per variant into oracle/_ref by oracle/Makefile
+layout = {}
+for tag in O.REF_LAYOUT_TAGS:
+    got = O.ref_layout(tag)
+    assert got is not None, "build oracle/_ref first (make -C oracle ref)"
+    macros, fields = got
+    layout[tag] = {"macros": macros, "fields": {"%s.%s" % k: list(v) for k, v in fields.items()}}
+json.dump(layout, open(os.path.join(HERE, "reference_layout.json"), "w"), indent=1, sort_keys=True)
 print(json.dumps(out))

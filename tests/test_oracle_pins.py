@@ -386,16 +386,68 @@ def test_adam_apply(orc):
     assert orc.lib().orc_learning_rate(999) == f32(0.075) and orc.lib().orc_learning_rate(1000) == f32(0.05)
 
 
+def np_adam(m, v, acc, w, g, lr, b1=0.9, b2=0.95, eps=1e-8, wd=0.01, limit=127):
+    """apply_adam_update (mgpu.cu:1040-1064) on arrays in numpy float32, one rounding per operation"""
+    f32 = np.float32
+    m, v, acc, g = m.astype(f32), v.astype(f32), acc.astype(f32), g.astype(f32)
+    w = w.astype(np.int32)
+    m1 = f32(b1) * m + (f32(1.0) - f32(b1)) * g
+    v1 = f32(b2) * v + (f32(1.0) - f32(b2)) * (g * g)
+    step = f32(-lr) * (m1 / (np.sqrt(v1) + f32(eps)) + f32(wd) * w.astype(f32))
+    acc1 = acc + step
+    up, dn = acc1 >= 1, acc1 <= -1
+    inc, dec = up & (w < limit), dn & (w > -limit)
+    w1 = w + inc - dec
+    acc2 = np.where(inc, acc1 - f32(1), np.where(up, f32(1), np.where(dec, acc1 + f32(1), np.where(dn, f32(-1), acc1))))
+    assert m1.dtype == v1.dtype == acc2.dtype == f32
+    return m1, v1, acc2.astype(f32), w1.astype(np.int8), int((inc | dec).sum())
+
+
 def test_vector_update_matches_definition(orc):
+    """update_vector_adam_kernel (mgpu.cu:1114-1152): votes from numpy hashes, AdamW in numpy float32 -- m, v, acc,
+    the weights and the change count bit for bit, over three steps from a state that includes saturated weights."""
     cfg = orc.config()
     rng = np.random.default_rng(10)
-    n, pairs, seed = 16, 30, 99
+    n, pairs = 48, 30
+    V = rng.integers(-127, 128, n).astype(np.int8); V[:4] = (127, 127, -127, -127)
+    st = np.zeros(n, orc.ADAM_DTYPE)
+    st["acc"] = rng.uniform(-0.99, 0.99, n).astype(np.float32); st["acc"][:4] = (0.99, -0.99, -0.99, 0.99)
+    st["m"] = rng.standard_normal(n).astype(np.float32) * 50; st["v"] = (rng.standard_normal(n).astype(np.float32) * 50) ** 2
+    m, v, acc, w = st["m"].copy(), st["v"].copy(), st["acc"].copy(), V.copy()
+    total_moved = 0
+    for step, (seed, lr) in enumerate(((99, 0.3), (0xFFFFFFF0, 0.9), (7, 0.05))):
+        fit = rng.integers(-1, 2, pairs).astype(np.int32)
+        got = orc.lib().orc_update_vector_adam(C.byref(cfg), P(V), P(st), n, 110, 111, 3000, P(fit), pairs, C.c_uint32(seed), C.c_float(lr))
+        vote = sum(int(fit[p]) * np_noise(seed + p + 3000 + 110, np.arange(n)).astype(np.int64) * np_noise(seed + p + 3000 + 111, np.arange(n))
+                   for p in range(pairs))
+        m, v, acc, w, changes = np_adam(m, v, acc, w, -vote.astype(np.float32), lr)
+        assert got == changes, step
+        assert np.array_equal(V, w), step
+        for name, want in (("m", m), ("v", v), ("acc", acc)):
+            assert np.array_equal(st[name].view(np.int32), want.view(np.int32)), (step, name)
+        total_moved += changes
+    assert total_moved > 0
+
+
+def test_matrix_update_matches_definition(orc):
+    """update_matrix_adam_kernel (mgpu.cu:1067-1111) bit for bit: blocked votes from numpy, AdamW in numpy float32."""
+    cfg = orc.config()
+    rng = np.random.default_rng(12)
+    rows, cols, pairs, seed, oa, ob, base, lr = 8, 12, 40, 4242, 206, 207, 1000, 0.7
+    n = rows * cols
+    W = rng.integers(-127, 128, n).astype(np.int8)
+    st = np.zeros(n, orc.ADAM_DTYPE); st["acc"] = rng.uniform(-0.99, 0.99, n).astype(np.float32)
     fit = rng.integers(-1, 2, pairs).astype(np.int32)
-    V = np.zeros(n, np.int8); st = np.zeros(n, orc.ADAM_DTYPE)
-    orc.lib().orc_update_vector_adam(C.byref(cfg), P(V), P(st), n, 100, 101, 3000, P(fit), pairs, seed, C.c_float(0.3))
-    vote = sum(int(fit[p]) * np_noise(seed + p + 3000 + 100, np.arange(n)) * np_noise(seed + p + 3000 + 101, np.arange(n)) for p in range(pairs))
-    g = -vote.astype(np.float32)
-    assert np.allclose(st["m"], np.float32(1 - np.float32(0.9)) * g)
+    m, v, acc, w = st["m"].copy(), st["v"].copy(), st["acc"].copy(), W.copy()
+    got = orc.lib().orc_update_matrix_adam(C.byref(cfg), P(W), P(st), rows, cols, oa, ob, base, P(fit), pairs, seed, C.c_float(lr))
+    A = np.stack([np_noise(seed + p + base + oa, np.arange(cols)) for p in range(pairs)]).astype(np.int64)
+    B = np.stack([np_noise(seed + p + base + ob, np.arange(rows)) for p in range(pairs)]).astype(np.int64)
+    full = B.T @ (fit[:, None] * A)
+    idx = np.arange(n); k = ((idx >> 2) // cols) * 4 + (idx & 3); nn = (idx >> 2) % cols       # mgpu.cu:1085-1089
+    m, v, acc, w, changes = np_adam(m, v, acc, w, -full[k, nn].astype(np.float32), lr)
+    assert got == changes and changes > 0 and np.array_equal(W, w)
+    for name, want in (("m", m), ("v", v), ("acc", acc)):
+        assert np.array_equal(st[name].view(np.int32), want.view(np.int32)), name
 
 
 # ------------------------------------------------------------------ Muon
@@ -419,6 +471,56 @@ def test_newton_schulz(orc):
     Z = (Q / math.sqrt(12)).copy()
     orc.lib().orc_newton_schulz_f64(P(Z), 12, 12, 0)
     assert np.allclose(Z, Q / math.sqrt(12) / np.linalg.norm(Q / math.sqrt(12)))
+
+
+def test_muon_update_matches_definition(orc):
+    """orc_update_matrix_muon (muon_internal.cuh:15-50 momentum, :53-74 gather, :112-170 apply; chain mgpu.cu:1587-1595)
+    against numpy: the momentum m = mu*m + vote in blocked order bit for bit; the row-major gather (k*cols + n) by feeding
+    the numpy-gathered matrix to the separately pinned Newton-Schulz and asking for identical output; the apply rule
+    (step = -lr*(u + wd*w), accumulator, +-1 move, saturation at the weight limit) in numpy float32 bit for bit."""
+    f32 = np.float32
+    rng = np.random.default_rng(13)
+    for (rows, cols), limit, lr in (((8, 24), 127, 40.0), ((24, 8), 1, 25.0), ((16, 16), 127, 3.0)):
+        cfg = orc.config(weight_limit=limit)
+        pairs, seed, oa, ob, base = 50, 777, 400, 401, 2000
+        n = rows * cols
+        W = rng.integers(-limit, limit + 1, n).astype(np.int8)
+        st = np.zeros(n, orc.MUON_DTYPE)
+        st["m"] = (rng.standard_normal(n) * 30).astype(f32); st["acc"] = rng.uniform(-0.99, 0.99, n).astype(f32)
+        W[:2] = (limit, -limit); st["acc"][:2] = (0.99, -0.99)
+        m0, acc0, w0 = st["m"].copy(), st["acc"].copy(), W.copy()
+        fit = rng.integers(-1, 2, pairs).astype(np.int32)
+        ortho = np.zeros((rows, cols), f32)
+        got = orc.lib().orc_update_matrix_muon(C.byref(cfg), P(W), P(st), rows, cols, oa, ob, base, P(fit), pairs, seed,
+                                               C.c_float(lr), P(ortho))
+        A = np.stack([np_noise(seed + p + base + oa, np.arange(cols)) for p in range(pairs)]).astype(np.int64)
+        B = np.stack([np_noise(seed + p + base + ob, np.arange(rows)) for p in range(pairs)]).astype(np.int64)
+        full = B.T @ (fit[:, None] * A)                                                          # [k][n]
+        idx = np.arange(n); k = ((idx >> 2) // cols) * 4 + (idx & 3); nn = (idx >> 2) % cols
+        m1 = f32(cfg.muon_momentum) * m0 + full[k, nn].astype(f32)
+        assert np.array_equal(st["m"].view(np.int32), m1.view(np.int32))
+        X = np.zeros((rows, cols), f32); X[k, nn] = m1                                           # gather, muon_internal.cuh:53-74
+        Xd = X.astype(np.float64)
+        orc.lib().orc_newton_schulz_f32(P(X), rows, cols, 5)
+        assert np.array_equal(X.view(np.int32), ortho.view(np.int32))
+        Y = Xd / np.linalg.norm(Xd)
+        for _ in range(5):
+            Y = 0.5 * (3 * np.eye(rows) - Y @ Y.T) @ Y if rows < cols else 0.5 * Y @ (3 * np.eye(cols) - Y.T @ Y)
+        assert np.linalg.norm(ortho - Y) / np.linalg.norm(Y) < 1e-5
+        # a transposed gather would orthogonalise a different matrix
+        assert np.linalg.norm(ortho - Y) < 0.1 * np.linalg.norm(ortho - Y.T.reshape(-1)[: n].reshape(rows, cols))
+        u = ortho[k, nn]
+        step = f32(-(f32(lr) * f32(cfg.muon_lr_scale))) * (u + f32(cfg.adam_weight_decay) * w0.astype(f32))
+        acc1 = acc0 + step
+        w = w0.astype(np.int32)
+        up, dn = acc1 >= 1, acc1 <= -1
+        inc, dec = up & (w < limit), dn & (w > -limit)
+        acc2 = np.where(inc, acc1 - f32(1), np.where(up, f32(1), np.where(dec, acc1 + f32(1), np.where(dn, f32(-1), acc1)))).astype(f32)
+        assert np.array_equal(W, (w + inc - dec).astype(np.int8))
+        assert np.array_equal(st["acc"].view(np.int32), acc2.view(np.int32))
+        assert got == int((inc | dec).sum()) and got > 0
+        assert (up & ~inc).any() or (dn & ~dec).any() or limit == 127      # the ternary case exercises saturation
+        assert np.abs(W).max() <= limit
 
 
 # ------------------------------------------------------------------ CPU GRU path (full_trained_egg.c)
