@@ -41,7 +41,7 @@ EXPORTS = [
     "egg_default_config", "egg_ctx_create", "egg_ctx_destroy", "egg_last_error", "egg_ctx_set_stream", "egg_sync",
     "egg_model_bytes", "egg_model_init", "egg_model_upload", "egg_model_download",
     "egg_opt_state_upload", "egg_opt_state_download", "egg_opt_state_reset", "egg_tables_download",
-    "egg_noise_fill", "egg_perturbed_linear", "egg_shared_linear", "egg_population_forward", "egg_population_forward_dev",
+    "egg_noise_fill", "egg_perturbed_linear", "egg_perturbed_linear_own_noise", "egg_shared_linear", "egg_population_forward", "egg_population_forward_dev",
     "egg_fitness", "egg_es_update", "egg_update_tensor", "egg_matrix_votes",
     "egg_adaptive_enable", "egg_overlay_upload", "egg_overlay_download",
     "egg_ternary_model_bytes", "egg_model_upload_ternary", "egg_model_download_ternary",
@@ -100,6 +100,7 @@ def lib():
         L.egg_tables_download.argtypes = [vp, vp, vp, vp]
         L.egg_noise_fill.argtypes = [vp, u32, u32, i32, vp]
         L.egg_perturbed_linear.argtypes = [vp, vp, vp, i32, i32, i32, i32, u32, i32, i32, i32, vp, vp]
+        L.egg_perturbed_linear_own_noise.argtypes = [vp, vp, vp, i32, i32, i32, i32, u32, i32, i32, i32, vp, vp]
         L.egg_shared_linear.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp]
         L.egg_population_forward.argtypes = [vp, vp, i64, i64, u32, i32, i32, vp]
         L.egg_population_forward_dev.argtypes = [vp, vp, i64, vp, vp, i32, i32, vp]
@@ -271,6 +272,12 @@ class Context:
                                             seed & 0xFFFFFFFF, off_a, off_b, shift,
                                             C.c_void_p(d_y32) if d_y32 else None, C.c_void_p(d_y8) if d_y8 else None),
                  "egg_perturbed_linear")
+
+    def perturbed_linear_own_noise(self, d_x, d_w, members, T, K, N, seed, off_a, off_b, shift, d_y32=None, d_y8=None):
+        self._ck(lib().egg_perturbed_linear_own_noise(self._h, C.c_void_p(d_x), C.c_void_p(d_w), members, T, K, N,
+                                                      seed & 0xFFFFFFFF, off_a, off_b, shift,
+                                                      C.c_void_p(d_y32) if d_y32 else None, C.c_void_p(d_y8) if d_y8 else None),
+                 "egg_perturbed_linear_own_noise")
 
     def shared_linear(self, d_x, d_w, members, T, K, N, shift, d_y32=None, d_y8=None):
         self._ck(lib().egg_shared_linear(self._h, C.c_void_p(d_x), C.c_void_p(d_w), members, T, K, N, shift,

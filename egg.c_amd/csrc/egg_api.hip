@@ -503,17 +503,21 @@ extern "C" int egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first, int n
 }
 
 static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
-                       uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8, int plain);
+                       uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8, int plain, int own_noise);
 extern "C" int egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
                                     uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8) {
-    return linear_impl(ctx, d_X, d_W, members, T, K, N, seed, off_a, off_b, shift, d_Y32, d_Y8, 0);
+    return linear_impl(ctx, d_X, d_W, members, T, K, N, seed, off_a, off_b, shift, d_Y32, d_Y8, 0, 0);
+}
+extern "C" int egg_perturbed_linear_own_noise(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
+                                              uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8) {
+    return linear_impl(ctx, d_X, d_W, members, T, K, N, seed, off_a, off_b, shift, d_Y32, d_Y8, 0, 1);
 }
 extern "C" int egg_shared_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
                                  int shift, int32_t *d_Y32, int8_t *d_Y8) {
-    return linear_impl(ctx, d_X, d_W, members, T, K, N, 0, 0, 0, shift, d_Y32, d_Y8, 1);
+    return linear_impl(ctx, d_X, d_W, members, T, K, N, 0, 0, 0, shift, d_Y32, d_Y8, 1, 0);
 }
 static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
-                       uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8, int plain) {
+                       uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8, int plain, int own_noise) {
     if (!ctx || !d_X || !d_W || members < 1 || T < 32 || T % 32 || (!d_Y32 && !d_Y8) || shift < 0 || shift > 31)
         return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear arguments");
     if (K < 64 || N < 64 || K % 64 || N % 64) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: K and N must be multiples of 64");
@@ -525,7 +529,7 @@ static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int m
         ctx->plin_frag_bytes = (size_t)K * N;
     }
     PlinParams p = {d_X, ctx->d_plin_frag, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
-                    noise_word(ctx->cfg), d_Y32, d_Y8, plain};
+                    noise_word(ctx->cfg), d_Y32, d_Y8, plain, own_noise};
     span_begin(ctx, EGG_K_PLINEAR);
     hipError_t e = egg_launch_plinear_swizzle(d_W, ctx->d_plin_frag, T, K, N, ctx->stream);
     if (e == hipSuccess) e = egg_launch_plinear(p, ctx->stream);

@@ -18,6 +18,7 @@ struct PlinParams {
     uint32_t seed; int off_a, off_b, shift, sigma, mask;
     int32_t *Y32; int8_t *Y8;
     int plain;              // the shared-weight product alone: no rank-1 term (the reference's ns == 0 case)
+    int own_noise;          // every member draws its own (A, B) with ns = +1 instead of sharing a pair's draw with ns = +-1
 };
 hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s);
 int egg_plinear_block(int K, int N);

@@ -74,8 +74,10 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear(PlinParams p) {
     int member = blockIdx.x * EGG_WAVES + wave;
     if (member >= p.members) member = p.members - 1;
     int32_t *y32 = p.Y32; int8_t *y8 = p.Y8;
-    const int ns = (member & 1) ? -1 : 1;
-    const uint32_t ps = p.seed + (uint32_t)(member / 2);
+    // reference indexing: a pair shares one draw, the odd member takes it negated (mgpu.cu:864-871); own_noise: every
+    // member its own draw, applied with ns = +1
+    const int ns = (!p.own_noise && (member & 1)) ? -1 : 1;
+    const uint32_t ps = p.seed + (uint32_t)(p.own_noise ? member : member / 2);
 
     // the W stream: unit u of a token tile (every tile walks the same UPP units), fragment-major blocks of B x B
     const Plan plan = dma_plan<P::PR, P::B>(B);
@@ -292,8 +294,10 @@ __global__ void __launch_bounds__(EGG_THREADS, 2) k_plinear2(PlinParams p) {
 
     int member = blockIdx.x * EGG_WAVES + wave;
     if (member >= p.members) member = p.members - 1;
-    const int ns = (member & 1) ? -1 : 1;
-    const uint32_t ps = p.seed + (uint32_t)(member / 2);
+    // reference indexing: a pair shares one draw, the odd member takes it negated (mgpu.cu:864-871); own_noise: every
+    // member its own draw, applied with ns = +1
+    const int ns = (!p.own_noise && (member & 1)) ? -1 : 1;
+    const uint32_t ps = p.seed + (uint32_t)(p.own_noise ? member : member / 2);
 
     const Plan plan = dma_plan<2 * P::KSU, P::BN>(BN);
     const int passes = p.T / 64, upp = nblk * P::UNITS_NB;      // units per pass: the whole of W, in stream order

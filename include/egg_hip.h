@@ -105,6 +105,13 @@ int  egg_noise_fill(egg_ctx *ctx, uint32_t seed, uint32_t first_idx, int n, int8
 int  egg_perturbed_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocked,
                           int members, int T, int K, int N, uint32_t seed, int off_a, int off_b,
                           int shift, int32_t *d_Y32, int8_t *d_Y8);
+/* The same layer with one noise draw per member instead of per antithetic pair: pair -> member, ns = +1 for every
+ * member (A[n] = noise(seed + member + off_a, n), B[k] = noise(seed + member + off_b, k)).  The reference has no such
+ * call site (its members always come in +- pairs, mgpu.cu:864-871); it is compute_linear_projection with those
+ * arguments, kept so that both indexings of the single-layer microbenchmark can be measured. */
+int  egg_perturbed_linear_own_noise(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocked,
+                                    int members, int T, int K, int N, uint32_t seed, int off_a, int off_b,
+                                    int shift, int32_t *d_Y32, int8_t *d_Y8);
 /* The same product without the rank-1 term: compute_linear_projection with ns == 0 (mgpu.cu:568, the guard the
  * reference's generation path takes), Y = (X . W) >> shift.  It is the shared-weight GEMM on its own. */
 int  egg_shared_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocked,
