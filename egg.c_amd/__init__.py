@@ -51,7 +51,7 @@ EXPORTS = [
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
-    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout",
+    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_newton_schulz_static",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
     "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
     "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
@@ -138,6 +138,7 @@ def lib():
         L.egg_opt_state_bytes.restype = i64
         L.egg_opt_state_bytes.argtypes = [vp]
         L.egg_describe_layout.argtypes = [vp, i32, vp, vp, vp, vp]
+        L.egg_newton_schulz_static.argtypes = [vp, i32, i32, i32, vp]
         L.egg_tensor_state_offset.restype = i64
         L.egg_tensor_state_offset.argtypes = [vp, i32]
         L.egg_newton_schulz.argtypes = [vp, vp, i32, i32, i32]
@@ -185,6 +186,13 @@ def describe_layout(cfg):
                         off_a=t.off_a, off_b=t.off_b, seed_base=t.seed_base, lr_scale=t.lr_scale, muon=t.muon,
                         state_offset=int(so.value)))
     return out, int(mb.value), int(sb.value)
+
+
+def newton_schulz_static(d_x, rows, cols, iters=5, stream=None):
+    """egg_newton_schulz_static: Newton-Schulz in place on a row-major fp32 device matrix, no context, no allocation."""
+    rc = lib().egg_newton_schulz_static(C.c_void_p(d_x), rows, cols, iters, C.c_void_p(stream))
+    if rc != 0:
+        raise EggError("egg_newton_schulz_static failed (%d): %s" % (rc, (lib().egg_last_error(None) or b"").decode()))
 
 
 def _np_ptr(a):

@@ -208,6 +208,7 @@ static void free_all(egg_ctx *ctx) {
 // why the last egg_ctx_create of this thread failed (there is no context to hold the message yet)
 static thread_local std::string g_create_err;
 static int refuse(const char *why) { g_create_err = why; return EGG_E_INVALID; }
+void egg_set_thread_error(const char *what) { g_create_err = what; }
 
 extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (!cfg || !out) return refuse("egg_ctx_create: null argument");

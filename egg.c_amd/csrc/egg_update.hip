@@ -5,8 +5,11 @@
 // The reference recomputes two noise hashes per (weight, pair); here the (rows+cols) x pairs noise
 // panels are generated once per matrix and the vote  sum_p fit_p A_p[n] B_p[k]  is an int8 MFMA GEMM
 // over the population axis whose epilogue applies AdamW in place (blocked element order).
+#include "../../include/egg_hip.h"
 #include "egg_device.h"
 #include "egg_launch.h"
+#include <mutex>
+#include <string>
 
 #pragma clang fp contract(off)
 
@@ -481,6 +484,61 @@ hipError_t egg_launch_newton_schulz(const MuonWork &w, int rows, int cols, int i
     }
     if (cur != w.x) hipLaunchKernelGGL(k_copy_f32, dim3((n + 255) / 256), dim3(256), 0, s, w.x, cur, n);
     return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- Newton-Schulz for callers that cannot allocate
+// The same kernels with their workspace (ping-pong matrix, 3I - G term, norm partials) in a file-scope device array
+// instead of a context's hipMalloc'd buffers.  Each GPU holds its own copy of the array; its address on a device is
+// looked up once per device with hipGetSymbolAddress and used from then on in place of the array's name.
+struct NsScratch {
+    float swap[EGG_NS_STATIC_MAX_ELEMS];
+    float bterm[EGG_NS_STATIC_MAX_SHORT * EGG_NS_STATIC_MAX_SHORT];
+    float partials[1024];
+    float norm[4];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(NsScratch)];
+static NsScratch *g_ns_scratch[EGG_MAX_DEVICES];      // per device; written once, under g_ns_mutex
+static std::mutex g_ns_mutex;
+
+static hipError_t ns_scratch_on_current_device(NsScratch **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= EGG_MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_ns_mutex);
+    if (!g_ns_scratch[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!ptr) return hipErrorInvalidSymbol;
+        g_ns_scratch[dev] = static_cast<NsScratch *>(ptr);
+    }
+    *out = g_ns_scratch[dev];
+    return hipSuccess;
+}
+
+extern "C" int egg_newton_schulz_static(float *d_X, int rows, int cols, int iters, void *hip_stream) {
+    if (!d_X || rows < 32 || cols < 32 || rows % 32 || cols % 32 || iters < 0 || iters > 64) {
+        egg_set_thread_error("egg_newton_schulz_static: need a device matrix with rows and cols multiples of 32 and 0 <= iters <= 64");
+        return EGG_E_INVALID;
+    }
+    if ((long long)rows * cols > EGG_NS_STATIC_MAX_ELEMS || (rows < cols ? rows : cols) > EGG_NS_STATIC_MAX_SHORT) {
+        egg_set_thread_error("egg_newton_schulz_static: matrix exceeds the static workspace (rows * cols <= 1,048,576 and min(rows, cols) <= 512)");
+        return EGG_E_INVALID;
+    }
+    NsScratch *sc = nullptr;
+    hipError_t e = ns_scratch_on_current_device(&sc);
+    if (e == hipSuccess) {
+        // nothing in the workspace has to start at zero: every partial, the norm, the 3I - G term and the ping-pong
+        // matrix are written in full before they are read
+        MuonWork w = {d_X, sc->swap, nullptr, sc->bterm, sc->partials, sc->norm};
+        e = egg_launch_newton_schulz(w, rows, cols, iters, static_cast<hipStream_t>(hip_stream));
+    }
+    if (e != hipSuccess) {
+        egg_set_thread_error((std::string("egg_newton_schulz_static: ") + hipGetErrorString(e)).c_str());
+        return EGG_E_HIP;
+    }
+    return EGG_OK;
 }
 
 // muon_apply_update_kernel (muon_internal.cuh:112-170)

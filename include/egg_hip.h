@@ -68,7 +68,8 @@ void egg_default_config(egg_config *cfg);
 /* init_tables + cudaMemcpyToSymbol + per-GPU allocation (mgpu.cu:394-426, :1442-1489) */
 int  egg_ctx_create(const egg_config *cfg, egg_ctx **out);
 void egg_ctx_destroy(egg_ctx *ctx);
-/* message of the last failed call on ctx; with ctx == NULL, why this thread's last egg_ctx_create failed */
+/* message of the last failed call on ctx; with ctx == NULL, why this thread's last egg_ctx_create (or last call of an
+ * entry point that takes no context) failed */
 const char *egg_last_error(const egg_ctx *ctx);
 /* run on a caller-provided hipStream_t instead of the context's own (d-eggs update_stream, de/src/worker.cu:352-357) */
 int  egg_ctx_set_stream(egg_ctx *ctx, void *hip_stream);
@@ -169,6 +170,17 @@ int  egg_matrix_votes(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const u
 /* perform_newton_schulz (muon_internal.cuh:182-342) on a row-major fp32 [rows][cols] device matrix, in place:
  * X /= ||X||_F, then `iters` times X <- 0.5 X (3I - X^T X) on the short side.  Needs a use_muon context. */
 int  egg_newton_schulz(egg_ctx *ctx, float *d_X, int rows, int cols, int iters);
+
+/* No counterpart in the reference.  egg_newton_schulz for callers that cannot allocate (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc): the same kernels and results, with the workspace (ping-pong matrix,
+ * 3I - G term, norm partials; about 5.3 MB) in a static device array of the library instead of a context's buffers, so
+ * no context is needed and the call makes no hipMalloc / hipFree.  Limits: rows * cols <= EGG_NS_STATIC_MAX_ELEMS and
+ * min(rows, cols) <= EGG_NS_STATIC_MAX_SHORT, else EGG_E_INVALID (message via egg_last_error(NULL)).  Runs on the
+ * current device, enqueued on hip_stream (NULL = the default stream).  Every call on a GPU shares that GPU's one
+ * workspace: calls that overlap on one GPU (two streams, two threads) race; serialise them. */
+#define EGG_NS_STATIC_MAX_ELEMS (512 * 2048)
+#define EGG_NS_STATIC_MAX_SHORT 512
+int  egg_newton_schulz_static(float *d_X, int rows, int cols, int iters, void *hip_stream);
 
 typedef struct egg_tensor_info {
     char    name[32];
