@@ -41,7 +41,7 @@ EXPORTS = [
     "egg_default_config", "egg_ctx_create", "egg_ctx_destroy", "egg_last_error", "egg_ctx_set_stream", "egg_sync",
     "egg_model_bytes", "egg_model_init", "egg_model_upload", "egg_model_download",
     "egg_opt_state_upload", "egg_opt_state_download", "egg_opt_state_reset", "egg_tables_download",
-    "egg_noise_fill", "egg_perturbed_linear", "egg_perturbed_linear_own_noise", "egg_shared_linear", "egg_population_forward", "egg_population_forward_dev",
+    "egg_noise_fill", "egg_perturbed_linear", "egg_perturbed_linear_own_noise", "egg_shared_linear", "egg_ctx_linear_kernel", "egg_population_forward", "egg_population_forward_dev",
     "egg_fitness", "egg_es_update", "egg_update_tensor", "egg_matrix_votes",
     "egg_adaptive_enable", "egg_overlay_upload", "egg_overlay_download",
     "egg_ternary_model_bytes", "egg_model_upload_ternary", "egg_model_download_ternary",
@@ -51,7 +51,7 @@ EXPORTS = [
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
-    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_newton_schulz_static",
+    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_newton_schulz_static", "egg_measure_mfma_int8",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
     "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
     "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
@@ -101,6 +101,7 @@ def lib():
         L.egg_noise_fill.argtypes = [vp, u32, u32, i32, vp]
         L.egg_perturbed_linear.argtypes = [vp, vp, vp, i32, i32, i32, i32, u32, i32, i32, i32, vp, vp]
         L.egg_perturbed_linear_own_noise.argtypes = [vp, vp, vp, i32, i32, i32, i32, u32, i32, i32, i32, vp, vp]
+        L.egg_ctx_linear_kernel.argtypes = [vp, i32]
         L.egg_shared_linear.argtypes = [vp, vp, vp, i32, i32, i32, i32, i32, vp, vp]
         L.egg_population_forward.argtypes = [vp, vp, i64, i64, u32, i32, i32, vp]
         L.egg_population_forward_dev.argtypes = [vp, vp, i64, vp, vp, i32, i32, vp]
@@ -139,6 +140,7 @@ def lib():
         L.egg_opt_state_bytes.argtypes = [vp]
         L.egg_describe_layout.argtypes = [vp, i32, vp, vp, vp, vp]
         L.egg_newton_schulz_static.argtypes = [vp, i32, i32, i32, vp]
+        L.egg_measure_mfma_int8.argtypes = [i32, i32, vp, C.POINTER(C.c_float), C.POINTER(C.c_double)]
         L.egg_tensor_state_offset.restype = i64
         L.egg_tensor_state_offset.argtypes = [vp, i32]
         L.egg_newton_schulz.argtypes = [vp, vp, i32, i32, i32]
@@ -193,6 +195,15 @@ def newton_schulz_static(d_x, rows, cols, iters=5, stream=None):
     rc = lib().egg_newton_schulz_static(C.c_void_p(d_x), rows, cols, iters, C.c_void_p(stream))
     if rc != 0:
         raise EggError("egg_newton_schulz_static failed (%d): %s" % (rc, (lib().egg_last_error(None) or b"").decode()))
+
+
+def measure_mfma_int8(d_sink, iters=20000, zero_operands=False):
+    """egg_measure_mfma_int8: (milliseconds, integer operations) of a register-only int8 MFMA loop on every SIMD."""
+    ms, ops = C.c_float(), C.c_double()
+    rc = lib().egg_measure_mfma_int8(iters, int(zero_operands), C.c_void_p(d_sink), C.byref(ms), C.byref(ops))
+    if rc != 0:
+        raise EggError("egg_measure_mfma_int8 failed (%d): %s" % (rc, (lib().egg_last_error(None) or b"").decode()))
+    return float(ms.value), float(ops.value)
 
 
 def _np_ptr(a):
@@ -286,6 +297,9 @@ class Context:
                                                       seed & 0xFFFFFFFF, off_a, off_b, shift,
                                                       C.c_void_p(d_y32) if d_y32 else None, C.c_void_p(d_y8) if d_y8 else None),
                  "egg_perturbed_linear_own_noise")
+
+    def linear_kernel(self, w_stationary=True):
+        self._ck(lib().egg_ctx_linear_kernel(self._h, 1 if w_stationary else 0), "egg_ctx_linear_kernel")
 
     def shared_linear(self, d_x, d_w, members, T, K, N, shift, d_y32=None, d_y8=None):
         self._ck(lib().egg_shared_linear(self._h, C.c_void_p(d_x), C.c_void_p(d_w), members, T, K, N, shift,

@@ -46,6 +46,7 @@ struct egg_ctx {
     MuonWork muon = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     int8_t *d_wfrag = nullptr;      // fragment-major copy of every matrix, same offsets as the model blob
     int8_t *d_plin_frag = nullptr; size_t plin_frag_bytes = 0;
+    bool plin_no_ws = false;        // egg_ctx_linear_kernel: run the W-streaming kernels also where the W-stationary one exists
     int32_t *d_exp = nullptr; int8_t *d_act = nullptr; int32_t *d_rope = nullptr;
     int chunk = 0;
     int8_t *d_x = nullptr, *d_q = nullptr, *d_k = nullptr, *d_v = nullptr, *d_ao = nullptr;
@@ -222,7 +223,11 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (c.n_layers < 1 || c.population < 2 || (c.population & 1)) return refuse("n_layers >= 1 and an even population >= 2 are required");
     // shift amounts and table scales the kernels can state in 32-bit shifts / 64-bit multiply-adds
     auto in_range = [](int v, int lo, int hi) { return v >= lo && v <= hi; };
-    if (!in_range(c.rope_scale_bit, 1, 30) || !in_range(c.softmax_scale_bit, 1, 30)) return refuse("rope_scale_bit and softmax_scale_bit must be 1..30");
+    if (!in_range(c.rope_scale_bit, 1, 30)) return refuse("rope_scale_bit must be 1..30");
+    // the attention kernels split every exp-table weight into three 7-bit planes for the int8 matrix pipe; the largest
+    // entry is exp(0) * 2^softmax_scale_bit, so it must stay below 2^21
+    if (!in_range(c.softmax_scale_bit, 1, 20)) return refuse("softmax_scale_bit must be 1..20 (table weights are split into three 7-bit planes)");
+    if (!(c.softmax_exp_scale > 0.0)) return refuse("softmax_exp_scale must be positive");
     if (!in_range(c.noise_mask, 0, 127) || !in_range(c.host_mask, 0, 127)) return refuse("noise_mask and host_mask must be 0..127");
     const int mag = c.device_gaussian ? 3 * c.noise_mask : c.noise_mask;        // largest |noise|
     if (mag > 127 || (c.host_gaussian ? 3 : 1) * c.host_mask > 127) return refuse("Gaussian noise needs 3 * mask <= 127");
@@ -235,6 +240,9 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (127 * (127 + ((mag * mag) >> c.sigma_shift_vector)) > (1 << 17))
         return refuse("noise_mask^2 >> sigma_shift_vector is too large for the norm's exact division");
     if (!in_range(c.weight_limit, 1, 127)) return refuse("weight_limit must be 1..127");
+    // the MLP's up accumulator carries (bias + 128 + noise) << shift_mlp_up on top of its matrix product
+    if (egg_mlp_up_acc_bound(c.hidden, noise_word(c), c.sigma_shift_vector, c.shift_mlp_up) >= (1LL << 31))
+        return refuse("shift_mlp_up is too large: (bias + 128 + noise) << shift_mlp_up plus the up projection's sum must stay below 2^31");
     egg_ctx *ctx = new egg_ctx();
     ctx->cfg = c;
     ctx->L = make_layout(c);
@@ -517,12 +525,18 @@ extern "C" int egg_shared_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *
                                  int shift, int32_t *d_Y32, int8_t *d_Y8) {
     return linear_impl(ctx, d_X, d_W, members, T, K, N, 0, 0, 0, shift, d_Y32, d_Y8, 1, 0);
 }
+extern "C" int egg_ctx_linear_kernel(egg_ctx *ctx, int w_stationary) {
+    if (!ctx) return EGG_E_INVALID;
+    ctx->plin_no_ws = !w_stationary;
+    return EGG_OK;
+}
 static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int members, int T, int K, int N,
                        uint32_t seed, int off_a, int off_b, int shift, int32_t *d_Y32, int8_t *d_Y8, int plain, int own_noise) {
     if (!ctx || !d_X || !d_W || members < 1 || T < 32 || T % 32 || (!d_Y32 && !d_Y8) || shift < 0 || shift > 31)
         return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear arguments");
     if (K < 64 || N < 64 || K % 64 || N % 64) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: K and N must be multiples of 64");
-    if ((size_t)K * N > ctx->plin_frag_bytes) {
+    const bool ws = egg_plinear_ws_shape(K, N) && !ctx->plin_no_ws;
+    if (!ws && (size_t)K * N > ctx->plin_frag_bytes) {
         HIP_TRY(hipStreamSynchronize(ctx->stream));
         if (ctx->d_plin_frag) (void)hipFree(ctx->d_plin_frag);
         ctx->d_plin_frag = nullptr; ctx->plin_frag_bytes = 0;
@@ -530,9 +544,9 @@ static int linear_impl(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W, int m
         ctx->plin_frag_bytes = (size_t)K * N;
     }
     PlinParams p = {d_X, ctx->d_plin_frag, members, T, K, N, seed, off_a, off_b, shift, ctx->cfg.fixed_point + ctx->cfg.sigma_shift,
-                    noise_word(ctx->cfg), d_Y32, d_Y8, plain, own_noise};
+                    noise_word(ctx->cfg), d_Y32, d_Y8, plain, own_noise, ws ? d_W : nullptr};
     span_begin(ctx, EGG_K_PLINEAR);
-    hipError_t e = egg_launch_plinear_swizzle(d_W, ctx->d_plin_frag, T, K, N, ctx->stream);
+    hipError_t e = ws ? hipSuccess : egg_launch_plinear_swizzle(d_W, ctx->d_plin_frag, T, K, N, ctx->stream);
     if (e == hipSuccess) e = egg_launch_plinear(p, ctx->stream);
     span_end(ctx);
     if (e == hipErrorInvalidValue) return fail(ctx, EGG_E_INVALID, "egg_perturbed_linear: unsupported (K, N)");

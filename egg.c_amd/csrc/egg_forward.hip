@@ -139,8 +139,8 @@ struct MlpCfg {
 };
 
 // FUSE: the host has checked sigma <= 7 and |noise| <= 15, which bounds |acc| * 2^sigma + |sb * a| below 2^31 for
-// GEMM depths up to 1024 (depth * 127 * 127 * 128 + depth * 127 * 225); the down projection (depth 4H) uses the
-// fused form only for 4H <= 1024.
+// GEMM depths up to 1024 (depth * 127 * 127 * 128 + depth * 127 * 225), and the same bound for the up accumulator
+// with its bias seed (egg_mlp_up_acc_bound); the down projection (depth 4H) uses the fused form only for 4H <= 1024.
 // ADAPT: the d-eggs adaptive noise overlay is on (de/include/model/layers.cuh:215-296, :432-438,
 // de/src/kernels.cu:139-158); see k_qkv.  The down projection's input-side sum follows the reference thread of a
 // hidden unit, which adds its four terms (k = unit, unit + H, ...) into an int one float addition at a time; the
@@ -1117,7 +1117,13 @@ static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
     const int sets = tile_map_sets(p.c.T, MlpCfg<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = MlpCfg<H>::total(sets, first);
-    const bool fuse = p.c.sigma <= 7 && egg_noise_magnitude(p.c.mask) <= 15;
+    // The up accumulator is seeded with (bias + 128 + noise) << shift_mlp_up (see the bias table), so its range is the
+    // GEMM's plus that seed; the fused perturb-and-shift needs |acc| * 2^sigma + |sb * a| below 2^31 for it as well.
+    const long long mag = egg_noise_magnitude(p.c.mask);
+    const long long up_acc = egg_mlp_up_acc_bound(H, p.c.mask, p.c.sigma_vec, p.c.shift_mlp_up);
+    const bool up_fits = p.c.sigma >= 0 && p.c.sigma < 31 && (up_acc << p.c.sigma) + (long long)H * 127 * mag * mag < (1LL << 31);
+    const bool fuse = p.c.sigma <= 7 && mag <= 15 && up_fits;
+    if (up_acc >= (1LL << 31)) return hipErrorInvalidValue;      // egg_ctx_create refuses such shifts
     if (p.q_ln_w) {      // adaptive noise overlay: one (unfused) variant
         if (first) hipLaunchKernelGGL((k_mlp<H, true, false, true>), grid, block, lds, s, p);
         else hipLaunchKernelGGL((k_mlp<H, false, false, true>), grid, block, lds, s, p);

@@ -19,7 +19,11 @@ struct PlinParams {
     int32_t *Y32; int8_t *Y8;
     int plain;              // the shared-weight product alone: no rank-1 term (the reference's ns == 0 case)
     int own_noise;          // every member draws its own (A, B) with ns = +1 instead of sharing a pair's draw with ns = +-1
+    const int8_t *Wblocked; // the canonical blocked matrix: set (with a shape egg_plinear_ws_shape accepts) to run the
+                            // W-stationary kernel, which needs no fragment-major copy
 };
+bool egg_plinear_ws_shape(int K, int N);
+hipError_t egg_launch_plinear_ws(const PlinParams &p, hipStream_t s);      // egg_linear_ws.hip
 hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s);
 int egg_plinear_block(int K, int N);
 // canonical blocked W -> the layout the kernel chosen for (T, K, N) reads

@@ -517,6 +517,7 @@ hipError_t egg_launch_plinear_swizzle(const int8_t *W, int8_t *Wf, int T, int K,
 
 hipError_t egg_launch_plinear(const PlinParams &p, hipStream_t s) {
     if (p.T % 32 || p.T < 32 || p.members < 1) return hipErrorInvalidValue;
+    if (p.Wblocked && egg_plinear_ws_shape(p.K, p.N)) return egg_launch_plinear_ws(p, s);
     if (two_tile_shape(p.T, p.K, p.N)) return p.K == 256 ? launch_two_k<256>(p, s) : launch_two_k<512>(p, s);
 #define CASE(K_, N_) if (p.K == K_ && p.N == N_) return launch_kn<K_, N_>(p, s);
     CASE(64, 64) CASE(64, 256) CASE(256, 64) CASE(128, 128) CASE(128, 512) CASE(512, 128)

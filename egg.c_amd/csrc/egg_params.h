@@ -24,6 +24,16 @@ enum {
 // largest |noise| a mask word can produce
 static inline int egg_noise_magnitude(int mask) { return (mask & EGG_NOISE_GAUSSIAN) ? 3 * (mask & 0xff) : (mask & 0xff); }
 
+// Largest |value| the MLP's up accumulator can hold: the GEMM over `hidden` int8 products plus the seed
+// (bias + 128 + vector noise) << shift_mlp_up that folds the bias and the GELU table's index offset into it.  The
+// vector noise is (n1 * n2 * ns) >> sigma_vec with |n| <= the noise magnitude (an arithmetic shift: one more on the
+// negative side).
+static inline long long egg_mlp_up_acc_bound(int hidden, int mask, int sigma_vec, int shift_mlp_up) {
+    const long long mag = egg_noise_magnitude(mask);
+    const long long seed = 127 + 128 + ((mag * mag) >> sigma_vec) + 1;
+    return (long long)hidden * 127 * 127 + (seed << shift_mlp_up);
+}
+
 // what every forward kernel needs to know about the run
 struct FwdCommon {
     const uint8_t  *data;        // token stream (device)

@@ -66,7 +66,9 @@ def test_unsupported_configurations_are_refused_with_a_reason(pkg):
                      (dict(noise_mask=60, sigma_shift_vector=0), "noise_mask"), (dict(weight_limit=0), "weight_limit"),
                      (dict(noise_mask=127), "noise too wide"), (dict(device_gaussian=1, noise_mask=50), "Gaussian"),
                      (dict(hidden=512, device_gaussian=1), "noise too wide"),
-                     (dict(shift_mlp_up=40), "shift")):
+                     (dict(shift_mlp_up=40), "shift"), (dict(softmax_scale_bit=21), "three 7-bit planes"),
+                     (dict(softmax_scale_bit=30), "softmax_scale_bit"), (dict(shift_mlp_up=23), "shift_mlp_up is too large"),
+                     (dict(shift_mlp_up=24, hidden=512), "shift_mlp_up is too large"), (dict(softmax_exp_scale=0.0), "softmax_exp_scale")):
         cfg = pkg.default_config(**kw)
         h = ctypes.c_void_p()
         rc = lib.egg_ctx_create(ctypes.byref(cfg), ctypes.byref(h))

@@ -111,6 +111,60 @@ def test_perturbed_linear(pkg, orc, dev, K, N, members, T, extra):
     ctx.close()
 
 
+# Shapes the W-stationary kernel serves (K x 512, K = 256 or 512), at member counts below, at and above the number of
+# workgroups (one per CU, members dealt round-robin), with one to five 32-token tiles per member, pair noise and own
+# noise, and the two-shift form (wide noise).  Every output is compared with the W-streaming kernel's, the first and
+# last pairs with the oracle, and the shared-weight product with the integer matrix product.
+@pytest.mark.parametrize("K,members,T,own,extra", [(256, 5, 64, 0, {}), (256, 300, 32, 0, {}), (512, 300, 96, 0, {}), (512, 517, 32, 1, {}),
+                                                   (256, 1, 32, 0, {}), (512, 1, 160, 1, {}), (512, 259, 160, 0, dict(sigma_shift=5, noise_mask=31)),
+                                                   (256, 258, 128, 1, dict(sigma_shift=5, noise_mask=31)), (512, 256, 32, 0, {}), (512, 2, 32, 0, {})])
+def test_w_stationary_linear(pkg, orc, dev, K, members, T, own, extra):
+    import torch
+    N = 512
+    rng = np.random.default_rng(K + members * 3 + T)
+    ctx = pkg.Context(pkg.default_config(**SMALL, **extra))
+    ocfg = orc.config(**SMALL, **extra)
+    X = rng.integers(-127, 128, size=(members * T, K), dtype=np.int8)
+    W = rng.integers(-127, 128, size=(K, N), dtype=np.int8)
+    Wb = np.zeros(K * N, np.int8)
+    orc.lib().orc_repack(Wb.ctypes.data_as(C.c_void_p), W.ctypes.data_as(C.c_void_p), K, N)
+    dX, dW = _t(dev, X), _t(dev, Wb)
+    call = ctx.perturbed_linear_own_noise if own else ctx.perturbed_linear
+    seed = 0xF00D0000 + members
+    for shift in (8, 3):
+        outs = []
+        # (the W-streaming kernels have no 256 x 512 instance for an odd number of 32-token tiles)
+        for ws in ((True, False) if K == 512 or T % 64 == 0 else (True,)):
+            ctx.linear_kernel(ws)
+            y32 = torch.full((members * T, N), 7, dtype=torch.int32, device=dev)
+            y8 = torch.full((members * T, N), 7, dtype=torch.int8, device=dev)
+            s32 = torch.full((members * T, N), 7, dtype=torch.int32, device=dev)
+            s8 = torch.full((members * T, N), 7, dtype=torch.int8, device=dev)
+            call(dX.data_ptr(), dW.data_ptr(), members, T, K, N, seed, 200, 201, shift, y32.data_ptr(), y8.data_ptr())
+            ctx.shared_linear(dX.data_ptr(), dW.data_ptr(), members, T, K, N, shift, s32.data_ptr(), s8.data_ptr())
+            ctx.sync()
+            outs.append((y32, y8, s32, s8))
+        for a, b, what in zip(outs[0], outs[-1], ("perturbed int32", "perturbed int8", "shared int32", "shared int8")):
+            assert torch.equal(a, b), f"W-stationary and W-streaming kernels differ: {what} K={K} members={members} T={T} shift={shift}"
+        plain = (torch.from_numpy(X).to(dev).double() @ torch.from_numpy(W).to(dev).double()).to(torch.int64) >> shift
+        assert torch.equal(outs[0][2].to(torch.int64), plain)
+        assert torch.equal(outs[0][3].to(torch.int64), plain.clamp(-127, 127))
+        assert torch.equal(outs[0][1].to(torch.int32), outs[0][0].clamp(-127, 127))
+        # the oracle evaluates pairs (member 2i with +noise, 2i + 1 with -noise, one seed per pair); with own noise every
+        # member is the first of a pair of its own seed
+        got = outs[0][0].cpu().numpy()
+        for m in sorted({0, members - 1}):
+            if own:
+                ref = orc.perturbed_linear(ocfg, np.concatenate([X[m * T:(m + 1) * T]] * 2), Wb, T, K, N, seed + m, 200, 201, shift)[:T]
+            elif m % 2 == 0 and m + 1 >= members:
+                ref = orc.perturbed_linear(ocfg, np.concatenate([X[m * T:(m + 1) * T]] * 2), Wb, T, K, N, seed + m // 2, 200, 201, shift)[:T]
+            else:
+                lo = m - (m % 2)
+                ref = orc.perturbed_linear(ocfg, X[lo * T:(lo + 2) * T], Wb, T, K, N, seed + lo // 2, 200, 201, shift)[(m - lo) * T:(m - lo + 1) * T]
+            assert np.array_equal(got[m * T:(m + 1) * T], ref), f"member {m} K={K} members={members} T={T} shift={shift}"
+    ctx.close()
+
+
 STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao", "x_attn", "x_mlp")]
 
 

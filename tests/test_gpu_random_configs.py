@@ -74,3 +74,57 @@ def test_random_configurations_follow_the_oracle(pkg, orc, dev, block):
         for f in ("m", "v", "acc"):
             assert np.array_equal(got[f].view(np.int32), state[f].view(np.int32)), (kw, f)
         ctx.close()
+
+
+def _extreme_cases():
+    """Shifts and table scales over the whole range egg_ctx_create accepts, the corners first."""
+    base = dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=2)
+    out = [dict(base, shift_mlp_up=22), dict(base, hidden=512, head_dim=64, shift_mlp_up=21),
+           dict(base, hidden=512, head_dim=64, shift_mlp_up=15, sigma_shift=3),       # the bias seed no longer fits the fused form
+           dict(base, hidden=256, head_dim=64, shift_mlp_up=16), dict(base, shift_mlp_up=0, shift_mlp_down=0, shift_out=0),
+           dict(base, softmax_scale_bit=20), dict(base, hidden=256, head_dim=64, seq_len=256, softmax_scale_bit=20, softmax_exp_scale=40.0),
+           dict(base, softmax_scale_bit=1), dict(base, shift_attn=0, shift_logit=0), dict(base, shift_attn=24, shift_logit=24, shift_out=24, shift_mlp_down=24),
+           dict(base, fixed_point=4, sigma_shift=20), dict(base, fixed_point=0, sigma_shift=0, noise_mask=7), dict(base, sigma_shift_vector=0, noise_mask=7),
+           dict(base, sigma_shift_vector=24)]
+    rng = np.random.default_rng(4711)
+    for _ in range(10):
+        H = int(rng.choice([64, 128, 256, 512]))
+        out.append(dict(hidden=H, head_dim=int(rng.choice([32, 64])), n_layers=1, seq_len=int(rng.choice([32, 64])), population=2,
+                        sigma_shift=int(rng.integers(0, 21)), sigma_shift_vector=int(rng.integers(0, 25)), shift_attn=int(rng.integers(0, 25)),
+                        shift_out=int(rng.integers(0, 25)), shift_logit=int(rng.integers(0, 25)), shift_mlp_up=int(rng.integers(0, 22)),
+                        shift_mlp_down=int(rng.integers(0, 25)), softmax_scale_bit=int(rng.integers(1, 21)), rope_scale_bit=int(rng.integers(1, 31)),
+                        noise_mask=int(rng.choice([1, 3, 7, 15]))))
+    return out
+
+
+def test_shift_and_table_scale_extremes_follow_the_oracle(pkg, orc, dev):
+    """Every stage, the logits and the loss at the edges of the accepted configuration space: the up projection's
+    bias is folded into its accumulator shifted left by shift_mlp_up, and the attention weights are split into three
+    7-bit planes, so both ends of both ranges are exercised (with biases that are not zero)."""
+    import torch
+    for kw in _extreme_cases():
+        rng = np.random.default_rng(kw["hidden"] + 7 * kw.get("shift_mlp_up", 8))
+        T, P = kw["seq_len"], kw["population"]
+        ocfg = orc.config(**kw)
+        model = orc.init_model(ocfg, 42)
+        for t in orc.tensor_table(ocfg):
+            if not t["is_matrix"]:
+                sl = slice(t["offset"], t["offset"] + t["cols"])
+                model[sl] = rng.integers(-127, 128, t["cols"]).astype(np.int8) if "bias" in t["name"] else rng.integers(1, 40, t["cols"]).astype(np.int8)
+        ctx = pkg.Context(pkg.default_config(**kw))
+        ctx.model_upload(model)
+        ctx.enable_taps(True)
+        data = orc.zipf_bytes(1 << 12)
+        d_data = torch.from_numpy(data).to(dev)
+        d_loss = torch.zeros(P, dtype=torch.int32, device=dev)
+        start, seed = 5 * T, 24680
+        ctx.population_forward(d_data.data_ptr(), len(data), start, seed, 0, P, d_loss.data_ptr())
+        ctx.sync()
+        for m in range(P):
+            ref_loss, tr = orc.forward_member(ocfg, model, data, start, seed, m, trace=True)
+            for st in ["x_init"] + [f"{n}.0" for n in ("q", "k", "v", "ao", "x_attn", "x_mlp")]:
+                exp = tr[st.split(".")[0]][0] if "." in st else tr[st]
+                assert np.array_equal(ctx.tap(st, m), exp), (kw, m, st)
+            assert np.array_equal(ctx.tap("logits", m), tr["logits"]), (kw, m)
+            assert int(d_loss[m].item()) == ref_loss, (kw, m)
+        ctx.close()
