@@ -51,7 +51,7 @@ EXPORTS = [
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
-    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_newton_schulz_static", "egg_measure_mfma_int8",
+    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_newton_schulz_static",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
     "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
     "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
@@ -140,7 +140,6 @@ def lib():
         L.egg_opt_state_bytes.argtypes = [vp]
         L.egg_describe_layout.argtypes = [vp, i32, vp, vp, vp, vp]
         L.egg_newton_schulz_static.argtypes = [vp, i32, i32, i32, vp]
-        L.egg_measure_mfma_int8.argtypes = [i32, i32, vp, C.POINTER(C.c_float), C.POINTER(C.c_double)]
         L.egg_tensor_state_offset.restype = i64
         L.egg_tensor_state_offset.argtypes = [vp, i32]
         L.egg_newton_schulz.argtypes = [vp, vp, i32, i32, i32]
@@ -195,15 +194,6 @@ def newton_schulz_static(d_x, rows, cols, iters=5, stream=None):
     rc = lib().egg_newton_schulz_static(C.c_void_p(d_x), rows, cols, iters, C.c_void_p(stream))
     if rc != 0:
         raise EggError("egg_newton_schulz_static failed (%d): %s" % (rc, (lib().egg_last_error(None) or b"").decode()))
-
-
-def measure_mfma_int8(d_sink, iters=20000, zero_operands=False):
-    """egg_measure_mfma_int8: (milliseconds, integer operations) of a register-only int8 MFMA loop on every SIMD."""
-    ms, ops = C.c_float(), C.c_double()
-    rc = lib().egg_measure_mfma_int8(iters, int(zero_operands), C.c_void_p(d_sink), C.byref(ms), C.byref(ops))
-    if rc != 0:
-        raise EggError("egg_measure_mfma_int8 failed (%d): %s" % (rc, (lib().egg_last_error(None) or b"").decode()))
-    return float(ms.value), float(ops.value)
 
 
 def _np_ptr(a):

@@ -435,48 +435,3 @@ hipError_t egg_launch_plinear_ws(const PlinParams &p, hipStream_t s) {
     if (p.K == 256 && p.N == 512) return launch_ws_kn<256, 512>(p, s);
     return hipErrorInvalidValue;
 }
-
-// ---- measurement: what the matrix pipes sustain on their own.  Every wave of a full grid (one workgroup per CU, one
-// wave per SIMD) issues dependent-free int8 MFMAs on register operands, random or zero; no memory traffic at all.
-__global__ void __launch_bounds__(EGG_THREADS, 1) k_mfma_i8_rate(int *out, int iters, int zero_operands) {
-    uint32_t h = (threadIdx.x + 1) * 2654435761u ^ (blockIdx.x * 40503u);
-    v4i a[4], b[4];
-    for (int i = 0; i < 4; i++)
-        for (int q = 0; q < 4; q++) {
-            h = hash_rng(h, 1); a[i][q] = zero_operands ? 0 : (int)h;
-            h = hash_rng(h, 2); b[i][q] = zero_operands ? 0 : (int)h;
-        }
-    v16i acc[8];
-    zero_acc<8>(acc);
-    for (int it = 0; it < iters; it++) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i & 3], b[(i + it) & 3], acc[i], 0, 0, 0);
-    }
-    int x = 0;
-    for (int i = 0; i < 8; i++)
-        for (int r = 0; r < 16; r++) x ^= acc[i][r];
-    if (x == 0x12345678) out[threadIdx.x] = x;          // keeps the loop alive; practically never taken
-}
-extern "C" int egg_measure_mfma_int8(int iters, int zero_operands, int *d_sink, float *ms, double *ops) {
-    if (iters < 1 || !d_sink || !ms || !ops) { egg_set_thread_error("egg_measure_mfma_int8: need iters >= 1, a device int[256] and two result pointers"); return 1; }
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    hipError_t e = hipEventCreate(&e0);
-    if (e == hipSuccess) e = hipEventCreate(&e1);
-    const int grid = egg_cu_count();
-    if (e == hipSuccess) {
-        hipLaunchKernelGGL(k_mfma_i8_rate, dim3(grid), dim3(EGG_THREADS), 0, 0, d_sink, 64, zero_operands);       // warm
-        e = hipEventRecord(e0, 0);
-    }
-    if (e == hipSuccess) {
-        hipLaunchKernelGGL(k_mfma_i8_rate, dim3(grid), dim3(EGG_THREADS), 0, 0, d_sink, iters, zero_operands);
-        e = hipGetLastError();
-    }
-    if (e == hipSuccess) e = hipEventRecord(e1, 0);
-    if (e == hipSuccess) e = hipEventSynchronize(e1);
-    if (e == hipSuccess) e = hipEventElapsedTime(ms, e0, e1);
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
-    if (e != hipSuccess) { egg_set_thread_error(hipGetErrorString(e)); return 1; }
-    *ops = (double)grid * EGG_WAVES * (double)iters * 8.0 * 2.0 * 32 * 32 * 32;
-    return 0;
-}

@@ -123,12 +123,6 @@ int  egg_shared_linear(egg_ctx *ctx, const int8_t *d_X, const int8_t *d_W_blocke
  * w_stationary = 0 makes them use the W-streaming kernels instead, which serve every other shape.  Results are
  * identical; the switch exists so that both can be measured and compared. */
 int  egg_ctx_linear_kernel(egg_ctx *ctx, int w_stationary);
-/* Measurement aid with no counterpart in the reference: runs `iters` x 8 independent int8 32x32x32 MFMAs per wave on
- * register operands (random, or all zero when zero_operands != 0) on every SIMD of the current device, with no memory
- * traffic, and reports the elapsed milliseconds and the integer operations executed.  It gives the rate the matrix
- * pipes sustain under the board's power limit, the practical ceiling beside the published peak.  d_sink is any device
- * int[256] (never written in practice).  Runs on the null stream and synchronises. */
-int  egg_measure_mfma_int8(int iters, int zero_operands, int *d_sink, float *ms, double *ops);
 
 /* train_sequence_kernel<<<batch,...>>> (mgpu.cu:847-1029, launch :1531): evaluates members
  * [pop_offset, pop_offset+pop_count) on tokens d_data[stream_pos + t], writes d_loss[member] (int32).
