@@ -46,7 +46,7 @@ EXPORTS = [
     "egg_adaptive_enable", "egg_overlay_upload", "egg_overlay_download",
     "egg_ternary_model_bytes", "egg_model_upload_ternary", "egg_model_download_ternary",
     "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
-    "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate",
+    "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate", "egg_generate_deggs", "egg_deggs_sampling_constants",
     "egg_shape_fitness", "egg_ternary_pack_size", "egg_ternary_pack", "egg_ternary_unpack",
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
@@ -117,6 +117,8 @@ def lib():
         L.egg_step_launch.argtypes = [vp, i64, u32, C.c_float]
         L.egg_step_losses.argtypes = [vp, vp, vp]
         L.egg_generate.argtypes = [vp, vp, i32, i32, u32]
+        L.egg_generate_deggs.argtypes = [vp, vp, i32, i32, u32, C.c_float, C.c_float, C.c_float]
+        L.egg_deggs_sampling_constants.argtypes = [vp, C.c_float, C.c_float, C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
         L.egg_shape_fitness.argtypes = [vp, i32, i32, C.c_double, i32, C.c_double, vp, vp]
         L.egg_ternary_pack_size.restype = C.c_size_t
         L.egg_ternary_pack_size.argtypes = [C.c_size_t]
@@ -194,6 +196,15 @@ def newton_schulz_static(d_x, rows, cols, iters=5, stream=None):
     rc = lib().egg_newton_schulz_static(C.c_void_p(d_x), rows, cols, iters, C.c_void_p(stream))
     if rc != 0:
         raise EggError("egg_newton_schulz_static failed (%d): %s" % (rc, (lib().egg_last_error(None) or b"").decode()))
+
+
+def deggs_sampling_constants(cfg, min_p, penalty):
+    """(penalty_int, min_p_limit) as egg_generate_deggs derives them (host only)."""
+    a, b = C.c_int32(), C.c_int32()
+    rc = lib().egg_deggs_sampling_constants(C.byref(cfg), min_p, penalty, C.byref(a), C.byref(b))
+    if rc != 0:
+        raise EggError("egg_deggs_sampling_constants failed (%d)" % rc)
+    return int(a.value), int(b.value)
 
 
 def _np_ptr(a):
@@ -379,6 +390,11 @@ class Context:
     def generate(self, d_buffer, seed_len, gen_len, seed):
         """Continue the seed_len prompt bytes at device pointer d_buffer by gen_len sampled bytes (in place)."""
         self._ck(lib().egg_generate(self._h, C.c_void_p(d_buffer), seed_len, gen_len, seed & 0xFFFFFFFF), "egg_generate")
+
+    def generate_deggs(self, d_buffer, seed_len, gen_len, seed, temp=0.6, min_p=0.08, penalty=0.2):
+        """The same with d-eggs' sampler: temperature, min-p filter and presence penalty (its defaults)."""
+        self._ck(lib().egg_generate_deggs(self._h, C.c_void_p(d_buffer), seed_len, gen_len, seed & 0xFFFFFFFF, temp, min_p, penalty),
+                 "egg_generate_deggs")
 
     def enable_taps(self, on=True):
         self._ck(lib().egg_ctx_enable_taps(self._h, 1 if on else 0), "egg_ctx_enable_taps")

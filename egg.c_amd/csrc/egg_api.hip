@@ -907,7 +907,8 @@ extern "C" uint32_t egg_next_seed(uint32_t seed, uint64_t step) {
 // token by token with a KV cache; here every new token re-runs the unperturbed forward of one member over the whole
 // window (noise mask 0 makes every perturbation term vanish, i.e. noise_sign = 0) and samples from the logits of
 // position t.  Causality makes the logits at t independent of the not yet generated tail.
-extern "C" int egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed) {
+struct DeggsSampling { float temp; int min_p_limit, penalty_int; };
+static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed, const DeggsSampling *de) {
     if (!ctx || !d_buffer) return EGG_E_INVALID;
     const egg_config &c = ctx->cfg; const int T = c.seq_len, total = seed_len + gen_len;
     if (seed_len < 1 || gen_len < 0 || total > T) return fail(ctx, EGG_E_INVALID, "egg_generate: need 1 <= seed_len and seed_len + gen_len <= seq_len");
@@ -929,7 +930,10 @@ extern "C" int egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int g
         // data_len = T + 1 puts the member's stream position at 0 (mgpu.cu:864-870 with len - T == 1)
         rc = forward_chunk(ctx, ctx->d_gen_tok, (int64_t)T + 1, &ctx->d_gen_scal->start, &ctx->d_gen_scal->seed, 0, 1);
         if (rc == EGG_OK) {
-            hipError_t e = egg_launch_sample(ctx->d_gen_logits + (size_t)t * c.vocab, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_tok + t + 1, s);
+            const int32_t *row = ctx->d_gen_logits + (size_t)t * c.vocab;
+            hipError_t e = de ? egg_launch_sample_deggs(row, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_tok, de->temp, de->min_p_limit, de->penalty_int,
+                                                        ctx->d_gen_tok + t + 1, s)
+                              : egg_launch_sample(row, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_tok + t + 1, s);
             if (e != hipSuccess) rc = fail(ctx, EGG_E_HIP, "egg_launch_sample", e);
         }
     }
@@ -937,6 +941,37 @@ extern "C" int egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int g
     if (rc) return rc;
     HIP_TRY(hipMemcpyAsync(d_buffer, ctx->d_gen_tok, (size_t)total, hipMemcpyDeviceToDevice, s));
     return EGG_OK;
+}
+extern "C" int egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed) {
+    return generate_impl(ctx, d_buffer, seed_len, gen_len, seed, nullptr);
+}
+// float -> int32 as the reference's GPU converts it: truncation, saturation at the ends, NaN -> 0
+static int sat_d2i(double x) {
+    if (x != x) return 0;
+    if (x >= 2147483648.0) return INT32_MAX;
+    if (x <= -2147483648.0) return INT32_MIN;
+    return (int)x;
+}
+// penalty_int = (int32_t)(penalty * (1 << SHIFT_LOGIT)) in float, min_p_limit = (int32_t)(logf(min_p) * SOFTMAX_EXP_SCALE)
+// in double (d-eggs/src/kernels.cu:386-387)
+extern "C" int egg_deggs_sampling_constants(const egg_config *cfg, float min_p, float penalty, int32_t *penalty_int, int32_t *min_p_limit) {
+    if (!cfg || !penalty_int || !min_p_limit || cfg->shift_logit < 0 || cfg->shift_logit > 30) return EGG_E_INVALID;
+    *penalty_int = sat_d2i((double)(penalty * (float)(1 << cfg->shift_logit)));
+    *min_p_limit = min_p > 0.0f ? sat_d2i((double)logf(min_p) * cfg->softmax_exp_scale) : (min_p <= 0.0f ? INT32_MIN : 0);
+    return EGG_OK;
+}
+extern "C" int egg_generate_deggs(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed, float temp, float min_p, float penalty) {
+    if (!ctx || !d_buffer) return EGG_E_INVALID;
+    int bt = (ctx->cfg.hidden + 31) & ~31; if (bt > 1024) bt = 1024;
+    // the reference keeps the tokens for the penalty in a 256-entry shared array that its first min(seed_len, block size)
+    // threads fill: beyond either limit it reads memory nobody wrote
+    if (seed_len + gen_len > 256 || seed_len > bt)
+        return fail(ctx, EGG_E_INVALID, "egg_generate_deggs: need seed_len + gen_len <= 256 and seed_len <= the reference's block size (hidden rounded up to 32)");
+    if (ctx->cfg.vocab > 256) return fail(ctx, EGG_E_INVALID, "egg_generate_deggs: byte vocabulary only");
+    DeggsSampling de; de.temp = temp;
+    int rc = egg_deggs_sampling_constants(&ctx->cfg, min_p, penalty, &de.penalty_int, &de.min_p_limit);
+    if (rc) return fail(ctx, rc, "egg_generate_deggs: configuration");
+    return generate_impl(ctx, d_buffer, seed_len, gen_len, seed, &de);
 }
 
 extern "C" int egg_ctx_enable_taps(egg_ctx *ctx, int enable) {

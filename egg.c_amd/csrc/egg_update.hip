@@ -363,6 +363,66 @@ hipError_t egg_launch_sample(const int32_t *logits, const int32_t *exp_lut, int 
     return hipGetLastError();
 }
 
+// The d-eggs form of the same sampler (d-eggs/src/kernels.cu:382-478): every occurrence of v among the tokens at
+// positions 0..t lowers v's logit by penalty_int (:398-402); the differences to the (penalised) maximum are divided by
+// the temperature in float and truncated (:430); entries whose scaled difference is below min_p_limit are left out
+// (:433); the rest weigh EXP_LUT[clamp(-scaled, 0, 255)] (layers.cuh:71-75).  Threshold and scan order as above.
+// The float -> int conversion is spelt out (truncation, saturation, NaN -> 0) so that it is defined for every input.
+__device__ __forceinline__ int sat_f2i(float x) {
+    if (x != x) return 0;
+    if (x >= 2147483648.0f) return INT_MAX;
+    if (x <= -2147483648.0f) return INT_MIN;
+    return (int)x;
+}
+__global__ void __launch_bounds__(256) k_sample_deggs(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
+                                                      const uint8_t *tokens, float temp, int min_p_limit, int penalty_int, uint8_t *out) {
+    __shared__ int lg[1024];
+    __shared__ int ex[1024];
+    __shared__ int red[256];
+    int mx = INT_MIN;
+    for (int v = threadIdx.x; v < vocab; v += 256) {
+        uint32_t count = 0;
+        for (int i = 0; i <= t; i++) count += tokens[i] == v;
+        const int l = (int)((uint32_t)logits[v] - count * (uint32_t)penalty_int);
+        lg[v] = l;
+        mx = max(mx, l);
+    }
+    red[threadIdx.x] = mx; __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) { if ((int)threadIdx.x < o) red[threadIdx.x] = max(red[threadIdx.x], red[threadIdx.x + o]); __syncthreads(); }
+    mx = red[0];
+    for (int v = threadIdx.x; v < vocab; v += 256) {
+        const int shifted = (int)((uint32_t)lg[v] - (uint32_t)mx);
+        const int scaled = sat_f2i((float)shifted / temp);
+        int e = 0;
+        if (scaled >= min_p_limit) {
+            int idx = (int)(0u - (uint32_t)scaled);
+            idx = idx < 0 ? 0 : (idx > 255 ? 255 : idx);
+            e = exp_lut[idx];
+        }
+        ex[v] = e;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        long long sum = 0;
+        for (int v = 0; v < vocab; v++) sum += ex[v];
+        const uint32_t r = hash_rng(seed + (uint32_t)t * 555u, 0);
+        const long long thresh = sum > 0 ? (long long)r % sum : 0;
+        int selected = 0; long long running = 0; bool done = false;
+        for (int tid = 0; tid < bt && !done; tid++)
+            for (int v = tid; v < vocab; v += bt) {
+                running += ex[v];
+                if (running > thresh) { selected = v; done = true; break; }
+            }
+        *out = (uint8_t)selected;
+    }
+}
+hipError_t egg_launch_sample_deggs(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
+                                   const uint8_t *tokens, float temp, int min_p_limit, int penalty_int, uint8_t *out, hipStream_t s) {
+    if (vocab > 256 || bt < 1 || t < 0) return hipErrorInvalidValue;       // tokens are bytes
+    hipLaunchKernelGGL(k_sample_deggs, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, tokens, temp, min_p_limit, penalty_int, out);
+    return hipGetLastError();
+}
+
 // canonical blocked weights -> fragment-major copy consumed by the GEMM kernels (layout in egg_device.h)
 __global__ void k_swizzle(const uint32_t *src, v4i *dst, int K, int N, int B, int nat) {
     int c = blockIdx.x * blockDim.x + threadIdx.x;

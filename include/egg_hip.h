@@ -227,6 +227,17 @@ uint32_t egg_next_seed(uint32_t seed, uint64_t step);
  * followed by room for gen_len more (seed_len + gen_len <= seq_len); the unperturbed model continues the prompt with
  * the reference's three-pass LUT sampling, threshold hash_rng(seed + t*555, 0) % sum.  Enqueued on the stream. */
 int  egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed);
+/* d-eggs' generate_sequence_kernel (d-eggs/src/kernels.cu:307-490, call site d-eggs/src/worker.cu:563-571): the same
+ * continuation with its sampler -- every earlier occurrence of a byte lowers that byte's logit by
+ * (int)(penalty * 2^shift_logit) (:398-402), differences to the maximum are divided by `temp` in float and truncated
+ * (:430), candidates whose scaled difference is below (int)(logf(min_p) * softmax_exp_scale) are left out (:433).
+ * temp = 1, min_p = 0, penalty = 0 is egg_generate.  The reference's defaults are 0.6 / 0.08 / 0.2
+ * (d-eggs/include/config.h:192-200).  seed_len + gen_len <= 256 and seed_len <= hidden rounded up to 32: beyond
+ * that the reference reads its 256-entry token history where nothing was written. */
+int  egg_generate_deggs(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed,
+                        float temp, float min_p, float penalty);
+/* the two integer constants that sampler derives from min_p and penalty (d-eggs/src/kernels.cu:386-387); host only */
+int  egg_deggs_sampling_constants(const egg_config *cfg, float min_p, float penalty, int32_t *penalty_int, int32_t *min_p_limit);
 
 /* ---- host-side companions of the GPU path (host code in the reference as well) ---- */
 /* d-eggs worker result shaping (de/src/worker.cu:636-687): loss[count] of `count/2` antithetic pairs -> diff = n - p,

@@ -326,6 +326,79 @@ def sample_token(logits_row, exp_lut, seed, t, hidden):
     return 0
 
 
+def _sat_f2i(x):
+    """float -> int32 as the GPU converts: truncation toward zero, saturation at the ends, NaN -> 0."""
+    x = np.float32(x)
+    if np.isnan(x):
+        return 0
+    if x >= np.float32(2147483648.0):
+        return 2147483647
+    if x <= np.float32(-2147483648.0):
+        return -2147483648
+    return int(x)
+
+
+def deggs_sampling_constants(cfg, min_p, penalty):
+    """penalty_int and min_p_limit of d-eggs/src/kernels.cu:386-387: the penalty in logit units, truncated, and
+    logf(min_p) * SOFTMAX_EXP_SCALE (a double product of a float logarithm), truncated; min_p <= 0 gives -inf,
+    which the conversion saturates to INT_MIN (nothing is filtered)."""
+    penalty_int = _sat_f2i(np.float32(penalty) * np.float32(1 << cfg.shift_logit))
+    if min_p <= 0:
+        limit = -2147483648
+    else:
+        prod = float(np.log(np.float32(min_p), dtype=np.float32)) * float(cfg.softmax_exp_scale)
+        limit = 2147483647 if prod >= 2147483648.0 else (-2147483648 if prod <= -2147483648.0 else int(prod))
+    return penalty_int, limit
+
+
+def sample_token_deggs(logits_row, exp_lut, seed, t, hidden, history, temp, min_p_limit, penalty_int):
+    """Three-pass sampling of d-eggs' generate_sequence_kernel (d-eggs/src/kernels.cu:382-478) for position t.
+    `history` is the token buffer up to and including position t: every occurrence of v in it lowers v's logit by
+    penalty_int (:398-402).  The differences to the maximum are divided by the temperature in float and truncated
+    (:430), entries below min_p_limit are left out (:433), the rest weigh EXP_LUT[clamp(-scaled, 0, 255)]
+    (layers.cuh:71-75).  Threshold and thread-major scan order as in the plain sampler (:443-474)."""
+    V = len(logits_row)
+    bt = min((hidden + 31) & ~31, 1024)
+    counts = np.bincount(np.asarray(history, np.int64), minlength=V)[:V]
+    lg = (logits_row.astype(np.int64) - counts * int(penalty_int))
+    lg = ((lg + (1 << 31)) % (1 << 32) - (1 << 31))                 # int32 wrap-around, as the repeated subtraction does
+    gmax = int(lg.max())
+    ex = np.zeros(V, np.int64)
+    for v in range(V):
+        shifted = int(lg[v]) - gmax
+        shifted = (shifted + (1 << 31)) % (1 << 32) - (1 << 31)
+        scaled = _sat_f2i(np.float32(shifted) / np.float32(temp))
+        if scaled >= min_p_limit:
+            idx = -scaled
+            ex[v] = int(exp_lut[0 if idx < 0 else (255 if idx > 255 else idx)])
+    total = int(ex.sum())
+    r = int(lib().orc_hash_rng(C.c_uint32((seed + t * 555) & 0xFFFFFFFF), C.c_uint32(0)))
+    thresh = r % total if total > 0 else 0
+    running = 0
+    for tid in range(bt):
+        for v in range(tid, V, bt):
+            running += int(ex[v])
+            if running > thresh:
+                return v
+    return 0
+
+
+def generate_deggs(cfg, model, prompt, gen_len, seed, temp, min_p, penalty):
+    """d-eggs' generate_sequence_kernel (d-eggs/src/kernels.cu:307-490) on this model's unperturbed forward: as
+    generate(), with the temperature / min-p / presence-penalty sampler."""
+    T = cfg.seq_len
+    seed_len = len(prompt)
+    assert 1 <= seed_len and seed_len + gen_len <= min(T, 256)
+    exp_lut = tables(cfg)[0]
+    penalty_int, limit = deggs_sampling_constants(cfg, min_p, penalty)
+    buf = np.zeros(T + 1, np.uint8)
+    buf[:seed_len] = prompt
+    for t in range(seed_len - 1, seed_len + gen_len - 1):
+        _, tr = forward_member(cfg, model, buf, 0, 0, 0, ns_override=0, trace=True)
+        buf[t + 1] = sample_token_deggs(tr["logits"][t], exp_lut, seed, t, cfg.hidden, buf[:t + 1], temp, limit, penalty_int)
+    return buf[:seed_len + gen_len].copy()
+
+
 def generate(cfg, model, prompt, gen_len, seed):
     """generate_sequence_kernel (mgpu.cu:1154-1283): unperturbed forward (noise_sign 0), token t+1 sampled from the
     logits of position t for t >= seed_len - 1.  The window is re-evaluated from position 0 for every new token,

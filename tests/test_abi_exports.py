@@ -74,3 +74,12 @@ def test_unsupported_configurations_are_refused_with_a_reason(pkg):
         rc = lib.egg_ctx_create(ctypes.byref(cfg), ctypes.byref(h))
         assert rc == -1 and not h.value, kw
         assert word in lib.egg_last_error(None).decode(), (kw, lib.egg_last_error(None))
+
+
+def test_deggs_sampling_constants_match_the_oracle(pkg, orc):
+    """Host-only: (int)(penalty * 2^shift_logit) and (int)(logf(min_p) * softmax_exp_scale), d-eggs/src/kernels.cu:386-387."""
+    for kw in (dict(), dict(shift_logit=6, softmax_exp_scale=10.0), dict(shift_logit=0)):
+        cfg, ocfg = pkg.default_config(**kw), orc.config(**kw)
+        for min_p in (0.08, 0.0, 1.0, 0.5, 1e-30, 2.0, -1.0, 0.3333):
+            for penalty in (0.2, 0.0, 1.0, -0.01, 7.77, 1e12):
+                assert pkg.deggs_sampling_constants(cfg, min_p, penalty) == orc.deggs_sampling_constants(ocfg, min_p, penalty), (kw, min_p, penalty)

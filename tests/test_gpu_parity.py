@@ -554,6 +554,47 @@ def test_generate(pkg, orc, dev, kw, seed_len, gen_len):
     ctx.close()
 
 
+@pytest.mark.parametrize("kw,seed_len,gen_len,sampling", [
+    (dict(hidden=64, head_dim=32, n_layers=1, seq_len=64, population=2), 5, 40, (0.6, 0.08, 0.2)),       # the reference's defaults
+    (dict(hidden=64, head_dim=32, n_layers=1, seq_len=64, population=2), 5, 40, (1.0, 0.0, 0.0)),        # neutral: the plain sampler
+    (dict(hidden=128, head_dim=32, n_layers=2, seq_len=128, population=2), 20, 100, (1.7, 0.3, 1.5)),
+    (dict(hidden=256, head_dim=64, n_layers=1, seq_len=256, population=2), 196, 60, (0.25, 0.01, -0.5)),
+    (dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=2), 1, 31, (3.0, 0.9, 4.0))])
+def test_generate_deggs(pkg, orc, dev, kw, seed_len, gen_len, sampling):
+    """d-eggs' sampler (temperature, min-p, presence penalty; d-eggs/src/kernels.cu:382-478) against the oracle."""
+    import torch
+    temp, min_p, penalty = sampling
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    rng = np.random.default_rng(3)
+    for t in orc.tensor_table(ocfg):
+        if not t["is_matrix"]:
+            sl = slice(t["offset"], t["offset"] + t["cols"])
+            model[sl] = rng.integers(-20, 21, t["cols"]).astype(np.int8) + (16 if t["name"].startswith("ln_") and "bias" not in t["name"] else 0)
+        elif t["name"] == "embedding":
+            n = t["rows"] * t["cols"]
+            model[t["offset"]:t["offset"] + n] = rng.integers(-5, 6, n).astype(np.int8)
+    prompt = orc.zipf_bytes(4096)[100:100 + seed_len].copy()
+    ref = orc.generate_deggs(ocfg, model, prompt, gen_len, 1041, temp, min_p, penalty)
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_upload(model)
+    buf = torch.zeros(seed_len + gen_len, dtype=torch.uint8, device=dev)
+    buf[:seed_len] = _t(dev, prompt)
+    ctx.generate_deggs(buf.data_ptr(), seed_len, gen_len, 1041, temp, min_p, penalty)
+    ctx.sync()
+    got = buf.cpu().numpy()
+    assert np.array_equal(got, ref), (got.tolist(), ref.tolist())
+    if sampling == (1.0, 0.0, 0.0):
+        assert np.array_equal(ref, orc.generate(ocfg, model, prompt, gen_len, 1041))
+    else:
+        assert not np.array_equal(ref, orc.generate(ocfg, model, prompt, gen_len, 1041))      # the settings matter
+    if penalty >= 1.5:
+        assert len(set(ref[seed_len:].tolist())) > 15          # a strong penalty spreads the continuation
+    with pytest.raises(pkg.EggError):
+        ctx.generate_deggs(buf.data_ptr(), 200, 100, 1)          # beyond the reference's 256-entry token history
+    ctx.close()
+
+
 def test_checkpoint_files_round_trip(pkg, orc, dev, tmp_path):
     """save_checkpoint / load_model (egg_disk_utils.h:46-82): raw model and optimizer-state files, "last" symlinks,
     byte-identical to what the oracle holds after the same steps; a file of another shape is refused."""

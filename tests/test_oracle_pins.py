@@ -645,6 +645,55 @@ def test_sampling_closed_forms(orc):
         assert orc.sample_token(two, exp_lut, 5, t, 256) == (10 if rr % (w0 + w1) < w0 else 20)
 
 
+def test_deggs_sampler_special_cases(orc):
+    """d-eggs' sampler (d-eggs/src/kernels.cu:382-478) has no fixture in the reference; these are the cases its
+    definition fixes: neutral settings reduce to the plain sampler, a temperature of 2 equals halved (even) differences,
+    min-p drops exactly the candidates below its limit, the penalty counts occurrences and can exclude a byte."""
+    cfg = orc.config(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=2)
+    exp_lut = orc.tables(cfg)[0]
+    rng = np.random.default_rng(11)
+    # the constants: (int)(penalty * 2^shift_logit) and (int)(logf(min_p) * 6.0), truncated toward zero
+    assert cfg.shift_logit == 8 and cfg.softmax_exp_scale == 6.0
+    assert orc.deggs_sampling_constants(cfg, 0.08, 0.2) == (51, -15)        # 0.2 * 256 = 51.2;  ln 0.08 * 6 = -15.15
+    assert orc.deggs_sampling_constants(cfg, 0.0, 0.0) == (0, -2147483648)
+    assert orc.deggs_sampling_constants(cfg, 1.0, 1.0) == (256, 0)
+    assert orc.deggs_sampling_constants(cfg, 0.5, -0.01) == (-2, -4)         # ln 0.5 * 6 = -4.16;  -2.56 truncates to -2
+    for seed, t in ((7, 0), (7, 13), (123456, 40)):
+        logits = rng.integers(-60, 60, 256).astype(np.int32)
+        hist = rng.integers(0, 256, t + 1)
+        plain = orc.sample_token(logits, exp_lut, seed, t, 256)
+        assert orc.sample_token_deggs(logits, exp_lut, seed, t, 256, hist, 1.0, -2147483648, 0) == plain
+        # temperature 2 on doubled differences is temperature 1 on the differences
+        assert orc.sample_token_deggs(2 * logits, exp_lut, seed, t, 256, hist, 2.0, -2147483648, 0) == plain
+        # truncation toward zero: differences -1 scale to 0 at temperature 2, i.e. weigh like the maximum
+        near = np.full(256, -1000, np.int32); near[3] = 5; near[9] = 4
+        got = {orc.sample_token_deggs(near, exp_lut, s2, t, 256, hist, 2.0, -2147483648, 0) for s2 in range(40)}
+        assert got == {3, 9}
+    # min-p: candidates at scaled difference -15 pass a limit of -15, those at -16 do not
+    lim = orc.deggs_sampling_constants(cfg, 0.08, 0.0)[1]
+    assert lim == -15 and exp_lut[15] > 0 and exp_lut[16] > 0
+    edge = np.full(256, -16, np.int32); edge[100] = 0; edge[200] = -15
+    seen = {orc.sample_token_deggs(edge, exp_lut, s2, 0, 256, [0], 1.0, lim, 0) for s2 in range(300)}
+    assert seen == {100, 200}
+    seen_all = {orc.sample_token_deggs(edge, exp_lut, s2, 0, 256, [0], 1.0, -2147483648, 0) for s2 in range(300)}
+    assert len(seen_all) > 50                       # without the filter the 254 small weights together matter
+    # a limit above zero leaves nothing: the sum is 0 and byte 0 is selected
+    assert orc.sample_token_deggs(edge, exp_lut, 5, 0, 256, [0], 1.0, 1, 0) == 0
+    # presence penalty: two equal peaks; three earlier occurrences of byte 10 push it 3 * 30 = 90 below byte 20, out of
+    # the table's range (EXP_LUT[75] is already 0), so only byte 20 is ever drawn; one occurrence of each leaves them equal
+    two = np.full(256, -1000, np.int32); two[10] = 0; two[20] = 0
+    assert exp_lut[90 if 90 < 256 else 255] == 0
+    assert {orc.sample_token_deggs(two, exp_lut, s2, 4, 256, [10, 10, 1, 10, 2], 1.0, -2147483648, 30) for s2 in range(60)} == {20}
+    assert {orc.sample_token_deggs(two, exp_lut, s2, 4, 256, [10, 20, 1, 3, 2], 1.0, -2147483648, 30) for s2 in range(60)} == {10, 20}
+    # the split between them follows the threshold exactly: weights EXP_LUT[0] each, byte 10 first in scan order
+    w = int(exp_lut[0])
+    for s2 in range(30):
+        r = int(orc.lib().orc_hash_rng(C.c_uint32((s2 + 4 * 555) & 0xFFFFFFFF), C.c_uint32(0)))
+        assert orc.sample_token_deggs(two, exp_lut, s2, 4, 256, [10, 20, 1, 3, 2], 1.0, -2147483648, 30) == (10 if r % (2 * w) < w else 20)
+    # only positions 0..t count: a later occurrence in the buffer is not seen
+    assert {orc.sample_token_deggs(two, exp_lut, s2, 1, 256, [1, 2], 1.0, -2147483648, 30) for s2 in range(60)} == {10, 20}
+
+
 # ------------------------------------------------------------------ d-eggs adaptive noise overlay
 def test_adaptive_overlay_special_cases(orc):
     """The overlay restatement has no reference fixture (parity unpinned); these are the cases arithmetic fixes:
