@@ -44,6 +44,8 @@ struct egg_ctx {
     int8_t *d_model = nullptr;
     uint8_t *d_state = nullptr; int64_t state_bytes = 0; std::vector<int64_t> t_state_off;   // optimizer state (AdamModel layout)
     MuonWork muon = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    std::vector<std::vector<int>> muon_groups;    // ids of the Muon matrices, grouped by shape; a group runs Newton-Schulz as batches
+    int muon_batch_max = 1;                       // matrices the Muon workspace holds at once
     int8_t *d_wfrag = nullptr;      // fragment-major copy of every matrix, same offsets as the model blob
     int8_t *d_plin_frag = nullptr; size_t plin_frag_bytes = 0;
     bool plin_no_ws = false;        // egg_ctx_linear_kernel: run the W-streaming kernels also where the W-stationary one exists
@@ -295,10 +297,31 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
         CR(hipMemcpy(ctx->d_vec_desc, vd.data(), vd.size() * sizeof(VecDesc), hipMemcpyHostToDevice));
     }
     if (c.use_muon) {
-        size_t mx = (size_t)4 * c.hidden * c.hidden;
-        CR(hipMalloc(&ctx->muon.x, mx * 4)); CR(hipMalloc(&ctx->muon.swap, mx * 4));
-        CR(hipMalloc(&ctx->muon.bterm, (size_t)c.hidden * c.hidden * 4));
-        CR(hipMalloc(&ctx->muon.partials, 1024 * 4)); CR(hipMalloc(&ctx->muon.norm, 16));
+        // Matrices of one shape go through Newton-Schulz together (one launch per stage for the whole batch).  The
+        // workspace holds the largest group, or as much of it as fits 16 Mi elements per buffer (and always one 4H x H).
+        for (int id = 0; id < (int)ctx->tensors.size(); id++) {
+            const egg_tensor_info &t = ctx->tensors[id];
+            if (!t.is_matrix || !t.muon) continue;
+            bool placed = false;
+            for (auto &g : ctx->muon_groups)
+                if (ctx->tensors[g[0]].rows == t.rows && ctx->tensors[g[0]].cols == t.cols) { g.push_back(id); placed = true; break; }
+            if (!placed) ctx->muon_groups.push_back(std::vector<int>(1, id));
+        }
+        size_t mx = (size_t)4 * c.hidden * c.hidden, cap = (size_t)16 << 20;
+        if (cap < mx) cap = mx;
+        size_t elems = mx, bt = (size_t)c.hidden * c.hidden; int nb = 1;
+        for (const auto &g : ctx->muon_groups) {
+            const egg_tensor_info &t = ctx->tensors[g[0]];
+            const size_t one = (size_t)t.rows * t.cols, k = (size_t)(t.rows < t.cols ? t.rows : t.cols);
+            size_t b = cap / one; if (b > g.size()) b = g.size(); if (b < 1) b = 1;
+            if (b * one > elems) elems = b * one;
+            if (b * k * k > bt) bt = b * k * k;
+            if ((int)b > nb) nb = (int)b;
+        }
+        ctx->muon_batch_max = nb;
+        CR(hipMalloc(&ctx->muon.x, elems * 4)); CR(hipMalloc(&ctx->muon.swap, elems * 4));
+        CR(hipMalloc(&ctx->muon.bterm, bt * 4));
+        CR(hipMalloc(&ctx->muon.partials, (size_t)nb * 256 * 4 + 1024 * 4)); CR(hipMalloc(&ctx->muon.norm, (size_t)nb * 4 + 16));
     }
     // activation workspace for one chunk of members
     // default: the whole population in one launch per kernel while its five activation buffers stay within 32 GiB
@@ -742,10 +765,36 @@ extern "C" int egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t 
     // matrices one by one (each needs the panel workspace), then every vector tensor in one launch; tensors are
     // independent, so the reference's launch order (mgpu.cu:1603-1643) does not matter
     for (int id = 0; id < (int)ctx->tensors.size(); id++) {
-        if (!ctx->tensors[id].is_matrix) continue;
+        if (!ctx->tensors[id].is_matrix || (ctx->cfg.use_muon && ctx->tensors[id].muon)) continue;
         int rc = update_one(ctx, id, d_fit, d_seed, d_lr, ctx->adaptive);
         if (rc) return rc;
     }
+    // Muon matrices (LAUNCH_ADAM_MATRIX under USE_MUON, mgpu.cu:1587-1595), a batch of one shape at a time: momentum of
+    // each into its slot of the workspace, Newton-Schulz of the whole batch, then each matrix's apply rule
+    if (ctx->cfg.use_muon)
+        for (const auto &g : ctx->muon_groups) {
+            const egg_tensor_info &t0 = ctx->tensors[g[0]];
+            const size_t one = (size_t)t0.rows * t0.cols;
+            for (size_t first = 0; first < g.size(); first += ctx->muon_batch_max) {
+                const int nb = (int)std::min(g.size() - first, (size_t)ctx->muon_batch_max);
+                span_begin(ctx, EGG_K_UPDATE_MATRIX);
+                for (int b = 0; b < nb; b++) {
+                    UpdParams p = make_upd(ctx, g[first + b], d_fit, d_seed, d_lr);
+                    p.muon_momentum = ctx->cfg.muon_momentum; p.muon_x = ctx->muon.x + (size_t)b * one;
+                    HIP_TRY(egg_launch_muon_momentum(p, ctx->stream));
+                }
+                HIP_TRY(egg_launch_newton_schulz_batched(ctx->muon, t0.rows, t0.cols, 5, nb, ctx->stream));
+                for (int b = 0; b < nb; b++) {
+                    const int id = g[first + b];
+                    UpdParams p = make_upd(ctx, id, d_fit, d_seed, d_lr);
+                    p.muon_x = ctx->muon.x + (size_t)b * one;
+                    p.lr_scale = ctx->tensors[id].lr_scale * ctx->cfg.muon_lr_scale;
+                    HIP_TRY(egg_launch_muon_apply(p, ctx->cfg.adam_weight_decay, ctx->stream));
+                }
+                span_end(ctx);
+                for (int b = 0; b < nb; b++) { int rc = refresh_frag(ctx, g[first + b]); if (rc) return rc; }
+            }
+        }
     UpdParams common = make_upd(ctx, 0, d_fit, d_seed, d_lr);
     span_begin(ctx, EGG_K_UPDATE_VECTOR);
     HIP_TRY(egg_launch_update_vectors(common, ctx->d_vec_desc, ctx->n_vec, ctx->vec_total, ctx->stream));
@@ -819,7 +868,8 @@ extern "C" int64_t egg_tensor_state_offset(const egg_ctx *ctx, int id) {
 // Newton-Schulz orthogonalisation of a row-major [rows][cols] fp32 device matrix, in place (test hook for
 // perform_newton_schulz, muon_internal.cuh:182-342)
 extern "C" int egg_newton_schulz(egg_ctx *ctx, float *d_X, int rows, int cols, int iters) {
-    if (!ctx || !d_X || rows < 32 || cols < 32 || rows % 32 || cols % 32) return fail(ctx, EGG_E_INVALID, "egg_newton_schulz arguments");
+    if (!ctx || !d_X || (reinterpret_cast<uintptr_t>(d_X) & 15) || rows < 32 || cols < 32 || rows % 32 || cols % 32)
+        return fail(ctx, EGG_E_INVALID, "egg_newton_schulz arguments (a 16-byte aligned matrix with rows and cols multiples of 32)");
     if (!ctx->muon.x) return fail(ctx, EGG_E_STATE, "context was created without use_muon");
     if ((size_t)rows * cols > (size_t)4 * ctx->cfg.hidden * ctx->cfg.hidden || (rows < cols ? rows : cols) > ctx->cfg.hidden)
         return fail(ctx, EGG_E_INVALID, "matrix larger than the Muon workspace");

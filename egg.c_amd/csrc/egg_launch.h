@@ -79,6 +79,7 @@ hipError_t egg_launch_ternary_pack(const int8_t *src, uint8_t *packed, int n_ele
 hipError_t egg_launch_muon_momentum(const UpdParams &p, hipStream_t s);
 struct MuonWork { float *x, *swap, *gram, *bterm, *partials, *norm; };   // x/swap: rows*cols, gram/bterm: K*K, partials: 1024
 hipError_t egg_launch_newton_schulz(const MuonWork &w, int rows, int cols, int iters, hipStream_t s);
+hipError_t egg_launch_newton_schulz_batched(const MuonWork &w, int rows, int cols, int iters, int batch, hipStream_t s);
 hipError_t egg_launch_muon_apply(const UpdParams &p, float wd, hipStream_t s);
 // message returned by egg_last_error(NULL) on this thread, for entry points that take no context
 void egg_set_thread_error(const char *what);

@@ -454,9 +454,12 @@ hipError_t egg_launch_muon_momentum(const UpdParams &p, hipStream_t s) {
 // ---------------------------------------------------------------- Newton-Schulz (muon_internal.cuh:182-342)
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-// sum of squares in two deterministic stages (cublasSnrm2 in the reference)
+// Every kernel of the chain takes a batch of same-shape matrices, one per blockIdx.y (matrix b's operands sit b strides
+// further on); what is computed for a matrix does not depend on the batch it runs in.
+// sum of squares in two deterministic stages (cublasSnrm2 in the reference): 256 partial sums per matrix
 __global__ void __launch_bounds__(256) k_sumsq_partial(const float *x, int n, float *partials) {
     __shared__ float sh[256];
+    x += (size_t)blockIdx.y * n; partials += (size_t)blockIdx.y * 256;
     float s = 0.f;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) { float v = x[i]; s += v * v; }
     sh[threadIdx.x] = s; __syncthreads();
@@ -465,38 +468,57 @@ __global__ void __launch_bounds__(256) k_sumsq_partial(const float *x, int n, fl
 }
 __global__ void __launch_bounds__(256) k_norm_finish(const float *partials, int n, float *norm) {
     __shared__ float sh[256];
+    partials += (size_t)blockIdx.y * 256;
     float s = 0.f;
     for (int i = threadIdx.x; i < n; i += 256) s += partials[i];
     sh[threadIdx.x] = s; __syncthreads();
     for (int o = 128; o > 0; o >>= 1) { if (threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o]; __syncthreads(); }
-    if (threadIdx.x == 0) norm[0] = sqrtf(sh[0]);
+    if (threadIdx.x == 0) norm[blockIdx.y] = sqrtf(sh[0]);
 }
 // muon_scale_by_norm_kernel (muon_internal.cuh:77-87)
 __global__ void k_scale_by_norm(float *x, const float *norm, int n) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) { float nv = *norm; if (nv > 1e-6f) x[i] /= nv; }
+    if (i < n) { float nv = norm[blockIdx.y]; if (nv > 1e-6f) x[(size_t)blockIdx.y * n + i] /= nv; }
 }
 
-// C[M][N] (row-major, ldc = N) = epilogue(sum_k A(i,k) B(k,j)), generic strides, one workgroup per 32x32 tile on
-// v_mfma_f32_32x32x2_f32.  The k range is dealt to the four waves in steps of two (wave w takes k = 2w, 2w + 8, ...),
-// the partial tiles are added in wave order in LDS (a fixed summation order, so results are reproducible), and wave q
-// writes rows 8q + 4g + e of the tile.  mode 0: C = alpha * acc.  mode 1: C = (i == j ? 3 : 0) - acc  (3I - G,
-// muon_internal.cuh:91-109).
-__global__ void __launch_bounds__(EGG_THREADS) k_sgemm(const float *A, long sa_i, long sa_k, const float *B, long sb_k, long sb_j,
+// C[M][N] (row-major, ldc = N) = epilogue(sum_k A(i,k) B(k,j)), one workgroup per 32x32 tile on
+// v_mfma_f32_32x32x2_f32.  Each operand is given by two strides of which one is 1 (a row-major matrix or its
+// transpose); AK / BK say that it is the k stride.  An operand whose k stride is 1 is read with one 16-byte load per lane
+// (four consecutive k of the lane's row or column); the other kind has its rows or columns side by side in memory and is
+// read with fully coalesced 4-byte loads.  The k range is dealt to the four waves in blocks of eight (wave w takes blocks
+// w, w + 4, ...); within a block, MFMA e multiplies the k pair {8c + e, 8c + 4 + e}.  The partial tiles are added in wave
+// order in LDS, so the summation order is fixed and results are reproducible; wave q writes rows 8q + 4g + e of the
+// tile.  mode 0: C = alpha * acc.  mode 1: C = (i == j ? 3 : 0) - acc  (3I - G, muon_internal.cuh:91-109).
+typedef float v4f __attribute__((ext_vector_type(4)));
+template <bool AK, bool BK>
+__global__ void __launch_bounds__(EGG_THREADS) k_sgemm(const float *A, long lda, long batch_a, const float *B, long ldb, long batch_b,
                                                       float *C, int M, int N, int K, float alpha, int mode) {
     __shared__ float red[EGG_WAVES][16][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const int tiles_n = N / 32, tile = blockIdx.x;
     const int i0 = (tile / tiles_n) * 32, j0 = (tile % tiles_n) * 32;
+    A += (long)blockIdx.y * batch_a; B += (long)blockIdx.y * batch_b; C += (size_t)blockIdx.y * M * N;
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
-    const float *ap = A + (long)(i0 + j) * sa_i + (long)g * sa_k;
-    const float *bp = B + (long)g * sb_k + (long)(j0 + j) * sb_j;
-#pragma unroll 8
-    for (int k = 2 * wave; k < K; k += 2 * EGG_WAVES) {
-        float a = ap[(long)k * sa_k], b = bp[(long)k * sb_k];
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+    // lane (j, g) supplies A(i0 + j, k) and B(k, j0 + j) for k = 8c + 4g + e
+    const float *ap = AK ? A + (long)(i0 + j) * lda + 4 * g : A + (long)(4 * g) * lda + i0 + j;
+    const float *bp = BK ? B + (long)(j0 + j) * ldb + 4 * g : B + (long)(4 * g) * ldb + j0 + j;
+#pragma unroll 4
+    for (int c = wave; c < K / 8; c += EGG_WAVES) {
+        v4f a4, b4;
+        if (AK) a4 = *reinterpret_cast<const v4f *>(ap + 8 * c);
+        else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) a4[e] = ap[(long)(8 * c + e) * lda];
+        }
+        if (BK) b4 = *reinterpret_cast<const v4f *>(bp + 8 * c);
+        else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) b4[e] = bp[(long)(8 * c + e) * ldb];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[e], b4[e], acc, 0, 0, 0);
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) red[wave][r][lane] = acc[r];
@@ -511,39 +533,59 @@ __global__ void __launch_bounds__(EGG_THREADS) k_sgemm(const float *A, long sa_i
         C[(size_t)i * N + jj] = (mode == 1) ? ((i == jj ? 3.0f : 0.0f) - v) : alpha * v;
     }
 }
-static void sgemm(const float *A, long sa_i, long sa_k, const float *B, long sb_k, long sb_j, float *C, int M, int N, int K,
-                  float alpha, int mode, hipStream_t s) {
-    int tiles = (M / 32) * (N / 32);
-    hipLaunchKernelGGL(k_sgemm, dim3(tiles), dim3(EGG_THREADS), 0, s, A, sa_i, sa_k, B, sb_k, sb_j, C, M, N, K, alpha, mode);
+// A(i,k) at A[i * sa_i + k * sa_k], B(k,j) at B[k * sb_k + j * sb_j]; one stride of each pair must be 1 and the other a
+// multiple of 4 (16-byte loads)
+static hipError_t sgemm(const float *A, long sa_i, long sa_k, long batch_a, const float *B, long sb_k, long sb_j, long batch_b, float *C, int M, int N, int K,
+                        float alpha, int mode, int batch, hipStream_t s) {
+    const bool ak = sa_k == 1, bk = sb_k == 1;
+    if ((!ak && sa_i != 1) || (!bk && sb_j != 1) || M % 32 || N % 32 || K % 32) return hipErrorInvalidValue;
+    const long lda = ak ? sa_i : sa_k, ldb = bk ? sb_j : sb_k;
+    if (lda % 4 || ldb % 4 || batch_a % 4 || batch_b % 4) return hipErrorInvalidValue;
+    const dim3 grid((M / 32) * (N / 32), batch), block(EGG_THREADS);
+    if (ak && bk) hipLaunchKernelGGL((k_sgemm<true, true>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    else if (ak) hipLaunchKernelGGL((k_sgemm<true, false>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    else if (bk) hipLaunchKernelGGL((k_sgemm<false, true>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    else hipLaunchKernelGGL((k_sgemm<false, false>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    return hipGetLastError();
 }
-__global__ void k_copy_f32(float *dst, const float *src, int n) {
-    int i = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ void k_copy_f32(float *dst, const float *src, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = src[i];
 }
 
-hipError_t egg_launch_newton_schulz(const MuonWork &w, int rows, int cols, int iters, hipStream_t s) {
-    if (rows % 32 || cols % 32) return hipErrorInvalidValue;
+// `batch` matrices of rows x cols, matrix b at w.x + b * rows * cols (w.swap likewise), its 3I - G term at
+// w.bterm + b * K * K (K = min(rows, cols)), its 256 norm partials at w.partials + 256 b, its norm at w.norm + b
+hipError_t egg_launch_newton_schulz_batched(const MuonWork &w, int rows, int cols, int iters, int batch, hipStream_t s) {
+    if (rows % 32 || cols % 32 || batch < 1 || batch > 65535) return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(w.x) | reinterpret_cast<uintptr_t>(w.swap) | reinterpret_cast<uintptr_t>(w.bterm)) & 15) return hipErrorInvalidValue;   // 16-byte loads
     const int n = rows * cols;
     const bool use_rows = rows < cols;
     const int K = use_rows ? rows : cols;
-    hipLaunchKernelGGL(k_sumsq_partial, dim3(256), dim3(256), 0, s, w.x, n, w.partials);
-    hipLaunchKernelGGL(k_norm_finish, dim3(1), dim3(256), 0, s, w.partials, 256, w.norm);
-    hipLaunchKernelGGL(k_scale_by_norm, dim3((n + 255) / 256), dim3(256), 0, s, w.x, w.norm, n);
+    const long kk = (long)K * K;
+    hipLaunchKernelGGL(k_sumsq_partial, dim3(256, batch), dim3(256), 0, s, w.x, n, w.partials);
+    hipLaunchKernelGGL(k_norm_finish, dim3(1, batch), dim3(256), 0, s, w.partials, 256, w.norm);
+    hipLaunchKernelGGL(k_scale_by_norm, dim3((n + 255) / 256, batch), dim3(256), 0, s, w.x, w.norm, n);
     float *cur = w.x, *nxt = w.swap;          // ping-pong instead of copying back after every iteration
-    for (int it = 0; it < iters; it++) {
+    hipError_t e = hipSuccess;
+    for (int it = 0; it < iters && e == hipSuccess; it++) {
         if (use_rows) {
             // G = X X^T (rows x rows); X <- 0.5 (3I - G) X
-            sgemm(cur, cols, 1, cur, 1, cols, w.bterm, K, K, cols, 1.f, 1, s);
-            sgemm(w.bterm, K, 1, cur, cols, 1, nxt, rows, cols, K, 0.5f, 0, s);
+            e = sgemm(cur, cols, 1, n, cur, 1, cols, n, w.bterm, K, K, cols, 1.f, 1, batch, s);
+            if (e == hipSuccess) e = sgemm(w.bterm, K, 1, kk, cur, cols, 1, n, nxt, rows, cols, K, 0.5f, 0, batch, s);
         } else {
             // G = X^T X (cols x cols); X <- 0.5 X (3I - G)
-            sgemm(cur, 1, cols, cur, cols, 1, w.bterm, K, K, rows, 1.f, 1, s);
-            sgemm(cur, cols, 1, w.bterm, K, 1, nxt, rows, cols, K, 0.5f, 0, s);
+            e = sgemm(cur, 1, cols, n, cur, cols, 1, n, w.bterm, K, K, rows, 1.f, 1, batch, s);
+            if (e == hipSuccess) e = sgemm(cur, cols, 1, n, w.bterm, K, 1, kk, nxt, rows, cols, K, 0.5f, 0, batch, s);
         }
         float *t = cur; cur = nxt; nxt = t;
     }
-    if (cur != w.x) hipLaunchKernelGGL(k_copy_f32, dim3((n + 255) / 256), dim3(256), 0, s, w.x, cur, n);
+    if (e != hipSuccess) return e;
+    const size_t total = (size_t)n * batch;
+    if (cur != w.x) hipLaunchKernelGGL(k_copy_f32, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, w.x, cur, total);
     return hipGetLastError();
+}
+hipError_t egg_launch_newton_schulz(const MuonWork &w, int rows, int cols, int iters, hipStream_t s) {
+    return egg_launch_newton_schulz_batched(w, rows, cols, iters, 1, s);
 }
 
 // ---------------------------------------------------------------- Newton-Schulz for callers that cannot allocate
@@ -578,8 +620,8 @@ static hipError_t ns_scratch_on_current_device(NsScratch **out) {
 }
 
 extern "C" int egg_newton_schulz_static(float *d_X, int rows, int cols, int iters, void *hip_stream) {
-    if (!d_X || rows < 32 || cols < 32 || rows % 32 || cols % 32 || iters < 0 || iters > 64) {
-        egg_set_thread_error("egg_newton_schulz_static: need a device matrix with rows and cols multiples of 32 and 0 <= iters <= 64");
+    if (!d_X || (reinterpret_cast<uintptr_t>(d_X) & 15) || rows < 32 || cols < 32 || rows % 32 || cols % 32 || iters < 0 || iters > 64) {
+        egg_set_thread_error("egg_newton_schulz_static: need a 16-byte aligned device matrix with rows and cols multiples of 32 and 0 <= iters <= 64");
         return EGG_E_INVALID;
     }
     if ((long long)rows * cols > EGG_NS_STATIC_MAX_ELEMS || (rows < cols ? rows : cols) > EGG_NS_STATIC_MAX_SHORT) {

@@ -174,7 +174,8 @@ int  egg_update_tensor(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const 
 int  egg_matrix_votes(egg_ctx *ctx, int tensor_id, const int32_t *d_fit, const uint32_t *d_seed, int32_t *d_votes);
 
 /* perform_newton_schulz (muon_internal.cuh:182-342) on a row-major fp32 [rows][cols] device matrix, in place:
- * X /= ||X||_F, then `iters` times X <- 0.5 X (3I - X^T X) on the short side.  Needs a use_muon context. */
+ * X /= ||X||_F, then `iters` times X <- 0.5 X (3I - X^T X) on the short side.  Needs a use_muon context; d_X must be
+ * 16-byte aligned, rows and cols multiples of 32. */
 int  egg_newton_schulz(egg_ctx *ctx, float *d_X, int rows, int cols, int iters);
 
 /* No counterpart in the reference.  egg_newton_schulz for callers that cannot allocate (code under HIP graph capture,

@@ -515,6 +515,40 @@ def test_muon_update(pkg, orc, dev):
     ctx.close()
 
 
+@pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=3, seq_len=32, population=64),
+                                dict(hidden=128, head_dim=32, n_layers=2, seq_len=32, population=32),
+                                dict(hidden=256, head_dim=64, n_layers=5, seq_len=32, population=16)])
+def test_muon_batched_update_equals_per_matrix_update(pkg, orc, dev, kw):
+    """egg_es_update sends the Muon matrices of one shape through Newton-Schulz as one batch per stage; what it leaves
+    (weights, momentum, accumulators, update count) is bit-identical to updating tensor by tensor."""
+    import torch
+    ocfg = orc.config(**kw)
+    model = orc.init_model(ocfg, 42)
+    rng = np.random.default_rng(5)
+    pairs = kw["population"] // 2
+    a = pkg.Context(pkg.default_config(use_muon=1, **kw))
+    b = pkg.Context(pkg.default_config(use_muon=1, **kw))
+    a.model_upload(model); b.model_upload(model)
+    shapes = {}
+    for t in a.tensors():
+        if t["muon"]:
+            shapes.setdefault((t["rows"], t["cols"]), []).append(t["id"])
+    assert max(len(v) for v in shapes.values()) >= 2 * kw["n_layers"]          # there is something to batch
+    d_lr = _t(dev, np.array([25.0], np.float32))
+    for step in range(3):
+        d_fit = _t(dev, rng.integers(-1, 2, pairs).astype(np.int32))
+        d_seed = _t(dev, np.array([900 + step], np.uint32).view(np.int32))
+        a.es_update(d_fit.data_ptr(), d_seed.data_ptr(), d_lr.data_ptr())
+        total = 0
+        for t in b.tensors():
+            b.update_tensor(t["id"], d_fit.data_ptr(), d_seed.data_ptr(), d_lr.data_ptr())
+        a.sync(); b.sync()
+        assert np.array_equal(a.model_download(), b.model_download()), step
+        assert np.array_equal(a.opt_state_download(), b.opt_state_download()), step
+    assert not np.array_equal(a.model_download(), model)
+    a.close(); b.close()
+
+
 @pytest.mark.parametrize("kw,seed_len,gen_len", [(dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4), 5, 27),
                                                  (dict(hidden=128, head_dim=32, n_layers=2, seq_len=64, population=4), 10, 30),
                                                  (dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4), 16, 40)],
