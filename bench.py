@@ -19,6 +19,47 @@ PEAK_INT8_OPS = 5.0e15      # MI355X dense int8 MFMA, published
 PEAK_HBM = 8.0e12
 
 
+def host_cpu():
+    """Model string, physical cores and hardware threads of the host, from /proc/cpuinfo."""
+    model, cores, threads = None, set(), 0
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "processor":
+                threads += 1
+            elif k == "model name" and model is None:
+                model = v
+            elif k == "physical id":
+                phys = v
+            elif k == "core id":
+                core = v
+            elif not k and phys is not None:
+                cores.add((phys, core)); phys = core = None
+        if phys is not None:
+            cores.add((phys, core))
+    except OSError:
+        pass
+    return {"model": model, "physical_cores": len(cores) or None, "hardware_threads": threads or os.cpu_count()}
+
+
+def profiled_traffic(path, kernel, members_per_launch, tokens):
+    """Bytes per launch from a line `TRAFFIC <kernel> members_per_launch=M tokens=T fetch_KiB=F write_KiB=W fetch_scale=a
+    write_scale=b` of a counter summary under profiles/, or None when there is no such line for this launch shape."""
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) < 3 or f[0] != "TRAFFIC" or f[1] != kernel:
+                continue
+            kv = dict(x.split("=", 1) for x in f[2:] if "=" in x)
+            if int(kv["members_per_launch"]) == members_per_launch and int(kv["tokens"]) == tokens:
+                return (float(kv["fetch_KiB"]) * float(kv["fetch_scale"]) + float(kv["write_KiB"]) * float(kv["write_scale"])) * 1024.0
+    except (OSError, KeyError, ValueError):
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -29,6 +70,7 @@ def main():
     ap.add_argument("--data-mib", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="skip the hipGraph replay leg")
+    ap.add_argument("--headline-only", action="store_true", help="only the headline steps (no side legs): the form counter runs use")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain elementwise copy of 256 MiB (reads 256 MiB, writes 256 MiB) so that a "
                          "counter run can scale FETCH_SIZE / WRITE_SIZE by what they read for known traffic")
@@ -100,12 +142,12 @@ def main():
     launches, tot_ms = timing[dom]
     tokens_per_launch = P * T * args.steps * (L if dom in ("mlp", "qkv", "attn") else 1) / max(launches, 1)
     achieved = ops_per_token[dom] * tokens_per_launch / (tot_ms / launches * 1e-3) if launches else 0.0
-    # HBM bytes per token of k_mlp<256,false>, from two rocprofv3 --pmc runs at 2048 members x 256 tokens per launch
-    # (FETCH_SIZE 260,192 KiB x 2.0, WRITE_SIZE 311,756 KiB x 1.0 per launch; the factors are what the same counters read
-    # for a plain 256 MiB elementwise copy in the same run: 131,091 KiB fetched, 262,144 KiB written); the kernel's
-    # traffic is per token, so a launch moves that figure times its tokens
-    traffic_per_token = (260192 * 2.0 + 311756 * 1.0) * 1024 / (2048 * 256)
-    traffic = traffic_per_token * tokens_per_launch if (dom == "mlp" and H == 256) else None
+    # HBM bytes per launch of the dominant kernel: read from the committed counter summary (two rocprofv3 --pmc runs,
+    # FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for a plain copy of known
+    # size), and only if that summary was taken at this run's launch shape; otherwise absent
+    traffic = None
+    if dom == "mlp":
+        traffic = profiled_traffic(os.path.join(ROOT, "profiles", "k_mlp_c4_hbm_traffic.txt"), f"k_mlp<{H},false>", chunk, T)
     roofline = {"kernel": "k_" + dom, "bound": "mfma", "achieved": achieved / 1e12, "peak": PEAK_INT8_OPS / 1e12,
                 "unit": "TOP/s", "frac": achieved / PEAK_INT8_OPS, "traffic": traffic,
                 "avg_launch_ms": tot_ms / launches if launches else None, "launches": launches}
@@ -125,20 +167,23 @@ def main():
                                       "GB/s": bytes_per_token[k] * tok / sec / 1e9,
                                       "frac_hbm": bytes_per_token[k] * tok / sec / PEAK_HBM}
 
+    side = not args.headline_only
     # ---- for comparison: the same eager steps with the block in front of the first attention layer evaluated at every
     # position instead of once per distinct byte value of a window (identical results, more work on repetitive data)
-    ctx.first_block_dedup(False)
-    s2 = run_steps(1, 1000, seed, False)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_steps(args.steps, 1001, s2, False)
-    torch.cuda.synchronize()
-    per_position_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ctx.first_block_dedup(True)
+    per_position_ms = None
+    if side:
+        ctx.first_block_dedup(False)
+        s2 = run_steps(1, 1000, seed, False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(args.steps, 1001, s2, False)
+        torch.cuda.synchronize()
+        per_position_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        ctx.first_block_dedup(True)
 
     # ---- the same steps replayed as one captured hipGraph per step
     graph_ms = None
-    if not args.no_graph:
+    if not args.no_graph and side:
         ctx.step_capture(d_data.data_ptr(), n)
         seed = run_steps(1, args.warmup + args.steps, seed, True)
         torch.cuda.synchronize()
@@ -154,31 +199,40 @@ def main():
         torch.cuda.synchronize()
         del a, b
 
-    # ---- perturbed-linear microbenchmark (P=8192, T=128, K=N=512), int32 output
+    # ---- perturbed-linear microbenchmark (8192 members x 128 tokens, K = N = 512): the reference's indexing (one noise
+    # vector pair per antithetic pair of members), every member with noise of its own, the shared-weight product alone
+    # (no rank-1 term: the reference's ns == 0 case), each with int8 and with int32 results; then the int8 legs again on
+    # the W-streaming kernels (the W-stationary kernel is the default for this shape)
     mb = {}
     try:
+        if not side:
+            raise RuntimeError("skipped (--headline-only)")
         members, Tm, K, N = 8192, 128, 512, 512
         X = torch.randint(-127, 128, (members * Tm, K), dtype=torch.int8, device=dev)
         W = torch.randint(-127, 128, (K * N,), dtype=torch.int8, device=dev)
         Y = torch.empty((members * Tm, N), dtype=torch.int32, device=dev)
         Y8 = torch.empty((members * Tm, N), dtype=torch.int8, device=dev)
-        # the last leg is the shared-weight GEMM alone (no rank-1 term: the reference's ns == 0 case)
-        for name, y32, y8, bytes_row in (("int32_out", Y.data_ptr(), None, K + 4 * N), ("int8_out", None, Y8.data_ptr(), K + N),
-                                         ("int8_out_shared_gemm_only", None, Y8.data_ptr(), K + N)):
-            if name.endswith("only"):
-                run = lambda: ctx.shared_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 8, y32, y8)
-            else:
-                run = lambda: ctx.perturbed_linear(X.data_ptr(), W.data_ptr(), members, Tm, K, N, 3, 200, 201, 8, y32, y8)
-            run()
+        xp, wp = X.data_ptr(), W.data_ptr()
+        forms = {"pair_noise": lambda y32, y8: ctx.perturbed_linear(xp, wp, members, Tm, K, N, 3, 200, 201, 8, y32, y8),
+                 "own_noise": lambda y32, y8: ctx.perturbed_linear_own_noise(xp, wp, members, Tm, K, N, 3, 200, 201, 8, y32, y8),
+                 "shared_gemm_only": lambda y32, y8: ctx.shared_linear(xp, wp, members, Tm, K, N, 8, y32, y8)}
+        legs = [(f"{out}_out_{form}", form, out, True) for out in ("int8", "int32") for form in forms]
+        legs += [(f"int8_out_{form}_w_streaming", form, "int8", False) for form in forms]
+        for name, form, out, ws in legs:
+            ctx.linear_kernel(ws)
+            y32, y8, bytes_row = (Y.data_ptr(), None, K + 4 * N) if out == "int32" else (None, Y8.data_ptr(), K + N)
+            forms[form](y32, y8)
             ctx.enable_timing(True); ctx.timing_reset()
             for _ in range(5):
-                run()
+                forms[form](y32, y8)
             nl, ms = ctx.timing()["plinear"]
             ctx.enable_timing(False)
             sec = ms / nl * 1e-3
             mb[name] = {"ms": ms / nl, "TOP/s": 2.0 * K * N * members * Tm / sec / 1e12,
                         "frac_mfma": 2.0 * K * N * members * Tm / sec / PEAK_INT8_OPS,
-                        "GB/s": bytes_row * members * Tm / sec / 1e9, "frac_hbm": bytes_row * members * Tm / sec / PEAK_HBM}
+                        "GB/s": bytes_row * members * Tm / sec / 1e9, "frac_hbm": bytes_row * members * Tm / sec / PEAK_HBM,
+                        "kernel": "k_plinear_ws (W stationary in registers)" if ws else "k_plinear2 (W streamed through LDS)"}
+        ctx.linear_kernel(True)
         del X, W, Y, Y8
     except Exception as e:   # the microbenchmark must not take the headline down
         mb = {"error": str(e)}
@@ -186,6 +240,8 @@ def main():
     # ---- the reference's CPU configuration (full_trained_egg.c defaults: GRU H=512 L=4 T=4096 P=128) on the GPU
     gru = None
     try:
+        if not side:
+            raise RuntimeError("skipped (--headline-only)")
         gcfg = pkg.gru_default_config()
         gctx = pkg.GruContext(gcfg)
         gctx.model_init(42)
@@ -204,6 +260,8 @@ def main():
     # ---- the d-eggs-style shape (hidden 512, 8 heads, seq 512, 8 layers, Muon) on one chunk of 2048 members
     c5 = None
     try:
+        if not side:
+            raise RuntimeError("skipped (--headline-only)")
         P5 = 2048
         c5ctx = pkg.Context(pkg.default_config(hidden=512, head_dim=64, n_layers=8, seq_len=512, population=P5, use_muon=1,
                                                weight_limit=1))
@@ -246,6 +304,8 @@ def main():
     # ---- the headline model with the d-eggs adaptive noise overlay on (fractional factors everywhere), one chunk
     adaptive = None
     try:
+        if not side:
+            raise RuntimeError("skipped (--headline-only)")
         PA = min(P, 2048)
         actx = pkg.Context(pkg.default_config(**dict(kw, population=PA)))
         actx.set_stream(stream.cuda_stream)
@@ -264,33 +324,38 @@ def main():
     except Exception as e:
         adaptive = {"error": str(e)}
 
-    # ---- CPU baseline: the oracle's restatement of the same forward on a bounded sample of members
+    # ---- CPU baseline: the oracle's scalar/OpenMP restatement of the reference's CPU program (full_trained_egg.c: GRU
+    # language model, H=512, L=4, T=4096, population 128) on a bounded sample of its pairs, and of the benchmarked
+    # transformer forward on a bounded sample of its members
     cpu = None
-    cpu_ref_path = None
-    if not args.no_cpu:
+    if not args.no_cpu and side:
         threads = orc.lib().orc_num_threads()
+        host = host_cpu()
+        g = orc.gru_config()                    # the compiled-in defaults, seq_len 4096
+        gm = orc.gru_init_model(g, 42)
+        states = np.zeros(g.population * g.n_layers * g.hidden, np.int8)
+        npairs = min(g.population // 2, max(threads, 16))
+        t0 = time.perf_counter()
+        orc.gru_population(g, gm, data, 0, 42, 0, npairs, states)
+        sec = time.perf_counter() - t0
+        cpu = {"value": 2 * npairs * g.seq_len / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
+               "cpu_model": host["model"], "physical_cores": host["physical_cores"], "hardware_threads": host["hardware_threads"],
+               "sample": f"full_trained_egg.c at its defaults (GRU H={g.hidden} L={g.n_layers} T={g.seq_len}), forward of {npairs} of "
+                         f"{g.population // 2} pairs x {g.seq_len} tokens, scalar C++/OpenMP oracle on {threads} threads, {sec:.1f}s"}
         ocfg = orc.config(**kw)
         model = orc.init_model(ocfg, 42)
         sample = 16 * threads
         t0 = time.perf_counter()
         orc.population_forward(ocfg, model, data, 0, 42, 0, sample)
         sec = time.perf_counter() - t0
-        cpu = {"value": sample * T / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
-               "sample": f"forward only of {sample} of {P} members (T={T}) of the same model, scalar C++/OpenMP oracle, {sec:.1f}s"}
-        # the reference's CPU program (full_trained_egg.c: GRU LM, H=512, L=4, P=128), scalar/OpenMP restatement
-        g = orc.gru_config(seq_len=2048)
-        gm = orc.gru_init_model(g, 42)
-        states = np.zeros(g.population * g.n_layers * g.hidden, np.int8)
-        npairs = min(64, 2 * threads)
-        t0 = time.perf_counter()
-        orc.gru_population(g, gm, data, 0, 42, 0, npairs, states)
-        sec = time.perf_counter() - t0
-        cpu_ref_path = {"value": 2 * npairs * g.seq_len / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
-                        "sample": f"full_trained_egg.c defaults (GRU H=512 L=4), forward of {npairs} pairs x {g.seq_len} tokens, {sec:.1f}s"}
+        cpu["transformer_forward"] = {"value": sample * T / sec, "unit": "member-tokens/s", "cores": threads, "kind": "port",
+                                      "sample": f"forward only of {sample} of {P} members (T={T}) of the benchmarked model, scalar C++/OpenMP oracle, {sec:.1f}s"}
 
     # ---- what HBM rate a plain copy / fill reaches on this box (torch elementwise kernels, 1 GiB each way)
     hbm = None
     try:
+        if not side:
+            raise RuntimeError("skipped (--headline-only)")
         n = 1 << 30
         a = torch.empty(n, dtype=torch.int8, device=dev); b = torch.empty_like(a)
         a.fill_(1); b.copy_(a); torch.cuda.synchronize()
@@ -305,15 +370,16 @@ def main():
         hbm = {"copy_GBs": 5 * 2 * n / (e0.elapsed_time(e1) * 1e-3) / 1e9, "fill_GBs": 5 * n / (e1.elapsed_time(e2) * 1e-3) / 1e9,
                "note": "read + write bytes of a 1 GiB device-to-device copy, and bytes of a 1 GiB fill, per second"}
         del a, b
-        if isinstance(mb, dict) and "int32_out" in mb:
-            mb["int32_out"]["frac_of_measured_copy_rate"] = mb["int32_out"]["GB/s"] / hbm["copy_GBs"]
+        for k in mb if isinstance(mb, dict) else ():
+            if k.startswith("int32_out"):
+                mb[k]["frac_of_measured_copy_rate"] = mb[k]["GB/s"] / hbm["copy_GBs"]
     except Exception as e:
         hbm = {"error": str(e)}
 
     # ---- what MFMA rate the GPU sustains on this box (child process: a bare loop of int8 MFMAs on register operands)
     sustained = None
     probe = os.path.join(ROOT, "egg.c_amd", "mfma_probe")
-    if os.path.exists(probe):
+    if os.path.exists(probe) and side:
         try:
             import subprocess
             torch.cuda.synchronize()
@@ -340,7 +406,7 @@ def main():
                    "distinct_bytes_per_window": round(distinct, 1),
                    "ms_per_step_first_block_at_every_position": per_position_ms},
         "roofline": roofline, "kernel_rooflines": kernel_rooflines, "mfma_sustained": sustained, "hbm_sustained": hbm, "kernels": per_class, "microbench_c2": mb,
-        "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu, "cpu_reference_path": cpu_ref_path,
+        "gru_c1_gpu": gru, "c5_shape_gpu": c5, "adaptive_overlay_gpu": adaptive, "cpu_baseline": cpu,
     }
     print(json.dumps(out))
     ctx.close()

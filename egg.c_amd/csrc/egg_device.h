@@ -67,8 +67,9 @@ __device__ __forceinline__ long long other_half64(long long v) {
 __device__ __forceinline__ int col_of(int nt, int r, int g) { return nt * 32 + ((r >> 2) << 3) + (g << 2) + (r & 3); }
 
 __device__ __forceinline__ int sx8(int packed, int e) { return (int)(int8_t)(packed >> (8 * e)); }
+// bytes 0 of four values side by side: two byte permutes and an or
 __device__ __forceinline__ int pack4(int a, int b, int c, int d) {
-    return (a & 255) | ((b & 255) << 8) | ((c & 255) << 16) | ((d & 255) << 24);
+    return (int)(__builtin_amdgcn_perm((unsigned)b, (unsigned)a, 0x0c0c0400u) | __builtin_amdgcn_perm((unsigned)d, (unsigned)c, 0x04000c0cu));
 }
 // dot of 4 signed bytes
 __device__ __forceinline__ int dot4(int a, int b, int c) {

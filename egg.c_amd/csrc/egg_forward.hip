@@ -332,8 +332,10 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
 #pragma unroll
                 for (int nt = 0; nt < NTS; nt++) store_op(p.x_mid + row + col0, nt, g, xs[nt]);
         }
-        // park the residual (this wave owns the slice; invalid padding waves only recompute)
-        if (valid)
+        // park the residual (this wave owns the slice; invalid padding waves only recompute, and so do the rows of the
+        // value table beyond the number of distinct values: nothing reads them, so nothing of them is written)
+        const bool keep = valid && (!(FIRST && dedup) || t < nrows);
+        if (keep)
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, g, xs[nt]);
 
@@ -453,7 +455,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         const int mx2 = xreduce<CS, true>(absmax_groups<NTS>(accd), red + 3 * M::SITE, tm, lane);
         v4i xnew[NTS];
         adaptive_scale<NTS>(accd, mx2, xnew);
-        if (valid)
+        if (keep)
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, g, xnew[nt]);
     }
@@ -628,17 +630,34 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
 // context positions are regrouped with byte permutes instead of shifts and masks; the sum of the weights is rebuilt
 // from per-plane byte sums.  Only the diagonal tile needs the causal mask.
 // den[pl] accumulates the plane sums; the sum of the weights is den[0] + 128 den[1] + 16384 den[2] (attn_den).
-__device__ __forceinline__ void attn_weights(const v16i &s, const int *lut, int mxs, int shift, bool diag, int ct, int t, int g,
+// `last4` is four times the last table index a lookup may use: the index of the first entry from which the table is zero to
+// its end (255 if the last entry is not zero).  Indices beyond it would read zeros anyway, and sending them all to one
+// entry turns most of a wave's gather into a broadcast instead of a spread over the LDS banks.  `mxs4` is four times
+// the shifted maximum: the byte offset 4 * (mxs - (s >> shift)) is one 24-bit multiply-add away from the shifted score.
+__device__ __forceinline__ int attn_lut_last4(const int32_t *exp_lut, int *spare, int wave, int lane) {
+    // last nonzero entry over the 256 threads of the workgroup (every thread looks at its own entry)
+    const unsigned long long nz = __ballot(exp_lut[threadIdx.x & 255] != 0);
+    if (lane == 0) spare[wave] = nz ? 64 * wave + 63 - __builtin_clzll(nz) : -1;
+    __syncthreads();
+    int last = -1;
+#pragma unroll
+    for (int w = 0; w < EGG_WAVES; w++) last = max(last, spare[w]);
+    return 4 * min(last + 1, 255);
+}
+__device__ __forceinline__ void attn_weights(const v16i &s, const int *lut, int mxs4, int last4, int shift, bool diag, int ct, int t, int g,
                                              v4i *pw, int *den) {
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         int pk[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            int idx = mxs - (s[4 * q + e] >> shift);
-            idx = min(255, max(0, idx));
-            pk[e] = lut[idx];
-            if (diag && (32 * ct + 8 * q + 4 * g + e) > t) pk[e] = 0;
+            // spelt out: the compiler turns the multiply into a shift and a subtraction and the clamp into two instructions
+            int off;
+            asm("v_mad_i32_i24 %0, %1, -4, %2\n\tv_med3_i32 %0, %0, 0, %3" : "=&v"(off) : "v"(s[4 * q + e] >> shift), "v"(mxs4), "v"(last4));
+            pk[e] = *reinterpret_cast<const int *>(reinterpret_cast<const int8_t *>(lut) + off);
+            // on the diagonal tile (ct == t / 32) the position 32 ct + 8q + 4g + e lies behind the query's when 8q + 4g + e > t % 32,
+            // which depends on the lane and the register only
+            if (diag && (8 * q + 4 * g + e) > (t & 31)) pk[e] = 0;
         }
         // bytes of pk[e]: plane0, plane1, plane2, 0  ->  one dword per plane holding the four positions
         const int ab_lo = __builtin_amdgcn_perm(pk[1], pk[0], 0x05010400);   // a0 b0 a1 b1
@@ -676,6 +695,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
         const int w = c.exp_lut[i];
         lut[i] = (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16);
     }
+    const int last4 = attn_lut_last4(c.exp_lut, lut + 256, wave, lane);
     // All three row sets of this (member, head) are requested at once, so the wave waits for global memory once: the K
     // rows stay in registers until the V rows have left the row area, the Q rows go to LDS in the K rows' layout
     // (chunk c of row r at c ^ ((r / RPL) % CH), see below), the V rows to LDS rows [ctx][HD].
@@ -784,8 +804,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                     s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qop[ks], s, 0, 0, 0);
                 }
                 v4i pw[3];
-                if (ct == qt) attn_weights(s, lut, mxs, c.shift_attn, true, ct, t, g, pw, dpl);
-                else attn_weights(s, lut, mxs, c.shift_attn, false, ct, t, g, pw, dpl);
+                if (ct == qt) attn_weights(s, lut, 4 * mxs, last4, c.shift_attn, true, ct, t, g, pw, dpl);
+                else attn_weights(s, lut, 4 * mxs, last4, c.shift_attn, false, ct, t, g, pw, dpl);
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -854,6 +874,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
         const int w = c.exp_lut[i];
         lut[i] = (w & 127) | (((w >> 7) & 127) << 8) | ((w >> 14) << 16);
     }
+    const int last4 = attn_lut_last4(c.exp_lut, lut + 256, wave, lane);
     // the K rows are requested now and held in registers until the V rows have left the shared row area, so that their
     // latency overlaps the V stage instead of following it
     constexpr int PER = T * CH / EGG_THREADS;
@@ -947,38 +968,44 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
             }
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                int cx = 32 * qt + ((r >> 2) << 3) + (g << 2) + (r & 3);
-                if (cx <= t) mx = max(mx, s[r]);
+                const int cx = ((r >> 2) << 3) + (g << 2) + (r & 3);      // position within the diagonal tile
+                if (cx <= j) mx = max(mx, s[r]);
             }
         }
         mx = max(mx, other_half(mx));
         const int mxs = mx >> c.shift_attn;
-        // pass 2: weights and weighted V sum (mgpu.cu:810-824)
+        // pass 2: weights and weighted V sum (mgpu.cu:810-824).  The first tile weighed starts the accumulators (a zero C
+        // operand instead of 96 cleared registers); the scores of the next tile are in flight while a tile is weighed.
         v16i o[3][DT];
-#pragma unroll
-        for (int pl = 0; pl < 3; pl++) zero_acc<DT>(o[pl]);
         int dpl[3] = {0, 0, 0};
-        auto weigh_tile = [&](const v16i &s, int ct, bool diag) {
+        const int mxs4 = 4 * mxs;
+        auto weigh_tile = [&](const v16i &s, int ct, bool diag, bool first) {      // diag and first are constants at every call
             v4i pw[3];
-            attn_weights(s, lut, mxs, c.shift_attn, diag, ct, t, g, pw, dpl);
+            attn_weights(s, lut, mxs4, last4, c.shift_attn, diag, ct, t, g, pw, dpl);
+            v16i z;
+#pragma unroll
+            for (int r = 0; r < 16; r++) z[r] = 0;
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
                 const v4i vt = *reinterpret_cast<const v4i *>(vfrag + ((size_t)(ct * DT + dt) * 64 + lane) * 16);
 #pragma unroll
-                for (int pl = 0; pl < 3; pl++) o[pl][dt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vt, pw[pl], o[pl][dt], 0, 0, 0);
+                for (int pl = 0; pl < 3; pl++) o[pl][dt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vt, pw[pl], first ? z : o[pl][dt], 0, 0, 0);
             }
             __builtin_amdgcn_s_setprio(0);
         };
         {
-            v16i s = score_tile(0, qop);
-#pragma unroll 2
+            // integer sums do not depend on the order: the diagonal tile goes first and starts the accumulators
+            v16i s = score_tile(qt, qop);
+            v16i sn = score_tile(0, qop);
+            weigh_tile(s, qt, true, true);
+            s = sn;
+#pragma unroll 1
             for (int ct = 0; ct < qt; ct++) {
-                const v16i sn = score_tile(ct + 1, qop);
-                weigh_tile(s, ct, false);
+                sn = score_tile(ct + 1 < qt ? ct + 1 : ct, qop);       // (the last one is not used)
+                weigh_tile(s, ct, false, false);
                 s = sn;
             }
-            weigh_tile(s, qt, true);
         }
         int den = attn_den(dpl);
         den += other_half(den);

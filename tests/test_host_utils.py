@@ -74,6 +74,43 @@ def test_shape_fitness_cases(pkg):
         pkg.shape_fitness(np.zeros(3, np.int32))
 
 
+def test_shape_fitness_properties_on_random_chunks(pkg):
+    """What the rule's definition fixes on random chunks (d-eggs/src/worker.cu:636-687): swapping the members of every
+    pair negates every vote, a larger alpha only turns votes into zeros and never flips one, the plain rule is the
+    sign of n - p, the filter moves every difference by the same truncated amount, and a vectorised numpy evaluation of
+    the same three steps agrees."""
+    rng = np.random.default_rng(77)
+    for trial in range(40):
+        pairs = int(rng.integers(1, 400))
+        spread = int(rng.choice([3, 50, 5000, 2_000_000]))
+        loss = rng.integers(100_000, 100_000 + spread, 2 * pairs).astype(np.int32)
+        if trial % 5 == 0:
+            loss[1::2] += int(rng.integers(-spread, spread + 1))          # a chunk-wide bias: the filter has something to add
+        swapped = loss.reshape(-1, 2)[:, ::-1].reshape(-1).copy()
+        p, n = loss[0::2].astype(np.int64), loss[1::2].astype(np.int64)
+        plain, total = pkg.shape_fitness(loss, chunk_mean_filter=False, adaptive_threshold=False)
+        assert np.array_equal(plain, np.sign(n - p)) and total == int(loss.astype(np.int64).sum())
+        for filt in (False, True):
+            exponent = float(rng.choice([1.0, 1.2, 0.5]))
+            mean = float((n - p).sum()) / pairs
+            shift = int(np.trunc(np.sign(mean) * abs(mean) ** exponent)) if filt else 0
+            d = n - p + shift
+            nofilter_votes, _ = pkg.shape_fitness(loss, chunk_mean_filter=filt, mean_exponent=exponent, adaptive_threshold=False)
+            assert np.array_equal(nofilter_votes, np.sign(d)), (trial, filt)
+            prev_zero = np.zeros(pairs, bool)
+            for alpha in (0.0, 0.05, 0.1, 0.5, 1.0, 3.0):
+                fit, _ = pkg.shape_fitness(loss, chunk_mean_filter=filt, mean_exponent=exponent, adaptive_threshold=True, alpha=alpha)
+                thr = np.abs(d).astype(np.float64).sum() / pairs * alpha
+                want = np.where(np.abs(d) < thr, 0, np.where(d > 0, 1, -1))
+                assert np.array_equal(fit, want), (trial, filt, alpha)
+                zero = fit == 0
+                assert np.all(zero | ~prev_zero)                              # zeros only grow with alpha
+                assert np.all((fit == nofilter_votes) | zero | (d == 0))      # a vote is never flipped (d == 0 votes -1 in this branch)
+                prev_zero = zero
+                back, _ = pkg.shape_fitness(swapped, chunk_mean_filter=filt, mean_exponent=exponent, adaptive_threshold=True, alpha=alpha)
+                assert np.array_equal(back[d != 0], -fit[d != 0]), (trial, filt, alpha)
+
+
 def test_eggc_checkpoints_interoperate_with_reference_header(pkg, orc, tmp_path):
     ref = orc.ref()
     d = str(tmp_path / "ckpt")
