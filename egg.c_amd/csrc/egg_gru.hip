@@ -473,7 +473,7 @@ extern "C" int egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out) {
     }
     add(ctx->off_head, (int)V, (int)H, 999, 8);
     ctx->noise_bytes = no; ctx->panel_bytes = po;
-    auto bail = [&](const char *what, hipError_t e) { fprintf(stderr, "egg_gru_create: %s: %s\n", what, hipGetErrorString(e)); delete ctx; return EGG_E_HIP; };
+    auto bail = [&](const char *what, hipError_t e) { fprintf(stderr, "egg_gru_create: %s: %s\n", what, hipGetErrorString(e)); egg_gru_destroy(ctx); return EGG_E_HIP; };   // frees what was allocated so far
 #define CR(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) return bail(#call, e_); } while (0)
     CR(hipStreamCreate(&ctx->stream));
     switch (c.hidden) {
@@ -546,8 +546,9 @@ extern "C" int egg_gru_state_reset(egg_gru_ctx *ctx) {
     return EGG_OK;
 }
 extern "C" int egg_gru_state_download(egg_gru_ctx *ctx, void *h, size_t bytes) {
-    size_t want = (size_t)ctx->cfg.population * ctx->cfg.n_layers * ctx->cfg.hidden;
-    if (!ctx || !h || bytes != want) return gfail(ctx, EGG_E_INVALID, "state size mismatch");
+    if (!ctx) return EGG_E_INVALID;
+    const size_t want = (size_t)ctx->cfg.population * ctx->cfg.n_layers * ctx->cfg.hidden;
+    if (!h || bytes != want) return gfail(ctx, EGG_E_INVALID, "state size mismatch");
     GTRY(hipStreamSynchronize(ctx->stream));
     GTRY(hipMemcpy(h, ctx->d_states, want, hipMemcpyDeviceToHost));
     return EGG_OK;
