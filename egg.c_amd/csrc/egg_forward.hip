@@ -630,6 +630,14 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
 // context positions are regrouped with byte permutes instead of shifts and masks; the sum of the weights is rebuilt
 // from per-plane byte sums.  Only the diagonal tile needs the causal mask.
 // den[pl] accumulates the plane sums; the sum of the weights is den[0] + 128 den[1] + 16384 den[2] (attn_den).
+// Workgroups go to the eight XCDs (each with an L2 of its own) in turn: block b runs on XCD b % 8.  The heads of a member
+// read 64-byte (or 32-byte) pieces of the same 128-byte lines of its Q, K and V rows, so they should meet in one L2: the
+// blocks of one XCD, in launch order, take consecutive (member, head) units.  Needs a grid that is a multiple of eight;
+// any other grid keeps the plain order.
+__device__ __forceinline__ int xcd_contiguous_unit(int block, int nblocks) {
+    if (nblocks & 7) return block;
+    return (block & 7) * (nblocks >> 3) + (block >> 3);
+}
 // `last4` is four times the last table index a lookup may use: the index of the first entry from which the table is zero to
 // its end (255 if the last entry is not zero).  Indices beyond it would read zeros anyway, and sending them all to one
 // entry turns most of a wave's gather into a broadcast instead of a spread over the LDS banks.  `mxs4` is four times
@@ -866,7 +874,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const FwdCommon &c = p.c;
     const int H = c.H, NH = H / HD;
-    const int unit = blockIdx.x;                                   // grid = n_members * heads exactly
+    const int unit = xcd_contiguous_unit(blockIdx.x, gridDim.x);   // grid = n_members * heads exactly
     const int mloc = unit / NH, h = unit % NH;
     const size_t base = (size_t)mloc * T * H + (size_t)h * HD;
 
