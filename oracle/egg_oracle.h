@@ -18,8 +18,17 @@
  *       host-compilable header (d-eggs/include/utils/egg_math.h) compiled
  *       into oracle/_ref, plus known answers committed under tests/golden.
  *   EXP / GELU / RoPE / EXP2 tables : closed forms + reference screenshot values.
- *   perturbed linear, norms, attention, loss, fitness, vote, AdamW : brute
+ *   seed offsets, shifts, defaults, model blob layout, optimizer-state layout,
+ *       Muon flags : the reference's own config.h / definitions.h / base.h,
+ *       compiled in place at four configurations (oracle/ref_layout_shim.cpp),
+ *       plus the values committed under tests/golden (tests/test_reference_headers.py).
+ *   perturbed linear, norms, attention, loss, fitness, vote : brute
  *       force and special cases in tests/test_oracle_*.py.
+ *   vector / matrix AdamW updates, Muon momentum + gather + apply rule : bitwise
+ *       numpy evaluations of their definitions (tests/test_oracle_pins.py).
+ *   d-eggs sampler (oracle_py.sample_token_deggs) : closed forms only (neutral
+ *       settings = the plain sampler, temperature 2 = halved differences, min-p
+ *       edge, penalty per occurrence); the reference holds no fixture for it.
  *   Muon Newton-Schulz : fp64 restatement + orthogonality invariants; the
  *       reference's cuBLAS summation order is unspecified => tolerance only.
  *   whole forward : no reference golden vectors exist, so its composition is
