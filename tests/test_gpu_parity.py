@@ -427,6 +427,35 @@ def test_fifty_graph_steps_follow_the_oracle_trajectory(pkg, orc, dev):
     ctx.close()
 
 
+def test_muon_step_graph_replays_equal_eager_steps(pkg, orc, dev):
+    """The whole step with the Muon update (momentum, batched Newton-Schulz, apply rule) captured once and replayed:
+    every replay leaves the weights, the optimizer state, the losses and the update count of the same step run eagerly
+    on a second context, with eager work and synchronisation between the replays."""
+    import torch
+    kw = dict(hidden=128, head_dim=32, n_layers=2, seq_len=32, population=64, use_muon=1)
+    data = orc.zipf_bytes(1 << 16)
+    d_data = _t(dev, data)
+    g, e = pkg.Context(pkg.default_config(**kw)), pkg.Context(pkg.default_config(**kw))
+    g.model_init(42); e.model_init(42)
+    g.step_capture(d_data.data_ptr(), len(data))
+    seed, moved = 4242, False
+    start_model = e.model_download()
+    for step in range(8):
+        lr, start = 30.0, step * kw["seq_len"]
+        g.step_launch(start, seed, lr)
+        e.step(d_data.data_ptr(), len(data), start, seed, lr)
+        # unrelated eager work on the card between the replays
+        junk = torch.randn(1 << 16, device=dev); junk = (junk * junk).sum().item()
+        gl, gf = g.step_losses(); el, ef = e.step_losses()
+        assert np.array_equal(gl, el) and np.array_equal(gf, ef), step
+        assert np.array_equal(g.model_download(), e.model_download()), f"weights differ after replay {step}"
+        assert g.opt_state_download().tobytes() == e.opt_state_download().tobytes(), f"optimizer state differs after replay {step}"
+        assert g.last_update_count() == e.last_update_count(), step
+        seed = pkg.next_seed(seed, step + 1)
+    assert not np.array_equal(e.model_download(), start_model)
+    g.close(); e.close()
+
+
 def test_error_paths(pkg, dev):
     with pytest.raises(pkg.EggError):
         pkg.Context(pkg.default_config(hidden=100))
