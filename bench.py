@@ -83,7 +83,7 @@ def main():
     import torch
     import __graft_entry__ as entry
     pkg = entry.load_package()
-    orc = entry.load_oracle()          # only for the synthetic data generator and the cpu_baseline leg
+    orc = entry.load_oracle()          # only for the cpu_baseline leg
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
 
@@ -97,7 +97,7 @@ def main():
     torch.cuda.set_stream(stream)
     ctx.set_stream(stream.cuda_stream)
     ctx.model_init(42)
-    data = orc.zipf_bytes(args.data_mib << 20, seed=1234)
+    data = pkg.zipf_bytes(args.data_mib << 20, seed=1234)
     d_data = torch.from_numpy(data).to(dev)
     n = len(data)
     # the block in front of the first attention layer is evaluated once per distinct byte value of a member's window

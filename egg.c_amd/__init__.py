@@ -51,7 +51,7 @@ EXPORTS = [
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
-    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_newton_schulz_static",
+    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_muon_plan", "egg_newton_schulz_static",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
     "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
     "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
@@ -141,6 +141,7 @@ def lib():
         L.egg_opt_state_bytes.restype = i64
         L.egg_opt_state_bytes.argtypes = [vp]
         L.egg_describe_layout.argtypes = [vp, i32, vp, vp, vp, vp]
+        L.egg_muon_plan.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp]
         L.egg_newton_schulz_static.argtypes = [vp, i32, i32, i32, vp]
         L.egg_tensor_state_offset.restype = i64
         L.egg_tensor_state_offset.argtypes = [vp, i32]
@@ -189,6 +190,20 @@ def describe_layout(cfg):
                         off_a=t.off_a, off_b=t.off_b, seed_base=t.seed_base, lr_scale=t.lr_scale, muon=t.muon,
                         state_offset=int(so.value)))
     return out, int(mb.value), int(sb.value)
+
+
+def muon_plan(cfg):
+    """Host-only: (groups, matrix_buffer_floats, term_buffer_floats); a group is a dict rows / cols / members / batch."""
+    a, b = C.c_int64(), C.c_int64()
+    n = lib().egg_muon_plan(C.byref(cfg), -1, None, None, None, None, C.byref(a), C.byref(b))
+    if n < 0:
+        raise EggError("egg_muon_plan: invalid configuration")
+    groups = []
+    for g in range(n):
+        r, c, m, bt = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+        lib().egg_muon_plan(C.byref(cfg), g, C.byref(r), C.byref(c), C.byref(m), C.byref(bt), None, None)
+        groups.append(dict(rows=r.value, cols=c.value, members=m.value, batch=bt.value))
+    return groups, int(a.value), int(b.value)
 
 
 def newton_schulz_static(d_x, rows, cols, iters=5, stream=None):
@@ -486,6 +501,33 @@ def eggc_load_latest(directory):
     if rc:
         return None
     return step.value, seed.value, buf[:n.value].copy()
+
+
+def zipf_bytes(n, seed=1234, s=1.1):
+    """Synthetic byte stream for benchmarks: i.i.d. Zipf(s) ranks over a fixed permutation of the 256 byte values.
+    Counter-based SplitMix64 -> inverse CDF (so any slice can be regenerated independently)."""
+    import numpy as _np
+    idx = _np.arange(1, n + 1, dtype=_np.uint64)
+    with _np.errstate(over="ignore"):
+        z = _np.uint64(seed) + idx * _np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> _np.uint64(30))) * _np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> _np.uint64(27))) * _np.uint64(0x94D049BB133111EB)
+        z = z ^ (z >> _np.uint64(31))
+    u = (z >> _np.uint64(11)).astype(_np.float64) * (1.0 / 9007199254740992.0)
+    w = 1.0 / _np.arange(1, 257, dtype=_np.float64) ** s
+    cdf = _np.cumsum(w) / _np.sum(w)
+    rank = _np.minimum(_np.searchsorted(cdf, u, side="right"), 255)
+    # fixed permutation of byte values from the same generator (Fisher-Yates with xorshift32)
+    perm = _np.arange(256, dtype=_np.uint8)
+    st = _np.uint32((seed * 2654435761 + 1) & 0xFFFFFFFF) or _np.uint32(1)
+    st = int(st)
+    for i in range(255, 0, -1):
+        st ^= (st << 13) & 0xFFFFFFFF
+        st ^= st >> 17
+        st ^= (st << 5) & 0xFFFFFFFF
+        j = st % (i + 1)
+        perm[i], perm[j] = perm[j], perm[i]
+    return perm[rank].astype(_np.uint8)
 
 
 def learning_rate(step):

@@ -45,7 +45,9 @@ struct egg_ctx {
     uint8_t *d_state = nullptr; int64_t state_bytes = 0; std::vector<int64_t> t_state_off;   // optimizer state (AdamModel layout)
     MuonWork muon = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     std::vector<std::vector<int>> muon_groups;    // ids of the Muon matrices, grouped by shape; a group runs Newton-Schulz as batches
-    int muon_batch_max = 1;                       // matrices the Muon workspace holds at once
+    std::vector<int> muon_group_batch;            // per group: matrices of that shape the Muon workspace holds at once
+    int muon_batch_max = 1;                       // the largest of them (sizes the per-matrix norm buffers)
+    size_t muon_elems = 0, muon_bterm = 0;        // floats in each of the two matrix buffers / in the 3I - G buffer
     int8_t *d_wfrag = nullptr;      // fragment-major copy of every matrix, same offsets as the model blob
     int8_t *d_plin_frag = nullptr; size_t plin_frag_bytes = 0;
     bool plin_no_ws = false;        // egg_ctx_linear_kernel: run the W-streaming kernels also where the W-stationary one exists
@@ -106,6 +108,12 @@ static void span_end(egg_ctx *ctx) {
     (void)hipEventRecord(ctx->spans[ctx->spans_used].b, ctx->stream);
     ctx->spans_used++;
 }
+// closes the span on every way out of a scope, error returns included
+struct SpanScope {
+    egg_ctx *ctx;
+    SpanScope(egg_ctx *c, int cls) : ctx(c) { span_begin(c, cls); }
+    ~SpanScope() { span_end(ctx); }
+};
 static void spans_collect(egg_ctx *ctx) {
     for (size_t i = 0; i < ctx->spans_used; i++) {
         float ms = 0.f;
@@ -178,6 +186,56 @@ static int64_t state_offsets(const egg_config &c, const std::vector<egg_tensor_i
     }
     return so;
 }
+// Muon workspace plan (host arithmetic only).  Matrices of one shape form a group and go through Newton-Schulz in
+// batches; a group's batch is as much of it as fits 16 Mi floats per matrix buffer, at least one matrix.  The
+// buffers hold the largest batch of any group: `elems` floats in each matrix buffer, `bterm` in the 3I - G buffer.
+struct MuonPlan { std::vector<std::vector<int>> groups; std::vector<int> batch; size_t elems = 0, bterm = 0; int batch_max = 1; };
+static MuonPlan muon_plan(const egg_config &c, const std::vector<egg_tensor_info> &tensors) {
+    MuonPlan pl;
+    for (int id = 0; id < (int)tensors.size(); id++) {
+        const egg_tensor_info &t = tensors[id];
+        if (!t.is_matrix || !t.muon) continue;
+        bool placed = false;
+        for (auto &g : pl.groups)
+            if (tensors[g[0]].rows == t.rows && tensors[g[0]].cols == t.cols) { g.push_back(id); placed = true; break; }
+        if (!placed) pl.groups.push_back(std::vector<int>(1, id));
+    }
+    // egg_update_tensor runs a single matrix of any Muon shape through the same buffers
+    const size_t mx = (size_t)4 * c.hidden * c.hidden;
+    size_t cap = (size_t)16 << 20;
+    if (cap < mx) cap = mx;
+    pl.elems = mx; pl.bterm = (size_t)c.hidden * c.hidden;
+    for (const auto &g : pl.groups) {
+        const egg_tensor_info &t = tensors[g[0]];
+        const size_t one = (size_t)t.rows * t.cols, k = (size_t)(t.rows < t.cols ? t.rows : t.cols);
+        size_t b = cap / one; if (b > g.size()) b = g.size(); if (b < 1) b = 1;
+        if (b * one > pl.elems) pl.elems = b * one;
+        if (b * k * k > pl.bterm) pl.bterm = b * k * k;
+        if ((int)b > pl.batch_max) pl.batch_max = (int)b;
+        pl.batch.push_back((int)b);
+    }
+    return pl;
+}
+// host-only: group `group` of the plan a context of this configuration would use (its shape, member count and batch
+// limit) and the workspace sizes in floats; returns the number of groups
+extern "C" int egg_muon_plan(const egg_config *cfg, int group, int *rows, int *cols, int *members, int *batch,
+                             int64_t *matrix_buffer_floats, int64_t *term_buffer_floats) {
+    if (!cfg || cfg->hidden < 4 || cfg->n_layers < 1 || cfg->vocab < 1) return EGG_E_INVALID;
+    const Layout L = make_layout(*cfg);
+    const std::vector<egg_tensor_info> tensors = build_tensor_table(*cfg, L);
+    const MuonPlan pl = muon_plan(*cfg, tensors);
+    if (matrix_buffer_floats) *matrix_buffer_floats = (int64_t)pl.elems;
+    if (term_buffer_floats) *term_buffer_floats = (int64_t)pl.bterm;
+    if (group < 0) return (int)pl.groups.size();
+    if (group >= (int)pl.groups.size()) return EGG_E_INVALID;
+    const egg_tensor_info &t = tensors[pl.groups[group][0]];
+    if (rows) *rows = t.rows;
+    if (cols) *cols = t.cols;
+    if (members) *members = (int)pl.groups[group].size();
+    if (batch) *batch = pl.batch[group];
+    return (int)pl.groups.size();
+}
+
 // host-only view of the same tables (no device is touched)
 extern "C" int egg_describe_layout(const egg_config *cfg, int tensor_id, egg_tensor_info *out, int64_t *state_offset,
                                    int64_t *model_bytes, int64_t *state_bytes) {
@@ -297,30 +355,12 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
         CR(hipMemcpy(ctx->d_vec_desc, vd.data(), vd.size() * sizeof(VecDesc), hipMemcpyHostToDevice));
     }
     if (c.use_muon) {
-        // Matrices of one shape go through Newton-Schulz together (one launch per stage for the whole batch).  The
-        // workspace holds the largest group, or as much of it as fits 16 Mi elements per buffer (and always one 4H x H).
-        for (int id = 0; id < (int)ctx->tensors.size(); id++) {
-            const egg_tensor_info &t = ctx->tensors[id];
-            if (!t.is_matrix || !t.muon) continue;
-            bool placed = false;
-            for (auto &g : ctx->muon_groups)
-                if (ctx->tensors[g[0]].rows == t.rows && ctx->tensors[g[0]].cols == t.cols) { g.push_back(id); placed = true; break; }
-            if (!placed) ctx->muon_groups.push_back(std::vector<int>(1, id));
-        }
-        size_t mx = (size_t)4 * c.hidden * c.hidden, cap = (size_t)16 << 20;
-        if (cap < mx) cap = mx;
-        size_t elems = mx, bt = (size_t)c.hidden * c.hidden; int nb = 1;
-        for (const auto &g : ctx->muon_groups) {
-            const egg_tensor_info &t = ctx->tensors[g[0]];
-            const size_t one = (size_t)t.rows * t.cols, k = (size_t)(t.rows < t.cols ? t.rows : t.cols);
-            size_t b = cap / one; if (b > g.size()) b = g.size(); if (b < 1) b = 1;
-            if (b * one > elems) elems = b * one;
-            if (b * k * k > bt) bt = b * k * k;
-            if ((int)b > nb) nb = (int)b;
-        }
-        ctx->muon_batch_max = nb;
-        CR(hipMalloc(&ctx->muon.x, elems * 4)); CR(hipMalloc(&ctx->muon.swap, elems * 4));
-        CR(hipMalloc(&ctx->muon.bterm, bt * 4));
+        const MuonPlan pl = muon_plan(c, ctx->tensors);
+        ctx->muon_groups = pl.groups; ctx->muon_group_batch = pl.batch; ctx->muon_batch_max = pl.batch_max;
+        ctx->muon_elems = pl.elems; ctx->muon_bterm = pl.bterm;
+        const int nb = pl.batch_max;
+        CR(hipMalloc(&ctx->muon.x, pl.elems * 4)); CR(hipMalloc(&ctx->muon.swap, pl.elems * 4));
+        CR(hipMalloc(&ctx->muon.bterm, pl.bterm * 4));
         CR(hipMalloc(&ctx->muon.partials, (size_t)nb * 256 * 4 + 1024 * 4)); CR(hipMalloc(&ctx->muon.norm, (size_t)nb * 4 + 16));
     }
     // activation workspace for one chunk of members
@@ -621,7 +661,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
             p.q_ln_w = Q + L.ln_init; p.q_ln_b = Q + L.ln_init_bias; p.q_b_up = Q + L.mlp_emb_bias_up; p.q_b_dn = Q + L.mlp_emb_bias_down;
             p.q_up = Q + L.w_emb_mlp_up; p.q_dn = Q + L.w_emb_mlp_down; p.q_emb = Q + L.embedding; p.q_emb_bias = Q + L.emb_bias;
         }
-        span_begin(ctx, EGG_K_MLP_FIRST); HIP_TRY(egg_launch_mlp(p, true, s)); span_end(ctx);
+        { SpanScope span(ctx, EGG_K_MLP_FIRST); HIP_TRY(egg_launch_mlp(p, true, s)); }
         if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 0), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
     }
     for (int l = 0; l < c.n_layers; l++) {
@@ -635,7 +675,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
                 p.q_ln_w = Q + L.ln_1 + (int64_t)l * H; p.q_ln_b = Q + L.ln_1_bias + (int64_t)l * H;
                 p.q_wq = Q + L.w_q + l * hh; p.q_wk = Q + L.w_k + l * hh; p.q_wv = Q + L.w_v + l * hh;
             }
-            span_begin(ctx, EGG_K_QKV); HIP_TRY(egg_launch_qkv(p, s)); span_end(ctx);
+            { SpanScope span(ctx, EGG_K_QKV); HIP_TRY(egg_launch_qkv(p, s)); }
             if (taps) {
                 HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 0), ctx->d_q, act_bytes, hipMemcpyDeviceToDevice, s));
                 HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 1), ctx->d_k, act_bytes, hipMemcpyDeviceToDevice, s));
@@ -644,7 +684,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         }
         {
             AttnParams p; memset(&p, 0, sizeof(p)); p.c = f; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v; p.ao = ctx->d_ao;
-            span_begin(ctx, EGG_K_ATTN); HIP_TRY(egg_launch_attn(p, s)); span_end(ctx);
+            { SpanScope span(ctx, EGG_K_ATTN); HIP_TRY(egg_launch_attn(p, s)); }
             if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 3), ctx->d_ao, act_bytes, hipMemcpyDeviceToDevice, s));
         }
         {
@@ -662,7 +702,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
                 p.q_b_up = Q + L.mlp_bias_up + (int64_t)l * 4 * H; p.q_b_dn = Q + L.mlp_bias_down + (int64_t)l * H;
                 p.q_up = Q + L.w_up + l * h4; p.q_dn = Q + L.w_down + l * h4; p.q_o = Q + L.w_o + l * hh;
             }
-            span_begin(ctx, EGG_K_MLP); HIP_TRY(egg_launch_mlp(p, false, s)); span_end(ctx);
+            { SpanScope span(ctx, EGG_K_MLP); HIP_TRY(egg_launch_mlp(p, false, s)); }
             if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 5), ctx->d_x, act_bytes, hipMemcpyDeviceToDevice, s));
         }
     }
@@ -671,7 +711,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.ln_w = M + L.ln_f; p.ln_b = M + L.ln_f_bias; p.embedding_frag = F + L.embedding; p.x = ctx->d_x;
         p.loss_acc = ctx->d_loss_acc; p.logits_tap = ctx->logits_override ? ctx->logits_override : (taps ? ctx->d_tap_logits : nullptr);
         if (Q) { p.q_ln_w = Q + L.ln_f; p.q_ln_b = Q + L.ln_f_bias; p.q_emb = Q + L.embedding; }
-        span_begin(ctx, EGG_K_HEAD); HIP_TRY(egg_launch_head(p, s)); span_end(ctx);
+        { SpanScope span(ctx, EGG_K_HEAD); HIP_TRY(egg_launch_head(p, s)); }
     }
     return EGG_OK;
 }
@@ -730,21 +770,22 @@ static int update_one(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t
     if (record_flags) p.flags = ctx->d_flags + t.offset;
     if (t.is_matrix && t.muon && ctx->cfg.use_muon) {
         // LAUNCH_ADAM_MATRIX under USE_MUON (mgpu.cu:1587-1595)
-        span_begin(ctx, EGG_K_UPDATE_MATRIX);
-        p.muon_momentum = ctx->cfg.muon_momentum; p.muon_x = ctx->muon.x;
-        HIP_TRY(egg_launch_muon_momentum(p, ctx->stream));
-        HIP_TRY(egg_launch_newton_schulz(ctx->muon, t.rows, t.cols, 5, ctx->stream));
-        p.lr_scale = t.lr_scale * ctx->cfg.muon_lr_scale;
-        HIP_TRY(egg_launch_muon_apply(p, ctx->cfg.adam_weight_decay, ctx->stream));
-        span_end(ctx);
+        {
+            SpanScope span(ctx, EGG_K_UPDATE_MATRIX);
+            p.muon_momentum = ctx->cfg.muon_momentum; p.muon_x = ctx->muon.x;
+            HIP_TRY(egg_launch_muon_momentum(p, ctx->stream));
+            HIP_TRY(egg_launch_newton_schulz(ctx->muon, t.rows, t.cols, 5, ctx->stream));
+            p.lr_scale = t.lr_scale * ctx->cfg.muon_lr_scale;
+            HIP_TRY(egg_launch_muon_apply(p, ctx->cfg.adam_weight_decay, ctx->stream));
+        }
         int rc = refresh_frag(ctx, id);
         if (rc) return rc;
     } else if (t.is_matrix) {
-        span_begin(ctx, EGG_K_UPDATE_MATRIX); HIP_TRY(egg_launch_update_matrix(p, ctx->stream)); span_end(ctx);
+        { SpanScope span(ctx, EGG_K_UPDATE_MATRIX); HIP_TRY(egg_launch_update_matrix(p, ctx->stream)); }
         int rc = refresh_frag(ctx, id);
         if (rc) return rc;
     }
-    else { span_begin(ctx, EGG_K_UPDATE_VECTOR); HIP_TRY(egg_launch_update_vector(p, ctx->stream)); span_end(ctx); }
+    else { SpanScope span(ctx, EGG_K_UPDATE_VECTOR); HIP_TRY(egg_launch_update_vector(p, ctx->stream)); }
     return EGG_OK;
 }
 extern "C" int egg_update_tensor(egg_ctx *ctx, int id, const int32_t *d_fit, const uint32_t *d_seed, const float *d_lr) {
@@ -772,33 +813,43 @@ extern "C" int egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t 
     // Muon matrices (LAUNCH_ADAM_MATRIX under USE_MUON, mgpu.cu:1587-1595), a batch of one shape at a time: momentum of
     // each into its slot of the workspace, Newton-Schulz of the whole batch, then each matrix's apply rule
     if (ctx->cfg.use_muon)
-        for (const auto &g : ctx->muon_groups) {
+        for (size_t gi = 0; gi < ctx->muon_groups.size(); gi++) {
+            const std::vector<int> &g = ctx->muon_groups[gi];
             const egg_tensor_info &t0 = ctx->tensors[g[0]];
-            const size_t one = (size_t)t0.rows * t0.cols;
-            for (size_t first = 0; first < g.size(); first += ctx->muon_batch_max) {
-                const int nb = (int)std::min(g.size() - first, (size_t)ctx->muon_batch_max);
-                span_begin(ctx, EGG_K_UPDATE_MATRIX);
-                for (int b = 0; b < nb; b++) {
-                    UpdParams p = make_upd(ctx, g[first + b], d_fit, d_seed, d_lr);
-                    p.muon_momentum = ctx->cfg.muon_momentum; p.muon_x = ctx->muon.x + (size_t)b * one;
-                    HIP_TRY(egg_launch_muon_momentum(p, ctx->stream));
+            const size_t one = (size_t)t0.rows * t0.cols, k = (size_t)(t0.rows < t0.cols ? t0.rows : t0.cols);
+            const size_t limit = (size_t)ctx->muon_group_batch[gi];
+            // the group's own limit, never the largest group's: the buffers hold `limit` matrices of this shape
+            if (limit < 1 || limit * one > ctx->muon_elems || limit * k * k > ctx->muon_bterm || (int)limit > ctx->muon_batch_max)
+                return fail(ctx, EGG_E_STATE, "Muon batch does not fit the workspace");
+            for (size_t first = 0; first < g.size(); first += limit) {
+                const int nb = (int)std::min(g.size() - first, limit);
+                int rc = EGG_OK;
+                {
+                    SpanScope span(ctx, EGG_K_UPDATE_MATRIX);
+                    for (int b = 0; b < nb; b++) {
+                        UpdParams p = make_upd(ctx, g[first + b], d_fit, d_seed, d_lr);
+                        p.muon_momentum = ctx->cfg.muon_momentum; p.muon_x = ctx->muon.x + (size_t)b * one;
+                        HIP_TRY(egg_launch_muon_momentum(p, ctx->stream));
+                    }
+                    HIP_TRY(egg_launch_newton_schulz_batched(ctx->muon, t0.rows, t0.cols, 5, nb, ctx->stream));
+                    // a failed launch must not leave earlier matrices of the batch with a stale fragment-major copy:
+                    // go on to the refresh below with what was applied, then report
+                    int applied = 0;
+                    for (; applied < nb; applied++) {
+                        const int id = g[first + applied];
+                        UpdParams p = make_upd(ctx, id, d_fit, d_seed, d_lr);
+                        p.muon_x = ctx->muon.x + (size_t)applied * one;
+                        p.lr_scale = ctx->tensors[id].lr_scale * ctx->cfg.muon_lr_scale;
+                        const hipError_t e = egg_launch_muon_apply(p, ctx->cfg.adam_weight_decay, ctx->stream);
+                        if (e != hipSuccess) { rc = fail(ctx, EGG_E_HIP, "egg_launch_muon_apply", e); break; }
+                    }
+                    for (int b = 0; b < applied; b++) { const int r2 = refresh_frag(ctx, g[first + b]); if (r2 && !rc) rc = r2; }
                 }
-                HIP_TRY(egg_launch_newton_schulz_batched(ctx->muon, t0.rows, t0.cols, 5, nb, ctx->stream));
-                for (int b = 0; b < nb; b++) {
-                    const int id = g[first + b];
-                    UpdParams p = make_upd(ctx, id, d_fit, d_seed, d_lr);
-                    p.muon_x = ctx->muon.x + (size_t)b * one;
-                    p.lr_scale = ctx->tensors[id].lr_scale * ctx->cfg.muon_lr_scale;
-                    HIP_TRY(egg_launch_muon_apply(p, ctx->cfg.adam_weight_decay, ctx->stream));
-                }
-                span_end(ctx);
-                for (int b = 0; b < nb; b++) { int rc = refresh_frag(ctx, g[first + b]); if (rc) return rc; }
+                if (rc) return rc;
             }
         }
     UpdParams common = make_upd(ctx, 0, d_fit, d_seed, d_lr);
-    span_begin(ctx, EGG_K_UPDATE_VECTOR);
-    HIP_TRY(egg_launch_update_vectors(common, ctx->d_vec_desc, ctx->n_vec, ctx->vec_total, ctx->stream));
-    span_end(ctx);
+    { SpanScope span(ctx, EGG_K_UPDATE_VECTOR); HIP_TRY(egg_launch_update_vectors(common, ctx->d_vec_desc, ctx->n_vec, ctx->vec_total, ctx->stream)); }
     // d-eggs runs the overlay rule after each tensor's update (de/src/worker.cu:446-523); tensors and their overlay
     // entries are independent, so one launch over every tensor's segment at the end gives the same values
     if (ctx->adaptive)
@@ -1007,7 +1058,9 @@ static int sat_d2i(double x) {
 extern "C" int egg_deggs_sampling_constants(const egg_config *cfg, float min_p, float penalty, int32_t *penalty_int, int32_t *min_p_limit) {
     if (!cfg || !penalty_int || !min_p_limit || cfg->shift_logit < 0 || cfg->shift_logit > 30) return EGG_E_INVALID;
     *penalty_int = sat_d2i((double)(penalty * (float)(1 << cfg->shift_logit)));
-    *min_p_limit = min_p > 0.0f ? sat_d2i((double)logf(min_p) * cfg->softmax_exp_scale) : (min_p <= 0.0f ? INT32_MIN : 0);
+    // logf(0) = -inf saturates to INT32_MIN (nothing is filtered); logf of a negative number is NaN, which the GPU's
+    // conversion turns into 0 (every token below the maximum is filtered)
+    *min_p_limit = sat_d2i((double)logf(min_p) * cfg->softmax_exp_scale);
     return EGG_OK;
 }
 extern "C" int egg_generate_deggs(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed, float temp, float min_p, float penalty) {

@@ -203,6 +203,13 @@ typedef struct egg_tensor_info {
  * that a context of this configuration has.  tensor_id < 0 only counts.  Returns the tensor count, or EGG_E_INVALID. */
 int  egg_describe_layout(const egg_config *cfg, int tensor_id, egg_tensor_info *out, int64_t *state_offset,
                          int64_t *model_bytes, int64_t *state_bytes);
+/* Host code only: the plan by which a use_muon context batches LAUNCH_ADAM_MATRIX's Newton-Schulz chain
+ * (mgpu.cu:1587-1595, muon_internal.cuh:182-342; the reference runs it matrix by matrix through one workspace,
+ * mgpu.cu:1477-1489).  Matrices of one shape form a group; `batch` of them share the workspace at a time, which holds
+ * `matrix_buffer_floats` floats in each of its two matrix buffers and `term_buffer_floats` in the 3I - G buffer, and
+ * batch * rows * cols / batch * min(rows, cols)^2 never exceed those.  group < 0 only counts.  Returns the group count. */
+int  egg_muon_plan(const egg_config *cfg, int group, int *rows, int *cols, int *members, int *batch,
+                   int64_t *matrix_buffer_floats, int64_t *term_buffer_floats);
 int  egg_tensor_count(const egg_ctx *ctx);
 int  egg_tensor_info_get(const egg_ctx *ctx, int tensor_id, egg_tensor_info *out);
 

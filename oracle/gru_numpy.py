@@ -165,14 +165,20 @@ def update_matrix(cfg, w, rows, cols, seed, fit):
     W += step.astype(np.int8)
 
 
-def update_all(cfg, model, step_seed, fit):
-    """egg.c:564-574: the four GRU matrices and two MLP matrices of every layer, then the head; embedding, biases and
-    norm gains are never updated"""
+def update_sites(cfg, model):
+    """egg.c:564-574: (matrix view, rows, cols, seed offset from step_seed) of every matrix the update touches: the
+    four GRU matrices and two MLP matrices of every layer, then the head; embedding, biases and norm gains are never
+    updated"""
     H = cfg.hidden
     for l in range(cfg.n_layers):
-        seed = step_seed + 100 * l
         for g in range(4):
-            update_matrix(cfg, model["gru_weights"][l][g], H, H, seed + 1 + g, fit)
-        update_matrix(cfg, model["mlp_weights"][l][0], 4 * H, H, seed + 5, fit)
-        update_matrix(cfg, model["mlp_weights"][l][1], H, 4 * H, seed + 6, fit)
-    update_matrix(cfg, model["head"], cfg.vocab, H, step_seed + 999, fit)
+            yield model["gru_weights"][l][g], H, H, 100 * l + 1 + g
+        yield model["mlp_weights"][l][0], 4 * H, H, 100 * l + 5
+        yield model["mlp_weights"][l][1], H, 4 * H, 100 * l + 6
+    yield model["head"], cfg.vocab, H, 999
+
+
+def update_all(cfg, model, step_seed, fit):
+    """egg.c:564-574"""
+    for w, rows, cols, off in update_sites(cfg, model):
+        update_matrix(cfg, w, rows, cols, step_seed + off, fit)

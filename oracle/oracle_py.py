@@ -340,10 +340,13 @@ def _sat_f2i(x):
 
 def deggs_sampling_constants(cfg, min_p, penalty):
     """penalty_int and min_p_limit of d-eggs/src/kernels.cu:386-387: the penalty in logit units, truncated, and
-    logf(min_p) * SOFTMAX_EXP_SCALE (a double product of a float logarithm), truncated; min_p <= 0 gives -inf,
-    which the conversion saturates to INT_MIN (nothing is filtered)."""
+    logf(min_p) * SOFTMAX_EXP_SCALE (a double product of a float logarithm), truncated; min_p = 0 gives -inf,
+    which the conversion saturates to INT_MIN (nothing is filtered); min_p < 0 gives NaN, which the GPU's conversion
+    turns into 0."""
     penalty_int = _sat_f2i(np.float32(penalty) * np.float32(1 << cfg.shift_logit))
-    if min_p <= 0:
+    if min_p < 0 or min_p != min_p:
+        limit = 0
+    elif min_p == 0:
         limit = -2147483648
     else:
         prod = float(np.log(np.float32(min_p), dtype=np.float32)) * float(cfg.softmax_exp_scale)

@@ -83,3 +83,34 @@ def test_deggs_sampling_constants_match_the_oracle(pkg, orc):
         for min_p in (0.08, 0.0, 1.0, 0.5, 1e-30, 2.0, -1.0, 0.3333):
             for penalty in (0.2, 0.0, 1.0, -0.01, 7.77, 1e12):
                 assert pkg.deggs_sampling_constants(cfg, min_p, penalty) == orc.deggs_sampling_constants(ocfg, min_p, penalty), (kw, min_p, penalty)
+
+
+def test_muon_workspace_plan_holds_every_batch(pkg):
+    """The batched Muon update runs each shape group at its own batch limit; the limit times the matrix size (and
+    times the Gram size) must fit the shared workspace for every group, also where the groups' limits differ
+    (hidden 512 with 16 or 32 layers: 64 or 128 square matrices at a limit of 64, 17 or 33 of each 4:1 shape at 16)."""
+    for hidden, layers in ((64, 2), (256, 4), (256, 5), (512, 8), (512, 16), (512, 32), (1024, 6)):
+        cfg = pkg.default_config(hidden=hidden, head_dim=64, n_layers=layers, seq_len=32, population=4, use_muon=1)
+        groups, elems, bterm = pkg.muon_plan(cfg)
+        assert {(g["rows"], g["cols"]) for g in groups} == {(hidden, hidden), (hidden, 4 * hidden), (4 * hidden, hidden)}
+        by = {(g["rows"], g["cols"]): g for g in groups}
+        assert by[(hidden, hidden)]["members"] == 4 * layers
+        assert by[(hidden, 4 * hidden)]["members"] == layers + 1 and by[(4 * hidden, hidden)]["members"] == layers + 1
+        for g in groups:
+            k = min(g["rows"], g["cols"])
+            assert 1 <= g["batch"] <= g["members"]
+            assert g["batch"] * g["rows"] * g["cols"] <= elems, (hidden, layers, g)
+            assert g["batch"] * k * k <= bterm, (hidden, layers, g)
+        assert elems >= 4 * hidden * hidden and bterm >= hidden * hidden        # a single matrix of any shape (egg_update_tensor)
+    groups, elems, _ = pkg.muon_plan(pkg.default_config(hidden=512, head_dim=64, n_layers=16, seq_len=32, population=4, use_muon=1))
+    by = {(g["rows"], g["cols"]): g["batch"] for g in groups}
+    assert by[(512, 512)] == 64 and by[(512, 2048)] == 16 and by[(2048, 512)] == 16 and elems == 16 << 20
+
+
+def test_benchmark_stream_generator(pkg, orc):
+    """The package's synthetic stream (what bench.py feeds the GPU) is the stream the tests feed the oracle."""
+    import numpy as np
+    a = pkg.zipf_bytes(1 << 16, seed=1234)
+    assert a.dtype == np.uint8 and np.array_equal(a, orc.zipf_bytes(1 << 16, seed=1234))
+    counts = np.sort(np.bincount(a, minlength=256))[::-1]
+    assert counts[0] > 4 * counts[15] > 0            # Zipf-like: rank 1 far above rank 16 (ratio 16^1.1 = 21)

@@ -117,7 +117,11 @@ def test_perturbed_linear(pkg, orc, dev, K, N, members, T, extra):
 # last pairs with the oracle, and the shared-weight product with the integer matrix product.
 @pytest.mark.parametrize("K,members,T,own,extra", [(256, 5, 64, 0, {}), (256, 300, 32, 0, {}), (512, 300, 96, 0, {}), (512, 517, 32, 1, {}),
                                                    (256, 1, 32, 0, {}), (512, 1, 160, 1, {}), (512, 259, 160, 0, dict(sigma_shift=5, noise_mask=31)),
-                                                   (256, 258, 128, 1, dict(sigma_shift=5, noise_mask=31)), (512, 256, 32, 0, {}), (512, 2, 32, 0, {})])
+                                                   (256, 258, 128, 1, dict(sigma_shift=5, noise_mask=31)), (512, 256, 32, 0, {}), (512, 2, 32, 0, {}),
+                                                   # K = 256 keeps a ring of 12 tile slots and waits on exact counts once 10 tiles
+                                                   # are in flight: 12 to 18 tiles per workgroup (slot wrap-around, steady-state
+                                                   # wait), 10 to 15 with an odd tile count per member, and 12 to 15 with a ragged tail
+                                                   (256, 600, 192, 0, {}), (256, 700, 160, 1, {}), (256, 1100, 96, 0, dict(sigma_shift=5, noise_mask=31))])
 def test_w_stationary_linear(pkg, orc, dev, K, members, T, own, extra):
     import torch
     N = 512

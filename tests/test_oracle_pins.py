@@ -657,6 +657,7 @@ def test_deggs_sampler_special_cases(orc):
     assert orc.deggs_sampling_constants(cfg, 0.08, 0.2) == (51, -15)        # 0.2 * 256 = 51.2;  ln 0.08 * 6 = -15.15
     assert orc.deggs_sampling_constants(cfg, 0.0, 0.0) == (0, -2147483648)
     assert orc.deggs_sampling_constants(cfg, 1.0, 1.0) == (256, 0)
+    assert orc.deggs_sampling_constants(cfg, -1.0, 0.0) == (0, 0)           # logf(-1) is NaN, (int32_t)NaN is 0 on the GPU
     assert orc.deggs_sampling_constants(cfg, 0.5, -0.01) == (-2, -4)         # ln 0.5 * 6 = -4.16;  -2.56 truncates to -2
     for seed, t in ((7, 0), (7, 13), (123456, 40)):
         logits = rng.integers(-60, 60, 256).astype(np.int32)

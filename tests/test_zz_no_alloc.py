@@ -14,7 +14,6 @@ def test_static_newton_schulz_matches_the_context_entry_point(pkg, orc, dev):
     ctx = pkg.Context(pkg.default_config(use_muon=1, hidden=512, head_dim=64, n_layers=1, seq_len=32, population=8))
     rng = np.random.default_rng(77)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
     for rows, cols, iters in ((512, 2048, 5), (128, 256, 5), (2048, 512, 4), (64, 96, 5), (512, 512, 5)):
         X = rng.integers(-300, 301, (rows, cols)).astype(np.float32)
         a = torch.from_numpy(X).to(dev)
@@ -41,8 +40,33 @@ def test_static_newton_schulz_matches_the_context_entry_point(pkg, orc, dev):
     s.synchronize()
     assert torch.equal(a, b)
     del a, b
-    assert torch.cuda.memory_allocated() == before
     ctx.close()
+
+
+@pytest.mark.gpu
+def test_static_newton_schulz_leaves_the_free_device_memory_unchanged(pkg, dev):
+    """hipMemGetInfo around a series of calls (every input allocated beforehand, one warm-up call so that the code
+    object and its static array are resident): the free byte count must not move, whatever allocator a hipMalloc
+    inside the library would have gone through.  A fresh 256 MiB tensor afterwards shows that the counter does see
+    device allocations."""
+    import torch
+    shapes = ((512, 2048, 5), (128, 256, 5), (2048, 512, 4), (64, 96, 5), (512, 512, 5))
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    xs = [torch.randint(-300, 301, (r, c), generator=gen).float().to(dev) for r, c, _ in shapes]
+    s = torch.cuda.Stream()
+    pkg.newton_schulz_static(xs[0].data_ptr(), *shapes[0], stream=None)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()          # so that the tensor at the end needs a fresh device allocation
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    for rep in range(3):
+        for x, (r, c, it) in zip(xs, shapes):
+            pkg.newton_schulz_static(x.data_ptr(), r, c, it, stream=s.cuda_stream if rep == 1 else None)
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info(dev)[0]
+    assert free_after == free_before, (free_before, free_after)
+    big = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    assert torch.cuda.mem_get_info(dev)[0] <= free_before - (256 << 20)
+    del big
 
 
 @pytest.mark.gpu
