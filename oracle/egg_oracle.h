@@ -31,13 +31,24 @@
  *       edge, penalty per occurrence); the reference holds no fixture for it.
  *   Muon Newton-Schulz : fp64 restatement + orthogonality invariants; the
  *       reference's cuBLAS summation order is unspecified => tolerance only.
- *   whole forward : no reference golden vectors exist, so its composition is
- *       stated a second time, independently and in a different shape (numpy, all
- *       tokens of the window at once: oracle/forward_numpy.py), and the two must
- *       agree on every residual-stream tap, logit and loss; the same file states
- *       the whole AdamW update a second time, and oracle/gru_numpy.py does so for
- *       the CPU program (egg_gru_oracle.cpp).  Beyond the per-stage checks above
- *       and that agreement the whole forward and the whole step are "parity unpinned".
+ *   whole forward (which seed offset, layer base and operand role each perturbation site uses) : the materialised-
+ *       perturbation identity.  With the perturbation shifts at zero the rank-1 term is linear in the weights, so
+ *       the perturbed forward of a member must equal the unperturbed forward of W + ns*B(x)A, v + ns*n1*n2 built
+ *       from the update's tensor table alone; that table is held against the reference's macros by name and against
+ *       the optimizer launch list in the reference's step loop (tests/golden/reference_update_launches.json,
+ *       re-parsed from the source where the checkout is present).  tests/test_materialised_identity.py requires
+ *       every tap, logit and loss to agree, shows that leaving out any one tensor, swapping A and B, borrowing a
+ *       neighbour's offsets or dropping the layer base breaks it, and does the same for the CPU program
+ *       (forward sites against the update's sites).  On top of that the composition is stated a second time in
+ *       numpy, all tokens of the window at once (oracle/forward_numpy.py, oracle/gru_numpy.py), and the two
+ *       restatements must agree on every residual-stream tap, logit and loss; the same files state the whole
+ *       AdamW update and the CPU program's update a second time.  Which of the five SHIFT_* macros follows which
+ *       product is outside the identity (both of its sides shift alike): the sites of mgpu.cu:737, :756, :815, :830,
+ *       :976 are held as a fixture parsed from the source (tests/golden/reference_shift_sites.json) and each
+ *       configuration field is shown to act at that site and no earlier (test_each_shift_acts_at_the_reference_site).
+ *   Still "parity unpinned" (the reference holds nothing to pin them to): Muon at the cuBLAS boundary (summation
+ *       order), the adaptive overlay and the d-eggs sampler beyond their closed forms, ternary-packed weights
+ *       (no reference counterpart).
  */
 #ifndef EGG_ORACLE_H
 #define EGG_ORACLE_H

@@ -299,3 +299,54 @@ def test_gpu_perturbed_forward_equals_forward_of_materialised_model(pkg, orc, de
     assert len(set(loss.tolist())) > 1
     noisy.close()
     plain.close()
+
+
+# ---------------------------------------------------------------- which shift follows which product
+SHIFT_GOLD = os.path.join(HERE, "golden", "reference_shift_sites.json")
+
+
+def parse_reference_shift_sites(text):
+    """every `<variable> >> SHIFT_<NAME>` of the training kernel and its device functions (mgpu.cu:553-1029)"""
+    body = text[text.index("__device__ __forceinline__ AccumType compute_linear_projection"):text.index("__global__ void compute_fitness_kernel")]
+    return sorted({(v.replace(" ", ""), m) for v, m in re.findall(r"([A-Za-z_]\w*(?:\[\w+\])?)\s*>>\s*SHIFT_(\w+)", body)})
+
+
+def test_each_shift_acts_at_the_reference_site(orc):
+    """The identity above cannot see a shift moved to another product (both of its sides shift alike).  The reference
+    applies SHIFT_MLP_UP to the up product `a`, SHIFT_MLP_DOWN to the down product `adn`, SHIFT_ATTN to the scores,
+    SHIFT_OUT to the O-projection `aco` and SHIFT_LOGIT to the head product `ah` (fixture parsed from the source);
+    here each configuration field is changed on its own and the first tap that moves must be that site's."""
+    gold = [tuple(x) for x in json.load(open(SHIFT_GOLD))]
+    if os.path.exists(REF_MGPU):
+        assert parse_reference_shift_sites(open(REF_MGPU).read()) == gold
+    assert gold == [("a", "MLP_UP"), ("aco", "OUT"), ("adn", "MLP_DOWN"), ("ah", "LOGIT"), ("my_h_max", "ATTN"), ("s_attn[h]", "ATTN")]
+
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=2)
+    base = orc.config(**kw)
+    tt = orc.tensor_table(base)
+    model = orc.init_model(base, 42)
+    data = orc.zipf_bytes(1 << 12)
+    order = ["x_emb", "x_init", "q", "k", "v", "ao", "x_attn", "x_mlp", "nf", "logits"]
+
+    def taps(model, ns=2, **change):
+        return orc.forward_member(orc.config(**kw, **change), model, data, 0, 77, 0, ns_override=ns, trace=True)[1]
+
+    def first_moved(model, ns=2, **change):
+        a, b = taps(model, ns), taps(model, ns, **change)
+        return next((n for n in order if not np.array_equal(a[n], b[n])), None)
+
+    assert first_moved(model, shift_attn=6) == "ao"               # scores: q, k, v untouched, the weighted sum moves
+    assert first_moved(model, shift_out=7) == "x_attn"            # O-projection: ao untouched
+    assert first_moved(model, shift_logit=6) == "logits"          # head: the final norm untouched
+    assert np.array_equal(taps(model, shift_logit=0)["logits"] >> 8, taps(model)["logits"])
+    assert first_moved(model, shift_mlp_up=6) == "x_init" and first_moved(model, shift_mlp_down=8) == "x_init"
+    # up against down: with every up matrix zero (and no noise) the up product is zero whatever its shift, the down
+    # product is not
+    no_up = model.copy()
+    for t in tt:
+        if t["name"].startswith(("w_up", "w_emb_mlp_up")):
+            no_up[t["offset"]:t["offset"] + t["rows"] * t["cols"]] = 0
+        if "bias_up" in t["name"]:
+            no_up[t["offset"]:t["offset"] + t["cols"]] = 40       # GELU(40/16) > 0 feeds the down product
+    assert first_moved(no_up, 0, shift_mlp_up=6) is None
+    assert first_moved(no_up, 0, shift_mlp_down=8) == "x_init"
