@@ -57,11 +57,21 @@ __device__ __forceinline__ int clip127(int a) { return min(127, max(-127, a)); }
 // ---------------------------------------------------------------- lane helpers
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 // value held by the same token's lane in the other half
-__device__ __forceinline__ int other_half(int v) { return __shfl_xor(v, 32, 64); }
-__device__ __forceinline__ long long other_half64(long long v) {
-    int lo = __shfl_xor((int)(v & 0xffffffffll), 32, 64);
-    int hi = __shfl_xor((int)(v >> 32), 32, 64);
-    return ((long long)hi << 32) | (unsigned int)lo;
+// A token's values sit in two lanes, 32 apart.  v_permlane32_swap on two copies of a register gives every lane the
+// value of the lower half's lane (first result) and of the upper half's lane (second result): a reduction over the
+// two halves is one swap and one operation, without the LDS crossbar or a lane index.
+__device__ __forceinline__ int sum_halves(int v) {
+    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+    return (int)(r[0] + r[1]);
+}
+__device__ __forceinline__ int max_halves(int v) {
+    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+    return max((int)r[0], (int)r[1]);
+}
+__device__ __forceinline__ long long sum_halves64(long long v) {
+    const auto lo = __builtin_amdgcn_permlane32_swap((unsigned)(v & 0xffffffffll), (unsigned)(v & 0xffffffffll), false, false);
+    const auto hi = __builtin_amdgcn_permlane32_swap((unsigned)(v >> 32), (unsigned)(v >> 32), false, false);
+    return (long long)(((unsigned long long)hi[0] << 32) | lo[0]) + (long long)(((unsigned long long)hi[1] << 32) | lo[1]);
 }
 // hidden index of accumulator register r of column group nt for lane half g
 __device__ __forceinline__ int col_of(int nt, int r, int g) { return nt * 32 + ((r >> 2) << 3) + (g << 2) + (r & 3); }
@@ -411,7 +421,7 @@ __device__ __forceinline__ int dot_noise(const v4i *xop, const int8_t *btab, int
             int kd = NAT ? (8 * ks + 4 * g + q) : (8 * ks + 2 * q + g);
             s = dot4(xop[ks][q], b32[kd], s);
         }
-    return s + other_half(s);
+    return sum_halves(s);
 }
 
 // x . B under the overlay: every term x[k] * B[k] is scaled by the input row's factor and truncated before it is added
@@ -431,7 +441,7 @@ __device__ __forceinline__ int dot_noise_ov(const v4i *xop, const int8_t *btab, 
 #pragma unroll
             for (int e = 0; e < 4; e++) s += div_pow2_trunc<6>(mul24(mul24(sx8(xb, e), sx8(nb, e)), sx8(qb, e)));
         }
-    return s + other_half(s);
+    return sum_halves(s);
 }
 
 // ---------------------------------------------------------------- norms on a token held as a packed operand
@@ -472,7 +482,7 @@ __device__ __forceinline__ void standard_scale(const v4i *x, v4i *out, int mn, c
 template <int KS>
 __device__ __forceinline__ void standard_norm(const v4i *x, v4i *out, const int *wt, const int *bt, int g) {
     int tot = sumabs_groups<KS>(x);
-    tot += other_half(tot);
+    tot = sum_halves(tot);
     int mn = tot / (32 * KS); if (!mn) mn = 1;
     standard_scale<KS>(x, out, mn, wt, bt, 0, g);
 }
@@ -491,7 +501,7 @@ __device__ __forceinline__ int absmax_groups(const v16i *val) {
             lo = min(min(lo, val[nt][r]), val[nt][r + 1]);
         }
     int mx = max(hi, -lo);
-    return max(mx, other_half(mx));
+    return max_halves(mx);
 }
 template <int NT>
 __device__ __forceinline__ void adaptive_scale(const v16i *val, int mx, v4i *out) {

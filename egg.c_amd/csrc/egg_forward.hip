@@ -184,7 +184,12 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         const int k = s * SC;
         w_prefetch2<M::PRDN, H>(ws, p.w_dn + (size_t)(k / H) * H * H + (size_t)((k % H) / 16 + du * M::PRDN) * H * 16, plan_dn);
     };
-    auto pf_o = [&](int u) { w_prefetch2<M::PRO, H>(ws, p.w_o + (size_t)u * M::PRO * H * 16, plan_o); };
+    // (the unit index passes through an empty asm so that the four unit addresses are formed where they are used:
+    // precomputed in front of the pass loop they overflow the scalar registers and are spilled through scratch)
+    auto pf_o = [&](int u) {
+        asm volatile("" : "+s"(u));
+        w_prefetch2<M::PRO, H>(ws, p.w_o + (size_t)(unsigned)u * (M::PRO * H * 16), plan_o);
+    };
     auto pf_pass_first = [&]() { if (FIRST) pf_up(0, 0); else pf_o(0); };
     pf_pass_first();
 
@@ -274,7 +279,13 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
     }
 
     for (int pass = 0; pass < npass; pass++) {
-        const int t = (tm.tile0 + M::TPW * pass) * 32 + j;     // token position; with dedup, row of the table
+        // The lane index is re-read behind an empty asm at the top of a pass and again behind the sub-chunk loop: the
+        // table and exchange addresses of the code around the loop are then formed where they are used instead of
+        // being computed once in front of the pass loop and held (or spilled) across the sub-chunk loop.
+        int laneA = lane;
+        asm volatile("" : "+v"(laneA));
+        const int gA = laneA >> 5, jA = laneA & 31;
+        const int t = (tm.tile0 + M::TPW * pass) * 32 + jA;     // token position; with dedup, row of the table
         const size_t row = ((size_t)mloc * T + t) * H;
         int8_t *xrow = (FIRST && dedup ? p.tab : p.x) + row + col0;   // this wave's slice of the residual row
         v4i xs[NTS];
@@ -289,7 +300,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             for (int nt = 0; nt < NTS; nt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    int n0 = col0 + 32 * nt + 8 * q + 4 * g;
+                    int n0 = col0 + 32 * nt + 8 * q + 4 * gA;
                     int e4 = (int)E32[(size_t)(n0 >> 2) * c.vocab + tok];
                     v4i b4 = *reinterpret_cast<const v4i *>(ex0 + n0);
                     v4i d4 = *reinterpret_cast<const v4i *>(ex1 + n0);
@@ -310,59 +321,62 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             {
                 v4i aop[KS];
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) aop[ks] = load_op(p.ao + row, ks, g);
-                sbo = ADAPT ? dot_noise_ov<KS, false>(aop, exB, p.q_o, 0, g) : dot_noise<KS, false>(aop, exB, 0, g);
+                for (int ks = 0; ks < KS; ks++) aop[ks] = load_op(p.ao + row, ks, gA);
+                sbo = ADAPT ? dot_noise_ov<KS, false>(aop, exB, p.q_o, 0, gA) : dot_noise<KS, false>(aop, exB, 0, gA);
 #pragma unroll
                 for (int u = 0; u < M::OU; u++) {
                     const int8_t *cur = w_acquire(ws);
                     if (u + 1 < M::OU) pf_o(u + 1); else pf_up(0, 0);
-                    mfma_cols<M::PRO / 2, NTS>(acc, aop + u * (M::PRO / 2), cur, H, col0, lane);
+                    mfma_cols<M::PRO / 2, NTS>(acc, aop + u * (M::PRO / 2), cur, H, col0, laneA);
                 }
             }
-            perturb_shift_groups<NTS, FUSE>(acc, sbo, oA, col0, c.sigma, c.shift_out, g);
+            perturb_shift_groups<NTS, FUSE>(acc, sbo, oA, col0, c.sigma, c.shift_out, gA);
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++) {
-                v4i xr = load_op(xrow, nt, g);
+                v4i xr = load_op(xrow, nt, gA);
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[nt][r] += sx8(xr[r >> 2], r & 3);
             }
-            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red, tm, lane);
+            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red, tm, laneA);
             adaptive_scale<NTS>(acc, mx, xs);
             if (p.x_mid && valid)
 #pragma unroll
-                for (int nt = 0; nt < NTS; nt++) store_op(p.x_mid + row + col0, nt, g, xs[nt]);
+                for (int nt = 0; nt < NTS; nt++) store_op(p.x_mid + row + col0, nt, gA, xs[nt]);
         }
         // park the residual (this wave owns the slice; invalid padding waves only recompute, and so do the rows of the
         // value table beyond the number of distinct values: nothing reads them, so nothing of them is written)
         const bool keep = valid && (!(FIRST && dedup) || t < nrows);
         if (keep)
 #pragma unroll
-            for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, g, xs[nt]);
+            for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, gA, xs[nt]);
 
         // MLP (mgpu.cu:708-759)
         v4i nrm[KS];
         {
             int tot = sumabs_groups<NTS>(xs);
-            tot += other_half(tot);
-            tot = xreduce<CS, false>(tot, red + M::SITE, tm, lane);
+            tot = sum_halves(tot);
+            tot = xreduce<CS, false>(tot, red + M::SITE, tm, laneA);
             int mn = tot / H; if (!mn) mn = 1;
-            if constexpr (CS == 1) standard_scale<NTS>(xs, nrm, mn, lnw, lnb, 0, g);
+            if constexpr (CS == 1) standard_scale<NTS>(xs, nrm, mn, lnw, lnb, 0, gA);
             else {
                 // ws.other holds the unit consumed last; every wave has passed a barrier since reading it, and the
                 // next prefetch into it is issued only after the barrier of the next w_acquire
                 v4i mine[NTS];
-                standard_scale<NTS>(xs, mine, mn, lnw, lnb, col0, g);
-                exchange_operand<CS, NTS, KS, M::TPW, M::UNIT>(ws.other, tm, lane, mine, nrm);
+                standard_scale<NTS>(xs, mine, mn, lnw, lnb, col0, gA);
+                exchange_operand<CS, NTS, KS, M::TPW, M::UNIT>(ws.other, tm, laneA, mine, nrm);
             }
         }
-        const int sbu = ADAPT ? dot_noise_ov<KS, false>(nrm, upB, p.q_up, 0, g) : dot_noise<KS, false>(nrm, upB, 0, g);
+        const int sbu = ADAPT ? dot_noise_ov<KS, false>(nrm, upB, p.q_up, 0, gA) : dot_noise<KS, false>(nrm, upB, 0, gA);
         v16i accd[NTS];
         zero_acc<NTS>(accd);
         int sbd = 0;
-        int pb[ADAPT ? NTU * 16 : 1];           // ADAPT: running sums of the reference threads this lane stands in for
+        int pb[ADAPT ? NTU * 16 : 1];           // ADAPT: running sums of the reference threads this laneA stands in for
         // ADAPT: iteration it visits sub-chunk (it % 4) * NSUB/4 + it / 4, so four consecutive iterations cover the
         // intermediate columns unit, unit + H, unit + 2H, unit + 3H of the same hidden units
         auto sub_chunk = [](int it) { return ADAPT ? (it & 3) * (M::NSUB / 4) + (it >> 2) : it; };
+        int laneL = lane;
+        asm volatile("" : "+v"(laneL));
+        const int gL = laneL >> 5;
 #pragma unroll 1
         for (int it = 0; it < M::NSUB; it++) {
             const int s = sub_chunk(it);
@@ -371,7 +385,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             for (int nt = 0; nt < NTU; nt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    v4i b4 = *reinterpret_cast<const v4i *>(bup + s * SC + tm.cs * 32 * NTU + 32 * nt + 8 * q + 4 * g);
+                    v4i b4 = *reinterpret_cast<const v4i *>(bup + s * SC + tm.cs * 32 * NTU + 32 * nt + 8 * q + 4 * gL);
 #pragma unroll
                     for (int e = 0; e < 4; e++) au[nt][4 * q + e] = b4[e];
                 }
@@ -379,7 +393,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             for (int ku = 0; ku < M::UPU; ku++) {
                 const int8_t *cur = w_acquire(ws);
                 if (ku + 1 < M::UPU) pf_up(s, ku + 1); else pf_dn(s, 0);
-                mfma_cols<M::PRUP / 2, NTU>(au, nrm + ku * (M::PRUP / 2), cur, SC, tm.cs * 32 * NTU, lane);
+                mfma_cols<M::PRUP / 2, NTU>(au, nrm + ku * (M::PRUP / 2), cur, SC, tm.cs * 32 * NTU, laneL);
             }
             v4i mid[CS * NTU];
             {
@@ -390,7 +404,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 for (int nt = 0; nt < NTU; nt++)
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
-                        int n0 = nb + 32 * nt + 8 * q + 4 * g;
+                        int n0 = nb + 32 * nt + 8 * q + 4 * gL;
                         int a4 = *reinterpret_cast<const int *>(upA + n0);
                         uint32_t r4[4];          // the activation of element e as an unsigned byte
 #pragma unroll
@@ -402,9 +416,9 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                         }
                         // bytes 0 of the four results side by side: two byte permutes and an or
                         mine[nt][q] = (int)(__builtin_amdgcn_perm(r4[1], r4[0], 0x0c0c0400u) | __builtin_amdgcn_perm(r4[3], r4[2], 0x04000c0cu));
-                        if (!ADAPT) sbd = dot4(mine[nt][q], dnb32[8 * nt + 2 * q + g], sbd);
+                        if (!ADAPT) sbd = dot4(mine[nt][q], dnb32[8 * nt + 2 * q + gL], sbd);
                         else {
-                            const int nz4 = dnb32[8 * nt + 2 * q + g], q4 = *reinterpret_cast<const int *>(p.q_dn + n0);
+                            const int nz4 = dnb32[8 * nt + 2 * q + gL], q4 = *reinterpret_cast<const int *>(p.q_dn + n0);
 #pragma unroll
                             for (int e = 0; e < 4; e++) {
                                 const int idx = ADAPT ? (nt * 4 + q) * 4 + e : 0;
@@ -423,7 +437,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                     for (int nt = 0; nt < NTU; nt++) mid[nt] = mine[nt];
                 } else {
 #pragma unroll
-                    for (int nt = 0; nt < NTU; nt++) xch_put(xch, CS * NTU, tm.tslot, tm.cs * NTU + nt, lane, mine[nt]);
+                    for (int nt = 0; nt < NTU; nt++) xch_put(xch, CS * NTU, tm.tslot, tm.cs * NTU + nt, laneL, mine[nt]);
                 }
             }
 #pragma unroll
@@ -431,33 +445,36 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 const int8_t *cur = w_acquire(ws);        // its barrier also publishes the intermediate slices
                 if (CS > 1 && du == 0)
 #pragma unroll
-                    for (int k = 0; k < CS * NTU; k++) mid[k] = xch_get(xch, CS * NTU, tm.tslot, k, lane);
+                    for (int k = 0; k < CS * NTU; k++) mid[k] = xch_get(xch, CS * NTU, tm.tslot, k, laneL);
                 if (du + 1 < M::DNU) pf_dn(s, du + 1);
                 else if (it + 1 < M::NSUB) pf_up(sub_chunk(it + 1), 0);
                 else if (pass + 1 < npass) pf_pass_first();
-                mfma_cols<M::PRDN / 2, NTS>(accd, mid + du * (M::PRDN / 2), cur, H, col0, lane);
+                mfma_cols<M::PRDN / 2, NTS>(accd, mid + du * (M::PRDN / 2), cur, H, col0, laneL);
             }
         }
-        sbd += other_half(sbd);
-        sbd = xreduce<CS, false>(sbd, red + 2 * M::SITE, tm, lane);
-        perturb_shift_groups<NTS, FUSE_DN>(accd, sbd, dnA, col0, c.sigma, c.shift_mlp_down, g);
+        int laneB = lane;
+        asm volatile("" : "+v"(laneB));
+        const int gB = laneB >> 5;
+        sbd = sum_halves(sbd);
+        sbd = xreduce<CS, false>(sbd, red + 2 * M::SITE, tm, laneB);
+        perturb_shift_groups<NTS, FUSE_DN>(accd, sbd, dnA, col0, c.sigma, c.shift_mlp_down, gB);
 #pragma unroll
         for (int nt = 0; nt < NTS; nt++) {
-            v4i xr = load_op(xrow, nt, g);          // the parked residual (for a padding wave: someone else's row, unused)
+            v4i xr = load_op(xrow, nt, gB);          // the parked residual (for a padding wave: someone else's row, unused)
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                v4i b4 = *reinterpret_cast<const v4i *>(bdn + col0 + 32 * nt + 8 * q + 4 * g);
+                v4i b4 = *reinterpret_cast<const v4i *>(bdn + col0 + 32 * nt + 8 * q + 4 * gB);
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                     accd[nt][4 * q + e] += sx8(xr[q], e) + b4[e];
             }
         }
-        const int mx2 = xreduce<CS, true>(absmax_groups<NTS>(accd), red + 3 * M::SITE, tm, lane);
+        const int mx2 = xreduce<CS, true>(absmax_groups<NTS>(accd), red + 3 * M::SITE, tm, laneB);
         v4i xnew[NTS];
         adaptive_scale<NTS>(accd, mx2, xnew);
         if (keep)
 #pragma unroll
-            for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, g, xnew[nt]);
+            for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, gB, xnew[nt]);
     }
     if (FIRST && dedup) {
         // every position takes the row of its byte value (16 bytes per thread and step)
@@ -582,7 +599,7 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++) x[nt] = load_op(p.x + row + col0, nt, g);
             int tot = sumabs_groups<NTS>(x);
-            tot += other_half(tot);
+            tot = sum_halves(tot);
             tot = xreduce<CS, false>(tot, red, tm, lane);        // sites alternate 0,1,0,1 through the pass
             int mn = tot / H; if (!mn) mn = 1;
             if constexpr (CS == 1) standard_scale<NTS>(x, nrm, mn, lnw, lnb, 0, g);
@@ -793,7 +810,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
                 }
             }
         }
-        mx = max(mx, other_half(mx));
+        mx = max_halves(mx);
         const int mxs = mx >> c.shift_attn;
         // pass 2: weights and weighted V sum (mgpu.cu:810-824)
         v16i o[3][DT];
@@ -822,7 +839,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
             }
         }
         int den = attn_den(dpl);
-        den += other_half(den);
+        den = sum_halves(den);
         // Truncating quotient num / den with one reciprocal per token.  num and den are integers below 2^53, the
         // quotient is at most 127 in magnitude, and a non-integer quotient is at least 1/den >= 2^-27 away from
         // the next integer.  Scaling the reciprocal by (1 + 2^-40) pushes an exactly integer quotient k to
@@ -980,7 +997,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
                 if (cx <= j) mx = max(mx, s[r]);
             }
         }
-        mx = max(mx, other_half(mx));
+        mx = max_halves(mx);
         const int mxs = mx >> c.shift_attn;
         // pass 2: weights and weighted V sum (mgpu.cu:810-824).  The first tile weighed starts the accumulators (a zero C
         // operand instead of 96 cleared registers); the scores of the next tile are in flight while a tile is weighed.
@@ -1016,7 +1033,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
             }
         }
         int den = attn_den(dpl);
-        den += other_half(den);
+        den = sum_halves(den);
         // truncating quotient with one reciprocal per token, see k_attn
         const double rden = (1.0 + 0x1p-40) / (double)(den ? den : 1);
 #pragma unroll
@@ -1104,7 +1121,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
         for (int nt = 0; nt < NV; nt++)
 #pragma unroll
             for (int r = 0; r < 16; r++) { acc[nt][r] >>= c.shift_logit; gmax = max(gmax, acc[nt][r]); }
-        gmax = max(gmax, other_half(gmax));
+        gmax = max_halves(gmax);
         const int target = c.data[spos + t + 1];
         long long sum_ex = 0; int tl = 0;
 #pragma unroll
@@ -1115,8 +1132,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
                 sum_ex += lut[idx];
                 if (col_of(nt, r, g) == target) tl = acc[nt][r];
             }
-        sum_ex += other_half64(sum_ex);
-        tl += other_half(tl);
+        sum_ex = sum_halves64(sum_ex);
+        tl = sum_halves(tl);
         if (p.logits_tap && valid)
 #pragma unroll
             for (int nt = 0; nt < NV; nt++)

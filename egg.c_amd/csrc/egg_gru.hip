@@ -136,7 +136,7 @@ __device__ __forceinline__ int gru_xb(const int8_t *ldsB, const int8_t *bvec, in
             for (int q = 0; q < 4; q++) s = dot4(b[q], n[u][q], s);
         }
     }
-    return s + other_half(s);
+    return sum_halves(s);
 }
 // rank-1 term, shift and clamp of one strip (egg.c:167-175); returns the 16 int8 results packed in slot order
 __device__ __forceinline__ v4i gru_finish(const v16i &acc, int xb, const int8_t *avec, int nt, int ns, int sigma, int shift, int g) {
@@ -191,7 +191,7 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
         if (own) {
 #pragma unroll
             for (int q = 0; q < 4; q++) part = sumabs4(x[q], part);
-            part += other_half(part);
+            part = sum_halves(part);
             if (g == 0) psum[wave * 32 + j] = part;
         }
         __syncthreads();
@@ -340,7 +340,7 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
                     part += lut[v + 128];
                     if (32 * wave + 8 * q + 4 * g + e == target) tl[j] = v;
                 }
-            part += other_half(part);
+            part = sum_halves(part);
         }
         if (g == 0) psum[wave * 32 + j] = part;
         __syncthreads();

@@ -356,7 +356,7 @@ __global__ void __launch_bounds__(EGG_THREADS, 1) k_plinear_ws(PlinParams p) {
                     }
                     if (!PLAIN) {
                         if (ks == QS) {
-                            sbp += other_half(sbp);
+                            sbp = sum_halves(sbp);
                             sbx[(((t & 1) * 32 + j) << 2) + wave] = sbp;
                         }
                         if (ks == MID + 1) {
