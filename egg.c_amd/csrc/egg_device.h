@@ -521,6 +521,39 @@ __device__ __forceinline__ void adaptive_norm(const v16i *val, v4i *out) {
     adaptive_scale<NT>(val, absmax_groups<NT>(val), out);
 }
 
+// The same two parts with the conversion to float first: (float) is monotonic, so the largest |(float)val| is the
+// float of the largest |val| the reference converts, and |.| is an operand modifier of the float maximum (one
+// three-operand maximum per two values instead of a maximum and a minimum).  The values are left as floats (bit
+// patterns) for the scaling; the result is the maximum's bit pattern, which orders like the float since it is not negative.
+template <int NT>
+__device__ __forceinline__ int absmax_to_float_groups(v16i *val) {
+    float m0 = 0.0f, m1 = 0.0f;
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int r = 0; r < 16; r += 4) {
+            const float a = (float)val[nt][r], b = (float)val[nt][r + 1], c2 = (float)val[nt][r + 2], d = (float)val[nt][r + 3];
+            m0 = fmaxf(fmaxf(m0, fabsf(a)), fabsf(b));
+            m1 = fmaxf(fmaxf(m1, fabsf(c2)), fabsf(d));
+            val[nt][r] = __float_as_int(a); val[nt][r + 1] = __float_as_int(b);
+            val[nt][r + 2] = __float_as_int(c2); val[nt][r + 3] = __float_as_int(d);
+        }
+    return max_halves(__float_as_int(fmaxf(m0, m1)));
+}
+template <int NT>
+__device__ __forceinline__ void adaptive_scale_floats(const v16i *valf, int mx_bits, v4i *out) {
+    const float scale = 127.0f / (__int_as_float(mx_bits) + 1e-9f);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            int o[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = round_half_away(__int_as_float(valf[nt][4 * q + e]) * scale);
+            out[nt][q] = pack4(o[0], o[1], o[2], o[3]);
+        }
+}
+
 // 128-bit load/store of a token's 16 bytes of column group `grp` in a slot-ordered [.][H] int8 buffer
 __device__ __forceinline__ v4i load_op(const int8_t *row, int grp, int g) {
     return *reinterpret_cast<const v4i *>(row + grp * 32 + g * 16);

@@ -123,19 +123,26 @@ struct MlpCfg {
     static constexpr int WBYTES = 2 * UNIT;
     static constexpr int I32 = 9 * H;        // ex0[H] ex1[H] lnw[H] lnb[H] bup[4H] bdn[H]
     static constexpr int I8 = 11 * H;        // exB[H] upB[H] dnB[4H] upA[4H] dnA[H]   (A noise already times the sign)
+    // The blocks behind the first one keep the up projection's output noise as int32 (UPA32): the GELU epilogue then
+    // multiplies by a table word as it stands instead of extracting a byte per element.  The first block has no room
+    // for it at three workgroups per CU (its value-rank tables take the space) and keeps the bytes.
+    static constexpr int UPA32 = 3 * 4 * H;  // extra bytes of the int32 form: upA occupies 16H instead of 4H
     static constexpr int PER_SET = I32 * 4 + I8;
     // The normalised input is exchanged through whichever W buffer is idle at that point (TPW*32*H <= UNIT bytes);
     // the intermediate slices have their own small area because both W buffers are busy inside the sub-chunk loop.
     static constexpr int XCHG = CS > 1 ? TPW * 32 * SC : 0;
     static constexpr int SITE = EGG_WAVES * 64;                       // ints per reduction site
-    static constexpr int RED = CS > 1 ? 4 * SITE * 4 : 0;
+    static constexpr int RED = CS > 1 ? 2 * SITE * 4 : 0;             // two reduction sites used alternately
     static constexpr int OCC = H == 256 ? 3 : 2;                      // workgroups per CU the kernel is built for
     // first block only: rank of every byte value among the values present in the member's window [256], wave counts
     // [4 ints], and below hidden 256 the list of present values [256] (from hidden 256 on it lives in the table slot
     // of the O projection's noise, which the first block does not use)
     static constexpr int DEDUP = 256 + 16 + (H < 256 ? 256 : 0);
     static constexpr int ACT = 256;          // GELU table: entry v + 128 holds the activation of the int8 value v
-    static int total(int sets, bool first) { return WBYTES + ACT + sets * PER_SET + XCHG + RED + (first ? DEDUP : 0); }
+    // (behind the first block ex1 does not exist: 4H bytes less.  At hidden 256 the total stays at 52 KB: the LDS is
+    // handed out in granules, three workgroups of 53 KB no longer share a CU, and the kernel then runs 9 % slower.)
+    static constexpr int per_set(bool first) { return PER_SET + (first ? 0 : UPA32 - 4 * H); }
+    static int total(int sets, bool first) { return WBYTES + ACT + sets * per_set(first) + XCHG + RED + (first ? DEDUP : 0); }
 };
 
 // FUSE: the host has checked sigma <= 7 and |noise| <= 15, which bounds |acc| * 2^sigma + |sb * a| below 2^31 for
@@ -161,15 +168,19 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
     const int T = c.T;
     const TileMap tm = tile_map<CS>(T, wave, blockIdx.x);
     const int col0 = tm.cs * HS;                      // first output column of this wave's slice
-    int8_t *tb = act + M::ACT + tm.set * M::PER_SET;
+    constexpr int PSET = M::per_set(FIRST);
+    constexpr bool UPA32 = !FIRST;
+    int8_t *tb = act + M::ACT + tm.set * PSET;
     int *ex0 = reinterpret_cast<int *>(tb);           // FIRST: emb_bias + noise   | else: O-proj A noise * ns as int8
-    int *ex1 = ex0 + H;                               // FIRST: b_dim noise * ns    | else: unused
-    int *lnw = ex1 + H, *lnb = lnw + H, *bup = lnb + H, *bdn = bup + 4 * H;
+    int *ex1 = ex0 + H;                               // FIRST: b_dim noise * ns    | else: absent
+    int *lnw = ex1 + (FIRST ? H : 0), *lnb = lnw + H, *bup = lnb + H, *bdn = bup + 4 * H;
     int8_t *exB = reinterpret_cast<int8_t *>(bdn + H);   // O-proj B noise
-    int8_t *upB = exB + H, *dnB = upB + H, *upA = dnB + 4 * H, *dnA = upA + 4 * H;
+    int8_t *upB = exB + H, *dnB = upB + H, *upA = dnB + 4 * H, *dnA = upA + (UPA32 ? 16 : 4) * H;
     const int8_t *oA = reinterpret_cast<const int8_t *>(ex0);
-    int8_t *xch = act + M::ACT + tm.sets * M::PER_SET;
+    int8_t *xch = act + M::ACT + tm.sets * PSET;
     int *red = reinterpret_cast<int *>(xch + M::XCHG);
+    int rsite = 0;          // the two reduction sites take turns, call by call (the same sequence in every wave)
+    auto next_site = [&]() { rsite ^= 1; return red + rsite * M::SITE; };
 
     WStream ws; wstream_init(ws, smem, M::UNIT);
     // unit sources inside the fragment-major copies (block size == H)
@@ -199,9 +210,9 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         int ml = blockIdx.x * tm.sets + ss; if (ml >= c.n_members) ml = c.n_members - 1;
         const int mem = c.pop_offset + ml, nsx = (mem & 1) ? -1 : 1;
         const uint32_t pseed = *c.d_step_seed + (uint32_t)(mem / 2), sbx = pseed + (uint32_t)p.seed_base;
-        int8_t *t2 = act + M::ACT + ss * M::PER_SET;
-        int *e0 = reinterpret_cast<int *>(t2), *e1 = e0 + H, *lw = e1 + H, *lb = lw + H, *bu = lb + H, *bd = bu + 4 * H;
-        int8_t *eB = reinterpret_cast<int8_t *>(bd + H), *uB = eB + H, *dB = uB + H, *uA = dB + 4 * H, *dA = uA + 4 * H;
+        int8_t *t2 = act + M::ACT + ss * PSET;
+        int *e0 = reinterpret_cast<int *>(t2), *e1 = e0 + H, *lw = e1 + (FIRST ? H : 0), *lb = lw + H, *bu = lb + H, *bd = bu + 4 * H;
+        int8_t *eB = reinterpret_cast<int8_t *>(bd + H), *uB = eB + H, *dB = uB + H, *uA = dB + 4 * H, *dA = uA + (UPA32 ? 16 : 4) * H;
         const int tid = threadIdx.x;
         if (ADAPT) {
             if (FIRST) {
@@ -214,7 +225,8 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             }
             fill_vec_i32_ov(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2, p.q_ln_w);
             fill_vec_i32_ov(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_b);
-            fill_noise_i8_ov(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx, p.q_up + H);
+            if (UPA32) fill_noise_i32_ov(reinterpret_cast<int *>(uA), sbx + p.off_up_a, 4 * H, c.mask, nsx, tid, EGG_THREADS, p.q_up + H);
+            else fill_noise_i8_ov(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx, p.q_up + H);
             fill_vec_i32_ov(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up, p.q_b_up, 128);
             fill_noise_i8_ov(dA, sbx + p.off_dn_a, H, c.mask, tid, EGG_THREADS, nsx, p.q_dn + 4 * H);
             fill_vec_i32_ov(bd, p.b_dn, sbx + p.off_bdn_a, sbx + p.off_bdn_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_b_dn);
@@ -231,7 +243,8 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         }
         fill_vec_i32(lw, p.ln_w, sbx + p.off_ln_a, sbx + p.off_ln_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2);     // 4 * gain, see standard_scale
         fill_vec_i32(lb, p.ln_b, sbx + p.off_lnb_a, sbx + p.off_lnb_b, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
-        fill_noise_i8(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx);
+        if (UPA32) fill_noise_i32(reinterpret_cast<int *>(uA), sbx + p.off_up_a, 4 * H, c.mask, nsx, tid, EGG_THREADS);
+        else fill_noise_i8(uA, sbx + p.off_up_a, 4 * H, c.mask, tid, EGG_THREADS, nsx);
         // the up bias is stored as (b + 128) << shift_mlp_up and seeds the up accumulator: ((a + (b << s)) >> s) == (a >> s) + b;
         // the 128 makes the clamped result (1..255) the GELU table's index
         fill_vec_i32(bu, p.b_up, sbx + p.off_bup_a, sbx + p.off_bup_b, 4 * H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, c.shift_mlp_up, 128);
@@ -337,8 +350,8 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[nt][r] += sx8(xr[r >> 2], r & 3);
             }
-            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red, tm, laneA);
-            adaptive_scale<NTS>(acc, mx, xs);
+            const int mx = xreduce<CS, true>(absmax_to_float_groups<NTS>(acc), next_site(), tm, laneA);
+            adaptive_scale_floats<NTS>(acc, mx, xs);
             if (p.x_mid && valid)
 #pragma unroll
                 for (int nt = 0; nt < NTS; nt++) store_op(p.x_mid + row + col0, nt, gA, xs[nt]);
@@ -355,7 +368,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         {
             int tot = sumabs_groups<NTS>(xs);
             tot = sum_halves(tot);
-            tot = xreduce<CS, false>(tot, red + M::SITE, tm, laneA);
+            tot = xreduce<CS, false>(tot, next_site(), tm, laneA);
             int mn = tot / H; if (!mn) mn = 1;
             if constexpr (CS == 1) standard_scale<NTS>(xs, nrm, mn, lnw, lnb, 0, gA);
             else {
@@ -405,13 +418,15 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
                         int n0 = nb + 32 * nt + 8 * q + 4 * gL;
-                        int a4 = *reinterpret_cast<const int *>(upA + n0);
+                        int a4 = 0; v4i a32 = {0, 0, 0, 0};
+                        if (UPA32) a32 = *reinterpret_cast<const v4i *>(reinterpret_cast<const int *>(upA) + n0);
+                        else a4 = *reinterpret_cast<const int *>(upA + n0);
                         uint32_t r4[4];          // the activation of element e as an unsigned byte
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             // the accumulator carries + 128 (see the bias table): clamping to 1..255 is the clamp to +-127,
                             // and the result is the table index as it stands
-                            const int idx = min(255, max(1, perturb_shift<FUSE>(au[nt][4 * q + e], sbu, sx8(a4, e), c.sigma, c.shift_mlp_up)));
+                            const int idx = min(255, max(1, perturb_shift<FUSE>(au[nt][4 * q + e], sbu, UPA32 ? a32[e] : sx8(a4, e), c.sigma, c.shift_mlp_up)));
                             r4[e] = reinterpret_cast<lds_u8_ptr>((uintptr_t)(uint32_t)idx)[M::WBYTES];
                         }
                         // bytes 0 of the four results side by side: two byte permutes and an or
@@ -456,7 +471,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         asm volatile("" : "+v"(laneB));
         const int gB = laneB >> 5;
         sbd = sum_halves(sbd);
-        sbd = xreduce<CS, false>(sbd, red + 2 * M::SITE, tm, laneB);
+        sbd = xreduce<CS, false>(sbd, next_site(), tm, laneB);
         perturb_shift_groups<NTS, FUSE_DN>(accd, sbd, dnA, col0, c.sigma, c.shift_mlp_down, gB);
 #pragma unroll
         for (int nt = 0; nt < NTS; nt++) {
@@ -469,9 +484,9 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                     accd[nt][4 * q + e] += sx8(xr[q], e) + b4[e];
             }
         }
-        const int mx2 = xreduce<CS, true>(absmax_groups<NTS>(accd), red + 3 * M::SITE, tm, laneB);
         v4i xnew[NTS];
-        adaptive_scale<NTS>(accd, mx2, xnew);
+        const int mx2 = xreduce<CS, true>(absmax_to_float_groups<NTS>(accd), next_site(), tm, laneB);
+        adaptive_scale_floats<NTS>(accd, mx2, xnew);
         if (keep)
 #pragma unroll
             for (int nt = 0; nt < NTS; nt++) store_op(xrow, nt, gB, xnew[nt]);
@@ -499,7 +514,8 @@ struct QkvCfg {
     static constexpr int PR = (H / 16) < (1024 / H) ? (H / 16) : (1024 / H), NU = (H / 16) / PR;   // p-rows per unit, units per matrix
     static constexpr int UNIT = 16 * PR * H;
     static constexpr int WBYTES = 2 * UNIT;
-    static constexpr int PER_SET = 2 * H * 4 + 6 * H;   // lnw lnb (int32) | qA kA vA (int8, times the sign) qB kB vB (int8)
+    // lnw lnb (int32) | qA kA vA (int32, times the sign: an operand of the multiply without a byte extraction) | qB kB vB (int8)
+    static constexpr int PER_SET = 5 * H * 4 + 3 * H;
     static constexpr int XCHG = 0;             // the normalised input is exchanged through the idle W buffer
     static constexpr int SITE = EGG_WAVES * 64;
     static constexpr int RED = CS > 1 ? 2 * SITE * 4 : 0;       // two reduction sites used alternately
@@ -550,7 +566,8 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
     const int col0 = tm.cs * HS;
     int8_t *tb = smem + Q::WBYTES + tm.set * Q::PER_SET;
     int *lnw = reinterpret_cast<int *>(tb), *lnb = lnw + H;
-    int8_t *qA = reinterpret_cast<int8_t *>(lnb + H), *kA = qA + H, *vA = kA + H, *qB = vA + H, *kB = qB + H, *vB = kB + H;
+    int *qA = lnb + H, *kA = qA + H, *vA = kA + H;
+    int8_t *qB = reinterpret_cast<int8_t *>(vA + H), *kB = qB + H, *vB = kB + H;
     int8_t *xch = smem + Q::WBYTES + tm.sets * Q::PER_SET;
     int *red = reinterpret_cast<int *>(xch + Q::XCHG);
 
@@ -565,20 +582,21 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
         const uint32_t sbx = *c.d_step_seed + (uint32_t)(mem / 2) + (uint32_t)p.seed_base;
         int8_t *t2 = smem + Q::WBYTES + ss * Q::PER_SET;
         int *lw = reinterpret_cast<int *>(t2), *lb = lw + H;
-        int8_t *a0 = reinterpret_cast<int8_t *>(lb + H), *a1 = a0 + H, *a2 = a1 + H, *b0 = a2 + H, *b1 = b0 + H, *b2 = b1 + H;
+        int *a0 = lb + H, *a1 = a0 + H, *a2 = a1 + H;
+        int8_t *b0 = reinterpret_cast<int8_t *>(a2 + H), *b1 = b0 + H, *b2 = b1 + H;
         const int tid = threadIdx.x;
         if (ADAPT) {
             fill_vec_i32_ov(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2, p.q_ln_w);
             fill_vec_i32_ov(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 0, p.q_ln_b);
-            fill_noise_i8_ov(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wq + H);
-            fill_noise_i8_ov(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wk + H);
-            fill_noise_i8_ov(a2, sbx + OFF_V_A, H, c.mask, tid, EGG_THREADS, nsx, p.q_wv + H);
+            fill_noise_i32_ov(a0, sbx + OFF_Q_A, H, c.mask, nsx, tid, EGG_THREADS, p.q_wq + H);
+            fill_noise_i32_ov(a1, sbx + OFF_K_A, H, c.mask, nsx, tid, EGG_THREADS, p.q_wk + H);
+            fill_noise_i32_ov(a2, sbx + OFF_V_A, H, c.mask, nsx, tid, EGG_THREADS, p.q_wv + H);
         } else {
             fill_vec_i32(lw, p.ln_w, sbx + OFF_LN_1_A, sbx + OFF_LN_1_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS, 2);     // 4 * gain, see standard_scale
             fill_vec_i32(lb, p.ln_b, sbx + OFF_LN_1_BIAS_A, sbx + OFF_LN_1_BIAS_B, H, c.mask, nsx, c.sigma_vec, tid, EGG_THREADS);
-            fill_noise_i8(a0, sbx + OFF_Q_A, H, c.mask, tid, EGG_THREADS, nsx);
-            fill_noise_i8(a1, sbx + OFF_K_A, H, c.mask, tid, EGG_THREADS, nsx);
-            fill_noise_i8(a2, sbx + OFF_V_A, H, c.mask, tid, EGG_THREADS, nsx);
+            fill_noise_i32(a0, sbx + OFF_Q_A, H, c.mask, nsx, tid, EGG_THREADS);
+            fill_noise_i32(a1, sbx + OFF_K_A, H, c.mask, nsx, tid, EGG_THREADS);
+            fill_noise_i32(a2, sbx + OFF_V_A, H, c.mask, nsx, tid, EGG_THREADS);
         }
         fill_noise_i8(b0, sbx + OFF_Q_B, H, c.mask, tid, EGG_THREADS);
         fill_noise_i8(b1, sbx + OFF_K_B, H, c.mask, tid, EGG_THREADS);
@@ -614,7 +632,7 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
             const int8_t *W = which == 0 ? p.w_q : (which == 1 ? p.w_k : p.w_v);
             const int8_t *nw = which == 0 ? p.w_k : (which == 1 ? p.w_v : ((pass + 1 < tm.passes) ? p.w_q : nullptr));
             const int8_t *Bn = which == 0 ? qB : (which == 1 ? kB : vB);
-            const int8_t *An = which == 0 ? qA : (which == 1 ? kA : vA);
+            const int *An = which == 0 ? qA : (which == 1 ? kA : vA);
             int8_t *dst = which == 0 ? p.q : (which == 1 ? p.k : p.v);
             const int sb = ADAPT ? dot_noise_ov<KS, false>(nrm, Bn, which == 0 ? p.q_wq : (which == 1 ? p.q_wk : p.q_wv), 0, g)
                                  : dot_noise<KS, false>(nrm, Bn, 0, g);
@@ -627,11 +645,11 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
                 else if (nw) pf(nw, 0);
                 mfma_cols<Q::PR / 2, NTS>(acc, nrm + u * (Q::PR / 2), cur, H, col0, lane);
             }
-            add_perturb8<NTS>(acc, sb, An, col0, c.sigma, g);
+            add_perturb<NTS>(acc, sb, An, col0, c.sigma, g);
             if (which < 2) rope_inplace<NTS>(acc, c.rope_lut + (size_t)t * c.head_dim, c.head_dim, g, c.rope_scale_bit);
-            const int mx = xreduce<CS, true>(absmax_groups<NTS>(acc), red + ((1 + which) & 1) * Q::SITE, tm, lane);
+            const int mx = xreduce<CS, true>(absmax_to_float_groups<NTS>(acc), red + ((1 + which) & 1) * Q::SITE, tm, lane);
             v4i o[NTS];
-            adaptive_scale<NTS>(acc, mx, o);
+            adaptive_scale_floats<NTS>(acc, mx, o);
             if (valid)
 #pragma unroll
                 for (int nt = 0; nt < NTS; nt++) store_op(dst + row + col0, nt, g, o[nt]);
