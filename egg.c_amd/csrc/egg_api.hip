@@ -831,7 +831,10 @@ extern "C" int egg_es_update(egg_ctx *ctx, const int32_t *d_fit, const uint32_t 
                         p.muon_momentum = ctx->cfg.muon_momentum; p.muon_x = ctx->muon.x + (size_t)b * one;
                         HIP_TRY(egg_launch_muon_momentum(p, ctx->stream));
                     }
-                    HIP_TRY(egg_launch_newton_schulz_batched(ctx->muon, t0.rows, t0.cols, 5, nb, ctx->stream));
+                }
+                { SpanScope span(ctx, EGG_K_MUON_NS); HIP_TRY(egg_launch_newton_schulz_batched(ctx->muon, t0.rows, t0.cols, 5, nb, ctx->stream)); }
+                {
+                    SpanScope span(ctx, EGG_K_UPDATE_MATRIX);
                     // a failed launch must not leave earlier matrices of the batch with a stale fragment-major copy:
                     // go on to the refresh below with what was applied, then report
                     int applied = 0;

@@ -277,20 +277,25 @@ __device__ __forceinline__ void mfma_unit2(v16i *acc, const v4i *xop, const int8
 
 // acc[nt] += unit^T . xop for the NTW column groups starting at column `colbase` of a staged unit that is
 // KSU k-steps deep and `cols` columns wide
-template <int KSU, int NTW>
+// MAXF: fragments (four registers each) read ahead of their MFMAs
+template <int KSU, int NTW, int MAXF = 8>
 __device__ __forceinline__ void mfma_cols(v16i *acc, const v4i *xop, const int8_t *lds, int cols, int colbase, int lane) {
     const int i = lane & 31, g = lane >> 5;
     // all fragment reads of a batch are issued before its first MFMA, so one LDS latency is exposed per batch
     // instead of one per fragment pair
-    constexpr int BK = (KSU * NTW <= 8) ? KSU : (8 / NTW > 0 ? 8 / NTW : 1);     // k-steps per batch
+    constexpr int NB = NTW < MAXF ? NTW : MAXF;                                   // column groups per batch
+    constexpr int BK = (KSU * NB <= MAXF) ? KSU : (MAXF / NB > 0 ? MAXF / NB : 1);   // k-steps per batch
+    static_assert(NTW % NB == 0 && KSU % BK == 0, "batches must tile the unit");
+#pragma unroll
+    for (int n0 = 0; n0 < NTW; n0 += NB)
 #pragma unroll
     for (int k0 = 0; k0 < KSU; k0 += BK) {
-        v4i a[BK * NTW];
+        v4i a[BK * NB];
 #pragma unroll
         for (int ks = 0; ks < BK; ks++)
 #pragma unroll
-            for (int nt = 0; nt < NTW; nt++)
-                a[ks * NTW + nt] = *reinterpret_cast<const v4i *>(lds + ((size_t)((k0 + ks) * 2 + g) * cols + colbase + nt * 32 + i) * 16);
+            for (int nt = 0; nt < NB; nt++)
+                a[ks * NB + nt] = *reinterpret_cast<const v4i *>(lds + ((size_t)((k0 + ks) * 2 + g) * cols + colbase + (n0 + nt) * 32 + i) * 16);
         __builtin_amdgcn_sched_barrier(0);
         // a wave that has its fragments goes first: the matrix pipe is the unit other waves cannot substitute for
         // (measured: 1.8 % on the MLP kernel, nothing elsewhere)
@@ -298,8 +303,8 @@ __device__ __forceinline__ void mfma_cols(v16i *acc, const v4i *xop, const int8_
 #pragma unroll
         for (int ks = 0; ks < BK; ks++)
 #pragma unroll
-            for (int nt = 0; nt < NTW; nt++)
-                acc[nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks * NTW + nt], xop[k0 + ks], acc[nt], 0, 0, 0);
+            for (int nt = 0; nt < NB; nt++)
+                acc[n0 + nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks * NB + nt], xop[k0 + ks], acc[n0 + nt], 0, 0, 0);
         __builtin_amdgcn_s_setprio(0);
     }
 }

@@ -157,6 +157,8 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
     typedef MlpCfg<H> M;
     constexpr bool FUSE_DN = FUSE && 4 * H <= 1024;
     constexpr int CS = M::CS, KS = M::KS, NTS = M::NTS, HS = M::HS, NTU = M::NTU, SC = M::SC;
+    // fragments read ahead of their MFMAs: at hidden 512 the accumulators and operands leave room for four
+    constexpr int MAXF = H == 512 ? 4 : 8;
     extern __shared__ __align__(16) int8_t smem[];
     int8_t *act = smem + M::WBYTES;
     // The GELU table is read through an LDS address formed from the index itself plus a constant offset, which assumes
@@ -340,7 +342,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 for (int u = 0; u < M::OU; u++) {
                     const int8_t *cur = w_acquire(ws);
                     if (u + 1 < M::OU) pf_o(u + 1); else pf_up(0, 0);
-                    mfma_cols<M::PRO / 2, NTS>(acc, aop + u * (M::PRO / 2), cur, H, col0, laneA);
+                    mfma_cols<M::PRO / 2, NTS, MAXF>(acc, aop + u * (M::PRO / 2), cur, H, col0, laneA);
                 }
             }
             perturb_shift_groups<NTS, FUSE>(acc, sbo, oA, col0, c.sigma, c.shift_out, gA);
@@ -406,7 +408,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
             for (int ku = 0; ku < M::UPU; ku++) {
                 const int8_t *cur = w_acquire(ws);
                 if (ku + 1 < M::UPU) pf_up(s, ku + 1); else pf_dn(s, 0);
-                mfma_cols<M::PRUP / 2, NTU>(au, nrm + ku * (M::PRUP / 2), cur, SC, tm.cs * 32 * NTU, laneL);
+                mfma_cols<M::PRUP / 2, NTU, MAXF>(au, nrm + ku * (M::PRUP / 2), cur, SC, tm.cs * 32 * NTU, laneL);
             }
             v4i mid[CS * NTU];
             {
@@ -464,7 +466,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
                 if (du + 1 < M::DNU) pf_dn(s, du + 1);
                 else if (it + 1 < M::NSUB) pf_up(sub_chunk(it + 1), 0);
                 else if (pass + 1 < npass) pf_pass_first();
-                mfma_cols<M::PRDN / 2, NTS>(accd, mid + du * (M::PRDN / 2), cur, H, col0, laneL);
+                mfma_cols<M::PRDN / 2, NTS, MAXF>(accd, mid + du * (M::PRDN / 2), cur, H, col0, laneL);
             }
         }
         int laneB = lane;

@@ -313,7 +313,9 @@ int  egg_gru_losses(egg_gru_ctx *ctx, int32_t *host_loss, int32_t *host_fit);  /
 /* per-kernel-class timing with hipEvent pairs recorded on the context's stream around each launch (the
  * reference only splits Fwd/Host/Upd wall time, full_cuda_train_egg.cu:1116-1126).  Not usable while capturing. */
 enum { EGG_K_MLP_FIRST = 0, EGG_K_QKV = 1, EGG_K_ATTN = 2, EGG_K_MLP = 3, EGG_K_HEAD = 4,
-       EGG_K_UPDATE_MATRIX = 5, EGG_K_UPDATE_VECTOR = 6, EGG_K_PLINEAR = 7, EGG_KCLASS_COUNT = 8 };
+       EGG_K_UPDATE_MATRIX = 5, EGG_K_UPDATE_VECTOR = 6, EGG_K_PLINEAR = 7,
+       EGG_K_MUON_NS = 8 /* the Newton-Schulz chain of a Muon batch; votes, momentum and apply count as UPDATE_MATRIX */,
+       EGG_KCLASS_COUNT = 9 };
 int  egg_ctx_enable_timing(egg_ctx *ctx, int enable);
 int  egg_timing_reset(egg_ctx *ctx);
 int  egg_timing_get(egg_ctx *ctx, int kclass, int64_t *launches, double *total_ms);   /* synchronises */
