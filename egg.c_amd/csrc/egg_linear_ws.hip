@@ -61,6 +61,11 @@ __device__ __forceinline__ int pack_bytes(int a, int b, int c, int d) {
     return (int)(__builtin_amdgcn_perm((unsigned)b, (unsigned)a, 0x0c0c0400u) | __builtin_amdgcn_perm((unsigned)d, (unsigned)c, 0x04000c0cu));
 }
 
+// bytes 1 of four values side by side
+__device__ __forceinline__ int pack_bytes1(int a, int b, int c, int d) {
+    return (int)(__builtin_amdgcn_perm((unsigned)b, (unsigned)a, 0x0c0c0501u) | __builtin_amdgcn_perm((unsigned)d, (unsigned)c, 0x05010c0cu));
+}
+
 // s_waitcnt vmcnt(n) for a run-time n (wave-uniform), n <= 63
 __device__ __forceinline__ void wait_vmcnt_upto(int n) {
 #define W_(c) case c: __builtin_amdgcn_s_waitcnt(0x0F70 | ((c) & 15) | (((c) >> 4) << 14)); break;
@@ -74,11 +79,15 @@ __device__ __forceinline__ void wait_vmcnt_upto(int n) {
 #undef W_
 }
 
-// MODE: 0 = the shared-weight product alone (no rank-1 term), 1 = perturbed, 2 = perturbed with the fused shift
+// MODE: 0 = the shared-weight product alone (no rank-1 term), 1 = perturbed, 2 = perturbed with the fused shift,
+// 3 = the shared-weight product alone with int8 results and a shift of exactly 8: the accumulator is clamped where it
+// stands (to [-127 * 256, 127 * 256 + 255]) and the result is its second byte, which the pack's byte permute picks,
+// so the shift costs no instruction
 template <int K, int N, bool OUT32, int MODE>
 __global__ void __launch_bounds__(EGG_THREADS, 1) k_plinear_ws(PlinParams p) {
     typedef PlinWS<K, N> P;
-    constexpr bool PLAIN = MODE == 0, FUSE = MODE == 2;
+    constexpr bool PLAIN = MODE == 0 || MODE == 3, FUSE = MODE == 2, BYTE1 = MODE == 3;
+    static_assert(!(BYTE1 && OUT32), "the byte-pick form packs int8 results");
     constexpr int KS = P::KS, NCT = P::NCT, NW = P::NW, CB = P::CB, NSLOT = P::NSLOT, PF = P::PF, NTAB = P::NTAB;
     constexpr int STORES = OUT32 ? NCT * 4 : NCT;                 // global store instructions per tile and wave
     constexpr int MID = KS / 2;                                   // k-step in front of which the tile's barrier sits
@@ -206,6 +215,7 @@ __global__ void __launch_bounds__(EGG_THREADS, 1) k_plinear_ws(PlinParams p) {
     // rank-1 term, clip for int8), ep_emit packs the four into the stage; the int32 form stores a 32 x 32 tile after
     // its fourth slice.
     auto ep_value = [&](int accv, int a, int sbv) -> int {
+        if (BYTE1) return min(127 * 256 + 255, max(-127 * 256, accv));
         const int o = PLAIN ? (accv >> p.shift) : ws_perturbed<FUSE>(accv, sbv, a, p.sigma, p.shift);
         return OUT32 ? o : clip127(o);
     };
@@ -227,7 +237,7 @@ __global__ void __launch_bounds__(EGG_THREADS, 1) k_plinear_ws(PlinParams p) {
                 wave_lds_fence();
             }
         } else {
-            o8[q] = pack_bytes(o[0], o[1], o[2], o[3]);
+            o8[q] = BYTE1 ? pack_bytes1(o[0], o[1], o[2], o[3]) : pack_bytes(o[0], o[1], o[2], o[3]);
             if (q == 3) {
                 const v4i v = {o8[0], o8[1], o8[2], o8[3]};
                 *reinterpret_cast<v4i *>(p.Y8 + (row0 + j) * N + wave * NW + 32 * ct + 16 * g) = v;
@@ -424,7 +434,8 @@ static hipError_t launch_ws_kn(const PlinParams &p, hipStream_t s) {
     const int mode = p.plain ? 0 : (fuse ? 2 : 1);
     hipError_t e = hipSuccess;
     if (p.Y32) e = mode == 0 ? launch_ws<K, N, true, 0>(p, s) : (mode == 1 ? launch_ws<K, N, true, 1>(p, s) : launch_ws<K, N, true, 2>(p, s));
-    if (e == hipSuccess && p.Y8) e = mode == 0 ? launch_ws<K, N, false, 0>(p, s) : (mode == 1 ? launch_ws<K, N, false, 1>(p, s) : launch_ws<K, N, false, 2>(p, s));
+    if (e == hipSuccess && p.Y8) e = mode == 0 ? (p.shift == 8 ? launch_ws<K, N, false, 3>(p, s) : launch_ws<K, N, false, 0>(p, s))
+                                               : (mode == 1 ? launch_ws<K, N, false, 1>(p, s) : launch_ws<K, N, false, 2>(p, s));
     return e;
 }
 // shapes the W-stationary kernel is built for
