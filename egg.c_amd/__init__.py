@@ -51,7 +51,7 @@ EXPORTS = [
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
-    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_muon_plan", "egg_newton_schulz_static",
+    "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_muon_plan", "egg_ctx_generate_kv_cache", "egg_newton_schulz_static",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
     "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
     "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
@@ -410,6 +410,10 @@ class Context:
         """The same with d-eggs' sampler: temperature, min-p filter and presence penalty (its defaults)."""
         self._ck(lib().egg_generate_deggs(self._h, C.c_void_p(d_buffer), seed_len, gen_len, seed & 0xFFFFFFFF, temp, min_p, penalty),
                  "egg_generate_deggs")
+
+    def generate_kv_cache(self, on=True):
+        """egg_generate / egg_generate_deggs with (default) or without the per-layer K / V cache; same tokens either way."""
+        self._ck(lib().egg_ctx_generate_kv_cache(self._h, 1 if on else 0), "egg_ctx_generate_kv_cache")
 
     def enable_taps(self, on=True):
         self._ck(lib().egg_ctx_enable_taps(self._h, 1 if on else 0), "egg_ctx_enable_taps")

@@ -67,6 +67,7 @@ struct egg_ctx {
     double t_ms[EGG_KCLASS_COUNT] = {0}; long t_n[EGG_KCLASS_COUNT] = {0};
     // generation (egg_generate): token buffer [T + 1], logits of one member [T][vocab], a zero start index / seed
     uint8_t *d_gen_tok = nullptr; int32_t *d_gen_logits = nullptr; Scalars *d_gen_scal = nullptr;
+    int8_t *d_gen_kv = nullptr; bool gen_kv_cache = true;      // per-layer K / V rows of the generated sequence (egg_ctx_generate_kv_cache)
     int mask_override = -1; int32_t *logits_override = nullptr;
     bool first_dedup = true;        // first block once per distinct byte value of a member's window (egg_ctx_first_block_dedup)
     VecDesc *d_vec_desc = nullptr; int n_vec = 0, vec_total = 0;       // all vector tensors, for the one-launch update
@@ -257,7 +258,7 @@ static void free_all(egg_ctx *ctx) {
     void *ptrs[] = {ctx->muon.x, ctx->muon.swap, ctx->muon.bterm, ctx->muon.partials, ctx->muon.norm,
                     ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
-                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal, ctx->d_vec_desc,
+                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal, ctx->d_gen_kv, ctx->d_vec_desc,
                     ctx->d_overlay, ctx->d_overlay_q, ctx->d_flags, ctx->d_ov_segs};
     for (void *p : ptrs) if (p) (void)hipFree(p);
     for (auto &sp : ctx->spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
@@ -625,6 +626,7 @@ static FwdCommon make_common(egg_ctx *ctx, const uint8_t *d_data, int64_t len, c
     f.data = d_data; f.data_len = len; f.d_start_idx = d_start; f.d_step_seed = d_seed;
     f.pop_offset = first_member; f.n_members = nm; f.population = c.population; f.same_data = c.use_same_data != 0;
     f.T = c.seq_len; f.H = c.hidden; f.head_dim = c.head_dim; f.vocab = c.vocab;
+    f.t0 = 0; f.tn = c.seq_len;
     f.sigma = c.fixed_point + c.sigma_shift; f.sigma_vec = c.sigma_shift_vector;
     f.mask = ctx->mask_override >= 0 ? ctx->mask_override : noise_word(c);
     f.shift_attn = c.shift_attn; f.shift_out = c.shift_out; f.shift_logit = c.shift_logit;
@@ -639,8 +641,12 @@ static int8_t *tap_ptr(egg_ctx *ctx, int slot) {
     return ctx->d_tap + (size_t)slot * ctx->tap_members * ctx->cfg.seq_len * ctx->cfg.hidden;
 }
 
+// `range` (generation only): evaluate the token positions [t0, t0 + tn) of the chunk's members and keep every layer's
+// K / V rows in `kv` ([layer][K, V][nm][T][H]) instead of the shared k / v buffers, so that a later call on a later
+// range finds the rows of the positions in front of it (the reference's d_gen_kv, mgpu.cu:1160-1170)
+struct FwdRange { int t0, tn; int8_t *kv; };
 static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const int64_t *d_start, const uint32_t *d_seed,
-                         int first_member, int nm) {
+                         int first_member, int nm, const FwdRange *range = nullptr) {
     const egg_config &c = ctx->cfg; const Layout &L = ctx->L; const int8_t *M = ctx->d_model; const int H = c.hidden;
     const int8_t *F = ctx->d_wfrag;
     const int8_t *Q = ctx->adaptive ? ctx->d_overlay_q : nullptr;      // same offsets as the model blob
@@ -648,6 +654,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
     const bool taps = ctx->taps && nm <= ctx->tap_members;
     const size_t act_bytes = (size_t)nm * c.seq_len * H;
     FwdCommon f = make_common(ctx, d_data, len, d_start, d_seed, first_member, nm);
+    if (range) { f.t0 = range->t0; f.tn = range->tn; }
     {
         MlpParams p; memset(&p, 0, sizeof(p)); p.c = f; p.seed_base = 0;
         p.off_ln_a = OFF_LN_INIT_A; p.off_ln_b = OFF_LN_INIT_B; p.off_lnb_a = OFF_LN_INIT_BIAS_A; p.off_lnb_b = OFF_LN_INIT_BIAS_B;
@@ -656,7 +663,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = F + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
         p.w_dn = F + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
         p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
-        p.tab = ctx->first_dedup ? ctx->d_q : nullptr;     // the q buffer is free until the first layer's QKV projection writes it
+        p.tab = (ctx->first_dedup && !range) ? ctx->d_q : nullptr;     // the q buffer is free until the first layer's QKV projection writes it
         if (Q) {
             p.q_ln_w = Q + L.ln_init; p.q_ln_b = Q + L.ln_init_bias; p.q_b_up = Q + L.mlp_emb_bias_up; p.q_b_dn = Q + L.mlp_emb_bias_down;
             p.q_up = Q + L.w_emb_mlp_up; p.q_dn = Q + L.w_emb_mlp_down; p.q_emb = Q + L.embedding; p.q_emb_bias = Q + L.emb_bias;
@@ -671,6 +678,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
             p.ln_w = M + L.ln_1 + (int64_t)l * H; p.ln_b = M + L.ln_1_bias + (int64_t)l * H;
             p.w_q = F + L.w_q + l * hh; p.w_k = F + L.w_k + l * hh; p.w_v = F + L.w_v + l * hh;
             p.x = ctx->d_x; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v;
+            if (range && range->kv) { p.k = range->kv + (size_t)(2 * l) * act_bytes; p.v = range->kv + (size_t)(2 * l + 1) * act_bytes; }
             if (Q) {
                 p.q_ln_w = Q + L.ln_1 + (int64_t)l * H; p.q_ln_b = Q + L.ln_1_bias + (int64_t)l * H;
                 p.q_wq = Q + L.w_q + l * hh; p.q_wk = Q + L.w_k + l * hh; p.q_wv = Q + L.w_v + l * hh;
@@ -684,6 +692,7 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         }
         {
             AttnParams p; memset(&p, 0, sizeof(p)); p.c = f; p.q = ctx->d_q; p.k = ctx->d_k; p.v = ctx->d_v; p.ao = ctx->d_ao;
+            if (range && range->kv) { p.k = range->kv + (size_t)(2 * l) * act_bytes; p.v = range->kv + (size_t)(2 * l + 1) * act_bytes; }
             { SpanScope span(ctx, EGG_K_ATTN); HIP_TRY(egg_launch_attn(p, s)); }
             if (taps) HIP_TRY(hipMemcpyAsync(tap_ptr(ctx, 1 + 6 * l + 3), ctx->d_ao, act_bytes, hipMemcpyDeviceToDevice, s));
         }
@@ -1008,9 +1017,13 @@ extern "C" uint32_t egg_next_seed(uint32_t seed, uint64_t step) {
 
 // ------------------------------------------------------------------ taps
 // generate_sequence_kernel (mgpu.cu:1154-1283) and its call site (:1701-1708).  The reference walks the sequence
-// token by token with a KV cache; here every new token re-runs the unperturbed forward of one member over the whole
-// window (noise mask 0 makes every perturbation term vanish, i.e. noise_sign = 0) and samples from the logits of
-// position t.  Causality makes the logits at t independent of the not yet generated tail.
+// token by token with a per-layer KV cache (d_gen_kv).  Here the unperturbed forward of one member (noise mask 0 makes
+// every perturbation term vanish, i.e. noise_sign = 0) runs once over the whole window for the prompt and fills every
+// layer's K / V rows; each new token then re-evaluates only the 32-token tile that holds position t -- embedding,
+// projections, the tile's queries against the cached K / V rows of everything in front of them, MLP, head -- and
+// samples from the logits of position t.  Causality makes what position t sees independent of the not yet generated
+// tail, and a tile's K / V rows are final once its last position has been generated.  With the cache switched off
+// (egg_ctx_generate_kv_cache) every new token re-runs the whole window instead; the tokens are the same.
 struct DeggsSampling { float temp; int min_p_limit, penalty_int; };
 static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed, const DeggsSampling *de) {
     if (!ctx || !d_buffer) return EGG_E_INVALID;
@@ -1023,6 +1036,7 @@ static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_
         HIP_TRY(hipMalloc(&ctx->d_gen_logits, (size_t)T * c.vocab * 4));
         HIP_TRY(hipMalloc(&ctx->d_gen_scal, sizeof(Scalars)));
         HIP_TRY(hipMemset(ctx->d_gen_scal, 0, sizeof(Scalars)));
+        HIP_TRY(hipMalloc(&ctx->d_gen_kv, (size_t)c.n_layers * 2 * T * c.hidden));
     }
     HIP_TRY(egg_launch_zero_u64(reinterpret_cast<unsigned long long *>(ctx->d_gen_tok), (T + 16) / 8, s));   // a fill kernel, not a memset node: a caller may be capturing this stream
     HIP_TRY(hipMemcpyAsync(ctx->d_gen_tok, d_buffer, (size_t)seed_len, hipMemcpyDeviceToDevice, s));
@@ -1032,7 +1046,10 @@ static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_
     int rc = EGG_OK;
     for (int t = seed_len - 1; t < total - 1 && rc == EGG_OK; t++) {
         // data_len = T + 1 puts the member's stream position at 0 (mgpu.cu:864-870 with len - T == 1)
-        rc = forward_chunk(ctx, ctx->d_gen_tok, (int64_t)T + 1, &ctx->d_gen_scal->start, &ctx->d_gen_scal->seed, 0, 1);
+        FwdRange range = {0, T, ctx->d_gen_kv};
+        if (t > seed_len - 1) { range.t0 = t & ~31; range.tn = 32; }       // the prompt: whole window; then the tile of position t
+        rc = forward_chunk(ctx, ctx->d_gen_tok, (int64_t)T + 1, &ctx->d_gen_scal->start, &ctx->d_gen_scal->seed, 0, 1,
+                           ctx->gen_kv_cache ? &range : nullptr);
         if (rc == EGG_OK) {
             const int32_t *row = ctx->d_gen_logits + (size_t)t * c.vocab;
             hipError_t e = de ? egg_launch_sample_deggs(row, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_tok, de->temp, de->min_p_limit, de->penalty_int,
@@ -1044,6 +1061,11 @@ static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_
     ctx->mask_override = -1; ctx->logits_override = nullptr; ctx->taps = taps;
     if (rc) return rc;
     HIP_TRY(hipMemcpyAsync(d_buffer, ctx->d_gen_tok, (size_t)total, hipMemcpyDeviceToDevice, s));
+    return EGG_OK;
+}
+extern "C" int egg_ctx_generate_kv_cache(egg_ctx *ctx, int enable) {
+    if (!ctx) return EGG_E_INVALID;
+    ctx->gen_kv_cache = enable != 0;
     return EGG_OK;
 }
 extern "C" int egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed) {

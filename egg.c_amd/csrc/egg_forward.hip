@@ -9,6 +9,7 @@
 //   k_attn<HD,CT>   causal exp-LUT attention core          (mgpu.cu:787-825)
 //   k_mlp<H,false>  O-projection + residual norm + MLP     (mgpu.cu:827-831, :708-759)
 //   k_head<H>       final norm + tied head + loss          (mgpu.cu:955-1028)
+#include <algorithm>
 #include "egg_device.h"
 #include "egg_params.h"
 #include "egg_launch.h"
@@ -168,7 +169,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const FwdCommon &c = p.c;
     const int T = c.T;
-    const TileMap tm = tile_map<CS>(T, wave, blockIdx.x);
+    const TileMap tm = tile_map<CS>(c.tn, wave, blockIdx.x);
     const int col0 = tm.cs * HS;                      // first output column of this wave's slice
     constexpr int PSET = M::per_set(FIRST);
     constexpr bool UPA32 = !FIRST;
@@ -300,7 +301,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
         int laneA = lane;
         asm volatile("" : "+v"(laneA));
         const int gA = laneA >> 5, jA = laneA & 31;
-        const int t = (tm.tile0 + M::TPW * pass) * 32 + jA;     // token position; with dedup, row of the table
+        const int t = c.t0 + (tm.tile0 + M::TPW * pass) * 32 + jA;     // token position; with dedup, row of the table
         const size_t row = ((size_t)mloc * T + t) * H;
         int8_t *xrow = (FIRST && dedup ? p.tab : p.x) + row + col0;   // this wave's slice of the residual row
         v4i xs[NTS];
@@ -564,7 +565,7 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const FwdCommon &c = p.c;
     const int T = c.T;
-    const TileMap tm = tile_map<CS>(T, wave, blockIdx.x);
+    const TileMap tm = tile_map<CS>(c.tn, wave, blockIdx.x);
     const int col0 = tm.cs * HS;
     int8_t *tb = smem + Q::WBYTES + tm.set * Q::PER_SET;
     int *lnw = reinterpret_cast<int *>(tb), *lnb = lnw + H;
@@ -611,7 +612,7 @@ __global__ void __launch_bounds__(EGG_THREADS, ADAPT ? 2 : QkvCfg<H>::OCC) k_qkv
     if (!valid) mloc = c.n_members - 1;
 
     for (int pass = 0; pass < tm.passes; pass++) {
-        const int t = (tm.tile0 + Q::TPW * pass) * 32 + j;
+        const int t = c.t0 + (tm.tile0 + Q::TPW * pass) * 32 + j;
         const size_t row = ((size_t)mloc * T + t) * H;
         v4i nrm[KS];
         {
@@ -799,7 +800,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (CT > 8 ? 1 : 2)) k_attn(AttnPara
     };
 
 #pragma unroll 1
-    for (int qt = 0; qt < CT; qt++) {
+    for (int qt = c.t0 >> 5; qt < ((c.t0 + c.tn) >> 5); qt++) {
         const int t = qt * 32 + j;
         v4i qop[KS];
 #pragma unroll
@@ -991,6 +992,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (AttnWg<HD, CT>::OCC)) k_attn_wg(
 #pragma unroll 1
     for (int qi = 0; qi < CT / 4; qi++) {
         const int qt = (qi >> 1) * 8 + ((qi & 1) ? 7 - wave : wave);
+        if (qt * 32 < c.t0 || qt * 32 >= c.t0 + c.tn) continue;      // (wave-uniform; the loop holds no barrier)
         const int t = qt * 32 + j;
         v4i qop[KS];
 #pragma unroll
@@ -1123,7 +1125,8 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
 
     const int64_t spos = stream_pos_of(c, member);
     long long wave_loss = 0;
-    for (int pass = 0; pass < T / 32; pass++) {
+    const int pass_end = (c.t0 + c.tn) >> 5;
+    for (int pass = c.t0 >> 5; pass < pass_end; pass++) {
         const int t = pass * 32 + j;
         const size_t row = ((size_t)mloc * T + t) * H;
         v4i x[KS], nf[KS];
@@ -1133,7 +1136,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
         const int sbh = ADAPT ? dot_noise_ov<KS, false>(nf, hB, p.q_emb, 0, g) : dot_noise<KS, false>(nf, hB, 0, g);
         v16i acc[NV];
         zero_acc<NV>(acc);
-        gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, ws, (pass + 1 < T / 32) ? w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0) : nullptr, lane);
+        gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, ws, (pass + 1 < pass_end) ? w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0) : nullptr, lane);
         add_perturb<NV>(acc, sbh, hA, 0, c.sigma, g);
         // two-pass softmax statistics (mgpu.cu:969-1009)
         int gmax = INT_MIN;
@@ -1186,7 +1189,7 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
 // ============================================================================ host launchers
 template <int H>
 static hipError_t launch_mlp_h(const MlpParams &p, bool first, hipStream_t s) {
-    const int sets = tile_map_sets(p.c.T, MlpCfg<H>::CS);
+    const int sets = tile_map_sets(p.c.tn, MlpCfg<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = MlpCfg<H>::total(sets, first);
     // The up accumulator is seeded with (bias + 128 + noise) << shift_mlp_up (see the bias table), so its range is the
@@ -1217,7 +1220,7 @@ hipError_t egg_launch_mlp(const MlpParams &p, bool first, hipStream_t s) {
 
 template <int H>
 static hipError_t launch_qkv_h(const QkvParams &p, hipStream_t s) {
-    const int sets = tile_map_sets(p.c.T, QkvCfg<H>::CS);
+    const int sets = tile_map_sets(p.c.tn, QkvCfg<H>::CS);
     dim3 grid((p.c.n_members + sets - 1) / sets), block(EGG_THREADS);
     size_t lds = QkvCfg<H>::total(sets);
     if (p.q_ln_w) hipLaunchKernelGGL((k_qkv<H, true>), grid, block, lds, s, p);
@@ -1298,8 +1301,9 @@ static hipError_t no_static_lds(K kern) {
 }
 template <int H>
 static hipError_t prepare_h(int T) {
-    const int sets = tile_map_sets(T, QkvCfg<H>::CS);
-    const int msets = tile_map_sets(T, MlpCfg<H>::CS);
+    // table sets per workgroup: the whole window's, or a single tile's (egg_generate evaluates one tile per new token)
+    const int sets = std::max(tile_map_sets(T, QkvCfg<H>::CS), tile_map_sets(32, QkvCfg<H>::CS));
+    const int msets = std::max(tile_map_sets(T, MlpCfg<H>::CS), tile_map_sets(32, MlpCfg<H>::CS));
     for (hipError_t e : {no_static_lds(&k_mlp<H, true, true, false>), no_static_lds(&k_mlp<H, false, true, false>),
                          no_static_lds(&k_mlp<H, true, false, false>), no_static_lds(&k_mlp<H, false, false, false>),
                          no_static_lds(&k_mlp<H, true, false, true>), no_static_lds(&k_mlp<H, false, false, true>)})

@@ -45,6 +45,8 @@ struct FwdCommon {
     int population;
     int same_data;               // USE_SAME_DATA: every pair reads the window at the start index
     int T, H, head_dim, vocab;
+    int t0, tn;                  // token positions [t0, t0 + tn) of every member are evaluated (multiples of 32; the whole window: 0, T);
+                                 // attention still reads the K / V rows of every position in front of them
     int sigma;                   // fixed_point + sigma_shift
     int sigma_vec;               // sigma_shift_vector
     int mask;                    // noise magnitude mask

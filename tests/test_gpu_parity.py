@@ -584,8 +584,11 @@ def test_muon_batched_update_equals_per_matrix_update(pkg, orc, dev, kw):
 
 @pytest.mark.parametrize("kw,seed_len,gen_len", [(dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4), 5, 27),
                                                  (dict(hidden=128, head_dim=32, n_layers=2, seq_len=64, population=4), 10, 30),
-                                                 (dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4), 16, 40)],
-                         ids=["h64", "h128", "h256"])
+                                                 (dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4), 16, 40),
+                                                 # the workgroup-per-head attention kernel (sequence 256 / 512), continuations that cross tile ends
+                                                 (dict(hidden=256, head_dim=64, n_layers=2, seq_len=256, population=2), 90, 40),
+                                                 (dict(hidden=512, head_dim=64, n_layers=1, seq_len=512, population=2), 60, 10)],
+                         ids=["h64", "h128", "h256", "h256_t256", "h512_t512"])
 def test_generate(pkg, orc, dev, kw, seed_len, gen_len):
     """Sampling continuation of a prompt by the unperturbed model against the oracle's token-by-token restatement."""
     import torch
@@ -610,6 +613,22 @@ def test_generate(pkg, orc, dev, kw, seed_len, gen_len):
     got = buf.cpu().numpy()
     assert np.array_equal(got, ref), (got.tolist(), ref.tolist())
     assert len(set(ref[seed_len:].tolist())) > 3      # the continuation is not degenerate
+    # without the per-layer K / V cache (every new token re-evaluates the whole window): the same tokens
+    ctx.generate_kv_cache(False)
+    buf2 = torch.zeros(seed_len + gen_len, dtype=torch.uint8, device=dev)
+    buf2[:seed_len] = _t(dev, prompt)
+    ctx.generate(buf2.data_ptr(), seed_len, gen_len, 1041)
+    ctx.sync()
+    assert np.array_equal(buf2.cpu().numpy(), ref)
+    ctx.generate_kv_cache(True)
+    # a second call on the same context starts from a fresh cache: another prompt, shorter continuation
+    prompt2 = orc.zipf_bytes(4096)[900:900 + seed_len].copy()
+    buf3 = torch.zeros(seed_len + gen_len, dtype=torch.uint8, device=dev)
+    buf3[:seed_len] = _t(dev, prompt2)
+    ctx.generate(buf3.data_ptr(), seed_len, max(1, gen_len // 2), 7)
+    ctx.sync()
+    n2 = seed_len + max(1, gen_len // 2)
+    assert np.array_equal(buf3.cpu().numpy()[:n2], orc.generate(ocfg, model, prompt2, max(1, gen_len // 2), 7))
     # a population forward afterwards is unaffected by the generation's mask / logits overrides
     data = orc.zipf_bytes(1 << 14)
     d_loss = torch.zeros(kw["population"], dtype=torch.int32, device=dev)
