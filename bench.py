@@ -254,7 +254,9 @@ def main():
         gctx.losses()
         sec = time.perf_counter() - t0
         gru = {"value": gcfg.population * gcfg.seq_len / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3,
-               "workload": "full_trained_egg.c defaults, one full step (forward of 128 members x 4096 tokens + update)"}
+               "workload": "full_trained_egg.c defaults, one full step (forward of 128 members x 4096 tokens + update)",
+               "note": "the bit-exact GPU twin of the CPU baseline's program, not a throughput path: 128 members of 4096 strictly sequential "
+                       "tokens fill four workgroups of the 256 CUs"}
         gctx.close()
     except Exception as e:
         gru = {"error": str(e)}
@@ -308,6 +310,8 @@ def main():
               "population": P5,
               "kernel_ms_per_step": {k: round(tm[k][1], 3) for k in fwd if tm[k][0]},
               "kernel_frac_mfma": {k: round(ops_tok[k] * toks * launches[k] / (tm[k][1] * 1e-3) / PEAK_INT8_OPS, 4) for k in fwd if tm[k][1] > 0},
+              "kernel_frac_mfma_note": "algorithmic int8 ops of the shared products at every position over event-timed kernel time, against 5.0 POP/s; "
+                                       "mlp_first evaluates its block once per distinct byte value of a member's window, so its figure is not a pipe utilisation",
               "muon": {"newton_schulz_ms": ns_ms, "matrices": sum(g["members"] for g in groups), "TFLOP/s_fp32": ns_flops / (ns_ms * 1e-3) / 1e12 if ns_ms > 0 else None,
                        "frac_fp32_mfma_peak": ns_flops / (ns_ms * 1e-3) / 157.3e12 if ns_ms > 0 else None,
                        "votes_momentum_apply_ms": tm["update_matrix"][1],
