@@ -533,6 +533,121 @@ __global__ void __launch_bounds__(EGG_THREADS) k_sgemm(const float *A, long lda,
         C[(size_t)i * N + jj] = (mode == 1) ? ((i == jj ? 3.0f : 0.0f) - v) : alpha * v;
     }
 }
+// The same product for M and N that are multiples of 64, with the operands staged once per workgroup through LDS and every
+// output element summed by one wave over the whole of K (no partial tiles to add up).  A workgroup owns a TILE x TILE
+// block of C, TILE = 64 WT: wave (wm, wn) owns the 32 WT x 32 WT quarter as WT x WT MFMA tiles.  A TILE x 32 chunk of A
+// and a 32 x TILE chunk of B go global -> registers -> LDS (the next chunk's loads are in flight while the MFMAs of the
+// current one run); with WT = 2 every value read from LDS feeds two MFMAs and the L2 traffic per flop is a quarter of
+// the 32 x 32 kernel's.  An operand whose k stride is 1 sits in LDS as [row][k] with rows 36 floats apart (16-byte
+// reads of four consecutive k, a 2-way bank conflict at most); the other kind as [k][row] with k rows TILE + 8 floats
+// apart (4-byte reads; the two lane halves, four k rows apart, fall on different banks).
+// Within a block of eight k, MFMA e multiplies the pair {8c + e, 8c + 4 + e}, blocks in ascending order, whatever WT
+// is: the two tile sizes give bit-identical results, so the host may pick by the size of the grid.  Epilogues as above.
+template <bool AK, bool BK, int WT>
+__global__ void __launch_bounds__(EGG_THREADS, 2) k_sgemm_lds(const float *A, long lda, long batch_a, const float *B, long ldb, long batch_b,
+                                                             float *C, int M, int N, int K, float alpha, int mode) {
+    constexpr int TILE = 64 * WT, KC = 32, LDK = 36, LDI = TILE + 8, PIECES = TILE * KC / 4 / EGG_THREADS;
+    constexpr int ASZ = AK ? TILE * LDK : KC * LDI, BSZ = BK ? TILE * LDK : KC * LDI;
+    constexpr int RPI = TILE / 4;                 // 16-byte pieces per k row of an [k][row] chunk
+    __shared__ __align__(16) float As[ASZ];
+    __shared__ __align__(16) float Bs[BSZ];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31, tid = threadIdx.x;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tiles_n = N / TILE, tile = blockIdx.x;
+    const int i0 = (tile / tiles_n) * TILE, j0 = (tile % tiles_n) * TILE;
+    A += (long)blockIdx.y * batch_a; B += (long)blockIdx.y * batch_b; C += (size_t)blockIdx.y * M * N;
+    v16f acc[WT][WT];
+#pragma unroll
+    for (int a = 0; a < WT; a++)
+#pragma unroll
+        for (int b = 0; b < WT; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+    // global -> registers: PIECES 16-byte pieces of each operand's chunk per thread
+    v4f ra[PIECES], rb[PIECES];
+    auto load_chunk = [&](int k0) {
+#pragma unroll
+        for (int p = 0; p < PIECES; p++) {
+            const int idx = tid + EGG_THREADS * p;
+            if (AK) ra[p] = *reinterpret_cast<const v4f *>(A + (long)(i0 + (idx >> 3)) * lda + k0 + 4 * (idx & 7));
+            else ra[p] = *reinterpret_cast<const v4f *>(A + (long)(k0 + idx / RPI) * lda + i0 + 4 * (idx % RPI));
+            if (BK) rb[p] = *reinterpret_cast<const v4f *>(B + (long)(j0 + (idx >> 3)) * ldb + k0 + 4 * (idx & 7));
+            else rb[p] = *reinterpret_cast<const v4f *>(B + (long)(k0 + idx / RPI) * ldb + j0 + 4 * (idx % RPI));
+        }
+    };
+    auto store_chunk = [&]() {
+#pragma unroll
+        for (int p = 0; p < PIECES; p++) {
+            const int idx = tid + EGG_THREADS * p;
+            if (AK) *reinterpret_cast<v4f *>(As + (idx >> 3) * LDK + 4 * (idx & 7)) = ra[p];
+            else *reinterpret_cast<v4f *>(As + (idx / RPI) * LDI + 4 * (idx % RPI)) = ra[p];
+            if (BK) *reinterpret_cast<v4f *>(Bs + (idx >> 3) * LDK + 4 * (idx & 7)) = rb[p];
+            else *reinterpret_cast<v4f *>(Bs + (idx / RPI) * LDI + 4 * (idx % RPI)) = rb[p];
+        }
+    };
+    load_chunk(0);
+    for (int k0 = 0; k0 < K; k0 += KC) {
+        __syncthreads();                    // every wave has finished reading the previous chunk
+        store_chunk();
+        __syncthreads();
+        if (k0 + KC < K) load_chunk(k0 + KC);
+#pragma unroll
+        for (int c = 0; c < KC / 8; c++) {
+            v4f a4[WT], b4[WT];
+#pragma unroll
+            for (int t = 0; t < WT; t++) {
+                const int row = 32 * WT * wm + 32 * t + j, col = 32 * WT * wn + 32 * t + j;
+                if (AK) a4[t] = *reinterpret_cast<const v4f *>(As + row * LDK + 8 * c + 4 * g);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) a4[t][e] = As[(8 * c + 4 * g + e) * LDI + row];
+                }
+                if (BK) b4[t] = *reinterpret_cast<const v4f *>(Bs + col * LDK + 8 * c + 4 * g);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) b4[t][e] = Bs[(8 * c + 4 * g + e) * LDI + col];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int ta = 0; ta < WT; ta++)
+#pragma unroll
+                    for (int tb = 0; tb < WT; tb++)
+                        acc[ta][tb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[ta][e], b4[tb][e], acc[ta][tb], 0, 0, 0);
+        }
+    }
+    // accumulator register r of lane (j, g) is row 8 (r / 4) + 4 g + r % 4, column j of its 32 x 32 tile
+#pragma unroll
+    for (int ta = 0; ta < WT; ta++)
+#pragma unroll
+        for (int tb = 0; tb < WT; tb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = i0 + 32 * WT * wm + 32 * ta + 8 * (r >> 2) + 4 * g + (r & 3), jj = j0 + 32 * WT * wn + 32 * tb + j;
+                const float v = acc[ta][tb][r];
+                C[(size_t)i * N + jj] = (mode == 1) ? ((i == jj ? 3.0f : 0.0f) - v) : alpha * v;
+            }
+}
+template <int WT>
+static hipError_t sgemm_lds(bool ak, bool bk, const float *A, long lda, long batch_a, const float *B, long ldb, long batch_b, float *C,
+                            int M, int N, int K, float alpha, int mode, int batch, hipStream_t s) {
+    const dim3 grid((M / (64 * WT)) * (N / (64 * WT)), batch), block(EGG_THREADS);
+    if (ak && bk) hipLaunchKernelGGL((k_sgemm_lds<true, true, WT>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    else if (ak) hipLaunchKernelGGL((k_sgemm_lds<true, false, WT>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    else if (bk) hipLaunchKernelGGL((k_sgemm_lds<false, true, WT>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    else hipLaunchKernelGGL((k_sgemm_lds<false, false, WT>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
+    return hipGetLastError();
+}
+static int egg_update_cu_count() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n = v;
+        else n = 256;
+    }
+    return n;
+}
 // A(i,k) at A[i * sa_i + k * sa_k], B(k,j) at B[k * sb_k + j * sb_j]; one stride of each pair must be 1 and the other a
 // multiple of 4 (16-byte loads)
 static hipError_t sgemm(const float *A, long sa_i, long sa_k, long batch_a, const float *B, long sb_k, long sb_j, long batch_b, float *C, int M, int N, int K,
@@ -541,6 +656,13 @@ static hipError_t sgemm(const float *A, long sa_i, long sa_k, long batch_a, cons
     if ((!ak && sa_i != 1) || (!bk && sb_j != 1) || M % 32 || N % 32 || K % 32) return hipErrorInvalidValue;
     const long lda = ak ? sa_i : sa_k, ldb = bk ? sb_j : sb_k;
     if (lda % 4 || ldb % 4 || batch_a % 4 || batch_b % 4) return hipErrorInvalidValue;
+    // The LDS-staged kernel where the shape allows it: 128 x 128 tiles when they still fill the GPU, 64 x 64 tiles otherwise
+    // (bit-identical results, so the choice may depend on the batch)
+    if (M % 64 == 0 && N % 64 == 0) {
+        const bool big = M % 128 == 0 && N % 128 == 0 && (long)(M / 128) * (N / 128) * batch >= 2 * egg_update_cu_count();
+        return big ? sgemm_lds<2>(ak, bk, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode, batch, s)
+                   : sgemm_lds<1>(ak, bk, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode, batch, s);
+    }
     const dim3 grid((M / 32) * (N / 32), batch), block(EGG_THREADS);
     if (ak && bk) hipLaunchKernelGGL((k_sgemm<true, true>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);
     else if (ak) hipLaunchKernelGGL((k_sgemm<true, false>), grid, block, 0, s, A, lda, batch_a, B, ldb, batch_b, C, M, N, K, alpha, mode);

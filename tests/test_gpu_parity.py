@@ -550,7 +550,10 @@ def test_muon_update(pkg, orc, dev):
 
 @pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=3, seq_len=32, population=64),
                                 dict(hidden=128, head_dim=32, n_layers=2, seq_len=32, population=32),
-                                dict(hidden=256, head_dim=64, n_layers=5, seq_len=32, population=16)])
+                                dict(hidden=256, head_dim=64, n_layers=5, seq_len=32, population=16),
+                                # shape groups with different batch limits (64 square matrices at once, 16 of each 4:1 shape
+                                # where a group has 17): every group must run at its own limit
+                                dict(hidden=512, head_dim=64, n_layers=16, seq_len=32, population=8)])
 def test_muon_batched_update_equals_per_matrix_update(pkg, orc, dev, kw):
     """egg_es_update sends the Muon matrices of one shape through Newton-Schulz as one batch per stage; what it leaves
     (weights, momentum, accumulators, update count) is bit-identical to updating tensor by tensor."""
