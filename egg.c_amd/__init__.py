@@ -54,7 +54,7 @@ EXPORTS = [
     "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_muon_plan", "egg_ctx_generate_kv_cache", "egg_newton_schulz_static",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
     "egg_gru_model_init", "egg_gru_model_upload", "egg_gru_model_download", "egg_gru_state_reset",
-    "egg_gru_state_download", "egg_gru_step", "egg_gru_losses",
+    "egg_gru_state_download", "egg_gru_step", "egg_gru_losses", "egg_gru_forward_mode",
 ]
 KCLASSES = ["mlp_first", "qkv", "attn", "mlp", "head", "update_matrix", "update_vector", "plinear", "muon_ns"]
 
@@ -596,6 +596,10 @@ class GruContext:
         out = np.zeros(self.model_bytes(), np.int8)
         self._ck(lib().egg_gru_model_download(self._h, _np_ptr(out), out.nbytes), "egg_gru_model_download")
         return out
+
+    def forward_mode(self, staged=True):
+        """one launch per stage over the whole GPU (default) or one persistent workgroup per 32 members; same results"""
+        self._ck(lib().egg_gru_forward_mode(self._h, 1 if staged else 0), "egg_gru_forward_mode")
 
     def state_reset(self):
         self._ck(lib().egg_gru_state_reset(self._h), "egg_gru_state_reset")

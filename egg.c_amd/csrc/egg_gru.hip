@@ -361,6 +361,281 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
     if (wave == 0 && g == 0) p.loss[member] = loss;
 }
 
+// ============================================================================ the same forward, one launch per stage
+// k_gru_forward keeps a member tile on one workgroup for the whole sequence, so four workgroups stream every weight
+// once per token from L2 and the rest of the GPU idles.  Here every dependent stage of a token is a launch of its own
+// whose grid spreads the output strips (32 rows of W) and the member tiles (32 members) over the CUs: a wave owns one
+// (strip, tile) pair, reads its W fragments and the members' input rows straight from global memory and writes its 32 x
+// 32 results back.  Activations live in global memory in slot order ([member][K]); the recurrent state stays in natural
+// order like the reference's.  The stages of one token are captured once as a hipGraph and launched seq_len times; the
+// token index and the step's arguments sit in device memory (GruStep).  Same arithmetic helpers, bit-identical results.
+// t: tokens finished (what the embedding stage reads); t_next = t + 1, written by the embedding stage for the head's target
+// lookup; the head hands it back as t when it is done.  Each is written only while no other stage of the token reads it.
+struct GruStep { const uint8_t *data; long long data_len, start_idx; int t, t_next, arrived; };
+struct GruStage {
+    const GruMat *mats;
+    const int8_t *model, *frag, *noise;
+    GruStep *step;
+    int8_t *states, *x, *xn, *gate, *ft, *m2, *mb;
+    int32_t *loss;
+    int H, L, V, T, population, sigma;
+    long long off_emb, off_gru_b, off_ln_w, off_ln_out;
+    const int32_t *exp2;
+};
+__device__ __forceinline__ long long gs_stream_pos(const GruStage &p, const GruStep &st, int member) {
+    const long long stride = st.data_len / (p.population / 2);                    // egg.c:553-554
+    return (st.start_idx + (long long)(member >> 1) * stride) % (st.data_len - p.T);
+}
+
+// KSN k-steps of a strip product starting at k-step ks0: acc += W[strip rows, k] . in[member, k], xb += in . B.
+// `in` is the lane's member row; SLOT: slot order (16 bytes of a k-step's lane half are contiguous) or natural order.
+template <int KSN, bool SLOT>
+__device__ __forceinline__ void gs_strip(v16i &acc, int &xb, const int8_t *ftile, const int8_t *in_row, const int8_t *bvec, int ks0, int lane) {
+    constexpr int BATCH = KSN < 8 ? KSN : 8;
+    static_assert(KSN % BATCH == 0, "k-steps come in whole batches");
+    const int j = lane & 31, g = lane >> 5;
+    const int8_t *fa = ftile + ((size_t)g * 32 + j) * 16;
+#pragma unroll 1
+    for (int k0 = 0; k0 < KSN; k0 += BATCH) {
+        v4i a[BATCH], b[BATCH], n[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; u++) {
+            const int ks = ks0 + k0 + u;
+            a[u] = *reinterpret_cast<const v4i *>(fa + (size_t)ks * 1024);
+            n[u] = *reinterpret_cast<const v4i *>(bvec + 32 * ks + 16 * g);
+            if (SLOT) b[u] = *reinterpret_cast<const v4i *>(in_row + 32 * ks + 16 * g);
+            else {
+                const int *r32 = reinterpret_cast<const int *>(in_row + 32 * ks);
+#pragma unroll
+                for (int q = 0; q < 4; q++) b[u][q] = r32[2 * q + g];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; u++) {
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u], b[u], acc, 0, 0, 0);
+#pragma unroll
+            for (int q = 0; q < 4; q++) xb = dot4(b[u][q], n[u][q], xb);
+        }
+    }
+}
+// one whole perturbed product of matrix mi for strip nt and the lane's member: the 16 packed int8 results (slot order)
+template <int KS, bool SLOT>
+__device__ __forceinline__ v4i gs_matmul(const GruStage &p, int mi, int nt, const int8_t *in_row, int member, int lane) {
+    const GruMat m = p.mats[mi];
+    const int pair = member >> 1, ns = (member & 1) ? -1 : 1, g = lane >> 5;
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+    int xb = 0;
+    gs_strip<KS, SLOT>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (KS * 32), in_row, p.noise + m.b_off + (long long)pair * (KS * 32), 0, lane);
+    xb = sum_halves(xb);
+    return gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g);
+}
+
+// egg_ln (egg.c:180-210) of every member's row, optionally after the embedding lookup (egg.c:238).  A lane owns one
+// 16-byte piece (32-group nt, half g) of one member's row; the H / 16 lanes of a member sit side by side.
+template <int H, bool EMBED>
+__global__ void __launch_bounds__(256) k_gs_ln(GruStage p, long long w_off) {
+    constexpr int PPM = H / 16;                     // pieces (lanes) per member
+    const int id = blockIdx.x * 256 + threadIdx.x, member = id / PPM, piece = id % PPM, nt = piece >> 1, g = piece & 1;
+    if (member >= p.population) return;            // whole waves only: population * PPM is a multiple of 64
+    const GruStep st = *p.step;
+    v4i x;
+    int8_t *xrow = p.x + (size_t)member * H + 32 * nt + 16 * g;
+    if (EMBED) {
+        const int tok = st.data[gs_stream_pos(p, st, member) + st.t];
+        const int *e = reinterpret_cast<const int *>(p.model + p.off_emb + (size_t)tok * H + 32 * nt);
+#pragma unroll
+        for (int q = 0; q < 4; q++) x[q] = e[2 * q + g];
+        *reinterpret_cast<v4i *>(xrow) = x;
+        if (id == 0) p.step->t_next = st.t + 1;
+    } else x = *reinterpret_cast<const v4i *>(xrow);
+    int sum = 0;
+#pragma unroll
+    for (int q = 0; q < 4; q++) sum = sumabs4(x[q], sum);
+#pragma unroll
+    for (int off = 1; off < PPM; off <<= 1) sum += __shfl_xor(sum, off, 64);
+    if (sum == 0) sum = 1;
+    int mean = sum / H; if (mean == 0) mean = 1;
+    const float rcp = 1.0f / (float)mean;
+    const int8_t *w = p.model + w_off;
+    v4i out;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int w4 = *reinterpret_cast<const int *>(w + 32 * nt + 8 * q + 4 * g);
+        int o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(sx8(x[q], e) * sx8(w4, e), rcp));
+        out[q] = pack4(o[0], o[1], o[2], o[3]);
+    }
+    *reinterpret_cast<v4i *>(p.xn + (size_t)member * H + 32 * nt + 16 * g) = out;
+}
+
+// gate products (egg.c:246-258): wave 0 W0.xn, wave 1 W1.h, wave 2 W2.xn of one (strip, member tile); then
+// ft = cadd(cadd(W0 x, W1 h), b_f) and gated = ((ft + 127) h) >> 8 for the strip
+template <int H>
+__global__ void __launch_bounds__(192) k_gs_gates1(GruStage p, int l) {
+    __shared__ v4i ex[2][64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int nt = blockIdx.x, member = blockIdx.y * 32 + j;
+    const int8_t *hrow = p.states + ((size_t)member * p.L + l) * H;
+    v4i r;
+    if (wave == 1) r = gs_matmul<H / 32, false>(p, 6 * l + 1, nt, hrow, member, lane);
+    else r = gs_matmul<H / 32, true>(p, 6 * l + (wave == 0 ? 0 : 2), nt, p.xn + (size_t)member * H, member, lane);
+    if (wave < 2) ex[wave][lane] = r;
+    else *reinterpret_cast<v4i *>(p.m2 + (size_t)member * H + 32 * nt + 16 * g) = r;
+    __syncthreads();
+    if (wave != 0) return;
+    const v4i b1 = ex[0][lane], b2 = ex[1][lane];
+    const int *h32 = reinterpret_cast<const int *>(hrow + 32 * nt);
+    const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
+    v4i ft, gated;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int bf4 = *reinterpret_cast<const int *>(gb + 32 * nt + 8 * q + 4 * g), h4 = h32[2 * q + g];
+        int f[4], gp[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            f[e] = cadd(cadd(sx8(b1[q], e), sx8(b2[q], e)), sx8(bf4, e));
+            gp[e] = ((f[e] + 127) * sx8(h4, e)) >> 8;
+        }
+        ft[q] = pack4(f[0], f[1], f[2], f[3]); gated[q] = pack4(gp[0], gp[1], gp[2], gp[3]);
+    }
+    *reinterpret_cast<v4i *>(p.ft + (size_t)member * H + 32 * nt + 16 * g) = ft;
+    *reinterpret_cast<v4i *>(p.gate + (size_t)member * H + 32 * nt + 16 * g) = gated;
+}
+
+// candidate and state update (egg.c:260-271): ht = cadd(cadd(W2 x, W3 gated), b_h); h += ((ft + 127)(ht - h)) >> 8; x = cadd(h, x)
+// (Measured: the same stage as one workgroup per member tile with a wave per strip, which holds whole rows and can apply
+// the following norm itself, saves a launch but draws all of a matrix through four CUs: 8.2 instead of 4.6 us per stage.)
+template <int H>
+__global__ void __launch_bounds__(64) k_gs_gates2(GruStage p, int l) {
+    const int lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int nt = blockIdx.x, member = blockIdx.y * 32 + j;
+    const v4i b2 = gs_matmul<H / 32, true>(p, 6 * l + 3, nt, p.gate + (size_t)member * H, member, lane);
+    const size_t piece = (size_t)member * H + 32 * nt + 16 * g;
+    const v4i b1 = *reinterpret_cast<const v4i *>(p.m2 + piece), ft = *reinterpret_cast<const v4i *>(p.ft + piece);
+    v4i x = *reinterpret_cast<const v4i *>(p.x + piece);
+    int *h32 = reinterpret_cast<int *>(p.states + ((size_t)member * p.L + l) * H + 32 * nt);
+    const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int bh4 = *reinterpret_cast<const int *>(gb + H + 32 * nt + 8 * q + 4 * g), h4 = h32[2 * q + g];
+        int hn[4], xo[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int ht = cadd(cadd(sx8(b1[q], e), sx8(b2[q], e)), sx8(bh4, e));
+            const int hv = sx8(h4, e);
+            const int upd = ((sx8(ft[q], e) + 127) * (ht - hv)) >> 8;
+            hn[e] = cadd(hv, upd);
+            xo[e] = cadd(hn[e], sx8(x[q], e));
+        }
+        h32[2 * q + g] = pack4(hn[0], hn[1], hn[2], hn[3]); x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
+    }
+    *reinterpret_cast<v4i *>(p.x + piece) = x;
+}
+
+// MLP expand (egg.c:276-278): one strip of the 4H-wide intermediate
+template <int H>
+__global__ void __launch_bounds__(64) k_gs_up(GruStage p, int l) {
+    const int lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int nt = blockIdx.x, member = blockIdx.y * 32 + j;
+    const v4i r = gs_matmul<H / 32, true>(p, 6 * l + 4, nt, p.xn + (size_t)member * H, member, lane);
+    *reinterpret_cast<v4i *>(p.mb + (size_t)member * 4 * H + 32 * nt + 16 * g) = r;
+}
+
+// MLP project + residual (egg.c:280-285): the 4H-deep product is dealt to the four waves of a workgroup by k range
+template <int H>
+__global__ void __launch_bounds__(256) k_gs_down(GruStage p, int l) {
+    constexpr int KS4 = 4 * H / 32, KSW = KS4 / 4;
+    __shared__ int red[3][16][64];
+    __shared__ int xbp[3][64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, pair = member >> 1, ns = (member & 1) ? -1 : 1;
+    const GruMat m = p.mats[6 * l + 5];
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0;
+    int xb = 0;
+    gs_strip<KSW, true>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (4 * H), p.mb + (size_t)member * 4 * H,
+                        p.noise + m.b_off + (long long)pair * (4 * H), wave * KSW, lane);
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) red[wave - 1][r][lane] = acc[r];
+        xbp[wave - 1][lane] = xb;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; w++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] += red[w][r][lane];
+        xb += xbp[w][lane];
+    }
+    xb = sum_halves(xb);
+    const v4i pr = gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g);
+    const size_t piece = (size_t)member * H + 32 * nt + 16 * g;
+    v4i x = *reinterpret_cast<const v4i *>(p.x + piece);
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        int xo[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) xo[e] = cadd(sx8(pr[q], e), sx8(x[q], e));
+        x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
+    }
+    *reinterpret_cast<v4i *>(p.x + piece) = x;
+}
+
+// head + loss (egg.c:288-294, :321-330) of one member tile: wave w owns strip w of the V logits; the last workgroup to
+// finish hands the token index on
+template <int H>
+__global__ void __launch_bounds__(512) k_gs_head(GruStage p) {
+    __shared__ int psum[8][32];
+    __shared__ int tl[32];
+    __shared__ int lut[256];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
+    const int member = blockIdx.x * 32 + j;
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) lut[i] = p.exp2[i];
+    __syncthreads();
+    const GruStep st = *p.step;
+    const int target = st.data[gs_stream_pos(p, st, member) + st.t_next];
+    const v4i lg = gs_matmul<H / 32, true>(p, 6 * p.L, wave, p.xn + (size_t)member * H, member, lane);
+    int part = 0;
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int v = sx8(lg[q], e);
+            part += lut[v + 128];
+            if (32 * wave + 8 * q + 4 * g + e == target) tl[j] = v;
+        }
+    part = sum_halves(part);
+    if (g == 0) psum[wave][j] = part;
+    __syncthreads();
+    if (wave == 0 && g == 0) {
+        int sum_exp = 0;
+        for (int w2 = 0; w2 < p.V / 32; w2++) sum_exp += psum[w2][j];
+        int lg2 = 0;                                   // log2_fixed (egg.c:309-319)
+        if (sum_exp > 0) {
+            const int k = 31 - __clz(sum_exp);
+            const int frac = (k >= 4) ? ((sum_exp - (1 << k)) >> (k - 4)) : ((sum_exp - (1 << k)) << (4 - k));
+            lg2 = (k << 4) + frac - 64;
+        }
+        p.loss[member] += lg2 - (tl[j] + 128);
+    }
+    // the token is done once every workgroup of this launch has read the step's arguments, which each does before its
+    // product: the last one to arrive here hands the index on (arrival counter in the step block, reset for the next token)
+    if (threadIdx.x == 0) {
+        __threadfence();
+        if (atomicAdd(&p.step->arrived, 1) == (int)gridDim.x - 1) { p.step->arrived = 0; p.step->t = st.t_next; }
+    }
+}
+__global__ void k_gs_begin(GruStep *st, const uint8_t *data, long long data_len, long long start_idx, int32_t *loss, int population) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i == 0) { st->data = data; st->data_len = data_len; st->start_idx = start_idx; st->t = 0; st->t_next = 0; st->arrived = 0; }
+    if (i < population) loss[i] = 0;
+}
+
 // A panel *= fitness of the pair (A_T[r][p] = A[r] * f, egg.c:362-366)
 __global__ void k_gru_scale_panel(int8_t *panel, long long n, int pairs_pad, int pairs, const int32_t *fit) {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -410,6 +685,10 @@ struct egg_gru_ctx {
     int pairs_pad = 0;
     int8_t *d_model = nullptr, *d_frag = nullptr, *d_noise = nullptr, *d_panels = nullptr, *d_states = nullptr;
     GruMat *d_mats = nullptr; int32_t *d_loss = nullptr, *d_fit = nullptr, *d_exp2 = nullptr;
+    // one launch per stage (egg_gru_forward_mode): activations in global memory, the step's arguments, the graph of one token
+    bool staged = true;
+    int8_t *d_act = nullptr; GruStep *d_step = nullptr;
+    hipGraph_t tok_graph = nullptr; hipGraphExec_t tok_exec = nullptr;
     std::string err;
 };
 static int gfail(egg_gru_ctx *c, int code, const char *what, hipError_t e = hipSuccess) {
@@ -493,6 +772,8 @@ extern "C" int egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out) {
     int32_t ex[256];
     for (int i = 0; i < 256; i++) ex[i] = (int32_t)(pow(2.0, (double)i / (1 << c.fixed_point)) * (1 << c.fixed_point));   // egg.c:57-60
     CR(hipMalloc(&ctx->d_exp2, 1024)); CR(hipMemcpy(ctx->d_exp2, ex, 1024, hipMemcpyHostToDevice));
+    CR(hipMalloc(&ctx->d_act, (size_t)c.population * H * 9));      // x xn gate ft m2 [P][H] each, mb [P][4H]
+    CR(hipMalloc(&ctx->d_step, sizeof(GruStep))); CR(hipMemset(ctx->d_step, 0, sizeof(GruStep)));
 #undef CR
     *out = ctx;
     return EGG_OK;
@@ -500,7 +781,10 @@ extern "C" int egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out) {
 extern "C" void egg_gru_destroy(egg_gru_ctx *ctx) {
     if (!ctx) return;
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    void *ptrs[] = {ctx->d_model, ctx->d_frag, ctx->d_noise, ctx->d_panels, ctx->d_states, ctx->d_mats, ctx->d_loss, ctx->d_fit, ctx->d_exp2};
+    if (ctx->tok_exec) (void)hipGraphExecDestroy(ctx->tok_exec);
+    if (ctx->tok_graph) (void)hipGraphDestroy(ctx->tok_graph);
+    void *ptrs[] = {ctx->d_model, ctx->d_frag, ctx->d_noise, ctx->d_panels, ctx->d_states, ctx->d_mats, ctx->d_loss, ctx->d_fit, ctx->d_exp2,
+                    ctx->d_act, ctx->d_step};
     for (void *q : ptrs) if (q) (void)hipFree(q);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -554,6 +838,70 @@ extern "C" int egg_gru_state_download(egg_gru_ctx *ctx, void *h, size_t bytes) {
     return EGG_OK;
 }
 
+// the stages of one token, in order, on the context's stream (captured once into a graph, or launched as they are)
+template <int H>
+static hipError_t gru_token_stages(egg_gru_ctx *ctx, const GruStage &p) {
+    const egg_gru_config &c = ctx->cfg;
+    hipStream_t s = ctx->stream;
+    const int tiles = c.population / 32, nth = H / 32;
+    const dim3 ln_grid((unsigned)((size_t)c.population * (H / 16) / 256 + 1));
+    for (int l = 0; l < c.n_layers; l++) {
+        const long long lnw = ctx->off_ln_w + (long long)l * 2 * H;
+        if (l == 0) hipLaunchKernelGGL((k_gs_ln<H, true>), ln_grid, dim3(256), 0, s, p, lnw);
+        else hipLaunchKernelGGL((k_gs_ln<H, false>), ln_grid, dim3(256), 0, s, p, lnw);
+        hipLaunchKernelGGL((k_gs_gates1<H>), dim3(nth, tiles), dim3(192), 0, s, p, l);
+        hipLaunchKernelGGL((k_gs_gates2<H>), dim3(nth, tiles), dim3(64), 0, s, p, l);
+        hipLaunchKernelGGL((k_gs_ln<H, false>), ln_grid, dim3(256), 0, s, p, lnw + H);
+        hipLaunchKernelGGL((k_gs_up<H>), dim3(4 * nth, tiles), dim3(64), 0, s, p, l);
+        hipLaunchKernelGGL((k_gs_down<H>), dim3(nth, tiles), dim3(256), 0, s, p, l);
+    }
+    hipLaunchKernelGGL((k_gs_ln<H, false>), ln_grid, dim3(256), 0, s, p, (long long)ctx->off_ln_out);
+    hipLaunchKernelGGL((k_gs_head<H>), dim3(tiles), dim3(c.vocab / 32 * 64), 0, s, p);
+    return hipGetLastError();
+}
+static hipError_t gru_token_stages_h(egg_gru_ctx *ctx, const GruStage &p) {
+    switch (ctx->cfg.hidden) {
+        case 64: return gru_token_stages<64>(ctx, p);
+        case 128: return gru_token_stages<128>(ctx, p);
+        case 256: return gru_token_stages<256>(ctx, p);
+        default: return gru_token_stages<512>(ctx, p);
+    }
+}
+static int gru_forward_staged(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx) {
+    const egg_gru_config &c = ctx->cfg;
+    const size_t PH = (size_t)c.population * c.hidden;
+    GruStage p;
+    p.mats = ctx->d_mats; p.model = ctx->d_model; p.frag = ctx->d_frag; p.noise = ctx->d_noise; p.step = ctx->d_step;
+    p.states = ctx->d_states; p.x = ctx->d_act; p.xn = p.x + PH; p.gate = p.xn + PH; p.ft = p.gate + PH; p.m2 = p.ft + PH; p.mb = p.m2 + PH;
+    p.loss = ctx->d_loss;
+    p.H = c.hidden; p.L = c.n_layers; p.V = c.vocab; p.T = c.seq_len; p.population = c.population; p.sigma = c.fixed_point + c.sigma_shift;
+    p.off_emb = ctx->off_emb; p.off_gru_b = ctx->off_gru_b; p.off_ln_w = ctx->off_ln_w; p.off_ln_out = ctx->off_ln_out; p.exp2 = ctx->d_exp2;
+    hipLaunchKernelGGL(k_gs_begin, dim3((c.population + 255) / 256), dim3(256), 0, ctx->stream, ctx->d_step, d_data, (long long)data_len,
+                       (long long)start_idx, ctx->d_loss, c.population);
+    GTRY(hipGetLastError());
+    // tokens per captured graph: a graph launch costs more than the gap between two of its nodes
+    const int TPG = c.seq_len % 8 == 0 ? 8 : 1;
+    if (!ctx->tok_exec) {
+        // every argument of the stages is fixed for the life of the context (the step's own arguments sit in *d_step)
+        GTRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+        hipError_t e = hipSuccess;
+        for (int i = 0; i < TPG && e == hipSuccess; i++) e = gru_token_stages_h(ctx, p);
+        hipGraph_t g = nullptr;
+        const hipError_t e2 = hipStreamEndCapture(ctx->stream, &g);
+        if (e != hipSuccess || e2 != hipSuccess) { if (g) (void)hipGraphDestroy(g); return gfail(ctx, EGG_E_HIP, "capture of a token's stages", e != hipSuccess ? e : e2); }
+        ctx->tok_graph = g;
+        GTRY(hipGraphInstantiate(&ctx->tok_exec, ctx->tok_graph, nullptr, nullptr, 0));
+    }
+    for (int t = 0; t < c.seq_len; t += TPG) GTRY(hipGraphLaunch(ctx->tok_exec, ctx->stream));
+    return EGG_OK;
+}
+// 1 (default): one launch per stage, spread over the whole GPU; 0: one persistent workgroup per 32 members
+extern "C" int egg_gru_forward_mode(egg_gru_ctx *ctx, int staged) {
+    if (!ctx) return EGG_E_INVALID;
+    ctx->staged = staged != 0;
+    return EGG_OK;
+}
+
 extern "C" int egg_gru_step(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx, uint32_t step_seed, int do_update) {
     if (!ctx || !d_data || data_len <= ctx->cfg.seq_len + 1) return gfail(ctx, EGG_E_INVALID, "egg_gru_step arguments");
     const egg_gru_config &c = ctx->cfg;
@@ -565,15 +913,20 @@ extern "C" int egg_gru_step(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t dat
     p.data = d_data; p.data_len = data_len; p.start_idx = start_idx; p.states = ctx->d_states; p.loss = ctx->d_loss;
     p.H = c.hidden; p.L = c.n_layers; p.T = c.seq_len; p.V = c.vocab; p.population = c.population; p.sigma = c.fixed_point + c.sigma_shift;
     p.off_emb = ctx->off_emb; p.off_gru_b = ctx->off_gru_b; p.off_ln_w = ctx->off_ln_w; p.off_ln_out = ctx->off_ln_out; p.exp2 = ctx->d_exp2;
-    dim3 grid(c.population / 32), block(GRU_THREADS);
-    size_t lds = gru_lds_bytes(c.hidden);
-    switch (c.hidden) {
-        case 64: hipLaunchKernelGGL((k_gru_forward<64>), grid, block, lds, ctx->stream, p); break;
-        case 128: hipLaunchKernelGGL((k_gru_forward<128>), grid, block, lds, ctx->stream, p); break;
-        case 256: hipLaunchKernelGGL((k_gru_forward<256>), grid, block, lds, ctx->stream, p); break;
-        default: hipLaunchKernelGGL((k_gru_forward<512>), grid, block, lds, ctx->stream, p); break;
+    if (ctx->staged) {
+        int rc = gru_forward_staged(ctx, d_data, data_len, start_idx);
+        if (rc) return rc;
+    } else {
+        dim3 grid(c.population / 32), block(GRU_THREADS);
+        size_t lds = gru_lds_bytes(c.hidden);
+        switch (c.hidden) {
+            case 64: hipLaunchKernelGGL((k_gru_forward<64>), grid, block, lds, ctx->stream, p); break;
+            case 128: hipLaunchKernelGGL((k_gru_forward<128>), grid, block, lds, ctx->stream, p); break;
+            case 256: hipLaunchKernelGGL((k_gru_forward<256>), grid, block, lds, ctx->stream, p); break;
+            default: hipLaunchKernelGGL((k_gru_forward<512>), grid, block, lds, ctx->stream, p); break;
+        }
+        GTRY(hipGetLastError());
     }
-    GTRY(hipGetLastError());
     // pair fitness (egg.c:559-561) has the same rule as the transformer's
     GTRY(egg_launch_fitness(ctx->d_loss, ctx->d_fit, pairs, ctx->stream));
     if (do_update) {

@@ -19,7 +19,8 @@ def _t(dev, arr):
     (dict(hidden=256, n_layers=2, seq_len=4, population=96, update_threshold=30), 2),
     (dict(hidden=64, n_layers=1, seq_len=9, population=32, update_threshold=5, sigma_shift=2), 3),
 ], ids=["h64", "h128", "h512", "h256_p96", "sigma_2"])
-def test_gru_steps(pkg, orc, dev, kw, steps):
+@pytest.mark.parametrize("staged", [True, False], ids=["launch_per_stage", "persistent_workgroups"])
+def test_gru_steps(pkg, orc, dev, kw, steps, staged):
     import ctypes as C
     g = orc.gru_config(**kw)
     data = orc.zipf_bytes(1 << 14)
@@ -30,6 +31,7 @@ def test_gru_steps(pkg, orc, dev, kw, steps):
     off_b = 256 * H + L * 4 * H * H
     model[off_b:off_b + L * 2 * H] = rng.integers(-30, 31, L * 2 * H).astype(np.int8)
     ctx = pkg.GruContext(pkg.gru_default_config(**kw))
+    ctx.forward_mode(staged)
     assert ctx.model_bytes() == model.size
     ctx.model_init(42)
     got0 = ctx.model_download()
