@@ -16,6 +16,7 @@
 #include <stdio.h>
 #include <string.h>
 #include <string>
+#include <tuple>
 #include <vector>
 
 #define GRU_WAVES 16
@@ -363,25 +364,44 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
 
 // ============================================================================ the same forward, one launch per stage
 // k_gru_forward keeps a member tile on one workgroup for the whole sequence, so four workgroups stream every weight
-// once per token from L2 and the rest of the GPU idles.  Here every dependent stage of a token is a launch of its own
-// whose grid spreads the output strips (32 rows of W) and the member tiles (32 members) over the CUs: a wave owns one
-// (strip, tile) pair, reads its W fragments and the members' input rows straight from global memory and writes its 32 x
-// 32 results back.  Activations live in global memory in slot order ([member][K]); the recurrent state stays in natural
-// order like the reference's.  The stages of one token are captured once as a hipGraph and launched seq_len times; the
-// token index and the step's arguments sit in device memory (GruStep).  Same arithmetic helpers, bit-identical results.
-// t: tokens finished (what the embedding stage reads); t_next = t + 1, written by the embedding stage for the head's target
-// lookup; the head hands it back as t when it is done.  Each is written only while no other stage of the token reads it.
-struct GruStep { const uint8_t *data; long long data_len, start_idx; int t, t_next, arrived; };
+// once per token from L2 and the rest of the GPU idles.  Here every dependent stage is a launch of its own whose grid
+// spreads the output strips (32 rows of W) and the member tiles (32 members) over the CUs: a wave owns one (strip, tile)
+// pair, reads its W fragments and the members' input rows straight from global memory and writes its 32 x 32 results
+// back.  Activations live in global memory in slot order ([member][K]); the recurrent state stays in natural order like
+// the reference's.  Same arithmetic helpers, bit-identical results.
+//
+// Launches that depend on each other cost about 4.6 us apiece however small they are, so the sequence is walked as a
+// pipeline over the layers: layer l of token t needs layer l - 1 of token t and layer l of token t - 1, nothing else, so
+// at pipeline step s every layer l works on its own token s - l, and the head ("layer L") on token s - L.  The six
+// stages of a step are six launches whose grids carry the layer in blockIdx.z; a sequence takes T + L steps of six
+// launches instead of T tokens of 6 L + 2.  For that every layer has its own temporaries, and the residual stream after
+// each layer is kept twice, by token parity: while layer l + 1 reads token t's stream, layer l writes token t + 1's.
+// The launches of several steps form one linear hipGraph; the step counter and the step's arguments sit in device
+// memory (GruStep).  s_base: pipeline steps finished before the running graph; a launch of the graph's step number
+// `step` belongs to pipeline step s_base + step.
+struct GruStep { const uint8_t *data; long long data_len, start_idx; int s_base; };
 struct GruStage {
     const GruMat *mats;
     const int8_t *model, *frag, *noise;
     GruStep *step;
-    int8_t *states, *x, *xn, *gate, *ft, *m2, *mb;
+    int8_t *states, *act;
+    int32_t *head_sum, *head_tl;                  // [P][V / 32] sums of exp2 over a strip of logits, [P] the target's logit
     int32_t *loss;
     int H, L, V, T, population, sigma;
     long long off_emb, off_gru_b, off_ln_w, off_ln_out;
     const int32_t *exp2;
 };
+// activations, [P][H] each unless noted: the residual stream after li layers (li 0..L, by token parity), the normed
+// row of layer li (li == L: of the head), the three gate temporaries and the [P][4H] MLP intermediate of layer l
+__device__ __forceinline__ size_t gs_ph(const GruStage &p) { return (size_t)p.population * p.H; }
+__device__ __forceinline__ int8_t *gs_x(const GruStage &p, int li, int par) { return p.act + (size_t)(2 * li + par) * gs_ph(p); }
+__device__ __forceinline__ int8_t *gs_xn(const GruStage &p, int li) { return p.act + (size_t)(2 * (p.L + 1) + li) * gs_ph(p); }
+__device__ __forceinline__ int8_t *gs_tmp(const GruStage &p, int which, int l) { return p.act + (size_t)(3 * (p.L + 1) + which * p.L + l) * gs_ph(p); }
+__device__ __forceinline__ int8_t *gs_mb(const GruStage &p, int l) { return p.act + (size_t)(3 * (p.L + 1) + 3 * p.L + 4 * l) * gs_ph(p); }
+enum { GS_GATE = 0, GS_FT = 1, GS_M2 = 2, GS_GRAPH_STEPS = 32 };
+static size_t gs_act_bytes(int population, int H, int L) { return (size_t)population * H * (3 * (L + 1) + 7 * L); }
+// the token that layer z works on in the graph's step `step`; out of [0, T) while the pipeline fills or drains
+__device__ __forceinline__ int gs_token(const GruStage &p, int step, int z) { return p.step->s_base + step - z; }
 __device__ __forceinline__ long long gs_stream_pos(const GruStage &p, const GruStep &st, int member) {
     const long long stride = st.data_len / (p.population / 2);                    // egg.c:553-554
     return (st.start_idx + (long long)(member >> 1) * stride) % (st.data_len - p.T);
@@ -432,23 +452,27 @@ __device__ __forceinline__ v4i gs_matmul(const GruStage &p, int mi, int nt, cons
     return gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g);
 }
 
-// egg_ln (egg.c:180-210) of every member's row, optionally after the embedding lookup (egg.c:238).  A lane owns one
-// 16-byte piece (32-group nt, half g) of one member's row; the H / 16 lanes of a member sit side by side.
-template <int H, bool EMBED>
-__global__ void __launch_bounds__(256) k_gs_ln(GruStage p, long long w_off) {
+// egg_ln (egg.c:180-210) of every member's row.  A lane owns one 16-byte piece (32-group nt, half g) of one member's
+// row; the H / 16 lanes of a member sit side by side.  blockIdx.z is the layer.  phase 0 (grid z 0..L): the norm in
+// front of the gates, for layer 0 after the embedding lookup (egg.c:238), and for z == L the output norm in front of
+// the head; phase 1 (grid z 0..L-1): the norm in front of the MLP.
+template <int H>
+__global__ void __launch_bounds__(256) k_gs_ln(GruStage p, int step, int phase) {
     constexpr int PPM = H / 16;                     // pieces (lanes) per member
     const int id = blockIdx.x * 256 + threadIdx.x, member = id / PPM, piece = id % PPM, nt = piece >> 1, g = piece & 1;
-    if (member >= p.population) return;            // whole waves only: population * PPM is a multiple of 64
-    const GruStep st = *p.step;
+    const int z = blockIdx.z, t = gs_token(p, step, z);
+    if (t < 0 || t >= p.T || member >= p.population) return;     // whole waves only: population * PPM is a multiple of 64
+    const int xi = phase == 0 ? z : z + 1;          // which residual stream is read: the one after xi layers
+    const long long w_off = z == p.L ? p.off_ln_out : p.off_ln_w + (long long)z * 2 * H + (phase ? H : 0);
     v4i x;
-    int8_t *xrow = p.x + (size_t)member * H + 32 * nt + 16 * g;
-    if (EMBED) {
-        const int tok = st.data[gs_stream_pos(p, st, member) + st.t];
-        const int *e = reinterpret_cast<const int *>(p.model + p.off_emb + (size_t)tok * H + 32 * nt);
+    int8_t *xrow = gs_x(p, xi, t & 1) + (size_t)member * H + 32 * nt + 16 * g;
+    if (phase == 0 && z == 0) {
+        const GruStep st = *p.step;
+        const int byte = st.data[gs_stream_pos(p, st, member) + t];
+        const int *e = reinterpret_cast<const int *>(p.model + p.off_emb + (size_t)byte * H + 32 * nt);
 #pragma unroll
         for (int q = 0; q < 4; q++) x[q] = e[2 * q + g];
         *reinterpret_cast<v4i *>(xrow) = x;
-        if (id == 0) p.step->t_next = st.t + 1;
     } else x = *reinterpret_cast<const v4i *>(xrow);
     int sum = 0;
 #pragma unroll
@@ -468,22 +492,46 @@ __global__ void __launch_bounds__(256) k_gs_ln(GruStage p, long long w_off) {
         for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(sx8(x[q], e) * sx8(w4, e), rcp));
         out[q] = pack4(o[0], o[1], o[2], o[3]);
     }
-    *reinterpret_cast<v4i *>(p.xn + (size_t)member * H + 32 * nt + 16 * g) = out;
+    *reinterpret_cast<v4i *>(gs_xn(p, z) + (size_t)member * H + 32 * nt + 16 * g) = out;
 }
 
-// gate products (egg.c:246-258): wave 0 W0.xn, wave 1 W1.h, wave 2 W2.xn of one (strip, member tile); then
-// ft = cadd(cadd(W0 x, W1 h), b_f) and gated = ((ft + 127) h) >> 8 for the strip
+// blockIdx.z < L, gate products (egg.c:246-258): wave 0 W0.xn, wave 1 W1.h, wave 2 W2.xn of one (strip, member tile);
+// then ft = cadd(cadd(W0 x, W1 h), b_f) and gated = ((ft + 127) h) >> 8 for the strip.
+// blockIdx.z == L, head (egg.c:288-294): wave 0 forms one strip of 32 logits of the members, sums their exp2 and keeps
+// the target's logit; the loss itself follows in the next launch.  The grid's x covers max(H, V) / 32 strips.
 template <int H>
-__global__ void __launch_bounds__(192) k_gs_gates1(GruStage p, int l) {
+__global__ void __launch_bounds__(192) k_gs_gates1(GruStage p, int step) {
     __shared__ v4i ex[2][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int nt = blockIdx.x, member = blockIdx.y * 32 + j;
+    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, l = blockIdx.z, t = gs_token(p, step, l);
+    if (t < 0 || t >= p.T) return;
+    if (l == p.L) {
+        if (nt >= p.V / 32 || wave != 0) return;
+        const GruStep st = *p.step;
+        const int target = st.data[gs_stream_pos(p, st, member) + t + 1];
+        const v4i lg = gs_matmul<H / 32, true>(p, 6 * p.L, nt, gs_xn(p, p.L) + (size_t)member * H, member, lane);
+        int part = 0, tl = 0;
+        bool mine = false;
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int v = sx8(lg[q], e);
+                part += p.exp2[v + 128];
+                if (32 * nt + 8 * q + 4 * g + e == target) { tl = v; mine = true; }
+            }
+        part = sum_halves(part);
+        if (g == 0) p.head_sum[(size_t)member * (p.V / 32) + nt] = part;
+        if (mine) p.head_tl[member] = tl;
+        return;
+    }
+    if (nt >= H / 32) return;
     const int8_t *hrow = p.states + ((size_t)member * p.L + l) * H;
     v4i r;
     if (wave == 1) r = gs_matmul<H / 32, false>(p, 6 * l + 1, nt, hrow, member, lane);
-    else r = gs_matmul<H / 32, true>(p, 6 * l + (wave == 0 ? 0 : 2), nt, p.xn + (size_t)member * H, member, lane);
+    else r = gs_matmul<H / 32, true>(p, 6 * l + (wave == 0 ? 0 : 2), nt, gs_xn(p, l) + (size_t)member * H, member, lane);
     if (wave < 2) ex[wave][lane] = r;
-    else *reinterpret_cast<v4i *>(p.m2 + (size_t)member * H + 32 * nt + 16 * g) = r;
+    else *reinterpret_cast<v4i *>(gs_tmp(p, GS_M2, l) + (size_t)member * H + 32 * nt + 16 * g) = r;
     __syncthreads();
     if (wave != 0) return;
     const v4i b1 = ex[0][lane], b2 = ex[1][lane];
@@ -501,21 +549,37 @@ __global__ void __launch_bounds__(192) k_gs_gates1(GruStage p, int l) {
         }
         ft[q] = pack4(f[0], f[1], f[2], f[3]); gated[q] = pack4(gp[0], gp[1], gp[2], gp[3]);
     }
-    *reinterpret_cast<v4i *>(p.ft + (size_t)member * H + 32 * nt + 16 * g) = ft;
-    *reinterpret_cast<v4i *>(p.gate + (size_t)member * H + 32 * nt + 16 * g) = gated;
+    *reinterpret_cast<v4i *>(gs_tmp(p, GS_FT, l) + (size_t)member * H + 32 * nt + 16 * g) = ft;
+    *reinterpret_cast<v4i *>(gs_tmp(p, GS_GATE, l) + (size_t)member * H + 32 * nt + 16 * g) = gated;
 }
 
-// candidate and state update (egg.c:260-271): ht = cadd(cadd(W2 x, W3 gated), b_h); h += ((ft + 127)(ht - h)) >> 8; x = cadd(h, x)
-// (Measured: the same stage as one workgroup per member tile with a wave per strip, which holds whole rows and can apply
+// blockIdx.z < L, candidate and state update (egg.c:260-271): ht = cadd(cadd(W2 x, W3 gated), b_h);
+// h += ((ft + 127)(ht - h)) >> 8; x = cadd(h, x).
+// blockIdx.z == L, the loss of the head's token (egg.c:321-330) from the strips' sums: one lane per member.
+// (Measured: the update as one workgroup per member tile with a wave per strip, which holds whole rows and can apply
 // the following norm itself, saves a launch but draws all of a matrix through four CUs: 8.2 instead of 4.6 us per stage.)
 template <int H>
-__global__ void __launch_bounds__(64) k_gs_gates2(GruStage p, int l) {
+__global__ void __launch_bounds__(64) k_gs_gates2(GruStage p, int step) {
     const int lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int nt = blockIdx.x, member = blockIdx.y * 32 + j;
-    const v4i b2 = gs_matmul<H / 32, true>(p, 6 * l + 3, nt, p.gate + (size_t)member * H, member, lane);
+    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, l = blockIdx.z, t = gs_token(p, step, l), par = t & 1;
+    if (t < 0 || t >= p.T) return;
+    if (l == p.L) {
+        if (nt != 0 || g != 0) return;
+        int sum_exp = 0;
+        for (int s = 0; s < p.V / 32; s++) sum_exp += p.head_sum[(size_t)member * (p.V / 32) + s];
+        int lg2 = 0;                                   // log2_fixed (egg.c:309-319)
+        if (sum_exp > 0) {
+            const int k = 31 - __clz(sum_exp);
+            const int frac = (k >= 4) ? ((sum_exp - (1 << k)) >> (k - 4)) : ((sum_exp - (1 << k)) << (4 - k));
+            lg2 = (k << 4) + frac - 64;
+        }
+        p.loss[member] += lg2 - (p.head_tl[member] + 128);
+        return;
+    }
+    const v4i b2 = gs_matmul<H / 32, true>(p, 6 * l + 3, nt, gs_tmp(p, GS_GATE, l) + (size_t)member * H, member, lane);
     const size_t piece = (size_t)member * H + 32 * nt + 16 * g;
-    const v4i b1 = *reinterpret_cast<const v4i *>(p.m2 + piece), ft = *reinterpret_cast<const v4i *>(p.ft + piece);
-    v4i x = *reinterpret_cast<const v4i *>(p.x + piece);
+    const v4i b1 = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_M2, l) + piece), ft = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_FT, l) + piece);
+    v4i x = *reinterpret_cast<const v4i *>(gs_x(p, l, par) + piece);
     int *h32 = reinterpret_cast<int *>(p.states + ((size_t)member * p.L + l) * H + 32 * nt);
     const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
 #pragma unroll
@@ -532,32 +596,36 @@ __global__ void __launch_bounds__(64) k_gs_gates2(GruStage p, int l) {
         }
         h32[2 * q + g] = pack4(hn[0], hn[1], hn[2], hn[3]); x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
     }
-    *reinterpret_cast<v4i *>(p.x + piece) = x;
+    *reinterpret_cast<v4i *>(gs_x(p, l + 1, par) + piece) = x;
 }
 
-// MLP expand (egg.c:276-278): one strip of the 4H-wide intermediate
+// MLP expand (egg.c:276-278): one strip of the 4H-wide intermediate of layer blockIdx.z
 template <int H>
-__global__ void __launch_bounds__(64) k_gs_up(GruStage p, int l) {
+__global__ void __launch_bounds__(64) k_gs_up(GruStage p, int step) {
     const int lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int nt = blockIdx.x, member = blockIdx.y * 32 + j;
-    const v4i r = gs_matmul<H / 32, true>(p, 6 * l + 4, nt, p.xn + (size_t)member * H, member, lane);
-    *reinterpret_cast<v4i *>(p.mb + (size_t)member * 4 * H + 32 * nt + 16 * g) = r;
+    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, l = blockIdx.z, t = gs_token(p, step, l);
+    if (t < 0 || t >= p.T) return;
+    const v4i r = gs_matmul<H / 32, true>(p, 6 * l + 4, nt, gs_xn(p, l) + (size_t)member * H, member, lane);
+    *reinterpret_cast<v4i *>(gs_mb(p, l) + (size_t)member * 4 * H + 32 * nt + 16 * g) = r;
 }
 
-// MLP project + residual (egg.c:280-285): the 4H-deep product is dealt to the four waves of a workgroup by k range
+// MLP project + residual (egg.c:280-285) of layer blockIdx.z: the 4H-deep product is dealt to the four waves of a
+// workgroup by k range
 template <int H>
-__global__ void __launch_bounds__(256) k_gs_down(GruStage p, int l) {
+__global__ void __launch_bounds__(256) k_gs_down(GruStage p, int step) {
     constexpr int KS4 = 4 * H / 32, KSW = KS4 / 4;
     __shared__ int red[3][16][64];
     __shared__ int xbp[3][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const int nt = blockIdx.x, member = blockIdx.y * 32 + j, pair = member >> 1, ns = (member & 1) ? -1 : 1;
+    const int l = blockIdx.z, t = gs_token(p, step, l);
+    if (t < 0 || t >= p.T) return;
     const GruMat m = p.mats[6 * l + 5];
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
     int xb = 0;
-    gs_strip<KSW, true>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (4 * H), p.mb + (size_t)member * 4 * H,
+    gs_strip<KSW, true>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (4 * H), gs_mb(p, l) + (size_t)member * 4 * H,
                         p.noise + m.b_off + (long long)pair * (4 * H), wave * KSW, lane);
     if (wave > 0) {
 #pragma unroll
@@ -574,8 +642,8 @@ __global__ void __launch_bounds__(256) k_gs_down(GruStage p, int l) {
     }
     xb = sum_halves(xb);
     const v4i pr = gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g);
-    const size_t piece = (size_t)member * H + 32 * nt + 16 * g;
-    v4i x = *reinterpret_cast<const v4i *>(p.x + piece);
+    int8_t *xrow = gs_x(p, l + 1, t & 1) + (size_t)member * H + 32 * nt + 16 * g;
+    v4i x = *reinterpret_cast<const v4i *>(xrow);
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         int xo[4];
@@ -583,56 +651,13 @@ __global__ void __launch_bounds__(256) k_gs_down(GruStage p, int l) {
         for (int e = 0; e < 4; e++) xo[e] = cadd(sx8(pr[q], e), sx8(x[q], e));
         x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
     }
-    *reinterpret_cast<v4i *>(p.x + piece) = x;
+    *reinterpret_cast<v4i *>(xrow) = x;
 }
-
-// head + loss (egg.c:288-294, :321-330) of one member tile: wave w owns strip w of the V logits; the last workgroup to
-// finish hands the token index on
-template <int H>
-__global__ void __launch_bounds__(512) k_gs_head(GruStage p) {
-    __shared__ int psum[8][32];
-    __shared__ int tl[32];
-    __shared__ int lut[256];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int member = blockIdx.x * 32 + j;
-    for (int i = threadIdx.x; i < 256; i += blockDim.x) lut[i] = p.exp2[i];
-    __syncthreads();
-    const GruStep st = *p.step;
-    const int target = st.data[gs_stream_pos(p, st, member) + st.t_next];
-    const v4i lg = gs_matmul<H / 32, true>(p, 6 * p.L, wave, p.xn + (size_t)member * H, member, lane);
-    int part = 0;
-#pragma unroll
-    for (int q = 0; q < 4; q++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int v = sx8(lg[q], e);
-            part += lut[v + 128];
-            if (32 * wave + 8 * q + 4 * g + e == target) tl[j] = v;
-        }
-    part = sum_halves(part);
-    if (g == 0) psum[wave][j] = part;
-    __syncthreads();
-    if (wave == 0 && g == 0) {
-        int sum_exp = 0;
-        for (int w2 = 0; w2 < p.V / 32; w2++) sum_exp += psum[w2][j];
-        int lg2 = 0;                                   // log2_fixed (egg.c:309-319)
-        if (sum_exp > 0) {
-            const int k = 31 - __clz(sum_exp);
-            const int frac = (k >= 4) ? ((sum_exp - (1 << k)) >> (k - 4)) : ((sum_exp - (1 << k)) << (4 - k));
-            lg2 = (k << 4) + frac - 64;
-        }
-        p.loss[member] += lg2 - (tl[j] + 128);
-    }
-    // the token is done once every workgroup of this launch has read the step's arguments, which each does before its
-    // product: the last one to arrive here hands the index on (arrival counter in the step block, reset for the next token)
-    if (threadIdx.x == 0) {
-        __threadfence();
-        if (atomicAdd(&p.step->arrived, 1) == (int)gridDim.x - 1) { p.step->arrived = 0; p.step->t = st.t_next; }
-    }
-}
+// last node of a graph: its pipeline steps are finished
+__global__ void k_gs_advance(GruStep *st, int steps) { if (threadIdx.x == 0) st->s_base += steps; }
 __global__ void k_gs_begin(GruStep *st, const uint8_t *data, long long data_len, long long start_idx, int32_t *loss, int population) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i == 0) { st->data = data; st->data_len = data_len; st->start_idx = start_idx; st->t = 0; st->t_next = 0; st->arrived = 0; }
+    if (i == 0) { st->data = data; st->data_len = data_len; st->start_idx = start_idx; st->s_base = 0; }
     if (i < population) loss[i] = 0;
 }
 
@@ -685,10 +710,12 @@ struct egg_gru_ctx {
     int pairs_pad = 0;
     int8_t *d_model = nullptr, *d_frag = nullptr, *d_noise = nullptr, *d_panels = nullptr, *d_states = nullptr;
     GruMat *d_mats = nullptr; int32_t *d_loss = nullptr, *d_fit = nullptr, *d_exp2 = nullptr;
-    // one launch per stage (egg_gru_forward_mode): activations in global memory, the step's arguments, the graph of one token
+    // one launch per stage (egg_gru_forward_mode): activations in global memory, the head's partial sums, the step's
+    // arguments, and two graphs: one of `graph_steps` pipeline steps, one of a single step for what is left of the sequence
     bool staged = true;
-    int8_t *d_act = nullptr; GruStep *d_step = nullptr;
-    hipGraph_t tok_graph = nullptr; hipGraphExec_t tok_exec = nullptr;
+    int8_t *d_act = nullptr; GruStep *d_step = nullptr; int32_t *d_head = nullptr;
+    int graph_steps = 0;
+    hipGraph_t tok_graph[2] = {nullptr, nullptr}; hipGraphExec_t tok_exec[2] = {nullptr, nullptr};
     std::string err;
 };
 static int gfail(egg_gru_ctx *c, int code, const char *what, hipError_t e = hipSuccess) {
@@ -772,7 +799,8 @@ extern "C" int egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out) {
     int32_t ex[256];
     for (int i = 0; i < 256; i++) ex[i] = (int32_t)(pow(2.0, (double)i / (1 << c.fixed_point)) * (1 << c.fixed_point));   // egg.c:57-60
     CR(hipMalloc(&ctx->d_exp2, 1024)); CR(hipMemcpy(ctx->d_exp2, ex, 1024, hipMemcpyHostToDevice));
-    CR(hipMalloc(&ctx->d_act, (size_t)c.population * H * 9));      // x xn gate ft m2 [P][H] each, mb [P][4H]
+    CR(hipMalloc(&ctx->d_act, gs_act_bytes(c.population, c.hidden, c.n_layers)));
+    CR(hipMalloc(&ctx->d_head, (size_t)c.population * (c.vocab / 32 + 1) * 4));
     CR(hipMalloc(&ctx->d_step, sizeof(GruStep))); CR(hipMemset(ctx->d_step, 0, sizeof(GruStep)));
 #undef CR
     *out = ctx;
@@ -781,10 +809,12 @@ extern "C" int egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out) {
 extern "C" void egg_gru_destroy(egg_gru_ctx *ctx) {
     if (!ctx) return;
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
-    if (ctx->tok_exec) (void)hipGraphExecDestroy(ctx->tok_exec);
-    if (ctx->tok_graph) (void)hipGraphDestroy(ctx->tok_graph);
+    for (int i = 0; i < 2; i++) {
+        if (ctx->tok_exec[i]) (void)hipGraphExecDestroy(ctx->tok_exec[i]);
+        if (ctx->tok_graph[i]) (void)hipGraphDestroy(ctx->tok_graph[i]);
+    }
     void *ptrs[] = {ctx->d_model, ctx->d_frag, ctx->d_noise, ctx->d_panels, ctx->d_states, ctx->d_mats, ctx->d_loss, ctx->d_fit, ctx->d_exp2,
-                    ctx->d_act, ctx->d_step};
+                    ctx->d_act, ctx->d_step, ctx->d_head};
     for (void *q : ptrs) if (q) (void)hipFree(q);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -838,61 +868,79 @@ extern "C" int egg_gru_state_download(egg_gru_ctx *ctx, void *h, size_t bytes) {
     return EGG_OK;
 }
 
-// the stages of one token, in order, on the context's stream (captured once into a graph, or launched as they are)
-template <int H>
-static hipError_t gru_token_stages(egg_gru_ctx *ctx, const GruStage &p) {
-    const egg_gru_config &c = ctx->cfg;
-    hipStream_t s = ctx->stream;
-    const int tiles = c.population / 32, nth = H / 32;
-    const dim3 ln_grid((unsigned)((size_t)c.population * (H / 16) / 256 + 1));
-    for (int l = 0; l < c.n_layers; l++) {
-        const long long lnw = ctx->off_ln_w + (long long)l * 2 * H;
-        if (l == 0) hipLaunchKernelGGL((k_gs_ln<H, true>), ln_grid, dim3(256), 0, s, p, lnw);
-        else hipLaunchKernelGGL((k_gs_ln<H, false>), ln_grid, dim3(256), 0, s, p, lnw);
-        hipLaunchKernelGGL((k_gs_gates1<H>), dim3(nth, tiles), dim3(192), 0, s, p, l);
-        hipLaunchKernelGGL((k_gs_gates2<H>), dim3(nth, tiles), dim3(64), 0, s, p, l);
-        hipLaunchKernelGGL((k_gs_ln<H, false>), ln_grid, dim3(256), 0, s, p, lnw + H);
-        hipLaunchKernelGGL((k_gs_up<H>), dim3(4 * nth, tiles), dim3(64), 0, s, p, l);
-        hipLaunchKernelGGL((k_gs_down<H>), dim3(nth, tiles), dim3(256), 0, s, p, l);
-    }
-    hipLaunchKernelGGL((k_gs_ln<H, false>), ln_grid, dim3(256), 0, s, p, (long long)ctx->off_ln_out);
-    hipLaunchKernelGGL((k_gs_head<H>), dim3(tiles), dim3(c.vocab / 32 * 64), 0, s, p);
-    return hipGetLastError();
+// A kernel node whose arguments are the values given (the graph keeps its own copy of them)
+template <typename... KA, typename... A>
+static hipError_t gs_node(hipGraph_t g, hipGraphNode_t *out, const std::vector<hipGraphNode_t> &deps, void (*fn)(KA...), dim3 grid, dim3 block, A... args) {
+    std::tuple<KA...> vals{static_cast<KA>(args)...};
+    void *params[sizeof...(KA)];
+    int n = 0;
+    std::apply([&](auto &...v) { ((params[n++] = (void *)&v), ...); }, vals);
+    hipKernelNodeParams kp = {};
+    kp.func = reinterpret_cast<void *>(fn); kp.gridDim = grid; kp.blockDim = block; kp.sharedMemBytes = 0; kp.kernelParams = params; kp.extra = nullptr;
+    return hipGraphAddKernelNode(out, g, deps.empty() ? nullptr : deps.data(), deps.size(), &kp);
 }
-static hipError_t gru_token_stages_h(egg_gru_ctx *ctx, const GruStage &p) {
+// The graph of `steps` pipeline steps of the forward: a chain of six launches per step, then the step counter moves on
+template <int H>
+static hipError_t gru_build_graph(egg_gru_ctx *ctx, const GruStage &p, int steps, hipGraph_t *out) {
+    const egg_gru_config &c = ctx->cfg;
+    const unsigned L = c.n_layers, tiles = c.population / 32, nth = H / 32, nv = c.vocab / 32;
+    const unsigned ln_blocks = (unsigned)((size_t)c.population * (H / 16) / 256 + 1);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipGraphCreate(&g, 0);
+    if (e != hipSuccess) return e;
+#define GR(call) do { e = (call); if (e != hipSuccess) { (void)hipGraphDestroy(g); return e; } } while (0)
+    hipGraphNode_t n = nullptr;
+    auto after = [&]() { return n ? std::vector<hipGraphNode_t>{n} : std::vector<hipGraphNode_t>{}; };
+    for (int i = 0; i < steps; i++) {
+        GR(gs_node(g, &n, after(), k_gs_ln<H>, dim3(ln_blocks, 1, L + 1), dim3(256), p, i, 0));
+        GR(gs_node(g, &n, after(), k_gs_gates1<H>, dim3(nth > nv ? nth : nv, tiles, L + 1), dim3(192), p, i));
+        GR(gs_node(g, &n, after(), k_gs_gates2<H>, dim3(nth, tiles, L + 1), dim3(64), p, i));
+        GR(gs_node(g, &n, after(), k_gs_ln<H>, dim3(ln_blocks, 1, L), dim3(256), p, i, 1));
+        GR(gs_node(g, &n, after(), k_gs_up<H>, dim3(4 * nth, tiles, L), dim3(64), p, i));
+        GR(gs_node(g, &n, after(), k_gs_down<H>, dim3(nth, tiles, L), dim3(256), p, i));
+    }
+    GR(gs_node(g, &n, after(), k_gs_advance, dim3(1), dim3(64), p.step, steps));
+#undef GR
+    *out = g;
+    return hipSuccess;
+}
+static hipError_t gru_build_graph_h(egg_gru_ctx *ctx, const GruStage &p, int steps, hipGraph_t *out) {
     switch (ctx->cfg.hidden) {
-        case 64: return gru_token_stages<64>(ctx, p);
-        case 128: return gru_token_stages<128>(ctx, p);
-        case 256: return gru_token_stages<256>(ctx, p);
-        default: return gru_token_stages<512>(ctx, p);
+        case 64: return gru_build_graph<64>(ctx, p, steps, out);
+        case 128: return gru_build_graph<128>(ctx, p, steps, out);
+        case 256: return gru_build_graph<256>(ctx, p, steps, out);
+        default: return gru_build_graph<512>(ctx, p, steps, out);
     }
 }
 static int gru_forward_staged(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx) {
     const egg_gru_config &c = ctx->cfg;
-    const size_t PH = (size_t)c.population * c.hidden;
     GruStage p;
     p.mats = ctx->d_mats; p.model = ctx->d_model; p.frag = ctx->d_frag; p.noise = ctx->d_noise; p.step = ctx->d_step;
-    p.states = ctx->d_states; p.x = ctx->d_act; p.xn = p.x + PH; p.gate = p.xn + PH; p.ft = p.gate + PH; p.m2 = p.ft + PH; p.mb = p.m2 + PH;
+    p.states = ctx->d_states; p.act = ctx->d_act; p.head_sum = ctx->d_head; p.head_tl = ctx->d_head + (size_t)c.population * (c.vocab / 32);
     p.loss = ctx->d_loss;
     p.H = c.hidden; p.L = c.n_layers; p.V = c.vocab; p.T = c.seq_len; p.population = c.population; p.sigma = c.fixed_point + c.sigma_shift;
     p.off_emb = ctx->off_emb; p.off_gru_b = ctx->off_gru_b; p.off_ln_w = ctx->off_ln_w; p.off_ln_out = ctx->off_ln_out; p.exp2 = ctx->d_exp2;
     hipLaunchKernelGGL(k_gs_begin, dim3((c.population + 255) / 256), dim3(256), 0, ctx->stream, ctx->d_step, d_data, (long long)data_len,
                        (long long)start_idx, ctx->d_loss, c.population);
     GTRY(hipGetLastError());
-    // tokens per captured graph: a graph launch costs more than the gap between two of its nodes
-    const int TPG = c.seq_len % 8 == 0 ? 8 : 1;
-    if (!ctx->tok_exec) {
+    // a sequence is T + L pipeline steps.  Steps per graph: the largest power of two up to 32 that fits (a graph launch
+    // costs more than the gap between two of its nodes); a one-step graph takes what is left
+    const int total = c.seq_len + c.n_layers;
+    if (!ctx->graph_steps) { int k = 1; while (2 * k <= total && 2 * k <= GS_GRAPH_STEPS) k *= 2; ctx->graph_steps = k; }
+    const int K = ctx->graph_steps;
+    for (int which = 0; which < 2; which++) {
+        const int steps = which == 0 ? K : 1;
+        if (ctx->tok_exec[which] || (which == 1 && (K == 1 || total % K == 0))) continue;
         // every argument of the stages is fixed for the life of the context (the step's own arguments sit in *d_step)
-        GTRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
-        hipError_t e = hipSuccess;
-        for (int i = 0; i < TPG && e == hipSuccess; i++) e = gru_token_stages_h(ctx, p);
         hipGraph_t g = nullptr;
-        const hipError_t e2 = hipStreamEndCapture(ctx->stream, &g);
-        if (e != hipSuccess || e2 != hipSuccess) { if (g) (void)hipGraphDestroy(g); return gfail(ctx, EGG_E_HIP, "capture of a token's stages", e != hipSuccess ? e : e2); }
-        ctx->tok_graph = g;
-        GTRY(hipGraphInstantiate(&ctx->tok_exec, ctx->tok_graph, nullptr, nullptr, 0));
+        const hipError_t e = gru_build_graph_h(ctx, p, steps, &g);
+        if (e != hipSuccess) return gfail(ctx, EGG_E_HIP, "graph of the forward's stages", e);
+        ctx->tok_graph[which] = g;
+        GTRY(hipGraphInstantiate(&ctx->tok_exec[which], g, nullptr, nullptr, 0));
     }
-    for (int t = 0; t < c.seq_len; t += TPG) GTRY(hipGraphLaunch(ctx->tok_exec, ctx->stream));
+    int t = 0;
+    for (; t + K <= total; t += K) GTRY(hipGraphLaunch(ctx->tok_exec[0], ctx->stream));
+    for (; t < total; t++) GTRY(hipGraphLaunch(ctx->tok_exec[1], ctx->stream));
     return EGG_OK;
 }
 // 1 (default): one launch per stage, spread over the whole GPU; 0: one persistent workgroup per 32 members

@@ -18,7 +18,8 @@ def _t(dev, arr):
     (dict(hidden=512, n_layers=4, seq_len=3, population=32, update_threshold=10), 2),
     (dict(hidden=256, n_layers=2, seq_len=4, population=96, update_threshold=30), 2),
     (dict(hidden=64, n_layers=1, seq_len=9, population=32, update_threshold=5, sigma_shift=2), 3),
-], ids=["h64", "h128", "h512", "h256_p96", "sigma_2"])
+    (dict(hidden=128, n_layers=4, seq_len=11, population=32, update_threshold=8), 2),    # an 8-token graph, four layers side by side
+], ids=["h64", "h128", "h512", "h256_p96", "sigma_2", "h128_l4_t11"])
 @pytest.mark.parametrize("staged", [True, False], ids=["launch_per_stage", "persistent_workgroups"])
 def test_gru_steps(pkg, orc, dev, kw, steps, staged):
     import ctypes as C
