@@ -16,6 +16,7 @@
 #include <stdio.h>
 #include <string.h>
 #include <string>
+#include <algorithm>
 #include <tuple>
 #include <vector>
 
@@ -48,9 +49,10 @@ __device__ __forceinline__ uint32_t xorshift32(uint32_t &x) { x ^= x << 13; x ^=
 __device__ __forceinline__ int slot_pos(int n) { int w = n & 31; return (n & ~31) + 16 * ((w >> 2) & 1) + 4 * (w >> 3) + (w & 3); }
 
 // gen_noise_vector_neon (egg.c:87-105) for every (matrix, pair): A[rows] then B[cols] from one stream seeded
-// step_seed + pair + seed_off.  Writes the vectors in slot order for the forward and the raw panels for the vote.
+// step_seed + pair + seed_off.  Writes the vectors in slot order for the forward, [pair][count], a second copy by tiles
+// of 16 pairs, [pair tile][32-group][half][pair][16 bytes], and the raw panels for the vote.
 __global__ void k_gru_noise(const GruMat *mats, int n_mats, int pairs, int pairs_pad, uint32_t step_seed,
-                            int8_t *noise, int8_t *panels) {
+                            int8_t *noise, int8_t *nfrag, int8_t *panels) {
     int id = blockIdx.x * blockDim.x + threadIdx.x;
     if (id >= n_mats * pairs) return;
     const GruMat m = mats[id / pairs]; const int p = id % pairs;
@@ -58,13 +60,16 @@ __global__ void k_gru_noise(const GruMat *mats, int n_mats, int pairs, int pairs
     for (int part = 0; part < 2; part++) {
         const int count = part ? m.cols : m.rows;
         int8_t *vec = noise + (part ? m.b_off + (long long)p * m.cols : m.a_off + (long long)p * m.rows);
+        int8_t *tvec = nfrag + (part ? m.b_off : m.a_off) + (long long)(p >> 4) * 16 * count + (p & 15) * 16;
         int8_t *pan = panels + (part ? m.pb_off : m.pa_off);
         for (int i = 0; i < count; i += 16) {
             xorshift32(rng); xorshift32(rng); xorshift32(rng); xorshift32(rng);
             for (int jj = 0; jj < 16 && i + jj < count; jj++) {
                 uint32_t r = xorshift32(rng);
                 int v = (int)((r >> 1) & 31u); if (!(r & 1)) v = -v;
-                vec[slot_pos(i + jj)] = (int8_t)v;
+                const int sp = slot_pos(i + jj);
+                vec[sp] = (int8_t)v;
+                tvec[(sp >> 4) * 256 + (sp & 15)] = (int8_t)v;
                 pan[(long long)(i + jj) * pairs_pad + p] = (int8_t)v;
             }
         }
@@ -140,8 +145,7 @@ __device__ __forceinline__ int gru_xb(const int8_t *ldsB, const int8_t *bvec, in
     return sum_halves(s);
 }
 // rank-1 term, shift and clamp of one strip (egg.c:167-175); returns the 16 int8 results packed in slot order
-__device__ __forceinline__ v4i gru_finish(const v16i &acc, int xb, const int8_t *avec, int nt, int ns, int sigma, int shift, int g) {
-    v4i a4 = *reinterpret_cast<const v4i *>(avec + 32 * nt + 16 * g);
+__device__ __forceinline__ v4i gru_finish(const v16i &acc, int xb, const v4i &a4, int ns, int sigma, int shift) {
     v4i out;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
@@ -154,6 +158,9 @@ __device__ __forceinline__ v4i gru_finish(const v16i &acc, int xb, const int8_t 
         out[q] = pack4(o[0], o[1], o[2], o[3]);
     }
     return out;
+}
+__device__ __forceinline__ v4i gru_finish(const v16i &acc, int xb, const int8_t *avec, int nt, int ns, int sigma, int shift, int g) {
+    return gru_finish(acc, xb, *reinterpret_cast<const v4i *>(avec + 32 * nt + 16 * g), ns, sigma, shift);
 }
 __device__ __forceinline__ int cadd(int a, int b) { return clip127(a + b); }   // clipped_add, egg.c:62-67
 
@@ -362,27 +369,53 @@ __global__ void __launch_bounds__(GRU_THREADS) k_gru_forward(GruParams p) {
     if (wave == 0 && g == 0) p.loss[member] = loss;
 }
 
-// ============================================================================ the same forward, one launch per stage
+// ============================================================================ the same forward, spread over the GPU
 // k_gru_forward keeps a member tile on one workgroup for the whole sequence, so four workgroups stream every weight
-// once per token from L2 and the rest of the GPU idles.  Here every dependent stage is a launch of its own whose grid
-// spreads the output strips (32 rows of W) and the member tiles (32 members) over the CUs: a wave owns one (strip, tile)
-// pair, reads its W fragments and the members' input rows straight from global memory and writes its 32 x 32 results
-// back.  Activations live in global memory in slot order ([member][K]); the recurrent state stays in natural order like
-// the reference's.  Same arithmetic helpers, bit-identical results.
+// once per token from L2 and the rest of the GPU idles.  Here the work is cut into stages whose units spread over the
+// CUs: a wave owns one (strip of 32 rows of W, tile of 32 members) pair, reads its W fragments and the tile's input
+// straight from global memory and writes its 32 x 32 results back.  Same arithmetic helpers, bit-identical results.
 //
-// Launches that depend on each other cost about 4.6 us apiece however small they are, so the sequence is walked as a
-// pipeline over the layers: layer l of token t needs layer l - 1 of token t and layer l of token t - 1, nothing else, so
-// at pipeline step s every layer l works on its own token s - l, and the head ("layer L") on token s - L.  The six
-// stages of a step are six launches whose grids carry the layer in blockIdx.z; a sequence takes T + L steps of six
-// launches instead of T tokens of 6 L + 2.  For that every layer has its own temporaries, and the residual stream after
-// each layer is kept twice, by token parity: while layer l + 1 reads token t's stream, layer l writes token t + 1's.
-// The launches of several steps form one linear hipGraph; the step counter and the step's arguments sit in device
-// memory (GruStep).  s_base: pipeline steps finished before the running graph; a launch of the graph's step number
-// `step` belongs to pipeline step s_base + step.
-struct GruStep { const uint8_t *data; long long data_len, start_idx; int s_base; };
+// Every operand of a product is kept in the order the MFMA wants it, so that a wave's load of one k-step is one
+// contiguous block: an activation buffer is [tile][k-step][half g][member j][16 bytes], the 16 bytes being a k-step's
+// lane half in slot order, which is also exactly what a wave's 32 x 32 result packs to; the noise vectors have a
+// second copy [pair tile][k-step][half][pair][16 bytes].  The recurrent state keeps its natural-order copy, the
+// reference's layout, beside a copy in this order.
+//
+// Launches that depend on each other cost some microseconds apiece however small they are, so the sequence is walked as
+// a pipeline in which one launch (a tick) carries every stage that is ready.  A layer's token passes six stages, one
+// per tick:
+//   0 norm (after the embedding for layer 0)   1 gate products, ft, gated   2 candidate, new state, residual
+//   3 norm                                     4 MLP expand                 5 MLP project, residual
+// Only stage 1 reads the state that stage 2 of the previous token wrote, so a layer starts a token every second tick;
+// layer l runs six ticks behind layer l - 1, whose stage 5 hands it the residual stream.  Stage k of layer l's token t
+// runs at tick 2 t + 6 l + k: even ticks carry stages 0, 2, 4 of every layer (tokens t, t - 1, t - 2), odd ticks stages
+// 1, 3, 5.  The head is "layer L" with three stages: output norm, logits with their partial sums, loss.  A sequence is
+// 2 T + 6 L + 1 ticks instead of T (6 L + 2) dependent launches.  Every layer has its own temporaries, each written at
+// one tick and read at the next; the residual stream after each layer lives from stage 2 of the layer that writes it to
+// stage 2 of the layer that reads it, seven ticks, so it is kept four times, by token number mod 4.
+// The launches of several ticks form one linear hipGraph; the tick counter and the step's arguments sit in device
+// memory (GruStep).  tick_base: ticks finished before the running graph (even); launch number `step` of the graph is
+// tick tick_base + step.
+struct GruStep { const uint8_t *data; long long data_len, start_idx; int tick_base; };
+// how a tick's workgroups (256 threads) are dealt to the stages
+struct GsGrid {
+    int ln, g2, up, loss;                          // even ticks: workgroups per layer of stages 0, 2, 4; of the loss
+    int g1, down, head;                            // odd ticks: per layer of stages 1 (3 waves a unit), 5 (4 waves a unit); of the logits
+    __host__ __device__ int even(int L) const { return (up + g2) * L + ln * (L + 1) + loss; }
+    __host__ __device__ int odd(int L) const { return (down + g1 + ln) * L + head; }
+};
+static GsGrid gs_grid(int population, int H, int V) {
+    const int tiles = population / 32, nth = H / 32;
+    GsGrid g;
+    g.ln = tiles;
+    g.g2 = (nth * tiles + 3) / 4; g.up = nth * tiles; g.loss = (population + 255) / 256;
+    g.g1 = nth * tiles; g.down = nth * tiles; g.head = (V / 32 * tiles + 3) / 4;
+    return g;
+}
+struct GsMat { long long w_off, a_off, b_off; int rows, shift; };      // what a product needs of a GruMat
+enum { GS_MAX_MATS = 6 * 8 + 1 };
 struct GruStage {
-    const GruMat *mats;
-    const int8_t *model, *frag, *noise;
+    const int8_t *model, *frag, *nfrag;            // nfrag: the noise vectors by pair tile, at the offsets of the plain copy
     GruStep *step;
     int8_t *states, *act;
     int32_t *head_sum, *head_tl;                  // [P][V / 32] sums of exp2 over a strip of logits, [P] the target's logit
@@ -390,31 +423,39 @@ struct GruStage {
     int H, L, V, T, population, sigma;
     long long off_emb, off_gru_b, off_ln_w, off_ln_out;
     const int32_t *exp2;
+    GsGrid grid;
+    GsMat m[GS_MAX_MATS];
 };
-// activations, [P][H] each unless noted: the residual stream after li layers (li 0..L, by token parity), the normed
-// row of layer li (li == L: of the head), the three gate temporaries and the [P][4H] MLP intermediate of layer l
+// activations, [P][H] bytes each unless noted: the residual stream after li layers (li 0..L, four copies by token), the
+// normed rows in front of layer li's gates (li == L: of the head) and in front of its MLP, the three gate temporaries,
+// the state's copy in product order and the [P][4H] MLP intermediate of layer l
 __device__ __forceinline__ size_t gs_ph(const GruStage &p) { return (size_t)p.population * p.H; }
-__device__ __forceinline__ int8_t *gs_x(const GruStage &p, int li, int par) { return p.act + (size_t)(2 * li + par) * gs_ph(p); }
-__device__ __forceinline__ int8_t *gs_xn(const GruStage &p, int li) { return p.act + (size_t)(2 * (p.L + 1) + li) * gs_ph(p); }
-__device__ __forceinline__ int8_t *gs_tmp(const GruStage &p, int which, int l) { return p.act + (size_t)(3 * (p.L + 1) + which * p.L + l) * gs_ph(p); }
-__device__ __forceinline__ int8_t *gs_mb(const GruStage &p, int l) { return p.act + (size_t)(3 * (p.L + 1) + 3 * p.L + 4 * l) * gs_ph(p); }
-enum { GS_GATE = 0, GS_FT = 1, GS_M2 = 2, GS_GRAPH_STEPS = 32 };
-static size_t gs_act_bytes(int population, int H, int L) { return (size_t)population * H * (3 * (L + 1) + 7 * L); }
-// the token that layer z works on in the graph's step `step`; out of [0, T) while the pipeline fills or drains
-__device__ __forceinline__ int gs_token(const GruStage &p, int step, int z) { return p.step->s_base + step - z; }
+__device__ __forceinline__ int8_t *gs_x(const GruStage &p, int li, int t) { return p.act + (size_t)(4 * li + (t & 3)) * gs_ph(p); }
+__device__ __forceinline__ int8_t *gs_xn(const GruStage &p, int li) { return p.act + (size_t)(4 * (p.L + 1) + li) * gs_ph(p); }
+__device__ __forceinline__ int8_t *gs_tmp(const GruStage &p, int which, int l) { return p.act + (size_t)(5 * (p.L + 1) + which * p.L + l) * gs_ph(p); }
+__device__ __forceinline__ int8_t *gs_mb(const GruStage &p, int l) { return p.act + (size_t)(5 * (p.L + 1) + 5 * p.L + 4 * l) * gs_ph(p); }
+enum { GS_XN2 = 0, GS_GATE = 1, GS_FT = 2, GS_M2 = 3, GS_HF = 4, GS_GRAPH_TICKS = 64 };
+static size_t gs_act_bytes(int population, int H, int L) { return (size_t)population * H * (5 * (L + 1) + 9 * L); }
+// where lane (g, j) keeps its 16 bytes of k-step ks of member tile `tile` in a buffer of K bytes per member
+__device__ __forceinline__ size_t gs_at(int K, int tile, int ks, int g, int j) { return (size_t)tile * 32 * K + ((size_t)(ks * 2 + g) * 32 + j) * 16; }
+// the same for a noise vector of `count` bytes per pair: the two members of a pair read the same 16 bytes
+__device__ __forceinline__ size_t gs_noise_at(int count, int tile, int ks, int g, int j) { return (size_t)tile * 16 * count + ((size_t)(ks * 2 + g) * 16 + (j >> 1)) * 16; }
+// the token whose stage k layer l runs at `tick` (their parities agree), or -1 while the pipeline fills or drains
+__device__ __forceinline__ int gs_token(const GruStage &p, int tick, int l, int k) {
+    const int d = tick - 6 * l - k;
+    return (d < 0 || (d >> 1) >= p.T) ? -1 : d >> 1;
+}
 __device__ __forceinline__ long long gs_stream_pos(const GruStage &p, const GruStep &st, int member) {
     const long long stride = st.data_len / (p.population / 2);                    // egg.c:553-554
     return (st.start_idx + (long long)(member >> 1) * stride) % (st.data_len - p.T);
 }
 
 // KSN k-steps of a strip product starting at k-step ks0: acc += W[strip rows, k] . in[member, k], xb += in . B.
-// `in` is the lane's member row; SLOT: slot order (16 bytes of a k-step's lane half are contiguous) or natural order.
-template <int KSN, bool SLOT>
-__device__ __forceinline__ void gs_strip(v16i &acc, int &xb, const int8_t *ftile, const int8_t *in_row, const int8_t *bvec, int ks0, int lane) {
+// fa, fb, fn: the lane's 16 bytes of k-step 0 of the W fragments, of the input tile and of the B noise.
+template <int KSN>
+__device__ __forceinline__ void gs_strip(v16i &acc, int &xb, const int8_t *fa, const int8_t *fb, const int8_t *fn, int ks0) {
     constexpr int BATCH = KSN < 8 ? KSN : 8;
     static_assert(KSN % BATCH == 0, "k-steps come in whole batches");
-    const int j = lane & 31, g = lane >> 5;
-    const int8_t *fa = ftile + ((size_t)g * 32 + j) * 16;
 #pragma unroll 1
     for (int k0 = 0; k0 < KSN; k0 += BATCH) {
         v4i a[BATCH], b[BATCH], n[BATCH];
@@ -422,13 +463,8 @@ __device__ __forceinline__ void gs_strip(v16i &acc, int &xb, const int8_t *ftile
         for (int u = 0; u < BATCH; u++) {
             const int ks = ks0 + k0 + u;
             a[u] = *reinterpret_cast<const v4i *>(fa + (size_t)ks * 1024);
-            n[u] = *reinterpret_cast<const v4i *>(bvec + 32 * ks + 16 * g);
-            if (SLOT) b[u] = *reinterpret_cast<const v4i *>(in_row + 32 * ks + 16 * g);
-            else {
-                const int *r32 = reinterpret_cast<const int *>(in_row + 32 * ks);
-#pragma unroll
-                for (int q = 0; q < 4; q++) b[u][q] = r32[2 * q + g];
-            }
+            b[u] = *reinterpret_cast<const v4i *>(fb + (size_t)ks * 1024);
+            n[u] = *reinterpret_cast<const v4i *>(fn + (size_t)ks * 512);
         }
 #pragma unroll
         for (int u = 0; u < BATCH; u++) {
@@ -438,212 +474,189 @@ __device__ __forceinline__ void gs_strip(v16i &acc, int &xb, const int8_t *ftile
         }
     }
 }
-// one whole perturbed product of matrix mi for strip nt and the lane's member: the 16 packed int8 results (slot order)
-template <int KS, bool SLOT>
-__device__ __forceinline__ v4i gs_matmul(const GruStage &p, int mi, int nt, const int8_t *in_row, int member, int lane) {
-    const GruMat m = p.mats[mi];
-    const int pair = member >> 1, ns = (member & 1) ? -1 : 1, g = lane >> 5;
+// one whole perturbed product of matrix mi for strip nt and member tile `tile`, whose input rows (KS * 32 bytes a
+// member) start at in_tile: the lane's 16 packed int8 results, which are its piece (nt, g, j) of the output tile
+template <int KS>
+__device__ __forceinline__ v4i gs_matmul(const GruStage &p, int mi, int nt, const int8_t *in_tile, int tile, int lane) {
+    const GsMat m = p.m[mi];
+    const int j = lane & 31, g = lane >> 5, ns = (j & 1) ? -1 : 1;
+    const v4i a4 = *reinterpret_cast<const v4i *>(p.nfrag + m.a_off + gs_noise_at(m.rows, tile, nt, g, j));
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
     int xb = 0;
-    gs_strip<KS, SLOT>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (KS * 32), in_row, p.noise + m.b_off + (long long)pair * (KS * 32), 0, lane);
+    gs_strip<KS>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (KS * 32) + gs_at(0, 0, 0, g, j), in_tile + gs_at(0, 0, 0, g, j),
+                 p.nfrag + m.b_off + gs_noise_at(KS * 32, tile, 0, g, j), 0);
     xb = sum_halves(xb);
-    return gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g);
+    return gru_finish(acc, xb, a4, ns, p.sigma, m.shift);
 }
 
-// egg_ln (egg.c:180-210) of every member's row.  A lane owns one 16-byte piece (32-group nt, half g) of one member's
-// row; the H / 16 lanes of a member sit side by side.  blockIdx.z is the layer.  phase 0 (grid z 0..L): the norm in
-// front of the gates, for layer 0 after the embedding lookup (egg.c:238), and for z == L the output norm in front of
-// the head; phase 1 (grid z 0..L-1): the norm in front of the MLP.
+// stages 0 and 3, and the head's stage 0: egg_ln (egg.c:180-210) of the rows of one member tile by one workgroup.
+// Wave w holds the 32-groups w, w + 4, ... of the tile's rows, lane (g, j) its half g of member j's group.  Reads the
+// residual stream after xi layers (embed: fills it first with the embedding row, egg.c:238) and writes `out`.
+// lds: 4 x 32 ints.
 template <int H>
-__global__ void __launch_bounds__(256) k_gs_ln(GruStage p, int step, int phase) {
-    constexpr int PPM = H / 16;                     // pieces (lanes) per member
-    const int id = blockIdx.x * 256 + threadIdx.x, member = id / PPM, piece = id % PPM, nt = piece >> 1, g = piece & 1;
-    const int z = blockIdx.z, t = gs_token(p, step, z);
-    if (t < 0 || t >= p.T || member >= p.population) return;     // whole waves only: population * PPM is a multiple of 64
-    const int xi = phase == 0 ? z : z + 1;          // which residual stream is read: the one after xi layers
-    const long long w_off = z == p.L ? p.off_ln_out : p.off_ln_w + (long long)z * 2 * H + (phase ? H : 0);
-    v4i x;
-    int8_t *xrow = gs_x(p, xi, t & 1) + (size_t)member * H + 32 * nt + 16 * g;
-    if (phase == 0 && z == 0) {
+__device__ __forceinline__ void gs_stage_ln(const GruStage &p, int tile, int t, int xi, bool embed, long long w_off, int8_t *out, int *lds) {
+    constexpr int NTH = H / 32, NP = (NTH + 3) / 4;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31, member = tile * 32 + j;
+    int8_t *xt = gs_x(p, xi, t);
+    const int8_t *erow = nullptr;
+    if (embed) {
         const GruStep st = *p.step;
-        const int byte = st.data[gs_stream_pos(p, st, member) + t];
-        const int *e = reinterpret_cast<const int *>(p.model + p.off_emb + (size_t)byte * H + 32 * nt);
-#pragma unroll
-        for (int q = 0; q < 4; q++) x[q] = e[2 * q + g];
-        *reinterpret_cast<v4i *>(xrow) = x;
-    } else x = *reinterpret_cast<const v4i *>(xrow);
+        erow = p.model + p.off_emb + (size_t)st.data[gs_stream_pos(p, st, member) + t] * H;
+    }
+    v4i x[NP];
     int sum = 0;
 #pragma unroll
-    for (int q = 0; q < 4; q++) sum = sumabs4(x[q], sum);
+    for (int i = 0; i < NP; i++) {
+        const int nt = wave + 4 * i;
+        if (nt < NTH) {
+            if (embed) {
+                const int *e = reinterpret_cast<const int *>(erow + 32 * nt);
 #pragma unroll
-    for (int off = 1; off < PPM; off <<= 1) sum += __shfl_xor(sum, off, 64);
+                for (int q = 0; q < 4; q++) x[i][q] = e[2 * q + g];
+                *reinterpret_cast<v4i *>(xt + gs_at(H, tile, nt, g, j)) = x[i];
+            } else x[i] = *reinterpret_cast<const v4i *>(xt + gs_at(H, tile, nt, g, j));
+#pragma unroll
+            for (int q = 0; q < 4; q++) sum = sumabs4(x[i][q], sum);
+        }
+    }
+    sum = sum_halves(sum);
+    if (g == 0) lds[wave * 32 + j] = sum;
+    __syncthreads();
+    sum = lds[j] + lds[32 + j] + lds[64 + j] + lds[96 + j];
     if (sum == 0) sum = 1;
     int mean = sum / H; if (mean == 0) mean = 1;
     const float rcp = 1.0f / (float)mean;
     const int8_t *w = p.model + w_off;
-    v4i out;
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int w4 = *reinterpret_cast<const int *>(w + 32 * nt + 8 * q + 4 * g);
-        int o[4];
+    for (int i = 0; i < NP; i++) {
+        const int nt = wave + 4 * i;
+        if (nt < NTH) {
+            v4i o4;
 #pragma unroll
-        for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(sx8(x[q], e) * sx8(w4, e), rcp));
-        out[q] = pack4(o[0], o[1], o[2], o[3]);
+            for (int q = 0; q < 4; q++) {
+                const int w4 = *reinterpret_cast<const int *>(w + 32 * nt + 8 * q + 4 * g);
+                int o[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(sx8(x[i][q], e) * sx8(w4, e), rcp));
+                o4[q] = pack4(o[0], o[1], o[2], o[3]);
+            }
+            *reinterpret_cast<v4i *>(out + gs_at(H, tile, nt, g, j)) = o4;
+        }
     }
-    *reinterpret_cast<v4i *>(gs_xn(p, z) + (size_t)member * H + 32 * nt + 16 * g) = out;
 }
 
-// blockIdx.z < L, gate products (egg.c:246-258): wave 0 W0.xn, wave 1 W1.h, wave 2 W2.xn of one (strip, member tile);
-// then ft = cadd(cadd(W0 x, W1 h), b_f) and gated = ((ft + 127) h) >> 8 for the strip.
-// blockIdx.z == L, head (egg.c:288-294): wave 0 forms one strip of 32 logits of the members, sums their exp2 and keeps
-// the target's logit; the loss itself follows in the next launch.  The grid's x covers max(H, V) / 32 strips.
+// stage 1, gate products (egg.c:246-258): wave 0 W0.xn, wave 1 W1.h, wave 2 W2.xn of one (strip, member tile); then
+// ft = cadd(cadd(W0 x, W1 h), b_f) and gated = ((ft + 127) h) >> 8 for the strip.  A whole workgroup; lds: 2 x 64 v4i.
 template <int H>
-__global__ void __launch_bounds__(192) k_gs_gates1(GruStage p, int step) {
-    __shared__ v4i ex[2][64];
+__device__ __forceinline__ void gs_stage_gates1(const GruStage &p, int l, int nt, int tile, int *lds) {
+    v4i *ex = reinterpret_cast<v4i *>(lds);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, l = blockIdx.z, t = gs_token(p, step, l);
-    if (t < 0 || t >= p.T) return;
-    if (l == p.L) {
-        if (nt >= p.V / 32 || wave != 0) return;
-        const GruStep st = *p.step;
-        const int target = st.data[gs_stream_pos(p, st, member) + t + 1];
-        const v4i lg = gs_matmul<H / 32, true>(p, 6 * p.L, nt, gs_xn(p, p.L) + (size_t)member * H, member, lane);
-        int part = 0, tl = 0;
-        bool mine = false;
-#pragma unroll
-        for (int q = 0; q < 4; q++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int v = sx8(lg[q], e);
-                part += p.exp2[v + 128];
-                if (32 * nt + 8 * q + 4 * g + e == target) { tl = v; mine = true; }
-            }
-        part = sum_halves(part);
-        if (g == 0) p.head_sum[(size_t)member * (p.V / 32) + nt] = part;
-        if (mine) p.head_tl[member] = tl;
-        return;
-    }
-    if (nt >= H / 32) return;
-    const int8_t *hrow = p.states + ((size_t)member * p.L + l) * H;
+    const size_t tile0 = gs_at(H, tile, 0, 0, 0), piece = gs_at(H, tile, nt, g, j);
+    const int8_t *hf = gs_tmp(p, GS_HF, l);
     v4i r;
-    if (wave == 1) r = gs_matmul<H / 32, false>(p, 6 * l + 1, nt, hrow, member, lane);
-    else r = gs_matmul<H / 32, true>(p, 6 * l + (wave == 0 ? 0 : 2), nt, gs_xn(p, l) + (size_t)member * H, member, lane);
-    if (wave < 2) ex[wave][lane] = r;
-    else *reinterpret_cast<v4i *>(gs_tmp(p, GS_M2, l) + (size_t)member * H + 32 * nt + 16 * g) = r;
+    if (wave == 1) r = gs_matmul<H / 32>(p, 6 * l + 1, nt, hf + tile0, tile, lane);
+    else if (wave != 3) r = gs_matmul<H / 32>(p, 6 * l + (wave == 0 ? 0 : 2), nt, gs_xn(p, l) + tile0, tile, lane);
+    if (wave < 2) ex[wave * 64 + lane] = r;
+    else if (wave == 2) *reinterpret_cast<v4i *>(gs_tmp(p, GS_M2, l) + piece) = r;
     __syncthreads();
     if (wave != 0) return;
-    const v4i b1 = ex[0][lane], b2 = ex[1][lane];
-    const int *h32 = reinterpret_cast<const int *>(hrow + 32 * nt);
+    const v4i b1 = ex[lane], b2 = ex[64 + lane], h = *reinterpret_cast<const v4i *>(hf + piece);
     const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
     v4i ft, gated;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int bf4 = *reinterpret_cast<const int *>(gb + 32 * nt + 8 * q + 4 * g), h4 = h32[2 * q + g];
+        const int bf4 = *reinterpret_cast<const int *>(gb + 32 * nt + 8 * q + 4 * g);
         int f[4], gp[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             f[e] = cadd(cadd(sx8(b1[q], e), sx8(b2[q], e)), sx8(bf4, e));
-            gp[e] = ((f[e] + 127) * sx8(h4, e)) >> 8;
+            gp[e] = ((f[e] + 127) * sx8(h[q], e)) >> 8;
         }
         ft[q] = pack4(f[0], f[1], f[2], f[3]); gated[q] = pack4(gp[0], gp[1], gp[2], gp[3]);
     }
-    *reinterpret_cast<v4i *>(gs_tmp(p, GS_FT, l) + (size_t)member * H + 32 * nt + 16 * g) = ft;
-    *reinterpret_cast<v4i *>(gs_tmp(p, GS_GATE, l) + (size_t)member * H + 32 * nt + 16 * g) = gated;
+    *reinterpret_cast<v4i *>(gs_tmp(p, GS_FT, l) + piece) = ft;
+    *reinterpret_cast<v4i *>(gs_tmp(p, GS_GATE, l) + piece) = gated;
 }
 
-// blockIdx.z < L, candidate and state update (egg.c:260-271): ht = cadd(cadd(W2 x, W3 gated), b_h);
-// h += ((ft + 127)(ht - h)) >> 8; x = cadd(h, x).
-// blockIdx.z == L, the loss of the head's token (egg.c:321-330) from the strips' sums: one lane per member.
-// (Measured: the update as one workgroup per member tile with a wave per strip, which holds whole rows and can apply
-// the following norm itself, saves a launch but draws all of a matrix through four CUs: 8.2 instead of 4.6 us per stage.)
+// stage 2, candidate and state update (egg.c:260-271): ht = cadd(cadd(W2 x, W3 gated), b_h);
+// h += ((ft + 127)(ht - h)) >> 8; x = cadd(h, x).  One wave per (strip, member tile); the new state goes to both copies.
+// (Measured: as one workgroup per member tile with a wave per strip, which holds whole rows and can apply the following
+// norm itself, it saves a stage but draws all of a matrix through four CUs: 8.2 instead of 4.6 us.)
 template <int H>
-__global__ void __launch_bounds__(64) k_gs_gates2(GruStage p, int step) {
-    const int lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, l = blockIdx.z, t = gs_token(p, step, l), par = t & 1;
-    if (t < 0 || t >= p.T) return;
-    if (l == p.L) {
-        if (nt != 0 || g != 0) return;
-        int sum_exp = 0;
-        for (int s = 0; s < p.V / 32; s++) sum_exp += p.head_sum[(size_t)member * (p.V / 32) + s];
-        int lg2 = 0;                                   // log2_fixed (egg.c:309-319)
-        if (sum_exp > 0) {
-            const int k = 31 - __clz(sum_exp);
-            const int frac = (k >= 4) ? ((sum_exp - (1 << k)) >> (k - 4)) : ((sum_exp - (1 << k)) << (4 - k));
-            lg2 = (k << 4) + frac - 64;
-        }
-        p.loss[member] += lg2 - (p.head_tl[member] + 128);
-        return;
-    }
-    const v4i b2 = gs_matmul<H / 32, true>(p, 6 * l + 3, nt, gs_tmp(p, GS_GATE, l) + (size_t)member * H, member, lane);
-    const size_t piece = (size_t)member * H + 32 * nt + 16 * g;
+__device__ __forceinline__ void gs_stage_gates2(const GruStage &p, int l, int t, int nt, int tile, int lane) {
+    const int g = lane >> 5, j = lane & 31, member = tile * 32 + j;
+    const size_t piece = gs_at(H, tile, nt, g, j);
+    int8_t *hf = gs_tmp(p, GS_HF, l) + piece;
     const v4i b1 = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_M2, l) + piece), ft = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_FT, l) + piece);
-    v4i x = *reinterpret_cast<const v4i *>(gs_x(p, l, par) + piece);
+    const v4i h = *reinterpret_cast<const v4i *>(hf);
+    v4i x = *reinterpret_cast<const v4i *>(gs_x(p, l, t) + piece);
+    const v4i b2 = gs_matmul<H / 32>(p, 6 * l + 3, nt, gs_tmp(p, GS_GATE, l) + gs_at(H, tile, 0, 0, 0), tile, lane);
     int *h32 = reinterpret_cast<int *>(p.states + ((size_t)member * p.L + l) * H + 32 * nt);
     const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
+    v4i hnew;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int bh4 = *reinterpret_cast<const int *>(gb + H + 32 * nt + 8 * q + 4 * g), h4 = h32[2 * q + g];
+        const int bh4 = *reinterpret_cast<const int *>(gb + H + 32 * nt + 8 * q + 4 * g);
         int hn[4], xo[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const int ht = cadd(cadd(sx8(b1[q], e), sx8(b2[q], e)), sx8(bh4, e));
-            const int hv = sx8(h4, e);
+            const int hv = sx8(h[q], e);
             const int upd = ((sx8(ft[q], e) + 127) * (ht - hv)) >> 8;
             hn[e] = cadd(hv, upd);
             xo[e] = cadd(hn[e], sx8(x[q], e));
         }
-        h32[2 * q + g] = pack4(hn[0], hn[1], hn[2], hn[3]); x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
+        hnew[q] = pack4(hn[0], hn[1], hn[2], hn[3]); x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
+        h32[2 * q + g] = hnew[q];
     }
-    *reinterpret_cast<v4i *>(gs_x(p, l + 1, par) + piece) = x;
+    *reinterpret_cast<v4i *>(hf) = hnew;
+    *reinterpret_cast<v4i *>(gs_x(p, l + 1, t) + piece) = x;
 }
 
-// MLP expand (egg.c:276-278): one strip of the 4H-wide intermediate of layer blockIdx.z
+// stage 4, MLP expand (egg.c:276-278): one wave per (strip of the 4H-wide intermediate, member tile)
 template <int H>
-__global__ void __launch_bounds__(64) k_gs_up(GruStage p, int step) {
-    const int lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, l = blockIdx.z, t = gs_token(p, step, l);
-    if (t < 0 || t >= p.T) return;
-    const v4i r = gs_matmul<H / 32, true>(p, 6 * l + 4, nt, gs_xn(p, l) + (size_t)member * H, member, lane);
-    *reinterpret_cast<v4i *>(gs_mb(p, l) + (size_t)member * 4 * H + 32 * nt + 16 * g) = r;
+__device__ __forceinline__ void gs_stage_up(const GruStage &p, int l, int nt, int tile, int lane) {
+    const v4i r = gs_matmul<H / 32>(p, 6 * l + 4, nt, gs_tmp(p, GS_XN2, l) + gs_at(H, tile, 0, 0, 0), tile, lane);
+    *reinterpret_cast<v4i *>(gs_mb(p, l) + gs_at(4 * H, tile, nt, lane >> 5, lane & 31)) = r;
 }
 
-// MLP project + residual (egg.c:280-285) of layer blockIdx.z: the 4H-deep product is dealt to the four waves of a
-// workgroup by k range
+// stage 5, MLP project + residual (egg.c:280-285): the 4H-deep product of one (strip, member tile) is dealt to the four
+// waves of a workgroup by k range.  lds: 3 x 16 x 64 + 3 x 64 ints.
 template <int H>
-__global__ void __launch_bounds__(256) k_gs_down(GruStage p, int step) {
+__device__ __forceinline__ void gs_stage_down(const GruStage &p, int l, int t, int nt, int tile, int *lds) {
     constexpr int KS4 = 4 * H / 32, KSW = KS4 / 4;
-    __shared__ int red[3][16][64];
-    __shared__ int xbp[3][64];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
-    const int nt = blockIdx.x, member = blockIdx.y * 32 + j, pair = member >> 1, ns = (member & 1) ? -1 : 1;
-    const int l = blockIdx.z, t = gs_token(p, step, l);
-    if (t < 0 || t >= p.T) return;
-    const GruMat m = p.mats[6 * l + 5];
+    int *red = lds, *xbp = lds + 3 * 16 * 64;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31, ns = (j & 1) ? -1 : 1;
+    const GsMat m = p.m[6 * l + 5];
+    int8_t *xrow = gs_x(p, l + 1, t) + gs_at(H, tile, nt, g, j);
+    v4i x, a4;
+    if (wave == 0) {
+        x = *reinterpret_cast<const v4i *>(xrow);
+        a4 = *reinterpret_cast<const v4i *>(p.nfrag + m.a_off + gs_noise_at(m.rows, tile, nt, g, j));
+    }
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0;
     int xb = 0;
-    gs_strip<KSW, true>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (4 * H), gs_mb(p, l) + (size_t)member * 4 * H,
-                        p.noise + m.b_off + (long long)pair * (4 * H), wave * KSW, lane);
+    gs_strip<KSW>(acc, xb, p.frag + m.w_off + (size_t)nt * 32 * (4 * H) + gs_at(0, 0, 0, g, j), gs_mb(p, l) + gs_at(4 * H, tile, 0, g, j),
+                  p.nfrag + m.b_off + gs_noise_at(4 * H, tile, 0, g, j), wave * KSW);
     if (wave > 0) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) red[wave - 1][r][lane] = acc[r];
-        xbp[wave - 1][lane] = xb;
+        for (int r = 0; r < 16; r++) red[((wave - 1) * 16 + r) * 64 + lane] = acc[r];
+        xbp[(wave - 1) * 64 + lane] = xb;
     }
     __syncthreads();
     if (wave != 0) return;
 #pragma unroll
     for (int w = 0; w < 3; w++) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] += red[w][r][lane];
-        xb += xbp[w][lane];
+        for (int r = 0; r < 16; r++) acc[r] += red[(w * 16 + r) * 64 + lane];
+        xb += xbp[w * 64 + lane];
     }
     xb = sum_halves(xb);
-    const v4i pr = gru_finish(acc, xb, p.noise + m.a_off + (long long)pair * m.rows, nt, ns, p.sigma, m.shift, g);
-    int8_t *xrow = gs_x(p, l + 1, t & 1) + (size_t)member * H + 32 * nt + 16 * g;
-    v4i x = *reinterpret_cast<const v4i *>(xrow);
+    const v4i pr = gru_finish(acc, xb, a4, ns, p.sigma, m.shift);
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         int xo[4];
@@ -653,12 +666,111 @@ __global__ void __launch_bounds__(256) k_gs_down(GruStage p, int step) {
     }
     *reinterpret_cast<v4i *>(xrow) = x;
 }
-// last node of a graph: its pipeline steps are finished
-__global__ void k_gs_advance(GruStep *st, int steps) { if (threadIdx.x == 0) st->s_base += steps; }
-__global__ void k_gs_begin(GruStep *st, const uint8_t *data, long long data_len, long long start_idx, int32_t *loss, int population) {
+
+// the head's stage 1 (egg.c:288-294): a wave forms one strip of 32 logits of a member tile, sums their exp2 and keeps
+// the target's logit
+template <int H>
+__device__ __forceinline__ void gs_stage_logits(const GruStage &p, int t, int nt, int tile, int lane) {
+    const int g = lane >> 5, member = tile * 32 + (lane & 31);
+    const GruStep st = *p.step;
+    const int target = st.data[gs_stream_pos(p, st, member) + t + 1];
+    const v4i lg = gs_matmul<H / 32>(p, 6 * p.L, nt, gs_xn(p, p.L) + gs_at(H, tile, 0, 0, 0), tile, lane);
+    int part = 0, tl = 0;
+    bool mine = false;
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int v = sx8(lg[q], e);
+            part += p.exp2[v + 128];
+            if (32 * nt + 8 * q + 4 * g + e == target) { tl = v; mine = true; }
+        }
+    part = sum_halves(part);
+    if (g == 0) p.head_sum[(size_t)member * (p.V / 32) + nt] = part;
+    if (mine) p.head_tl[member] = tl;
+}
+// the head's stage 2: a member's loss for the token (egg.c:321-330) from the strips' sums
+__device__ __forceinline__ void gs_stage_loss(const GruStage &p, int member) {
+    int sum_exp = 0;
+    for (int s = 0; s < p.V / 32; s++) sum_exp += p.head_sum[(size_t)member * (p.V / 32) + s];
+    int lg2 = 0;                                   // log2_fixed (egg.c:309-319)
+    if (sum_exp > 0) {
+        const int k = 31 - __clz(sum_exp);
+        const int frac = (k >= 4) ? ((sum_exp - (1 << k)) >> (k - 4)) : ((sum_exp - (1 << k)) << (4 - k));
+        lg2 = (k << 4) + frac - 64;
+    }
+    p.loss[member] += lg2 - (p.head_tl[member] + 128);
+}
+
+// One tick.  ODD false: stages 4, 2, 0 of every layer, the output norm and the loss; true: stages 5, 1, 3 and the logits.
+// The workgroups are dealt to the stages in that order (the deepest products first); every branch below is taken by a
+// whole workgroup, except that waves past a stage's last unit leave where the stage has no barrier.
+template <int H, bool ODD>
+__global__ void __launch_bounds__(256) k_gs_tick(GruStage p, int step) {
+    __shared__ int lds[3 * 16 * 64 + 3 * 64];
+    const int tick = p.step->tick_base + step, L = p.L, tiles = p.population / 32, nth = H / 32;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const GsGrid &gr = p.grid;
+    int b = blockIdx.x;
+    if (!ODD) {
+        if (b < gr.up * L) {
+            const int l = b / gr.up, unit = (b % gr.up) * 4 + wave, t = gs_token(p, tick, l, 4);
+            if (t >= 0) gs_stage_up<H>(p, l, unit % (4 * nth), unit / (4 * nth), lane);
+            return;
+        }
+        b -= gr.up * L;
+        if (b < gr.g2 * L) {
+            const int l = b / gr.g2, unit = (b % gr.g2) * 4 + wave, t = gs_token(p, tick, l, 2);
+            if (t >= 0 && unit < nth * tiles) gs_stage_gates2<H>(p, l, t, unit % nth, unit / nth, lane);
+            return;
+        }
+        b -= gr.g2 * L;
+        if (b < gr.ln * (L + 1)) {
+            const int l = b / gr.ln, t = gs_token(p, tick, l, 0);
+            if (t >= 0) gs_stage_ln<H>(p, b % gr.ln, t, l, l == 0, l == L ? p.off_ln_out : p.off_ln_w + (long long)l * 2 * H, gs_xn(p, l), lds);
+            return;
+        }
+        b -= gr.ln * (L + 1);
+        const int member = b * 256 + threadIdx.x;
+        if (gs_token(p, tick, L, 2) >= 0 && member < p.population) gs_stage_loss(p, member);
+    } else {
+        if (b < gr.down * L) {
+            const int l = b / gr.down, unit = b % gr.down, t = gs_token(p, tick, l, 5);
+            if (t >= 0) gs_stage_down<H>(p, l, t, unit % nth, unit / nth, lds);
+            return;
+        }
+        b -= gr.down * L;
+        if (b < gr.g1 * L) {
+            const int l = b / gr.g1, unit = b % gr.g1;
+            if (gs_token(p, tick, l, 1) >= 0) gs_stage_gates1<H>(p, l, unit % nth, unit / nth, lds);
+            return;
+        }
+        b -= gr.g1 * L;
+        if (b < gr.ln * L) {
+            const int l = b / gr.ln, t = gs_token(p, tick, l, 3);
+            if (t >= 0) gs_stage_ln<H>(p, b % gr.ln, t, l + 1, false, p.off_ln_w + (long long)l * 2 * H + H, gs_tmp(p, GS_XN2, l), lds);
+            return;
+        }
+        b -= gr.ln * L;
+        const int nv = p.V / 32, unit = b * 4 + wave, t = gs_token(p, tick, L, 1);
+        if (t >= 0 && unit < nv * tiles) gs_stage_logits<H>(p, t, unit % nv, unit / nv, lane);
+    }
+}
+// last node of a graph: its ticks are finished
+__global__ void k_gs_advance(GruStep *st, int ticks) { if (threadIdx.x == 0) st->tick_base += ticks; }
+// before the first tick: the step's arguments, zero losses, and the state's copy in product order from the natural one
+__global__ void k_gs_begin(GruStage p, const uint8_t *data, long long data_len, long long start_idx) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i == 0) { st->data = data; st->data_len = data_len; st->start_idx = start_idx; st->s_base = 0; }
-    if (i < population) loss[i] = 0;
+    if (i == 0) { GruStep *st = p.step; st->data = data; st->data_len = data_len; st->start_idx = start_idx; st->tick_base = 0; }
+    if (i < p.population) p.loss[i] = 0;
+    const int H = p.H, per_member = p.L * (H / 16);
+    if (i >= p.population * per_member) return;
+    const int member = i / per_member, r = i % per_member, l = r / (H / 16), piece = r % (H / 16), nt = piece >> 1, g = piece & 1;
+    const int *h32 = reinterpret_cast<const int *>(p.states + ((size_t)member * p.L + l) * H + 32 * nt);
+    v4i h;
+#pragma unroll
+    for (int q = 0; q < 4; q++) h[q] = h32[2 * q + g];
+    *reinterpret_cast<v4i *>(gs_tmp(p, GS_HF, l) + gs_at(H, member >> 5, nt, g, member & 31)) = h;
 }
 
 // A panel *= fitness of the pair (A_T[r][p] = A[r] * f, egg.c:362-366)
@@ -710,11 +822,11 @@ struct egg_gru_ctx {
     int pairs_pad = 0;
     int8_t *d_model = nullptr, *d_frag = nullptr, *d_noise = nullptr, *d_panels = nullptr, *d_states = nullptr;
     GruMat *d_mats = nullptr; int32_t *d_loss = nullptr, *d_fit = nullptr, *d_exp2 = nullptr;
-    // one launch per stage (egg_gru_forward_mode): activations in global memory, the head's partial sums, the step's
-    // arguments, and two graphs: one of `graph_steps` pipeline steps, one of a single step for what is left of the sequence
+    // the forward spread over the GPU (egg_gru_forward_mode): activations in global memory, the head's partial sums, the
+    // step's arguments, and two graphs: one of `graph_ticks` ticks, one of two ticks for what is left of the sequence
     bool staged = true;
-    int8_t *d_act = nullptr; GruStep *d_step = nullptr; int32_t *d_head = nullptr;
-    int graph_steps = 0;
+    int8_t *d_act = nullptr, *d_nfrag = nullptr; GruStep *d_step = nullptr; int32_t *d_head = nullptr;
+    int graph_ticks = 0;
     hipGraph_t tok_graph[2] = {nullptr, nullptr}; hipGraphExec_t tok_exec[2] = {nullptr, nullptr};
     std::string err;
 };
@@ -800,6 +912,7 @@ extern "C" int egg_gru_create(const egg_gru_config *cfg, egg_gru_ctx **out) {
     for (int i = 0; i < 256; i++) ex[i] = (int32_t)(pow(2.0, (double)i / (1 << c.fixed_point)) * (1 << c.fixed_point));   // egg.c:57-60
     CR(hipMalloc(&ctx->d_exp2, 1024)); CR(hipMemcpy(ctx->d_exp2, ex, 1024, hipMemcpyHostToDevice));
     CR(hipMalloc(&ctx->d_act, gs_act_bytes(c.population, c.hidden, c.n_layers)));
+    CR(hipMalloc(&ctx->d_nfrag, ctx->noise_bytes));
     CR(hipMalloc(&ctx->d_head, (size_t)c.population * (c.vocab / 32 + 1) * 4));
     CR(hipMalloc(&ctx->d_step, sizeof(GruStep))); CR(hipMemset(ctx->d_step, 0, sizeof(GruStep)));
 #undef CR
@@ -814,7 +927,7 @@ extern "C" void egg_gru_destroy(egg_gru_ctx *ctx) {
         if (ctx->tok_graph[i]) (void)hipGraphDestroy(ctx->tok_graph[i]);
     }
     void *ptrs[] = {ctx->d_model, ctx->d_frag, ctx->d_noise, ctx->d_panels, ctx->d_states, ctx->d_mats, ctx->d_loss, ctx->d_fit, ctx->d_exp2,
-                    ctx->d_act, ctx->d_step, ctx->d_head};
+                    ctx->d_act, ctx->d_step, ctx->d_head, ctx->d_nfrag};
     for (void *q : ptrs) if (q) (void)hipFree(q);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -879,71 +992,69 @@ static hipError_t gs_node(hipGraph_t g, hipGraphNode_t *out, const std::vector<h
     kp.func = reinterpret_cast<void *>(fn); kp.gridDim = grid; kp.blockDim = block; kp.sharedMemBytes = 0; kp.kernelParams = params; kp.extra = nullptr;
     return hipGraphAddKernelNode(out, g, deps.empty() ? nullptr : deps.data(), deps.size(), &kp);
 }
-// The graph of `steps` pipeline steps of the forward: a chain of six launches per step, then the step counter moves on
+// The graph of `ticks` ticks (an even number) of the forward: a chain of launches, then the tick counter moves on
 template <int H>
-static hipError_t gru_build_graph(egg_gru_ctx *ctx, const GruStage &p, int steps, hipGraph_t *out) {
-    const egg_gru_config &c = ctx->cfg;
-    const unsigned L = c.n_layers, tiles = c.population / 32, nth = H / 32, nv = c.vocab / 32;
-    const unsigned ln_blocks = (unsigned)((size_t)c.population * (H / 16) / 256 + 1);
+static hipError_t gru_build_graph(egg_gru_ctx *ctx, const GruStage &p, int ticks, hipGraph_t *out) {
+    const int L = ctx->cfg.n_layers;
     hipGraph_t g = nullptr;
     hipError_t e = hipGraphCreate(&g, 0);
     if (e != hipSuccess) return e;
 #define GR(call) do { e = (call); if (e != hipSuccess) { (void)hipGraphDestroy(g); return e; } } while (0)
     hipGraphNode_t n = nullptr;
     auto after = [&]() { return n ? std::vector<hipGraphNode_t>{n} : std::vector<hipGraphNode_t>{}; };
-    for (int i = 0; i < steps; i++) {
-        GR(gs_node(g, &n, after(), k_gs_ln<H>, dim3(ln_blocks, 1, L + 1), dim3(256), p, i, 0));
-        GR(gs_node(g, &n, after(), k_gs_gates1<H>, dim3(nth > nv ? nth : nv, tiles, L + 1), dim3(192), p, i));
-        GR(gs_node(g, &n, after(), k_gs_gates2<H>, dim3(nth, tiles, L + 1), dim3(64), p, i));
-        GR(gs_node(g, &n, after(), k_gs_ln<H>, dim3(ln_blocks, 1, L), dim3(256), p, i, 1));
-        GR(gs_node(g, &n, after(), k_gs_up<H>, dim3(4 * nth, tiles, L), dim3(64), p, i));
-        GR(gs_node(g, &n, after(), k_gs_down<H>, dim3(nth, tiles, L), dim3(256), p, i));
+    for (int i = 0; i < ticks; i++) {
+        if (i & 1) GR(gs_node(g, &n, after(), k_gs_tick<H, true>, dim3((unsigned)p.grid.odd(L)), dim3(256), p, i));
+        else GR(gs_node(g, &n, after(), k_gs_tick<H, false>, dim3((unsigned)p.grid.even(L)), dim3(256), p, i));
     }
-    GR(gs_node(g, &n, after(), k_gs_advance, dim3(1), dim3(64), p.step, steps));
+    GR(gs_node(g, &n, after(), k_gs_advance, dim3(1), dim3(64), p.step, ticks));
 #undef GR
     *out = g;
     return hipSuccess;
 }
-static hipError_t gru_build_graph_h(egg_gru_ctx *ctx, const GruStage &p, int steps, hipGraph_t *out) {
+static hipError_t gru_build_graph_h(egg_gru_ctx *ctx, const GruStage &p, int ticks, hipGraph_t *out) {
     switch (ctx->cfg.hidden) {
-        case 64: return gru_build_graph<64>(ctx, p, steps, out);
-        case 128: return gru_build_graph<128>(ctx, p, steps, out);
-        case 256: return gru_build_graph<256>(ctx, p, steps, out);
-        default: return gru_build_graph<512>(ctx, p, steps, out);
+        case 64: return gru_build_graph<64>(ctx, p, ticks, out);
+        case 128: return gru_build_graph<128>(ctx, p, ticks, out);
+        case 256: return gru_build_graph<256>(ctx, p, ticks, out);
+        default: return gru_build_graph<512>(ctx, p, ticks, out);
     }
 }
 static int gru_forward_staged(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx) {
     const egg_gru_config &c = ctx->cfg;
     GruStage p;
-    p.mats = ctx->d_mats; p.model = ctx->d_model; p.frag = ctx->d_frag; p.noise = ctx->d_noise; p.step = ctx->d_step;
+    p.model = ctx->d_model; p.frag = ctx->d_frag; p.nfrag = ctx->d_nfrag; p.step = ctx->d_step;
     p.states = ctx->d_states; p.act = ctx->d_act; p.head_sum = ctx->d_head; p.head_tl = ctx->d_head + (size_t)c.population * (c.vocab / 32);
     p.loss = ctx->d_loss;
     p.H = c.hidden; p.L = c.n_layers; p.V = c.vocab; p.T = c.seq_len; p.population = c.population; p.sigma = c.fixed_point + c.sigma_shift;
     p.off_emb = ctx->off_emb; p.off_gru_b = ctx->off_gru_b; p.off_ln_w = ctx->off_ln_w; p.off_ln_out = ctx->off_ln_out; p.exp2 = ctx->d_exp2;
-    hipLaunchKernelGGL(k_gs_begin, dim3((c.population + 255) / 256), dim3(256), 0, ctx->stream, ctx->d_step, d_data, (long long)data_len,
-                       (long long)start_idx, ctx->d_loss, c.population);
+    p.grid = gs_grid(c.population, c.hidden, c.vocab);
+    for (size_t i = 0; i < ctx->mats.size(); i++) { const GruMat &m = ctx->mats[i]; p.m[i] = GsMat{m.w_off, m.a_off, m.b_off, m.rows, m.shift}; }
+    const long long pieces = (long long)c.population * c.n_layers * (c.hidden / 16);
+    hipLaunchKernelGGL(k_gs_begin, dim3((unsigned)((std::max<long long>(pieces, c.population) + 255) / 256)), dim3(256), 0, ctx->stream, p, d_data,
+                       (long long)data_len, (long long)start_idx);
     GTRY(hipGetLastError());
-    // a sequence is T + L pipeline steps.  Steps per graph: the largest power of two up to 32 that fits (a graph launch
-    // costs more than the gap between two of its nodes); a one-step graph takes what is left
-    const int total = c.seq_len + c.n_layers;
-    if (!ctx->graph_steps) { int k = 1; while (2 * k <= total && 2 * k <= GS_GRAPH_STEPS) k *= 2; ctx->graph_steps = k; }
-    const int K = ctx->graph_steps;
+    // a sequence is 2 T + 6 L + 1 ticks, rounded up to an even number (a tick past the end finds no token).  Ticks per
+    // graph: the largest power of two up to 64 that fits (a graph launch costs more than the gap between two of its
+    // nodes); a two-tick graph takes what is left
+    const int total = (2 * c.seq_len + 6 * c.n_layers + 2) & ~1;
+    if (!ctx->graph_ticks) { int k = 2; while (2 * k <= total && 2 * k <= GS_GRAPH_TICKS) k *= 2; ctx->graph_ticks = k; }
+    const int K = ctx->graph_ticks;
     for (int which = 0; which < 2; which++) {
-        const int steps = which == 0 ? K : 1;
-        if (ctx->tok_exec[which] || (which == 1 && (K == 1 || total % K == 0))) continue;
-        // every argument of the stages is fixed for the life of the context (the step's own arguments sit in *d_step)
+        const int ticks = which == 0 ? K : 2;
+        if (ctx->tok_exec[which] || (which == 1 && (K == 2 || total % K == 0))) continue;
+        // every argument of the launches is fixed for the life of the context (the step's own arguments sit in *d_step)
         hipGraph_t g = nullptr;
-        const hipError_t e = gru_build_graph_h(ctx, p, steps, &g);
-        if (e != hipSuccess) return gfail(ctx, EGG_E_HIP, "graph of the forward's stages", e);
+        const hipError_t e = gru_build_graph_h(ctx, p, ticks, &g);
+        if (e != hipSuccess) return gfail(ctx, EGG_E_HIP, "graph of the forward's ticks", e);
         ctx->tok_graph[which] = g;
         GTRY(hipGraphInstantiate(&ctx->tok_exec[which], g, nullptr, nullptr, 0));
     }
     int t = 0;
     for (; t + K <= total; t += K) GTRY(hipGraphLaunch(ctx->tok_exec[0], ctx->stream));
-    for (; t < total; t++) GTRY(hipGraphLaunch(ctx->tok_exec[1], ctx->stream));
+    for (; t < total; t += 2) GTRY(hipGraphLaunch(ctx->tok_exec[1], ctx->stream));
     return EGG_OK;
 }
-// 1 (default): one launch per stage, spread over the whole GPU; 0: one persistent workgroup per 32 members
+// 1 (default): the stages spread over the whole GPU, a launch per pipeline tick; 0: one persistent workgroup per 32 members
 extern "C" int egg_gru_forward_mode(egg_gru_ctx *ctx, int staged) {
     if (!ctx) return EGG_E_INVALID;
     ctx->staged = staged != 0;
@@ -955,7 +1066,7 @@ extern "C" int egg_gru_step(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t dat
     const egg_gru_config &c = ctx->cfg;
     const int pairs = c.population / 2, nm = (int)ctx->mats.size();
     hipLaunchKernelGGL(k_gru_noise, dim3((nm * pairs + 63) / 64), dim3(64), 0, ctx->stream, ctx->d_mats, nm, pairs, ctx->pairs_pad,
-                       step_seed, ctx->d_noise, ctx->d_panels);
+                       step_seed, ctx->d_noise, ctx->d_nfrag, ctx->d_panels);
     GruParams p;
     p.mats = ctx->d_mats; p.model = ctx->d_model; p.frag = ctx->d_frag; p.noise = ctx->d_noise;
     p.data = d_data; p.data_len = data_len; p.start_idx = start_idx; p.states = ctx->d_states; p.loss = ctx->d_loss;
