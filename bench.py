@@ -255,8 +255,9 @@ def main():
         sec = time.perf_counter() - t0
         gru = {"value": gcfg.population * gcfg.seq_len / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3,
                "workload": "full_trained_egg.c defaults, one full step (forward of 128 members x 4096 tokens + update)",
-               "note": "the bit-exact GPU twin of the CPU baseline's program, not a throughput path: 128 members of 4096 strictly sequential "
-                       "tokens fill four workgroups of the 256 CUs"}
+               "note": "the bit-exact GPU twin of the CPU baseline's program: 128 members of 4096 strictly sequential tokens, walked as a "
+                       "pipeline over the layers with one launch per tick (2 T + 6 L + 1 launches); a tick is bound by streaming the "
+                       "tick's weights into the L2s again, which do not keep them across launches"}
         gctx.close()
     except Exception as e:
         gru = {"error": str(e)}

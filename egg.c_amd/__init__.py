@@ -598,7 +598,7 @@ class GruContext:
         return out
 
     def forward_mode(self, staged=True):
-        """one launch per stage over the whole GPU (default) or one persistent workgroup per 32 members; same results"""
+        """stages spread over the whole GPU, one launch per pipeline tick (default), or one persistent workgroup per 32 members; same results"""
         self._ck(lib().egg_gru_forward_mode(self._h, 1 if staged else 0), "egg_gru_forward_mode")
 
     def state_reset(self):

@@ -313,10 +313,11 @@ int  egg_gru_state_download(egg_gru_ctx *ctx, void *host_states, size_t bytes);
  * do_update, update_matrix on every GRU / MLP / head matrix (:564-574) */
 int  egg_gru_step(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx, uint32_t step_seed, int do_update);
 int  egg_gru_losses(egg_gru_ctx *ctx, int32_t *host_loss, int32_t *host_fit);  /* synchronises */
-/* How egg_gru_step evaluates forward_pass (full_trained_egg.c:213-296) -- same results either way.  1 (default): one
- * launch per dependent stage of a token (norm, gate products, state update, expand, project, head), each spread over
- * the GPU by output strip and member tile, the stages of a token captured once as a hipGraph; 0: one persistent
- * workgroup per 32 members for the whole sequence. */
+/* How egg_gru_step evaluates forward_pass (full_trained_egg.c:213-296) -- same results either way.  1 (default): the
+ * stages of a layer's token (norm, gate products, state update, norm, expand, project; for the head norm, logits,
+ * loss) are spread over the GPU by output strip and member tile, and the sequence is walked as a pipeline over the
+ * layers with one launch per tick that carries every stage that is ready (2 T + 6 L + 1 launches, 64 to a hipGraph);
+ * 0: one persistent workgroup per 32 members for the whole sequence. */
 int  egg_gru_forward_mode(egg_gru_ctx *ctx, int staged);
 
 /* per-kernel-class timing with hipEvent pairs recorded on the context's stream around each launch (the

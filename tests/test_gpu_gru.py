@@ -18,9 +18,10 @@ def _t(dev, arr):
     (dict(hidden=512, n_layers=4, seq_len=3, population=32, update_threshold=10), 2),
     (dict(hidden=256, n_layers=2, seq_len=4, population=96, update_threshold=30), 2),
     (dict(hidden=64, n_layers=1, seq_len=9, population=32, update_threshold=5, sigma_shift=2), 3),
-    (dict(hidden=128, n_layers=4, seq_len=11, population=32, update_threshold=8), 2),    # an 8-token graph, four layers side by side
-], ids=["h64", "h128", "h512", "h256_p96", "sigma_2", "h128_l4_t11"])
-@pytest.mark.parametrize("staged", [True, False], ids=["launch_per_stage", "persistent_workgroups"])
+    (dict(hidden=128, n_layers=4, seq_len=11, population=32, update_threshold=8), 2),
+    (dict(hidden=64, n_layers=2, seq_len=70, population=64, update_threshold=12), 2),     # more ticks than one graph holds
+], ids=["h64", "h128", "h512", "h256_p96", "sigma_2", "h128_l4_t11", "h64_t70"])
+@pytest.mark.parametrize("staged", [True, False, None], ids=["launch_per_tick", "persistent_workgroups", "alternating"])
 def test_gru_steps(pkg, orc, dev, kw, steps, staged):
     import ctypes as C
     g = orc.gru_config(**kw)
@@ -32,7 +33,8 @@ def test_gru_steps(pkg, orc, dev, kw, steps, staged):
     off_b = 256 * H + L * 4 * H * H
     model[off_b:off_b + L * 2 * H] = rng.integers(-30, 31, L * 2 * H).astype(np.int8)
     ctx = pkg.GruContext(pkg.gru_default_config(**kw))
-    ctx.forward_mode(staged)
+    if staged is not None:
+        ctx.forward_mode(staged)
     assert ctx.model_bytes() == model.size
     ctx.model_init(42)
     got0 = ctx.model_download()
@@ -45,6 +47,8 @@ def test_gru_steps(pkg, orc, dev, kw, steps, staged):
     for step in range(steps):
         seed = 1000 + 77 * step
         start = step * kw["seq_len"]
+        if staged is None:                      # the recurrent state is handed from one way of evaluating to the other
+            ctx.forward_mode(step % 2 == 0)
         ctx.step(d_data.data_ptr(), len(data), start, seed, True)
         loss, fit = ctx.losses()
         ref_loss, ref_fit = orc.gru_population(g, model, data, start, seed, 0, P // 2, states)
