@@ -68,6 +68,8 @@ def main():
     ap.add_argument("--population", type=int, default=40960)
     ap.add_argument("--c5-population", type=int, default=16384, help="population of the d-eggs-style side measurement")
     ap.add_argument("--chunk", type=int, default=0, help="members per forward chunk (0 = library default)")
+    ap.add_argument("--gru-seq-len", type=int, default=0,
+                    help="sequence length of the full_trained_egg.c side measurement (0 = the program's 4096); counter runs use a short one")
     ap.add_argument("--data-mib", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="skip the hipGraph replay leg")
@@ -245,6 +247,8 @@ def main():
         if not side:
             raise RuntimeError("skipped (--headline-only)")
         gcfg = pkg.gru_default_config()
+        if args.gru_seq_len:
+            gcfg.seq_len = args.gru_seq_len
         gctx = pkg.GruContext(gcfg)
         gctx.model_init(42)
         gctx.step(d_data.data_ptr(), n, 0, 42, True)
@@ -254,7 +258,7 @@ def main():
         gctx.losses()
         sec = time.perf_counter() - t0
         gru = {"value": gcfg.population * gcfg.seq_len / sec, "unit": "member-tokens/s", "ms_per_step": sec * 1e3,
-               "workload": "full_trained_egg.c defaults, one full step (forward of 128 members x 4096 tokens + update)",
+               "workload": "full_trained_egg.c defaults, one full step (forward of %d members x %d tokens + update)" % (gcfg.population, gcfg.seq_len),
                "note": "the bit-exact GPU twin of the CPU baseline's program: 128 members of 4096 strictly sequential tokens, walked as a "
                        "pipeline over the layers with one launch per tick (2 T + 6 L + 1 launches); a tick is bound by streaming the "
                        "tick's weights into the L2s again, which do not keep them across launches"}
