@@ -424,7 +424,7 @@ class Context:
     def tap(self, name, member):
         import numpy as np
         T, H = self.cfg.seq_len, self.cfg.hidden
-        out = np.zeros((T, 256), np.int32) if name == "logits" else np.zeros((T, H), np.int8)
+        out = np.zeros((T, self.cfg.vocab), np.int32) if name == "logits" else np.zeros((T, H), np.int8)
         self._ck(lib().egg_tap_download(self._h, name.encode(), member, _np_ptr(out)), "egg_tap_download")
         return out
 

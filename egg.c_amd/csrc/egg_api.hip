@@ -280,7 +280,9 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     if (!(c.head_dim == 32 || c.head_dim == 64) || c.hidden % c.head_dim) return refuse("head_dim must be 32 or 64 and divide hidden");
     if (!(c.seq_len == 32 || c.seq_len == 64 || c.seq_len == 128 || c.seq_len == 256 || c.seq_len == 512))
         return refuse("seq_len must be 32, 64, 128, 256 or 512");
-    if (c.vocab != 256) return refuse("vocab must be 256 (byte-level model)");
+    // 256: the byte-level model, the token stream is bytes.  Larger (d-eggs' VOCAB_SIZE, de/include/config.h:22-28): uint32
+    // tokens; the head takes the vocabulary in blocks of 256 columns
+    if (c.vocab < 256 || c.vocab % 256 || c.vocab > 65536) return refuse("vocab must be a multiple of 256, at most 65536");
     if (c.n_layers < 1 || c.population < 2 || (c.population & 1)) return refuse("n_layers >= 1 and an even population >= 2 are required");
     // shift amounts and table scales the kernels can state in 32-bit shifts / 64-bit multiply-adds
     auto in_range = [](int v, int lo, int hi) { return v >= lo && v <= hi; };
@@ -383,8 +385,9 @@ extern "C" int egg_ctx_create(const egg_config *cfg, egg_ctx **out) {
     CR(hipMalloc(&ctx->d_loss, (size_t)c.population * 4)); CR(hipMalloc(&ctx->d_fit, (size_t)(c.population / 2) * 4));
     CR(hipMalloc(&ctx->d_scal, sizeof(Scalars)));
     ctx->pairs_pad = ((c.population / 2) + 63) / 64 * 64;
-    CR(hipMalloc(&ctx->d_panel_a, (size_t)4 * c.hidden * ctx->pairs_pad));
-    CR(hipMalloc(&ctx->d_panel_b, (size_t)4 * c.hidden * ctx->pairs_pad));
+    const size_t panel_rows = std::max(4 * c.hidden, c.vocab);       // the widest side of any matrix: 4 * hidden, or the embedding's vocabulary
+    CR(hipMalloc(&ctx->d_panel_a, panel_rows * ctx->pairs_pad));
+    CR(hipMalloc(&ctx->d_panel_b, panel_rows * ctx->pairs_pad));
 #undef CR
     *out = ctx;
     return EGG_OK;
@@ -626,6 +629,7 @@ static FwdCommon make_common(egg_ctx *ctx, const uint8_t *d_data, int64_t len, c
     f.data = d_data; f.data_len = len; f.d_start_idx = d_start; f.d_step_seed = d_seed;
     f.pop_offset = first_member; f.n_members = nm; f.population = c.population; f.same_data = c.use_same_data != 0;
     f.T = c.seq_len; f.H = c.hidden; f.head_dim = c.head_dim; f.vocab = c.vocab;
+    f.token_bytes = c.vocab > 256 ? 4 : 1;
     f.t0 = 0; f.tn = c.seq_len;
     f.sigma = c.fixed_point + c.sigma_shift; f.sigma_vec = c.sigma_shift_vector;
     f.mask = ctx->mask_override >= 0 ? ctx->mask_override : noise_word(c);
@@ -663,7 +667,9 @@ static int forward_chunk(egg_ctx *ctx, const uint8_t *d_data, int64_t len, const
         p.ln_w = M + L.ln_init; p.ln_b = M + L.ln_init_bias; p.w_up = F + L.w_emb_mlp_up; p.b_up = M + L.mlp_emb_bias_up;
         p.w_dn = F + L.w_emb_mlp_down; p.b_dn = M + L.mlp_emb_bias_down;
         p.embedding = M + L.embedding; p.emb_bias = M + L.emb_bias; p.x = ctx->d_x;
-        p.tab = (ctx->first_dedup && !range) ? ctx->d_q : nullptr;     // the q buffer is free until the first layer's QKV projection writes it
+        // the q buffer is free until the first layer's QKV projection writes it; one row per distinct value only pays (and
+        // is only built) for byte tokens
+        p.tab = (ctx->first_dedup && !range && c.vocab == 256) ? ctx->d_q : nullptr;
         if (Q) {
             p.q_ln_w = Q + L.ln_init; p.q_ln_b = Q + L.ln_init_bias; p.q_b_up = Q + L.mlp_emb_bias_up; p.q_b_dn = Q + L.mlp_emb_bias_down;
             p.q_up = Q + L.w_emb_mlp_up; p.q_dn = Q + L.w_emb_mlp_down; p.q_emb = Q + L.embedding; p.q_emb_bias = Q + L.emb_bias;
@@ -1030,6 +1036,7 @@ static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_
     const egg_config &c = ctx->cfg; const int T = c.seq_len, total = seed_len + gen_len;
     if (seed_len < 1 || gen_len < 0 || total > T) return fail(ctx, EGG_E_INVALID, "egg_generate: need 1 <= seed_len and seed_len + gen_len <= seq_len");
     if (ctx->captured) return fail(ctx, EGG_E_STATE, "egg_generate cannot run on a context whose step is captured");
+    if (c.vocab != 256) return fail(ctx, EGG_E_INVALID, "egg_generate: byte vocabulary only (the buffer holds bytes)");
     hipStream_t s = ctx->stream;
     if (!ctx->d_gen_tok) {
         HIP_TRY(hipMalloc(&ctx->d_gen_tok, (size_t)T + 16));
@@ -1111,7 +1118,7 @@ extern "C" int egg_ctx_enable_taps(egg_ctx *ctx, int enable) {
         ctx->tap_members = ctx->chunk < 64 ? ctx->chunk : 64;
         size_t one = (size_t)ctx->tap_members * c.seq_len * c.hidden;
         HIP_TRY(hipMalloc(&ctx->d_tap, one * (1 + 6 * c.n_layers)));
-        HIP_TRY(hipMalloc(&ctx->d_tap_logits, (size_t)ctx->tap_members * c.seq_len * 256 * 4));
+        HIP_TRY(hipMalloc(&ctx->d_tap_logits, (size_t)ctx->tap_members * c.seq_len * c.vocab * 4));
     }
     ctx->taps = enable != 0;
     return EGG_OK;
@@ -1127,7 +1134,7 @@ extern "C" int egg_tap_download(egg_ctx *ctx, const char *name, int member, void
     const egg_config &c = ctx->cfg; const int T = c.seq_len, H = c.hidden;
     HIP_TRY(hipStreamSynchronize(ctx->stream));
     if (!strcmp(name, "logits")) {
-        HIP_TRY(hipMemcpy(host_out, ctx->d_tap_logits + (size_t)member * T * 256, (size_t)T * 256 * 4, hipMemcpyDeviceToHost));
+        HIP_TRY(hipMemcpy(host_out, ctx->d_tap_logits + (size_t)member * T * c.vocab, (size_t)T * c.vocab * 4, hipMemcpyDeviceToHost));
         return EGG_OK;
     }
     int slot = -1, layer = 0; char base[32] = {0};

@@ -23,6 +23,11 @@ __device__ __forceinline__ int64_t stream_pos_of(const FwdCommon &c, int member)
     return (*c.d_start_idx + pair * stride) % (c.data_len - c.T);
 }
 
+// token i of the stream: bytes, or uint32 where the vocabulary is larger than 256 (TokenType, de/include/config.h:26-28)
+__device__ __forceinline__ int token_at(const FwdCommon &c, int64_t i) {
+    return c.token_bytes == 4 ? (int)reinterpret_cast<const uint32_t *>(c.data)[i] : (int)c.data[i];
+}
+
 // acc[nt][r] += (sb * At[n]) >> sigma for NT column groups starting at table offset n_off
 template <int NT>
 __device__ __forceinline__ void add_perturb(v16i *acc, int sb, const int *At, int n_off, int sigma, int g) {
@@ -308,7 +313,7 @@ __global__ void __launch_bounds__(EGG_THREADS, MlpCfg<H>::OCC) k_mlp(MlpParams p
 
         if (FIRST) {
             // embedding stage (mgpu.cu:901-931)
-            const int tok = dedup ? uniq[min(t, nrows - 1)] : c.data[spos + t];
+            const int tok = dedup ? uniq[min(t, nrows - 1)] : token_at(c, spos + t);
             int a_tok = noise_from_hash(pair_seed + OFF_EMB, (uint32_t)tok, c.mask);
             if (ADAPT) a_tok *= p.q_emb[H + tok];        // a_tok * q(token); the table holds b_dim * q(hidden) * ns
             const uint32_t *E32 = reinterpret_cast<const uint32_t *>(p.embedding);
@@ -1088,7 +1093,8 @@ struct HeadLds {
 
 // ADAPT: adaptive noise overlay; the tied head takes the embedding's per-hidden q values on its input side and the
 // per-token values on its output side (de/src/kernels.cu:200-240)
-template <int H, bool ADAPT>
+// BIG: a vocabulary of more than 256 entries
+template <int H, bool ADAPT, bool BIG>
 __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadParams p) {
     constexpr int KS = H / 32, NV = 256 / 32, BLK = H < 256 ? H : 256;
     extern __shared__ __align__(16) int8_t smem[];
@@ -1108,17 +1114,25 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
     const int ns = (member & 1) ? -1 : 1;
     const uint32_t pair_seed = *c.d_step_seed + (uint32_t)(member / 2);
 
+    // The vocabulary is taken in blocks of 256 columns.  One block (the byte-level model): the logits stay in registers
+    // between the maximum and the sum.  More: like the reference (de/src/kernels.cu:233-272) the projection runs twice,
+    // first for the maximum, then for the sum of the table weights and the target's logit; the output-side noise of a
+    // block is rebuilt in front of it (noise(seed, 256 b + i) is the hash of seed + 256 b * 0x9e3779b9 at index i).
+    const int V = BIG ? c.vocab : 256, nvb = BIG ? V >> 8 : 1;
+    constexpr bool single = !BIG;
     WStream ws; wstream_init(ws, wlds, WUnit<BLK>::BYTES);
-    w_prefetch<BLK>(ws, w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0));
+    w_prefetch<BLK>(ws, w_unit_ptr<BLK>(p.embedding_frag, V, 0, 0, 0));
     for (int i = threadIdx.x; i < 256; i += EGG_THREADS) lut[i] = c.exp_lut[i];
     if (ADAPT) {
         fill_vec_i32_ov(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane, 64, 2, p.q_ln_w);
         fill_vec_i32_ov(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane, 64, 0, p.q_ln_b);
-        fill_noise_i32_ov(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane, 64, p.q_emb + H);
     } else {
         fill_vec_i32(lnw, p.ln_w, pair_seed + OFF_LN_F_A, pair_seed + OFF_LN_F_B, H, c.mask, ns, c.sigma_vec, lane, 64, 2);   // 4 * gain, see standard_scale
         fill_vec_i32(lnb, p.ln_b, pair_seed + OFF_LN_F_BIAS_A, pair_seed + OFF_LN_F_BIAS_B, H, c.mask, ns, c.sigma_vec, lane);
-        fill_noise_i32(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane);
+    }
+    if (single) {
+        if (ADAPT) fill_noise_i32_ov(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane, 64, p.q_emb + H);
+        else fill_noise_i32(hA, pair_seed + OFF_EMB, 256, c.mask, ns, lane);
     }
     fill_noise_i8(hB, pair_seed + OFF_EMB + H, H, c.mask, lane);
     __syncthreads();
@@ -1134,39 +1148,90 @@ __global__ void __launch_bounds__(EGG_THREADS, (H > 256 ? 1 : 2)) k_head(HeadPar
         for (int ks = 0; ks < KS; ks++) x[ks] = load_op(p.x + row, ks, g);
         standard_norm<KS>(x, nf, lnw, lnb, g);
         const int sbh = ADAPT ? dot_noise_ov<KS, false>(nf, hB, p.q_emb, 0, g) : dot_noise<KS, false>(nf, hB, 0, g);
-        v16i acc[NV];
-        zero_acc<NV>(acc);
-        gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, ws, (pass + 1 < pass_end) ? w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0) : nullptr, lane);
-        add_perturb<NV>(acc, sbh, hA, 0, c.sigma, g);
+        int gmax = INT_MIN, target;
+        long long sum_ex; int tl;
         // two-pass softmax statistics (mgpu.cu:969-1009)
-        int gmax = INT_MIN;
-#pragma unroll
-        for (int nt = 0; nt < NV; nt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) { acc[nt][r] >>= c.shift_logit; gmax = max(gmax, acc[nt][r]); }
-        gmax = max_halves(gmax);
-        const int target = c.data[spos + t + 1];
-        long long sum_ex = 0; int tl = 0;
-#pragma unroll
-        for (int nt = 0; nt < NV; nt++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                int idx = min(255, max(0, gmax - acc[nt][r]));
-                sum_ex += lut[idx];
-                if (col_of(nt, r, g) == target) tl = acc[nt][r];
-            }
-        sum_ex = sum_halves64(sum_ex);
-        tl = sum_halves(tl);
-        if (p.logits_tap && valid)
+        if constexpr (single) {
+            v16i acc[NV];
+            zero_acc<NV>(acc);
+            gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, 256, 0, 0, ws, (pass + 1 < pass_end) ? w_unit_ptr<BLK>(p.embedding_frag, 256, 0, 0, 0) : nullptr, lane);
+            add_perturb<NV>(acc, sbh, hA, 0, c.sigma, g);
 #pragma unroll
             for (int nt = 0; nt < NV; nt++)
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    v4i o4;
+                for (int r = 0; r < 16; r++) { acc[nt][r] >>= c.shift_logit; gmax = max(gmax, acc[nt][r]); }
+            gmax = max_halves(gmax);
+            target = c.data[spos + t + 1];
+            sum_ex = 0; tl = 0;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o4[e] = acc[nt][4 * q + e];
-                    *reinterpret_cast<v4i *>(p.logits_tap + ((size_t)mloc * T + t) * 256 + 32 * nt + 8 * q + 4 * g) = o4;
+            for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    int idx = min(255, max(0, gmax - acc[nt][r]));
+                    sum_ex += lut[idx];
+                    if (col_of(nt, r, g) == target) tl = acc[nt][r];
                 }
+            sum_ex = sum_halves64(sum_ex);
+            tl = sum_halves(tl);
+            if (p.logits_tap && valid)
+#pragma unroll
+                for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        v4i o4;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o4[e] = acc[nt][4 * q + e];
+                        *reinterpret_cast<v4i *>(p.logits_tap + ((size_t)mloc * T + t) * 256 + 32 * nt + 8 * q + 4 * g) = o4;
+                    }
+        } else {
+            target = token_at(c, spos + t + 1);
+            sum_ex = 0; tl = 0;
+#pragma unroll 1
+            for (int phase = 0; phase < 2; phase++) {
+#pragma unroll 1
+                for (int vb = 0; vb < nvb; vb++) {
+                    {                                   // read behind the barriers of the product below, by this wave only
+                        const uint32_t seed = pair_seed + OFF_EMB + (uint32_t)(vb * 256) * 0x9e3779b9u;
+                        if (ADAPT) fill_noise_i32_ov(hA, seed, 256, c.mask, ns, lane, 64, p.q_emb + H + vb * 256);
+                        else fill_noise_i32(hA, seed, 256, c.mask, ns, lane);
+                    }
+                    const bool last = vb + 1 == nvb && phase == 1;
+                    const int8_t *next = !last ? w_unit_ptr<BLK>(p.embedding_frag, V, 0, (vb + 1 == nvb ? 0 : vb + 1) * 256, 0)
+                                               : ((pass + 1 < pass_end) ? w_unit_ptr<BLK>(p.embedding_frag, V, 0, 0, 0) : nullptr);
+                    v16i acc[NV];
+                    zero_acc<NV>(acc);
+                    gemm_stream<H, 256, BLK>(acc, nf, p.embedding_frag, V, 0, vb * 256, ws, next, lane);
+                    add_perturb<NV>(acc, sbh, hA, 0, c.sigma, g);
+                    if (phase == 0) {
+#pragma unroll
+                        for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+                            for (int r = 0; r < 16; r++) { acc[nt][r] >>= c.shift_logit; gmax = max(gmax, acc[nt][r]); }
+                        if (p.logits_tap && valid)
+#pragma unroll
+                            for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+                                for (int q = 0; q < 4; q++) {
+                                    v4i o4;
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) o4[e] = acc[nt][4 * q + e];
+                                    *reinterpret_cast<v4i *>(p.logits_tap + ((size_t)mloc * T + t) * V + vb * 256 + 32 * nt + 8 * q + 4 * g) = o4;
+                                }
+                    } else {
+#pragma unroll
+                        for (int nt = 0; nt < NV; nt++)
+#pragma unroll
+                            for (int r = 0; r < 16; r++) {
+                                const int lg = acc[nt][r] >> c.shift_logit;
+                                sum_ex += lut[min(255, max(0, gmax - lg))];
+                                if (vb * 256 + col_of(nt, r, g) == target) tl = lg;
+                            }
+                    }
+                }
+                if (phase == 0) gmax = max_halves(gmax);
+            }
+        }
+        if constexpr (!single) { sum_ex = sum_halves64(sum_ex); tl = sum_halves(tl); }
         // loss (mgpu.cu:1012-1024)
         long long log_sum = 0;
         if (sum_ex > 0) {
@@ -1273,8 +1338,12 @@ template <int H>
 static hipError_t launch_head_h(const HeadParams &p, hipStream_t s) {
     dim3 grid((p.c.n_members + EGG_WAVES - 1) / EGG_WAVES), block(EGG_THREADS);
     size_t lds = HeadLds<H>::TOTAL;
-    if (p.q_ln_w) hipLaunchKernelGGL((k_head<H, true>), grid, block, lds, s, p);
-    else hipLaunchKernelGGL((k_head<H, false>), grid, block, lds, s, p);
+    if (p.c.vocab < 256 || p.c.vocab % 256) return hipErrorInvalidValue;
+    if (p.c.vocab > 256) {
+        if (p.q_ln_w) hipLaunchKernelGGL((k_head<H, true, true>), grid, block, lds, s, p);
+        else hipLaunchKernelGGL((k_head<H, false, true>), grid, block, lds, s, p);
+    } else if (p.q_ln_w) hipLaunchKernelGGL((k_head<H, true, false>), grid, block, lds, s, p);
+    else hipLaunchKernelGGL((k_head<H, false, false>), grid, block, lds, s, p);
     return hipGetLastError();
 }
 hipError_t egg_launch_head(const HeadParams &p, hipStream_t s) {
@@ -1316,8 +1385,10 @@ static hipError_t prepare_h(int T) {
     SET_LDS((k_mlp<H, false, false, true>), MlpCfg<H>::total(msets, false));
     SET_LDS((k_qkv<H, false>), QkvCfg<H>::total(sets));
     SET_LDS((k_qkv<H, true>), QkvCfg<H>::total(sets));
-    SET_LDS((k_head<H, false>), HeadLds<H>::TOTAL);
-    SET_LDS((k_head<H, true>), HeadLds<H>::TOTAL);
+    SET_LDS((k_head<H, false, false>), HeadLds<H>::TOTAL);
+    SET_LDS((k_head<H, true, false>), HeadLds<H>::TOTAL);
+    SET_LDS((k_head<H, false, true>), HeadLds<H>::TOTAL);
+    SET_LDS((k_head<H, true, true>), HeadLds<H>::TOTAL);
     return hipSuccess;
 }
 template <int HD, int CT>

@@ -36,7 +36,7 @@ static inline long long egg_mlp_up_acc_bound(int hidden, int mask, int sigma_vec
 
 // what every forward kernel needs to know about the run
 struct FwdCommon {
-    const uint8_t  *data;        // token stream (device)
+    const uint8_t  *data;        // token stream (device): bytes, or uint32 tokens when token_bytes is 4
     int64_t         data_len;
     const int64_t  *d_start_idx; // device scalar: step * seq_len
     const uint32_t *d_step_seed; // device scalar
@@ -45,6 +45,7 @@ struct FwdCommon {
     int population;
     int same_data;               // USE_SAME_DATA: every pair reads the window at the start index
     int T, H, head_dim, vocab;
+    int token_bytes;             // 1 (vocab 256) or 4 (larger vocabularies); data_len counts tokens
     int t0, tn;                  // token positions [t0, t0 + tn) of every member are evaluated (multiples of 32; the whole window: 0, T);
                                  // attention still reads the K / V rows of every position in front of them
     int sigma;                   // fixed_point + sigma_shift

@@ -40,7 +40,7 @@ typedef struct egg_config {
     int head_dim;            /* HEAD_DIM: 32 or 64, divides hidden                    */
     int n_layers;            /* N_LAYERS                                              */
     int seq_len;             /* SEQ_LEN: multiple of 32                               */
-    int vocab;               /* VOCAB_SIZE: 256 (byte level)                          */
+    int vocab;               /* VOCAB_SIZE: 256 (byte level), or a multiple of 256 <= 65536 */
     int population;          /* POPULATION_SIZE: even                                 */
     int fixed_point;         /* 4                                                     */
     int sigma_shift;         /* 3                                                     */
@@ -126,7 +126,9 @@ int  egg_ctx_linear_kernel(egg_ctx *ctx, int w_stationary);
 
 /* train_sequence_kernel<<<batch,...>>> (mgpu.cu:847-1029, launch :1531): evaluates members
  * [pop_offset, pop_offset+pop_count) on tokens d_data[stream_pos + t], writes d_loss[member] (int32).
- * pop_offset and pop_count must be even. */
+ * pop_offset and pop_count must be even.  With vocab 256 the stream is bytes; with a larger vocabulary d_data points at
+ * uint32 tokens (d-eggs' TokenType, de/include/config.h:22-28), every one below vocab.  data_len counts tokens either
+ * way.  The same holds for egg_population_forward_dev, egg_step and egg_step_capture. */
 int  egg_population_forward(egg_ctx *ctx, const uint8_t *d_data, int64_t data_len, int64_t start_idx,
                             uint32_t step_seed, int pop_offset, int pop_count, int32_t *d_loss);
 /* same, with the step seed and start index read from device memory when the launch executes

@@ -518,6 +518,12 @@ static Tables make_tables(const orc_config *c) {
     return t;
 }
 
+/* token i of the stream: bytes for the byte-level model; d-eggs' TokenType is uint32 for any other VOCAB_SIZE
+ * (de/include/config.h:22-28), and `data` then points at uint32 tokens, data_len counting tokens */
+static inline int tok_at(const orc_config *c, const uint8_t *data, int64_t i) {
+    return c->vocab > 256 ? (int)reinterpret_cast<const uint32_t *>(data)[i] : (int)data[i];
+}
+
 /* mgpu.cu:847-1029 (one block == one member) */
 static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_t *model,
                               const uint8_t *data, int64_t data_len, int64_t start_idx,
@@ -539,7 +545,7 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
 
     for (int t = 0; t < T; t++) {
         /* 1. embedding, mgpu.cu:901-931 */
-        int tok = data[stream_pos + t];
+        int tok = tok_at(c, data, stream_pos + t);
         uint32_t seed_emb = pair_seed + OFF_EMB;
         for (int tid = 0; tid < H; tid++) {
             int8_t emb = blk(model + L.embedding, V, tid, tok);
@@ -623,7 +629,7 @@ static int32_t forward_member(const orc_config *c, const Tables &tb, const int8_
             logits[v] = ah >> c->shift_logit;
         }
         if (tr && tr->logits) memcpy(tr->logits + (size_t)t * V, logits.data(), sizeof(int32_t) * V);
-        int target = data[stream_pos + t + 1];
+        int target = tok_at(c, data, stream_pos + t + 1);
         int64_t lt = orc_token_loss(c, tb.exp_lut.data(), logits.data(), V, target);
         if (tr && tr->loss_t) tr->loss_t[t] = lt;
         my_loss += lt;

@@ -13,7 +13,10 @@ SMALL = dict(hidden=64, head_dim=32, n_layers=2, seq_len=32, population=8)
 
 def _t(dev, arr):
     import torch
-    return torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+    arr = np.ascontiguousarray(arr)
+    if arr.dtype == np.uint32:          # same bytes; torch's own uint32 support is partial
+        arr = arr.view(np.int32)
+    return torch.from_numpy(arr).to(dev)
 
 
 def _mapping_hint(got, exp):
@@ -169,6 +172,14 @@ def test_w_stationary_linear(pkg, orc, dev, K, members, T, own, extra):
     ctx.close()
 
 
+def _stream(orc, ocfg, n):
+    """the synthetic token stream: bytes for the byte-level model, uint32 tokens that reach the whole vocabulary otherwise"""
+    data = orc.zipf_bytes(n if ocfg.vocab == 256 else 2 * n)
+    if ocfg.vocab > 256:
+        data = ((data[0::2].astype(np.uint32) << 8 | data[1::2]) % ocfg.vocab).astype(np.uint32)
+    return data
+
+
 STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao", "x_attn", "x_mlp")]
 
 
@@ -193,12 +204,18 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
                                 # DEVICE_GAUSSIAN / HOST_GAUSSIAN: noise up to +-45 (the kernels' unfused shift path)
                                 dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4, device_gaussian=1, host_gaussian=1),
                                 # USE_SAME_DATA: every pair reads the same window
-                                dict(hidden=128, head_dim=64, n_layers=1, seq_len=128, population=6, use_same_data=1)],
-                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30", "gaussian", "same_data"])
+                                dict(hidden=128, head_dim=64, n_layers=1, seq_len=128, population=6, use_same_data=1),
+                                # vocabularies of more than 256 entries: uint32 tokens, the head in blocks of 256 columns
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4, vocab=512),
+                                dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4, vocab=1024),
+                                dict(hidden=512, head_dim=64, n_layers=1, seq_len=32, population=4, vocab=768),
+                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=64, population=6, vocab=2048, sigma_shift=5, noise_mask=31)],
+                         ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30", "gaussian", "same_data",
+                              "vocab_512", "h256_vocab_1024", "h512_vocab_768", "vocab_2048_wide_noise"])
 def test_forward_stages_and_loss(pkg, orc, dev, kw):
     """Every stage tap of every member against the oracle's trace, then the per-member losses."""
-    data = orc.zipf_bytes(1 << 15)
     ocfg = orc.config(**kw)
+    data = _stream(orc, ocfg, 1 << 15)
     model = orc.init_model(ocfg, 42)
     # make biases / gains non-trivial so every term of the arithmetic is exercised
     rng = np.random.default_rng(5)
@@ -318,8 +335,9 @@ def test_fitness(pkg, orc, dev):
 @pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=200),
                                 dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=66),
                                 dict(hidden=512, head_dim=64, n_layers=1, seq_len=128, population=40),
-                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=200, device_gaussian=1)],
-                         ids=["p200", "p66", "h512", "gaussian"])
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=200, device_gaussian=1),
+                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=66, vocab=768)],
+                         ids=["p200", "p66", "h512", "gaussian", "vocab_768"])
 def test_votes_and_adam_update(pkg, orc, dev, kw):
     import torch
     ocfg = orc.config(**kw)
@@ -370,11 +388,12 @@ def test_votes_and_adam_update(pkg, orc, dev, kw):
     ctx.close()
 
 
-def test_full_step_eager_and_graph(pkg, orc, dev):
+@pytest.mark.parametrize("kw", [dict(hidden=64, head_dim=32, n_layers=2, seq_len=32, population=16),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=16, vocab=512)], ids=["bytes", "vocab_512"])
+def test_full_step_eager_and_graph(pkg, orc, dev, kw):
     """Whole ES steps (forward + fitness + update): eager and hipGraph replays follow the oracle's weight trajectory."""
-    kw = dict(hidden=64, head_dim=32, n_layers=2, seq_len=32, population=16)
-    data = orc.zipf_bytes(1 << 15)
     ocfg = orc.config(**kw)
+    data = _stream(orc, ocfg, 1 << 15)
     d_data = _t(dev, data)
     for mode in ("eager", "graph"):
         model = orc.init_model(ocfg, 42)
@@ -465,6 +484,14 @@ def test_error_paths(pkg, dev):
         pkg.Context(pkg.default_config(hidden=100))
     with pytest.raises(pkg.EggError):
         pkg.Context(pkg.default_config(seq_len=48))
+    with pytest.raises(pkg.EggError):
+        pkg.Context(pkg.default_config(vocab=300))        # multiples of 256 only
+    big = pkg.Context(pkg.default_config(vocab=512, **SMALL))
+    import torch
+    buf = torch.zeros(SMALL["seq_len"], dtype=torch.uint8, device=dev)
+    with pytest.raises(pkg.EggError):
+        big.generate(buf.data_ptr(), 4, 4, 1)              # the generation buffer holds bytes
+    big.close()
     ctx = pkg.Context(pkg.default_config(**SMALL))
     with pytest.raises(pkg.EggError):
         ctx.step_launch(0, 1, 0.1)            # launch before capture

@@ -306,6 +306,13 @@ def test_token_loss(orc):
     S = int(ex[np.clip(lg.max() - lg, 0, 255)].astype(np.int64).sum())
     exp = ((((S.bit_length() - 1) << 4) - (18 << 4)) >> 1) + int(lg.max()) - int(lg[11])
     assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), 256, 11) == exp
+    # a larger vocabulary (de/src/kernels.cu:233-290 loops over VOCAB_SIZE): uniform logits give log2(V) * 16 / 2
+    for V in (512, 8192):
+        lg = np.full(V, -3, np.int32)
+        assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), V, V - 1) == 8 * (V.bit_length() - 1)
+        lg = np.full(V, -1000, np.int32); lg[V - 2] = 300
+        assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), V, V - 2) == 0
+        assert orc.lib().orc_token_loss(C.byref(cfg), P(ex), P(lg), V, 300) == 1300
 
 
 def test_forward_invariants(orc):
@@ -845,8 +852,9 @@ def test_ternary_model_packing_and_weight_limit(orc):
                                      shift_out=8, shift_mlp_up=7, shift_mlp_down=9, sigma_shift_vector=3),
                                 dict(hidden=256, head_dim=64, n_layers=4, seq_len=8, population=2),
                                 dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=4, device_gaussian=1, host_gaussian=1),
-                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=6, use_same_data=1)],
-                         ids=["h64", "h128", "other_shifts", "h256_l4", "gaussian", "same_data"])
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=6, use_same_data=1),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=16, population=4, vocab=768)],
+                         ids=["h64", "h128", "other_shifts", "h256_l4", "gaussian", "same_data", "vocab_768"])
 def test_two_restatements_of_the_forward_agree(orc, kw):
     """Nothing external pins the composition of the whole forward (the reference ships no golden vectors), so it is
     stated twice: the C++ oracle walks token by token with a K/V cache as the reference kernel does, the numpy
@@ -855,6 +863,8 @@ def test_two_restatements_of_the_forward_agree(orc, kw):
     from oracle import forward_numpy as fn
     cfg = orc.config(**kw)
     data = orc.zipf_bytes(1 << 13)
+    if cfg.vocab > 256:                      # uint32 tokens, every value of the vocabulary reachable
+        data = ((data[0::2].astype(np.uint32) << 8 | data[1::2]) % cfg.vocab).astype(np.uint32)
     model = orc.init_model(cfg, 42)
     rng = np.random.default_rng(21)
     for t in orc.tensor_table(cfg):          # non-trivial gains and biases
