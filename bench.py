@@ -326,6 +326,31 @@ def main():
               "workload": f"hidden {H5}, 8 heads, seq {T5}, {L5} layers, ternary-packed weights (unpacked on upload, weight limit 1), "
                           f"population {P5} in one launch per kernel, one full step: forward + fitness + votes + Muon"}
         c5ctx.close()
+        # the same shape with d-eggs' default vocabulary (VOCAB_SIZE 8192, uint32 tokens): the head then costs 2 x 2 H V
+        # ops per token (the projection runs twice, like the reference's) beside the layers' 2 x 12 H^2 each
+        try:
+            PV = min(P5, 4096)
+            raw = d_data[: 1 << 23].to(torch.int32)
+            d_tok = ((raw[0::2] << 8 | raw[1::2]) % 8192).contiguous()
+            vctx = pkg.Context(pkg.default_config(hidden=H5, head_dim=64, n_layers=L5, seq_len=T5, population=PV, use_muon=1, vocab=8192))
+            vctx.set_stream(stream.cuda_stream)
+            vctx.model_init(42)
+            vctx.step(d_tok.data_ptr(), d_tok.numel(), 0, 42, 0.3)
+            torch.cuda.synchronize()
+            vctx.enable_timing(True); vctx.timing_reset()
+            t0 = time.perf_counter()
+            vctx.step(d_tok.data_ptr(), d_tok.numel(), T5, 43, 0.3)
+            torch.cuda.synchronize()
+            vsec = time.perf_counter() - t0
+            vtm = vctx.timing()
+            c5["vocab_8192"] = {"value": PV * T5 / vsec, "unit": "member-tokens/s", "ms_per_step": vsec * 1e3, "population": PV,
+                                "kernel_ms_per_step": {k: round(vtm[k][1], 3) for k in fwd if vtm[k][0]},
+                                "head_frac_mfma": round(2 * 2.0 * H5 * 8192 * PV * T5 / (vtm["head"][1] * 1e-3) / PEAK_INT8_OPS, 4) if vtm["head"][1] > 0 else None,
+                                "workload": f"as above with vocabulary 8192 and uint32 tokens, population {PV}, int8 weights from the reference initialisation"}
+            vctx.close()
+            del d_tok, raw
+        except Exception as e:
+            c5["vocab_8192"] = {"error": str(e)}
     except Exception as e:
         c5 = {"error": str(e)}
 

@@ -8,7 +8,10 @@ pytestmark = pytest.mark.gpu
 
 def _t(dev, arr):
     import torch
-    return torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
+    arr = np.ascontiguousarray(arr)
+    if arr.dtype == np.uint32:          # same bytes; torch's own uint32 support is partial
+        arr = arr.view(np.int32)
+    return torch.from_numpy(arr).to(dev)
 
 
 def _model_with_nontrivial_vectors(orc, ocfg, seed):
@@ -25,12 +28,15 @@ def _model_with_nontrivial_vectors(orc, ocfg, seed):
                                 dict(hidden=128, head_dim=32, n_layers=1, seq_len=64, population=4),
                                 dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4),
                                 dict(hidden=512, head_dim=64, n_layers=1, seq_len=32, population=2),
-                                dict(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=4, sigma_shift=5, noise_mask=31)],
-                         ids=["h64", "h128", "h256", "h512", "wide_noise"])
+                                dict(hidden=256, head_dim=64, n_layers=1, seq_len=64, population=4, sigma_shift=5, noise_mask=31),
+                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=4, vocab=768)],
+                         ids=["h64", "h128", "h256", "h512", "wide_noise", "vocab_768"])
 def test_adaptive_forward_stages_and_loss(pkg, orc, dev, kw):
     import torch
-    data = orc.zipf_bytes(1 << 15)
     ocfg = orc.config(**kw)
+    data = orc.zipf_bytes(1 << 15)
+    if ocfg.vocab > 256:                     # uint32 tokens over the whole vocabulary
+        data = ((data[0::2].astype(np.uint32) << 8 | data[1::2]) % ocfg.vocab).astype(np.uint32)
     model = _model_with_nontrivial_vectors(orc, ocfg, 5)
     rng = np.random.default_rng(17)
     # every regime of the factor: below zero, fractional, saturated

@@ -220,3 +220,49 @@ def test_deggs_style_h512_l8_t512_ternary_muon_population_16384(pkg, orc, dev):
         assert np.allclose(got_st["acc"][same], st["acc"][same], atol=2e-3), name
         assert np.count_nonzero(W != model[t["offset"]:t["offset"] + n]) > 0, "the oracle moved no weight of " + name
     ctx.close()
+
+
+def test_deggs_default_vocabulary_8192(pkg, orc, dev):
+    """The d-eggs-style configuration with d-eggs' default vocabulary (VOCAB_SIZE 8192, uint32 tokens): 2048 members in
+    one launch per kernel -- determinism, sampled pairs and the embedding's votes against the oracle."""
+    import torch
+    pop, pairs = 2048, 1024
+    kw = dict(hidden=512, head_dim=64, n_layers=8, seq_len=512, population=pop, weight_limit=1, vocab=8192)
+    ocfg = orc.config(**kw)
+    model = _ternary_model(orc, ocfg, 6)
+    raw = orc.zipf_bytes(1 << 23)
+    # 13-bit tokens from two Zipf bytes: frequent tokens stay frequent, the whole vocabulary is reachable
+    data = ((raw[0::2].astype(np.uint32) << 8 | raw[1::2]) % 8192).astype(np.uint32)
+    assert int(data.max()) == 8191
+    d_data = _t(dev, data.view(np.int32))
+    start, seed = 5 * 512, 0xBEE5
+    ctx = pkg.Context(pkg.default_config(use_muon=1, **kw))
+    ctx.model_upload_ternary(orc.ternary_model_pack(ocfg, model))
+    assert np.array_equal(ctx.model_download(), model)
+    d_loss = torch.full((pop,), -1, dtype=torch.int32, device=dev)
+    runs = []
+    for rep in range(2):
+        ctx.population_forward(d_data.data_ptr(), len(data), start, seed, 0, pop, d_loss.data_ptr())
+        ctx.sync()
+        runs.append(d_loss.cpu().numpy())
+    loss = runs[0]
+    assert np.array_equal(loss, runs[1]), "two evaluations of the same step differ"
+    assert loss.min() > 0
+    for first in (0, pop - 2):
+        ref = orc.population_forward(ocfg, model, data, start, seed, first, 2)
+        assert np.array_equal(loss[first:first + 2], ref[first:first + 2]), (first, loss[first:first + 2], ref[first:first + 2])
+    # the embedding (512 x 8192, the widest vote panel) against the oracle's votes
+    fit = orc.fitness(loss)
+    d_fit = _t(dev, fit)
+    d_seed = _t(dev, np.array([seed], np.uint32).view(np.int32))
+    t = {t["name"]: t for t in ctx.tensors()}["embedding"]
+    assert (t["rows"], t["cols"]) == (512, 8192)
+    n = t["rows"] * t["cols"]
+    d_votes = torch.zeros(n, dtype=torch.int32, device=dev)
+    ctx.matrix_votes(t["id"], d_fit.data_ptr(), d_seed.data_ptr(), d_votes.data_ptr())
+    ctx.sync()
+    ref = np.zeros(n, np.int32)
+    orc.lib().orc_matrix_votes(C.byref(ocfg), t["rows"], t["cols"], t["off_a"], t["off_b"], t["seed_base"],
+                               fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed), ref.ctypes.data_as(C.c_void_p))
+    assert np.array_equal(d_votes.cpu().numpy(), ref)
+    ctx.close()
