@@ -211,3 +211,59 @@ def test_population_40960_one_launch_equals_chunks_of_8192(pkg, orc, dev):
         ctx.close()
     assert got[0].min() > 0
     assert np.array_equal(got[0], got[8192])
+
+
+def test_population_40960_steps_checked_link_by_link(pkg, orc, dev):
+    """A trajectory at the headline size whose every link is held against the oracle on samples: before each of ten
+    steps the weights and the optimizer state come back from the GPU; the oracle then evaluates two sampled pairs on
+    those weights (they depend on every tensor of the model), and applies the step's update to a matrix and a vector
+    tensor of its own from that state and the step's fitness.  Losses, updated weights and float state must agree bit
+    for bit at every step; the sampled pairs and tensors change from step to step."""
+    import torch
+    pop = 40960
+    pairs = pop // 2
+    kw = dict(population=pop, **SHAPE)
+    data = orc.zipf_bytes(1 << 23)
+    ocfg = orc.config(**kw)
+    d_data = _t(dev, data)
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_init(42)
+    tensors = {t["name"]: t for t in ctx.tensors()}
+    plan = [("w_q.0", "ln_1.2"), ("w_o.3", "mlp_bias_up.1"), ("embedding", "ln_f"), ("w_k.2", "emb_bias"), ("w_v.1", "ln_2_bias.0"),
+            ("w_up.2", "ln_init"), ("w_down.0", "mlp_bias_down.3"), ("w_emb_mlp_up", "ln_f_bias"), ("w_emb_mlp_down", "ln_1_bias.1"),
+            ("w_q.3", "mlp_emb_bias_up")]
+    seed, lr = 42, 8.0
+    changed = 0
+    for step, names in enumerate(plan):
+        start = step * SHAPE["seq_len"]
+        model = ctx.model_download().copy()
+        state = ctx.opt_state_download().view(orc.ADAM_DTYPE).copy()
+        ctx.step(d_data.data_ptr(), len(data), start, seed, lr)
+        loss, fit = ctx.step_losses()
+        assert np.array_equal(fit, orc.fitness(loss))
+        for first in ((7919 * (step + 1)) % pop & ~1, (20011 * (step + 3)) % pop & ~1, pop - 2 - 2 * step):
+            ref = orc.population_forward(ocfg, model, data, start, seed, first, 2)
+            assert np.array_equal(loss[first:first + 2], ref[first:first + 2]), (step, first)
+        got_m = ctx.model_download()
+        got_s = ctx.opt_state_download().view(orc.ADAM_DTYPE)
+        changed += ctx.last_update_count()
+        for name in names:
+            t = tensors[name]
+            n = t["rows"] * t["cols"]
+            sl = slice(t["offset"], t["offset"] + n)
+            w = model[sl].copy()
+            st = state[sl].copy()
+            if t["is_matrix"]:
+                orc.lib().orc_update_matrix_adam(C.byref(ocfg), w.ctypes.data_as(C.c_void_p), st.ctypes.data_as(C.c_void_p),
+                                                 t["rows"], t["cols"], t["off_a"], t["off_b"], t["seed_base"],
+                                                 fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed), C.c_float(lr * t["lr_scale"]))
+            else:
+                orc.lib().orc_update_vector_adam(C.byref(ocfg), w.ctypes.data_as(C.c_void_p), st.ctypes.data_as(C.c_void_p),
+                                                 n, t["off_a"], t["off_b"], t["seed_base"],
+                                                 fit.ctypes.data_as(C.c_void_p), pairs, C.c_uint32(seed), C.c_float(lr * t["lr_scale"]))
+            assert np.array_equal(got_m[sl], w), (step, name, np.count_nonzero(got_m[sl] != w))
+            for f in ("m", "v", "acc"):
+                assert np.array_equal(got_s[f][sl].view(np.int32), st[f].view(np.int32)), (step, name, f)
+        seed = pkg.next_seed(seed, step + 1)
+    assert changed > 0, "no weight changed: the trajectory would not test the update"
+    ctx.close()
