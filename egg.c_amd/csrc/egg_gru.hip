@@ -505,8 +505,16 @@ __device__ __forceinline__ void gs_stage_ln(const GruStage &p, int tile, int t, 
         const GruStep st = *p.step;
         erow = p.model + p.off_emb + (size_t)st.data[gs_stream_pos(p, st, member) + t] * H;
     }
-    v4i x[NP];
+    v4i x[NP], wv[NP];
     int sum = 0;
+    const int8_t *w = p.model + w_off;
+#pragma unroll
+    for (int i = 0; i < NP; i++) {                 // the gains are asked for here so that they arrive with the rows
+        const int nt = wave + 4 * i;
+        if (nt < NTH)
+#pragma unroll
+            for (int q = 0; q < 4; q++) wv[i][q] = *reinterpret_cast<const int *>(w + 32 * nt + 8 * q + 4 * g);
+    }
 #pragma unroll
     for (int i = 0; i < NP; i++) {
         const int nt = wave + 4 * i;
@@ -528,7 +536,6 @@ __device__ __forceinline__ void gs_stage_ln(const GruStage &p, int tile, int t, 
     if (sum == 0) sum = 1;
     int mean = sum / H; if (mean == 0) mean = 1;
     const float rcp = 1.0f / (float)mean;
-    const int8_t *w = p.model + w_off;
 #pragma unroll
     for (int i = 0; i < NP; i++) {
         const int nt = wave + 4 * i;
@@ -536,7 +543,7 @@ __device__ __forceinline__ void gs_stage_ln(const GruStage &p, int tile, int t, 
             v4i o4;
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const int w4 = *reinterpret_cast<const int *>(w + 32 * nt + 8 * q + 4 * g);
+                const int w4 = wv[i][q];
                 int o[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) o[e] = clip127(div_trunc(sx8(x[i][q], e) * sx8(w4, e), rcp));
@@ -555,6 +562,13 @@ __device__ __forceinline__ void gs_stage_gates1(const GruStage &p, int l, int nt
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 5, j = lane & 31;
     const size_t tile0 = gs_at(H, tile, 0, 0, 0), piece = gs_at(H, tile, nt, g, j);
     const int8_t *hf = gs_tmp(p, GS_HF, l);
+    const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
+    v4i h, bf;                                     // what wave 0 needs behind the products, asked for in front of them
+    if (wave == 0) {
+        h = *reinterpret_cast<const v4i *>(hf + piece);
+#pragma unroll
+        for (int q = 0; q < 4; q++) bf[q] = *reinterpret_cast<const int *>(gb + 32 * nt + 8 * q + 4 * g);
+    }
     v4i r;
     if (wave == 1) r = gs_matmul<H / 32>(p, 6 * l + 1, nt, hf + tile0, tile, lane);
     else if (wave != 3) r = gs_matmul<H / 32>(p, 6 * l + (wave == 0 ? 0 : 2), nt, gs_xn(p, l) + tile0, tile, lane);
@@ -562,12 +576,11 @@ __device__ __forceinline__ void gs_stage_gates1(const GruStage &p, int l, int nt
     else if (wave == 2) *reinterpret_cast<v4i *>(gs_tmp(p, GS_M2, l) + piece) = r;
     __syncthreads();
     if (wave != 0) return;
-    const v4i b1 = ex[lane], b2 = ex[64 + lane], h = *reinterpret_cast<const v4i *>(hf + piece);
-    const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
+    const v4i b1 = ex[lane], b2 = ex[64 + lane];
     v4i ft, gated;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int bf4 = *reinterpret_cast<const int *>(gb + 32 * nt + 8 * q + 4 * g);
+        const int bf4 = bf[q];
         int f[4], gp[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
@@ -592,13 +605,16 @@ __device__ __forceinline__ void gs_stage_gates2(const GruStage &p, int l, int t,
     const v4i b1 = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_M2, l) + piece), ft = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_FT, l) + piece);
     const v4i h = *reinterpret_cast<const v4i *>(hf);
     v4i x = *reinterpret_cast<const v4i *>(gs_x(p, l, t) + piece);
+    const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
+    v4i bh;
+#pragma unroll
+    for (int q = 0; q < 4; q++) bh[q] = *reinterpret_cast<const int *>(gb + H + 32 * nt + 8 * q + 4 * g);
     const v4i b2 = gs_matmul<H / 32>(p, 6 * l + 3, nt, gs_tmp(p, GS_GATE, l) + gs_at(H, tile, 0, 0, 0), tile, lane);
     int *h32 = reinterpret_cast<int *>(p.states + ((size_t)member * p.L + l) * H + 32 * nt);
-    const int8_t *gb = p.model + p.off_gru_b + (size_t)l * 2 * H;
     v4i hnew;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int bh4 = *reinterpret_cast<const int *>(gb + H + 32 * nt + 8 * q + 4 * g);
+        const int bh4 = bh[q];
         int hn[4], xo[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
