@@ -594,12 +594,13 @@ __device__ __forceinline__ void gs_stage_gates1(const GruStage &p, int l, int nt
 }
 
 // stage 2, candidate and state update (egg.c:260-271): ht = cadd(cadd(W2 x, W3 gated), b_h);
-// h += ((ft + 127)(ht - h)) >> 8; x = cadd(h, x).  One wave per (strip, member tile); the new state goes to both copies.
+// h += ((ft + 127)(ht - h)) >> 8; x = cadd(h, x).  One wave per (strip, member tile).  The new state goes to the copy in
+// product order only; the natural-order copy is brought up to date once, behind the last tick (k_gs_end).
 // (Measured: as one workgroup per member tile with a wave per strip, which holds whole rows and can apply the following
 // norm itself, it saves a stage but draws all of a matrix through four CUs: 8.2 instead of 4.6 us.)
 template <int H>
 __device__ __forceinline__ void gs_stage_gates2(const GruStage &p, int l, int t, int nt, int tile, int lane) {
-    const int g = lane >> 5, j = lane & 31, member = tile * 32 + j;
+    const int g = lane >> 5, j = lane & 31;
     const size_t piece = gs_at(H, tile, nt, g, j);
     int8_t *hf = gs_tmp(p, GS_HF, l) + piece;
     const v4i b1 = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_M2, l) + piece), ft = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_FT, l) + piece);
@@ -610,7 +611,6 @@ __device__ __forceinline__ void gs_stage_gates2(const GruStage &p, int l, int t,
 #pragma unroll
     for (int q = 0; q < 4; q++) bh[q] = *reinterpret_cast<const int *>(gb + H + 32 * nt + 8 * q + 4 * g);
     const v4i b2 = gs_matmul<H / 32>(p, 6 * l + 3, nt, gs_tmp(p, GS_GATE, l) + gs_at(H, tile, 0, 0, 0), tile, lane);
-    int *h32 = reinterpret_cast<int *>(p.states + ((size_t)member * p.L + l) * H + 32 * nt);
     v4i hnew;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
@@ -625,7 +625,6 @@ __device__ __forceinline__ void gs_stage_gates2(const GruStage &p, int l, int t,
             xo[e] = cadd(hn[e], sx8(x[q], e));
         }
         hnew[q] = pack4(hn[0], hn[1], hn[2], hn[3]); x[q] = pack4(xo[0], xo[1], xo[2], xo[3]);
-        h32[2 * q + g] = hnew[q];
     }
     *reinterpret_cast<v4i *>(hf) = hnew;
     *reinterpret_cast<v4i *>(gs_x(p, l + 1, t) + piece) = x;
@@ -787,6 +786,17 @@ __global__ void k_gs_begin(GruStage p, const uint8_t *data, long long data_len, 
 #pragma unroll
     for (int q = 0; q < 4; q++) h[q] = h32[2 * q + g];
     *reinterpret_cast<v4i *>(gs_tmp(p, GS_HF, l) + gs_at(H, member >> 5, nt, g, member & 31)) = h;
+}
+// behind the last tick: the natural-order state from its copy in product order
+__global__ void k_gs_end(GruStage p) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const int H = p.H, per_member = p.L * (H / 16);
+    if (i >= p.population * per_member) return;
+    const int member = i / per_member, r = i % per_member, l = r / (H / 16), piece = r % (H / 16), nt = piece >> 1, g = piece & 1;
+    const v4i h = *reinterpret_cast<const v4i *>(gs_tmp(p, GS_HF, l) + gs_at(H, member >> 5, nt, g, member & 31));
+    int *h32 = reinterpret_cast<int *>(p.states + ((size_t)member * p.L + l) * H + 32 * nt);
+#pragma unroll
+    for (int q = 0; q < 4; q++) h32[2 * q + g] = h[q];
 }
 
 // A panel *= fitness of the pair (A_T[r][p] = A[r] * f, egg.c:362-366)
@@ -1068,6 +1078,8 @@ static int gru_forward_staged(egg_gru_ctx *ctx, const uint8_t *d_data, int64_t d
     int t = 0;
     for (; t + K <= total; t += K) GTRY(hipGraphLaunch(ctx->tok_exec[0], ctx->stream));
     for (; t < total; t += 2) GTRY(hipGraphLaunch(ctx->tok_exec[1], ctx->stream));
+    hipLaunchKernelGGL(k_gs_end, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, ctx->stream, p);
+    GTRY(hipGetLastError());
     return EGG_OK;
 }
 // 1 (default): the stages spread over the whole GPU, a launch per pipeline tick; 0: one persistent workgroup per 32 members
