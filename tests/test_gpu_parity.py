@@ -209,9 +209,10 @@ STAGES = ["x_init"] + [f"{n}.{l}" for l in range(2) for n in ("q", "k", "v", "ao
                                 dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=4, vocab=512),
                                 dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=4, vocab=1024),
                                 dict(hidden=512, head_dim=64, n_layers=1, seq_len=32, population=4, vocab=768),
-                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=64, population=6, vocab=2048, sigma_shift=5, noise_mask=31)],
+                                dict(hidden=128, head_dim=32, n_layers=1, seq_len=64, population=6, vocab=2048, sigma_shift=5, noise_mask=31),
+                                dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=2, vocab=65536)],
                          ids=["h64", "h128", "h256", "h256_t32", "h64_t256", "h256_t256", "h512_t32", "h512_t128", "h512_t512", "wide_noise", "other_shifts", "h64_t512", "h128_t512", "rope_2_30", "gaussian", "same_data",
-                              "vocab_512", "h256_vocab_1024", "h512_vocab_768", "vocab_2048_wide_noise"])
+                              "vocab_512", "h256_vocab_1024", "h512_vocab_768", "vocab_2048_wide_noise", "vocab_65536"])
 def test_forward_stages_and_loss(pkg, orc, dev, kw):
     """Every stage tap of every member against the oracle's trace, then the per-member losses."""
     ocfg = orc.config(**kw)
