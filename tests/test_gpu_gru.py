@@ -22,7 +22,8 @@ def _t(dev, arr):
     (dict(hidden=64, n_layers=2, seq_len=70, population=64, update_threshold=12), 2),     # more ticks than one graph holds
     (dict(hidden=128, n_layers=1, seq_len=100, population=32, update_threshold=6), 2),    # two graph launches in the pipeline's steady state
     (dict(hidden=64, n_layers=1, seq_len=1, population=32, update_threshold=3), 2),
-], ids=["h64", "h128", "h512", "h256_p96", "sigma_2", "h128_l4_t11", "h64_t70", "h128_t100", "t1"])
+    (dict(hidden=256, n_layers=2, seq_len=16, population=1024, update_threshold=200), 1),  # 32 member tiles
+], ids=["h64", "h128", "h512", "h256_p96", "sigma_2", "h128_l4_t11", "h64_t70", "h128_t100", "t1", "h256_p1024"])
 @pytest.mark.parametrize("staged", [True, False, None], ids=["launch_per_tick", "persistent_workgroups", "alternating"])
 def test_gru_steps(pkg, orc, dev, kw, steps, staged):
     import ctypes as C
