@@ -46,6 +46,8 @@
  *       product is outside the identity (both of its sides shift alike): the sites of mgpu.cu:737, :756, :815, :830,
  *       :976 are held as a fixture parsed from the source (tests/golden/reference_shift_sites.json) and each
  *       configuration field is shown to act at that site and no earlier (test_each_shift_acts_at_the_reference_site).
+ *   vocabularies above 256 (uint32 tokens, d-eggs/include/config.h:22-28) : the same functions with V as a parameter;
+ *       the loss's closed forms at V = 512 and 8192, and the two restatements of the forward agreeing at V = 768.
  *   Still "parity unpinned" (the reference holds nothing to pin them to): Muon at the cuBLAS boundary (summation
  *       order), the adaptive overlay and the d-eggs sampler beyond their closed forms, ternary-packed weights
  *       (no reference counterpart).
