@@ -66,7 +66,7 @@ struct egg_ctx {
     std::vector<Span> spans; size_t spans_used = 0;
     double t_ms[EGG_KCLASS_COUNT] = {0}; long t_n[EGG_KCLASS_COUNT] = {0};
     // generation (egg_generate): token buffer [T + 1], logits of one member [T][vocab], a zero start index / seed
-    uint8_t *d_gen_tok = nullptr; int32_t *d_gen_logits = nullptr; Scalars *d_gen_scal = nullptr;
+    uint8_t *d_gen_tok = nullptr; int32_t *d_gen_logits = nullptr, *d_gen_ws = nullptr; Scalars *d_gen_scal = nullptr;
     int8_t *d_gen_kv = nullptr; bool gen_kv_cache = true;      // per-layer K / V rows of the generated sequence (egg_ctx_generate_kv_cache)
     int mask_override = -1; int32_t *logits_override = nullptr;
     bool first_dedup = true;        // first block once per distinct byte value of a member's window (egg_ctx_first_block_dedup)
@@ -258,7 +258,7 @@ static void free_all(egg_ctx *ctx) {
     void *ptrs[] = {ctx->muon.x, ctx->muon.swap, ctx->muon.bterm, ctx->muon.partials, ctx->muon.norm,
                     ctx->d_wfrag, ctx->d_plin_frag, ctx->d_model, ctx->d_state, ctx->d_exp, ctx->d_act, ctx->d_rope, ctx->d_x, ctx->d_q, ctx->d_k, ctx->d_v,
                     ctx->d_ao, ctx->d_loss_acc, ctx->d_counter, ctx->d_loss, ctx->d_fit, ctx->d_scal, ctx->d_panel_a,
-                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_scal, ctx->d_gen_kv, ctx->d_vec_desc,
+                    ctx->d_panel_b, ctx->d_tap, ctx->d_tap_logits, ctx->d_gen_tok, ctx->d_gen_logits, ctx->d_gen_ws, ctx->d_gen_scal, ctx->d_gen_kv, ctx->d_vec_desc,
                     ctx->d_overlay, ctx->d_overlay_q, ctx->d_flags, ctx->d_ov_segs};
     for (void *p : ptrs) if (p) (void)hipFree(p);
     for (auto &sp : ctx->spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
@@ -1036,17 +1036,18 @@ static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_
     const egg_config &c = ctx->cfg; const int T = c.seq_len, total = seed_len + gen_len;
     if (seed_len < 1 || gen_len < 0 || total > T) return fail(ctx, EGG_E_INVALID, "egg_generate: need 1 <= seed_len and seed_len + gen_len <= seq_len");
     if (ctx->captured) return fail(ctx, EGG_E_STATE, "egg_generate cannot run on a context whose step is captured");
-    if (c.vocab != 256) return fail(ctx, EGG_E_INVALID, "egg_generate: byte vocabulary only (the buffer holds bytes)");
+    const int tb = c.vocab > 256 ? 4 : 1;          // bytes per token of the buffer
     hipStream_t s = ctx->stream;
     if (!ctx->d_gen_tok) {
-        HIP_TRY(hipMalloc(&ctx->d_gen_tok, (size_t)T + 16));
+        HIP_TRY(hipMalloc(&ctx->d_gen_tok, ((size_t)T + 16) * tb));
+        HIP_TRY(hipMalloc(&ctx->d_gen_ws, (size_t)2 * c.vocab * 4));
         HIP_TRY(hipMalloc(&ctx->d_gen_logits, (size_t)T * c.vocab * 4));
         HIP_TRY(hipMalloc(&ctx->d_gen_scal, sizeof(Scalars)));
         HIP_TRY(hipMemset(ctx->d_gen_scal, 0, sizeof(Scalars)));
         HIP_TRY(hipMalloc(&ctx->d_gen_kv, (size_t)c.n_layers * 2 * T * c.hidden));
     }
-    HIP_TRY(egg_launch_zero_u64(reinterpret_cast<unsigned long long *>(ctx->d_gen_tok), (T + 16) / 8, s));   // a fill kernel, not a memset node: a caller may be capturing this stream
-    HIP_TRY(hipMemcpyAsync(ctx->d_gen_tok, d_buffer, (size_t)seed_len, hipMemcpyDeviceToDevice, s));
+    HIP_TRY(egg_launch_zero_u64(reinterpret_cast<unsigned long long *>(ctx->d_gen_tok), (T + 16) * tb / 8, s));   // a fill kernel, not a memset node: a caller may be capturing this stream
+    HIP_TRY(hipMemcpyAsync(ctx->d_gen_tok, d_buffer, (size_t)seed_len * tb, hipMemcpyDeviceToDevice, s));
     int bt = (c.hidden + 31) & ~31; if (bt > 1024) bt = 1024;          // BLOCK_THREADS (mgpu.cu:74-75)
     const bool taps = ctx->taps; ctx->taps = false;
     ctx->mask_override = 0; ctx->logits_override = ctx->d_gen_logits;
@@ -1059,15 +1060,16 @@ static int generate_impl(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_
                            ctx->gen_kv_cache ? &range : nullptr);
         if (rc == EGG_OK) {
             const int32_t *row = ctx->d_gen_logits + (size_t)t * c.vocab;
+            uint8_t *next = ctx->d_gen_tok + (size_t)(t + 1) * tb;
             hipError_t e = de ? egg_launch_sample_deggs(row, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_tok, de->temp, de->min_p_limit, de->penalty_int,
-                                                        ctx->d_gen_tok + t + 1, s)
-                              : egg_launch_sample(row, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_tok + t + 1, s);
+                                                        ctx->d_gen_ws, next, tb, s)
+                              : egg_launch_sample(row, ctx->d_exp, c.vocab, bt, seed, t, ctx->d_gen_ws, next, tb, s);
             if (e != hipSuccess) rc = fail(ctx, EGG_E_HIP, "egg_launch_sample", e);
         }
     }
     ctx->mask_override = -1; ctx->logits_override = nullptr; ctx->taps = taps;
     if (rc) return rc;
-    HIP_TRY(hipMemcpyAsync(d_buffer, ctx->d_gen_tok, (size_t)total, hipMemcpyDeviceToDevice, s));
+    HIP_TRY(hipMemcpyAsync(d_buffer, ctx->d_gen_tok, (size_t)total * tb, hipMemcpyDeviceToDevice, s));
     return EGG_OK;
 }
 extern "C" int egg_ctx_generate_kv_cache(egg_ctx *ctx, int enable) {
@@ -1102,7 +1104,6 @@ extern "C" int egg_generate_deggs(egg_ctx *ctx, uint8_t *d_buffer, int seed_len,
     // threads fill: beyond either limit it reads memory nobody wrote
     if (seed_len + gen_len > 256 || seed_len > bt)
         return fail(ctx, EGG_E_INVALID, "egg_generate_deggs: need seed_len + gen_len <= 256 and seed_len <= the reference's block size (hidden rounded up to 32)");
-    if (ctx->cfg.vocab > 256) return fail(ctx, EGG_E_INVALID, "egg_generate_deggs: byte vocabulary only");
     DeggsSampling de; de.temp = temp;
     int rc = egg_deggs_sampling_constants(&ctx->cfg, min_p, penalty, &de.penalty_int, &de.min_p_limit);
     if (rc) return fail(ctx, rc, "egg_generate_deggs: configuration");

@@ -36,10 +36,11 @@ hipError_t egg_launch_noise_fill(uint32_t seed, uint32_t first, int n, int mask,
 hipError_t egg_launch_zero_u64(unsigned long long *p, int64_t n, hipStream_t s);
 hipError_t egg_launch_loss_finalize(const unsigned long long *acc, int32_t *loss, int first, int count, hipStream_t s);
 hipError_t egg_launch_fitness(const int32_t *loss, int32_t *fit, int pairs, hipStream_t s);
+// ws: vocab ints (plain sampler) or 2 * vocab ints (d-eggs sampler) of device scratch; token_bytes: 1 or 4
 hipError_t egg_launch_sample(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
-                             uint8_t *out, hipStream_t s);
+                             int *ws, void *out, int token_bytes, hipStream_t s);
 hipError_t egg_launch_sample_deggs(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
-                                   const uint8_t *tokens, float temp, int min_p_limit, int penalty_int, uint8_t *out, hipStream_t s);
+                                   const void *tokens, float temp, int min_p_limit, int penalty_int, int *ws, void *out, int token_bytes, hipStream_t s);
 
 struct UpdParams {
     int8_t *W; float *state;           // tensor weights and optimizer state ({m,v,acc} per element)

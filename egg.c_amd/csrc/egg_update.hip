@@ -326,11 +326,38 @@ hipError_t egg_launch_update_vector(const UpdParams &p, hipStream_t s) {
 // sum of EXP_LUT[clamp(max - logit)], threshold hash_rng(seed + t*555, 0) % sum, then the first vocabulary entry
 // whose running sum exceeds the threshold.  The reference accumulates in thread order with thread `tid` owning
 // v = tid, tid + bt, ... (bt = its block size = hidden rounded up to 32, at most 1024), so for bt < vocab the scan
-// order is thread-major, not natural; `bt` reproduces that.  One workgroup; vocab <= 1024.
+// order is thread-major, not natural; `bt` reproduces that: every reference thread's sum is formed (in parallel), the
+// thread in whose range the threshold falls is found from their prefix sums, and its entries are walked.
+// One workgroup; `ws` holds the vocab weights.  TOK: the token type of the buffer (bytes, or uint32 above vocab 256).
+__device__ __forceinline__ void sample_select(const int *ex, int vocab, int bt, uint32_t seed, int t, long long *tsum, int *selected) {
+    for (int tid = threadIdx.x; tid < bt; tid += 256) {
+        long long sum = 0;
+        for (int v = tid; v < vocab; v += bt) sum += ex[v];
+        tsum[tid] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        long long total = 0;
+        for (int tid = 0; tid < bt; tid++) total += tsum[tid];
+        const uint32_t r = hash_rng(seed + (uint32_t)t * 555u, 0);
+        const long long thresh = total > 0 ? (long long)r % total : 0;
+        int sel = 0; long long running = 0; bool done = false;
+        for (int tid = 0; tid < bt && !done; tid++) {
+            if (running + tsum[tid] <= thresh) { running += tsum[tid]; continue; }
+            for (int v = tid; v < vocab; v += bt) {
+                running += ex[v];
+                if (running > thresh) { sel = v; done = true; break; }
+            }
+        }
+        *selected = sel;
+    }
+}
+template <typename TOK>
 __global__ void __launch_bounds__(256) k_sample(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt,
-                                                uint32_t seed, int t, uint8_t *out) {
-    __shared__ int ex[1024];
+                                                uint32_t seed, int t, int *ws, TOK *out) {
+    __shared__ long long tsum[1024];
     __shared__ int red[256];
+    __shared__ int sel;
     int mx = INT_MIN;
     for (int v = threadIdx.x; v < vocab; v += 256) mx = max(mx, logits[v]);
     red[threadIdx.x] = mx; __syncthreads();
@@ -339,50 +366,42 @@ __global__ void __launch_bounds__(256) k_sample(const int32_t *logits, const int
     for (int v = threadIdx.x; v < vocab; v += 256) {
         int idx = mx - logits[v];
         idx = idx < 0 ? 0 : (idx > 255 ? 255 : idx);
-        ex[v] = exp_lut[idx];
+        ws[v] = exp_lut[idx];
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        long long sum = 0;
-        for (int v = 0; v < vocab; v++) sum += ex[v];
-        const uint32_t r = hash_rng(seed + (uint32_t)t * 555u, 0);
-        const long long thresh = sum > 0 ? (long long)r % sum : 0;
-        int selected = 0; long long running = 0; bool done = false;
-        for (int tid = 0; tid < bt && !done; tid++)
-            for (int v = tid; v < vocab; v += bt) {
-                running += ex[v];
-                if (running > thresh) { selected = v; done = true; break; }
-            }
-        *out = (uint8_t)selected;
-    }
+    sample_select(ws, vocab, bt, seed, t, tsum, &sel);
+    if (threadIdx.x == 0) *out = (TOK)sel;
 }
 hipError_t egg_launch_sample(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
-                             uint8_t *out, hipStream_t s) {
-    if (vocab > 1024 || bt < 1) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(k_sample, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, out);
+                             int *ws, void *out, int token_bytes, hipStream_t s) {
+    if (bt < 1 || bt > 1024 || !ws) return hipErrorInvalidValue;
+    if (token_bytes == 4) hipLaunchKernelGGL(k_sample<uint32_t>, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, ws, (uint32_t *)out);
+    else hipLaunchKernelGGL(k_sample<uint8_t>, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, ws, (uint8_t *)out);
     return hipGetLastError();
 }
 
-// The d-eggs form of the same sampler (d-eggs/src/kernels.cu:382-478): every occurrence of v among the tokens at
-// positions 0..t lowers v's logit by penalty_int (:398-402); the differences to the (penalised) maximum are divided by
-// the temperature in float and truncated (:430); entries whose scaled difference is below min_p_limit are left out
-// (:433); the rest weigh EXP_LUT[clamp(-scaled, 0, 255)] (layers.cuh:71-75).  Threshold and scan order as above.
-// The float -> int conversion is spelt out (truncation, saturation, NaN -> 0) so that it is defined for every input.
+// The d-eggs sampler (d-eggs/src/kernels.cu:382-478): every occurrence of v among the tokens up to position t lowers
+// v's logit by penalty_int (repeated int32 subtraction: wraps), the differences to the maximum are divided by the
+// temperature in float and truncated, entries below min_p_limit are left out, the rest weigh
+// EXP_LUT[clamp(-scaled, 0, 255)]; threshold and scan order as above.  `ws` holds 2 * vocab ints.
+// float -> int32 as the GPU's conversion does it: truncation toward zero, saturation at the ends, NaN -> 0
 __device__ __forceinline__ int sat_f2i(float x) {
     if (x != x) return 0;
     if (x >= 2147483648.0f) return INT_MAX;
     if (x <= -2147483648.0f) return INT_MIN;
     return (int)x;
 }
+template <typename TOK>
 __global__ void __launch_bounds__(256) k_sample_deggs(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
-                                                      const uint8_t *tokens, float temp, int min_p_limit, int penalty_int, uint8_t *out) {
-    __shared__ int lg[1024];
-    __shared__ int ex[1024];
+                                                      const TOK *tokens, float temp, int min_p_limit, int penalty_int, int *ws, TOK *out) {
+    __shared__ long long tsum[1024];
     __shared__ int red[256];
+    __shared__ int sel;
+    int *lg = ws, *ex = ws + vocab;
     int mx = INT_MIN;
     for (int v = threadIdx.x; v < vocab; v += 256) {
         uint32_t count = 0;
-        for (int i = 0; i <= t; i++) count += tokens[i] == v;
+        for (int i = 0; i <= t; i++) count += (int)tokens[i] == v;
         const int l = (int)((uint32_t)logits[v] - count * (uint32_t)penalty_int);
         lg[v] = l;
         mx = max(mx, l);
@@ -402,24 +421,18 @@ __global__ void __launch_bounds__(256) k_sample_deggs(const int32_t *logits, con
         ex[v] = e;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        long long sum = 0;
-        for (int v = 0; v < vocab; v++) sum += ex[v];
-        const uint32_t r = hash_rng(seed + (uint32_t)t * 555u, 0);
-        const long long thresh = sum > 0 ? (long long)r % sum : 0;
-        int selected = 0; long long running = 0; bool done = false;
-        for (int tid = 0; tid < bt && !done; tid++)
-            for (int v = tid; v < vocab; v += bt) {
-                running += ex[v];
-                if (running > thresh) { selected = v; done = true; break; }
-            }
-        *out = (uint8_t)selected;
-    }
+    sample_select(ex, vocab, bt, seed, t, tsum, &sel);
+    if (threadIdx.x == 0) *out = (TOK)sel;
 }
 hipError_t egg_launch_sample_deggs(const int32_t *logits, const int32_t *exp_lut, int vocab, int bt, uint32_t seed, int t,
-                                   const uint8_t *tokens, float temp, int min_p_limit, int penalty_int, uint8_t *out, hipStream_t s) {
-    if (vocab > 256 || bt < 1 || t < 0) return hipErrorInvalidValue;       // tokens are bytes
-    hipLaunchKernelGGL(k_sample_deggs, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, tokens, temp, min_p_limit, penalty_int, out);
+                                   const void *tokens, float temp, int min_p_limit, int penalty_int, int *ws, void *out, int token_bytes, hipStream_t s) {
+    if (bt < 1 || bt > 1024 || t < 0 || !ws) return hipErrorInvalidValue;
+    if (token_bytes == 4)
+        hipLaunchKernelGGL(k_sample_deggs<uint32_t>, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, (const uint32_t *)tokens, temp,
+                           min_p_limit, penalty_int, ws, (uint32_t *)out);
+    else
+        hipLaunchKernelGGL(k_sample_deggs<uint8_t>, dim3(1), dim3(256), 0, s, logits, exp_lut, vocab, bt, seed, t, (const uint8_t *)tokens, temp,
+                           min_p_limit, penalty_int, ws, (uint8_t *)out);
     return hipGetLastError();
 }
 

@@ -238,7 +238,8 @@ uint32_t egg_next_seed(uint32_t seed, uint64_t step);
  * the reference's three-pass LUT sampling, threshold hash_rng(seed + t*555, 0) % sum.  Enqueued on the stream.
  * Like the reference (d_gen_kv, mgpu.cu:1160-1170, :1199-1202) it keeps every layer's K / V rows of the sequence: the
  * prompt is evaluated once, each new token costs one 32-token tile.  egg_ctx_generate_kv_cache(ctx, 0) makes every new
- * token re-evaluate the whole window instead (same tokens; for checks). */
+ * token re-evaluate the whole window instead (same tokens; for checks).  With a vocabulary above 256 the buffer holds
+ * uint32 tokens (d-eggs' TokenType), here and in egg_generate_deggs; the lengths count tokens. */
 int  egg_generate(egg_ctx *ctx, uint8_t *d_buffer, int seed_len, int gen_len, uint32_t seed);
 int  egg_ctx_generate_kv_cache(egg_ctx *ctx, int enable);
 /* d-eggs' generate_sequence_kernel (d-eggs/src/kernels.cu:307-490, call site d-eggs/src/worker.cu:563-571): the same

@@ -394,7 +394,7 @@ def generate_deggs(cfg, model, prompt, gen_len, seed, temp, min_p, penalty):
     assert 1 <= seed_len and seed_len + gen_len <= min(T, 256)
     exp_lut = tables(cfg)[0]
     penalty_int, limit = deggs_sampling_constants(cfg, min_p, penalty)
-    buf = np.zeros(T + 1, np.uint8)
+    buf = np.zeros(T + 1, np.uint8 if cfg.vocab <= 256 else np.uint32)      # TokenType, d-eggs/include/config.h:26-28
     buf[:seed_len] = prompt
     for t in range(seed_len - 1, seed_len + gen_len - 1):
         _, tr = forward_member(cfg, model, buf, 0, 0, 0, ns_override=0, trace=True)
@@ -410,7 +410,7 @@ def generate(cfg, model, prompt, gen_len, seed):
     seed_len = len(prompt)
     assert 1 <= seed_len and seed_len + gen_len <= T
     exp_lut = tables(cfg)[0]
-    buf = np.zeros(T + 1, np.uint8)
+    buf = np.zeros(T + 1, np.uint8 if cfg.vocab <= 256 else np.uint32)
     buf[:seed_len] = prompt
     for t in range(seed_len - 1, seed_len + gen_len - 1):
         _, tr = forward_member(cfg, model, buf, 0, 0, 0, ns_override=0, trace=True)

@@ -487,12 +487,6 @@ def test_error_paths(pkg, dev):
         pkg.Context(pkg.default_config(seq_len=48))
     with pytest.raises(pkg.EggError):
         pkg.Context(pkg.default_config(vocab=300))        # multiples of 256 only
-    big = pkg.Context(pkg.default_config(vocab=512, **SMALL))
-    import torch
-    buf = torch.zeros(SMALL["seq_len"], dtype=torch.uint8, device=dev)
-    with pytest.raises(pkg.EggError):
-        big.generate(buf.data_ptr(), 4, 4, 1)              # the generation buffer holds bytes
-    big.close()
     ctx = pkg.Context(pkg.default_config(**SMALL))
     with pytest.raises(pkg.EggError):
         ctx.step_launch(0, 1, 0.1)            # launch before capture
@@ -709,6 +703,47 @@ def test_generate_deggs(pkg, orc, dev, kw, seed_len, gen_len, sampling):
         assert len(set(ref[seed_len:].tolist())) > 15          # a strong penalty spreads the continuation
     with pytest.raises(pkg.EggError):
         ctx.generate_deggs(buf.data_ptr(), 200, 100, 1)          # beyond the reference's 256-entry token history
+    ctx.close()
+
+
+@pytest.mark.parametrize("sampling", [None, (0.6, 0.08, 0.2), (1.7, 0.3, 1.5)], ids=["plain", "deggs_defaults", "deggs_other"])
+@pytest.mark.parametrize("kw,seed_len,gen_len", [(dict(hidden=64, head_dim=32, n_layers=1, seq_len=64, population=2, vocab=768), 6, 40),
+                                                 (dict(hidden=256, head_dim=64, n_layers=2, seq_len=64, population=2, vocab=8192), 12, 30)],
+                         ids=["vocab_768", "h256_vocab_8192"])
+def test_generate_with_a_larger_vocabulary(pkg, orc, dev, kw, seed_len, gen_len, sampling):
+    """Both samplers over a vocabulary of more than 256 entries: the buffer holds uint32 tokens."""
+    import torch
+    ocfg = orc.config(**kw)
+    V = kw["vocab"]
+    model = orc.init_model(ocfg, 42)
+    rng = np.random.default_rng(3)
+    for t in orc.tensor_table(ocfg):
+        if not t["is_matrix"]:
+            sl = slice(t["offset"], t["offset"] + t["cols"])
+            model[sl] = rng.integers(-20, 21, t["cols"]).astype(np.int8) + (16 if t["name"].startswith("ln_") and "bias" not in t["name"] else 0)
+        elif t["name"] == "embedding":      # a small tied head keeps the next-token distribution broad
+            n = t["rows"] * t["cols"]
+            model[t["offset"]:t["offset"] + n] = rng.integers(-5, 6, n).astype(np.int8)
+    prompt = rng.integers(0, V, seed_len).astype(np.uint32)
+    prompt[0] = V - 1
+    if sampling is None:
+        ref = orc.generate(ocfg, model, prompt, gen_len, 1041)
+    else:
+        ref = orc.generate_deggs(ocfg, model, prompt, gen_len, 1041, *sampling)
+    assert ref.dtype == np.uint32 and int(ref[seed_len:].max()) > 255 and len(set(ref[seed_len:].tolist())) > 3
+    ctx = pkg.Context(pkg.default_config(**kw))
+    ctx.model_upload(model)
+    for cache in (True, False):
+        ctx.generate_kv_cache(cache)
+        buf = torch.zeros(seed_len + gen_len, dtype=torch.int32, device=dev)
+        buf[:seed_len] = _t(dev, prompt)
+        if sampling is None:
+            ctx.generate(buf.data_ptr(), seed_len, gen_len, 1041)
+        else:
+            ctx.generate_deggs(buf.data_ptr(), seed_len, gen_len, 1041, *sampling)
+        ctx.sync()
+        got = buf.cpu().numpy().view(np.uint32)
+        assert np.array_equal(got, ref), (cache, got.tolist(), ref.tolist())
     ctx.close()
 
 
