@@ -65,6 +65,28 @@ def test_gru_steps(pkg, orc, dev, kw, steps, staged):
     ctx.close()
 
 
+def test_gru_training_reduces_the_loss(pkg, orc, dev):
+    """full_trained_egg.c prints its loss while it trains (:576-586); 200 steps of a small model on the synthetic stream
+    bring the mean loss per token down by a tenth or more, in both ways of evaluating the forward alike."""
+    data = orc.zipf_bytes(1 << 22)
+    d_data = _t(dev, data)
+    runs = []
+    for staged in (True, False):
+        ctx = pkg.GruContext(pkg.gru_default_config(hidden=64, n_layers=1, seq_len=64, population=128, update_threshold=20))
+        ctx.forward_mode(staged)
+        ctx.model_init(42)
+        hist = []
+        for step in range(200):
+            ctx.step(d_data.data_ptr(), len(data), step * 64, 1000 + step, True)
+            if step < 3 or step >= 197:
+                hist.append(float(ctx.losses()[0].mean()) / 64)
+        runs.append(hist)
+        ctx.close()
+    assert runs[0] == runs[1]
+    first, last = np.mean(runs[0][:3]), np.mean(runs[0][3:])
+    assert last < 0.9 * first, (first, last)
+
+
 def test_gru_config_errors(pkg, dev):
     with pytest.raises(pkg.EggError):
         pkg.GruContext(pkg.gru_default_config(hidden=100))

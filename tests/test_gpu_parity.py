@@ -480,11 +480,12 @@ def test_muon_step_graph_replays_equal_eager_steps(pkg, orc, dev):
     g.close(); e.close()
 
 
-def test_training_reduces_the_loss(pkg, orc, dev):
+@pytest.mark.parametrize("muon", [0, 1], ids=["adamw", "muon"])
+def test_training_reduces_the_loss(pkg, orc, dev, muon):
     """What the reference itself checks (sweep_hyperparams.sh:146-178 trains and reads the last "Loss:"): 160 whole
     steps of the small model on the synthetic stream at the reference's starting learning rate bring the population's
     mean loss per token down by a quarter or more; the same run twice gives the same numbers."""
-    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=2048)
+    kw = dict(hidden=64, head_dim=32, n_layers=1, seq_len=32, population=2048, use_muon=muon)
     data = orc.zipf_bytes(1 << 22)
     d_data = _t(dev, data)
     runs = []
