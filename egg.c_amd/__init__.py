@@ -48,6 +48,7 @@ EXPORTS = [
     "egg_tensor_count", "egg_tensor_info_get", "egg_last_update_count",
     "egg_step", "egg_step_capture", "egg_step_launch", "egg_step_losses", "egg_generate", "egg_generate_deggs", "egg_deggs_sampling_constants",
     "egg_shape_fitness", "egg_ternary_pack_size", "egg_ternary_pack", "egg_ternary_unpack",
+    "egg_vocab_load", "egg_vocab_free", "egg_vocab_size", "egg_vocab_save", "egg_detokenize",
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
     "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
@@ -123,6 +124,13 @@ def lib():
         L.egg_ternary_pack_size.restype = C.c_size_t
         L.egg_ternary_pack_size.argtypes = [C.c_size_t]
         L.egg_ternary_pack.argtypes = [vp, C.c_size_t, vp]
+        L.egg_vocab_load.argtypes = [C.c_char_p, C.POINTER(vp)]
+        L.egg_vocab_free.argtypes = [vp]
+        L.egg_vocab_free.restype = None
+        L.egg_vocab_size.argtypes = [vp]
+        L.egg_vocab_save.argtypes = [C.c_char_p, vp, vp, C.c_uint32]
+        L.egg_detokenize.argtypes = [vp, vp, i32, vp, C.c_int64]
+        L.egg_detokenize.restype = C.c_int64
         L.egg_ternary_unpack.argtypes = [vp, C.c_size_t, vp]
         L.egg_checkpoint_save.argtypes = [vp, C.c_char_p, C.c_long]
         L.egg_checkpoint_load.argtypes = [vp, C.c_char_p, C.c_char_p]
@@ -453,6 +461,45 @@ Context.timing = _timing
 
 
 # ---- host-side companions (no GPU needed)
+class Vocabulary:
+    """d-eggs' token table for printing generated tokens ("decoding.bin", d-eggs/src/worker.cu:36-81)."""
+
+    def __init__(self, path):
+        h = C.c_void_p()
+        rc = lib().egg_vocab_load(str(path).encode(), C.byref(h))
+        if rc:
+            raise EggError(f"egg_vocab_load failed ({rc}): {path}")
+        self._h = h
+
+    @staticmethod
+    def save(path, entries):
+        """entries: a sequence of bytes objects, token id = position"""
+        entries = [bytes(e) for e in entries]
+        arr = (C.c_char_p * len(entries))(*entries)
+        lens = (C.c_uint32 * len(entries))(*[len(e) for e in entries])
+        rc = lib().egg_vocab_save(str(path).encode(), arr, lens, len(entries))
+        if rc:
+            raise EggError(f"egg_vocab_save failed ({rc}): {path}")
+
+    def __len__(self):
+        return lib().egg_vocab_size(self._h)
+
+    def detokenize(self, tokens):
+        import numpy as np
+        tokens = np.ascontiguousarray(tokens, np.uint32)
+        n = lib().egg_detokenize(self._h, _np_ptr(tokens), len(tokens), None, 0)
+        if n < 0:
+            raise EggError(f"egg_detokenize failed ({n})")
+        buf = C.create_string_buffer(max(int(n), 1))
+        lib().egg_detokenize(self._h, _np_ptr(tokens), len(tokens), buf, n)
+        return buf.raw[:n]
+
+    def close(self):
+        if self._h:
+            lib().egg_vocab_free(self._h)
+            self._h = None
+
+
 def shape_fitness(loss, chunk_mean_filter=True, mean_exponent=1.2, adaptive_threshold=True, alpha=None):
     """d-eggs worker shaping of one chunk's losses -> (fit[count/2] in {-1,0,1}, sum of losses)."""
     import numpy as np

@@ -182,3 +182,56 @@ extern "C" int egg_eggc_load_latest(const char *dir, uint64_t *step, uint64_t *s
     fclose(f);
     return rc;
 }
+
+// ---------------------------------------------------------------- token vocabulary (worker.cu:36-81)
+// "decoding.bin": uint32 count, then per token uint32 length + bytes.  The reference prints a generated token run as the
+// concatenation of its tokens' strings and "<id>" for an id beyond the table.
+struct egg_vocab { std::vector<std::string> entries; };
+extern "C" int egg_vocab_load(const char *path, egg_vocab **out) {
+    if (!path || !out) return EGG_E_INVALID;
+    *out = nullptr;
+    FILE *f = fopen(path, "rb");
+    if (!f) return EGG_E_INVALID;
+    uint32_t n = 0;
+    int rc = fread(&n, 4, 1, f) == 1 ? EGG_OK : EGG_E_INVALID;
+    egg_vocab *v = new egg_vocab();
+    for (uint32_t i = 0; rc == EGG_OK && i < n; i++) {
+        uint32_t len = 0;
+        if (fread(&len, 4, 1, f) != 1) { rc = EGG_E_INVALID; break; }
+        std::string s;
+        // a length is checked against what is left of the file before it is trusted with an allocation
+        const long here = ftell(f);
+        if (fseek(f, 0, SEEK_END) != 0) { rc = EGG_E_INVALID; break; }
+        const long end = ftell(f);
+        if (here < 0 || end < here || (unsigned long)(end - here) < len || fseek(f, here, SEEK_SET) != 0) { rc = EGG_E_INVALID; break; }
+        s.resize(len);
+        if (len && fread(&s[0], 1, len, f) != len) { rc = EGG_E_INVALID; break; }
+        v->entries.push_back(std::move(s));
+    }
+    fclose(f);
+    if (rc != EGG_OK) { delete v; return rc; }
+    *out = v;
+    return EGG_OK;
+}
+extern "C" void egg_vocab_free(egg_vocab *v) { delete v; }
+extern "C" int egg_vocab_size(const egg_vocab *v) { return v ? (int)v->entries.size() : 0; }
+extern "C" int egg_vocab_save(const char *path, const char *const *entries, const uint32_t *lengths, uint32_t count) {
+    if (!path || (count && (!entries || !lengths))) return EGG_E_INVALID;
+    FILE *f = fopen(path, "wb");
+    if (!f) return EGG_E_INVALID;
+    bool ok = fwrite(&count, 4, 1, f) == 1;
+    for (uint32_t i = 0; ok && i < count; i++)
+        ok = fwrite(&lengths[i], 4, 1, f) == 1 && (lengths[i] == 0 || fwrite(entries[i], 1, lengths[i], f) == lengths[i]);
+    return (fclose(f) == 0 && ok) ? EGG_OK : EGG_E_INVALID;
+}
+extern "C" int64_t egg_detokenize(const egg_vocab *v, const uint32_t *tokens, int count, char *out, int64_t capacity) {
+    if (!v || (count && !tokens) || count < 0 || capacity < 0 || (capacity && !out)) return EGG_E_INVALID;
+    std::string text;
+    for (int i = 0; i < count; i++) {
+        if (tokens[i] < v->entries.size()) text += v->entries[tokens[i]];
+        else text += "<" + std::to_string(tokens[i]) + ">";
+    }
+    const int64_t n = (int64_t)text.size();
+    if (capacity > 0) { const int64_t c = n < capacity ? n : capacity; memcpy(out, text.data(), (size_t)c); }
+    return n;
+}

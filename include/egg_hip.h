@@ -265,6 +265,16 @@ int  egg_shape_fitness(const int32_t *loss, int count, int chunk_mean_filter, do
 size_t egg_ternary_pack_size(size_t count);
 int  egg_ternary_pack(const int32_t *src, size_t count, uint8_t *dst);
 int  egg_ternary_unpack(const uint8_t *src, size_t count, int32_t *dst);
+/* d-eggs' token vocabulary for printing generated tokens (de/src/worker.cu:36-81): "decoding.bin" holds a uint32 count and
+ * per token a uint32 length and its bytes.  egg_detokenize concatenates the tokens' strings, "<id>" for an id beyond the
+ * table, like the reference's detokenize; it returns the length of the text and writes at most `capacity` bytes of it
+ * (no terminator), so a first call with capacity 0 sizes the buffer.  egg_vocab_save writes the same format. */
+typedef struct egg_vocab egg_vocab;
+int  egg_vocab_load(const char *path, egg_vocab **out);
+void egg_vocab_free(egg_vocab *v);
+int  egg_vocab_size(const egg_vocab *v);
+int  egg_vocab_save(const char *path, const char *const *entries, const uint32_t *lengths, uint32_t count);
+int64_t egg_detokenize(const egg_vocab *v, const uint32_t *tokens, int count, char *out, int64_t capacity);
 /* save_checkpoint / load_model (egg_disk_utils.h:46-82): <dir>/egg_step-%08ld.model.bin and .adam.bin hold the raw
  * model blob and optimizer state, "egg_transformer_last.*" symlinks point at the newest; dir NULL = "models".
  * Loading checks the file size against this context's shapes; state_path may be NULL.  Both synchronise. */

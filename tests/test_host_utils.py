@@ -143,3 +143,39 @@ def test_eggc_checkpoints_interoperate_with_reference_header(pkg, orc, tmp_path)
     d3 = str(tmp_path / "bad"); os.mkdir(d3)
     open(os.path.join(d3, "checkpoint_00000001.bin"), "wb").write(b"\0" * 64)
     assert pkg.eggc_load_latest(d3) is None
+
+
+def test_token_vocabulary_file_and_detokenize(pkg, tmp_path):
+    """d-eggs' "decoding.bin" (d-eggs/src/worker.cu:36-81): uint32 count, then per token uint32 length + bytes; a run of
+    tokens prints as the concatenation of their strings, an id beyond the table as "<id>"."""
+    import struct
+    entries = [b"the", b" ", b"", b"\xe2\x82\xac", b"egg", bytes(range(256))]
+    path = tmp_path / "decoding.bin"
+    # the file written by hand, byte for byte as the reference's reader expects it
+    with open(path, "wb") as f:
+        f.write(struct.pack("<I", len(entries)))
+        for e in entries:
+            f.write(struct.pack("<I", len(e)) + e)
+    v = pkg.Vocabulary(path)
+    assert len(v) == len(entries)
+    assert v.detokenize([0, 1, 4, 2, 3]) == b"the egg\xe2\x82\xac"
+    assert v.detokenize([4, 6, 1, 4000000000]) == b"egg<6> <4000000000>"
+    assert v.detokenize([5]) == bytes(range(256)) and v.detokenize([]) == b""
+    v.close()
+    # the library's writer produces the same bytes
+    path2 = tmp_path / "again.bin"
+    pkg.Vocabulary.save(path2, entries)
+    assert open(path2, "rb").read() == open(path, "rb").read()
+    # a file that ends early, or whose length field points past its end, is refused
+    whole = open(path, "rb").read()
+    for cut in (2, 7, len(whole) - 1):
+        bad = tmp_path / f"cut{cut}.bin"
+        open(bad, "wb").write(whole[:cut])
+        with pytest.raises(pkg.EggError):
+            pkg.Vocabulary(bad)
+    huge = tmp_path / "huge.bin"
+    open(huge, "wb").write(struct.pack("<II", 1, 0xFFFFFFF0) + b"abc")
+    with pytest.raises(pkg.EggError):
+        pkg.Vocabulary(huge)
+    with pytest.raises(pkg.EggError):
+        pkg.Vocabulary(tmp_path / "missing.bin")
