@@ -11,6 +11,10 @@
 // usage: egg_train [--data FILE] [--steps N] [--population P] [--seq T] [--hidden H] [--layers L] [--muon] [--graph]
 //                  [--gen-every N] [--save-every N] [--save-dir DIR] [--load MODEL.bin [--load-state ADAM.bin]]
 //                  [--adaptive]   (the d-eggs worker's adaptive noise overlay, d-eggs/src/worker.cu:331-333, :446-523)
+//                  [--vocab V]    (d-eggs' VOCAB_SIZE: above 256 the data file holds uint32 tokens like its input.bin,
+//                                  d-eggs/src/worker.cu:301-311; without --data a synthetic token stream is made)
+//                  [--decoding FILE]  (d-eggs' decoding.bin: generated tokens are printed as text, worker.cu:320, :577)
+//                  [--deggs-sampler]  (temperature / min-p / presence penalty at the reference's defaults, config.h:192-200)
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -49,7 +53,7 @@ int main(int argc, char **argv) {
     egg_config cfg; egg_default_config(&cfg);
     cfg.seq_len = 256; cfg.population = 40960;
     const char *data_file = nullptr; long steps = 10; bool graph = false; size_t synth_bytes = 64u << 20;
-    bool adaptive = false;
+    bool adaptive = false, deggs_sampler = false; const char *decoding_file = nullptr;
     long gen_every = 5, save_every = 0; const char *save_dir = "models", *load_model = nullptr, *load_state = nullptr;
     for (int i = 1; i < argc; i++) {
         auto next = [&](const char *name) -> const char * { if (i + 1 >= argc) { fprintf(stderr, "%s needs a value\n", name); exit(2); } return argv[++i]; };
@@ -62,6 +66,9 @@ int main(int argc, char **argv) {
         else if (!strcmp(argv[i], "--muon")) cfg.use_muon = 1;
         else if (!strcmp(argv[i], "--graph")) graph = true;
         else if (!strcmp(argv[i], "--adaptive")) adaptive = true;
+        else if (!strcmp(argv[i], "--vocab")) cfg.vocab = atoi(next("--vocab"));
+        else if (!strcmp(argv[i], "--decoding")) decoding_file = next("--decoding");
+        else if (!strcmp(argv[i], "--deggs-sampler")) deggs_sampler = true;
         else if (!strcmp(argv[i], "--gen-every")) gen_every = atol(next("--gen-every"));
         else if (!strcmp(argv[i], "--save-every")) save_every = atol(next("--save-every"));
         else if (!strcmp(argv[i], "--save-dir")) save_dir = next("--save-dir");
@@ -79,8 +86,20 @@ int main(int argc, char **argv) {
         fclose(f);
     } else {
         data = zipf_bytes(synth_bytes, 1234, 1.1);
+        if (cfg.vocab > 256) {          // uint32 tokens from pairs of Zipf bytes: frequent tokens stay frequent, every id is reachable
+            std::vector<uint8_t> tok(data.size() / 2 * 4);
+            for (size_t i = 0; i + 1 < data.size(); i += 2) {
+                const uint32_t t = (((uint32_t)data[i] << 8) | data[i + 1]) % (uint32_t)cfg.vocab;
+                memcpy(&tok[i / 2 * 4], &t, 4);
+            }
+            data.swap(tok);
+        }
     }
-    printf("data: %zu bytes (%s)\n", data.size(), data_file ? data_file : "synthetic Zipf(1.1)");
+    const size_t tb = cfg.vocab > 256 ? 4 : 1;                 // bytes per token (TokenType, d-eggs/include/model/definitions.h:9-13)
+    const size_t n_tokens = data.size() / tb;
+    printf("data: %zu tokens of %zu byte(s) (%s)\n", n_tokens, tb, data_file ? data_file : "synthetic Zipf(1.1)");
+    egg_vocab *vocab = nullptr;
+    if (decoding_file && egg_vocab_load(decoding_file, &vocab) != EGG_OK) { fprintf(stderr, "cannot read %s\n", decoding_file); return 1; }
 
     egg_ctx *ctx = nullptr;
     int rc = egg_ctx_create(&cfg, &ctx);
@@ -98,19 +117,19 @@ int main(int argc, char **argv) {
     if (gen_every > 0) {
         egg_config gcfg = cfg; gcfg.population = 2; gcfg.chunk_members = 2;
         if (egg_ctx_create(&gcfg, &gen_ctx) != EGG_OK) { fprintf(stderr, "generation context failed\n"); return 1; }
-        HK(hipMalloc(&d_gen, (size_t)cfg.seq_len));
+        HK(hipMalloc(&d_gen, (size_t)cfg.seq_len * tb));
         h_model.resize((size_t)egg_model_bytes(ctx));
     }
-    if (graph) CK(egg_step_capture(ctx, d_data, (int64_t)data.size()));
+    if (graph) CK(egg_step_capture(ctx, d_data, (int64_t)n_tokens));
 
     std::vector<int32_t> loss((size_t)cfg.population), fit((size_t)cfg.population / 2);
     uint32_t seed = 42;
-    long max_steps = (long)((data.size() - 1) / (size_t)cfg.seq_len);
+    long max_steps = (long)((n_tokens - 1) / (size_t)cfg.seq_len);
     for (long step = 0; step < steps && step < max_steps; step++) {
         struct timespec t0, t1; clock_gettime(CLOCK_MONOTONIC, &t0);
         float lr = egg_learning_rate(step);
         if (graph) CK(egg_step_launch(ctx, step * cfg.seq_len, seed, lr));
-        else CK(egg_step(ctx, d_data, (int64_t)data.size(), step * cfg.seq_len, seed, lr));
+        else CK(egg_step(ctx, d_data, (int64_t)n_tokens, step * cfg.seq_len, seed, lr));
         uint64_t updates = 0;
         CK(egg_last_update_count(ctx, &updates));          // synchronises, like the reference's cudaMemcpy of d_total_updates
         clock_gettime(CLOCK_MONOTONIC, &t1);
@@ -123,22 +142,37 @@ int main(int argc, char **argv) {
         if (gen_every > 0 && step % gen_every == 0) {
             CK(egg_model_download(ctx, h_model.data(), h_model.size()));
             if (egg_model_upload(gen_ctx, h_model.data(), h_model.size()) != EGG_OK) return 1;
-            size_t pos = (size_t)(step * cfg.seq_len) % (data.size() - (size_t)cfg.seq_len);
-            HK(hipMemcpy(d_gen, d_data + pos, (size_t)gen_seed_len, hipMemcpyDeviceToDevice));
-            if (egg_generate(gen_ctx, d_gen, gen_seed_len, gen_total - gen_seed_len, seed + 999) != EGG_OK) { fprintf(stderr, "egg_generate: %s\n", egg_last_error(gen_ctx)); return 1; }
+            size_t pos = (size_t)(step * cfg.seq_len) % (n_tokens - (size_t)cfg.seq_len);
+            HK(hipMemcpy(d_gen, d_data + pos * tb, (size_t)gen_seed_len * tb, hipMemcpyDeviceToDevice));
+            const int grc = deggs_sampler ? egg_generate_deggs(gen_ctx, d_gen, gen_seed_len, gen_total - gen_seed_len, seed + 999, 0.6f, 0.08f, 0.2f)
+                                          : egg_generate(gen_ctx, d_gen, gen_seed_len, gen_total - gen_seed_len, seed + 999);
+            if (grc != EGG_OK) { fprintf(stderr, "egg_generate: %s\n", egg_last_error(gen_ctx)); return 1; }
             if (egg_sync(gen_ctx) != EGG_OK) return 1;
-            std::vector<uint8_t> h((size_t)gen_total);
+            std::vector<uint8_t> h((size_t)gen_total * tb);
             HK(hipMemcpy(h.data(), d_gen, h.size(), hipMemcpyDeviceToHost));
             printf("\n--- GENERATION ---\n\033[32m");
-            for (int i = 0; i < gen_total; i++) {
-                if (i == gen_seed_len) printf("\033[36m");
-                char c = (char)h[(size_t)i]; putchar((c >= 32 && c <= 126) ? c : '.');
+            for (int part = 0; part < 2; part++) {           // the prompt, then the continuation
+                const int first = part ? gen_seed_len : 0, count = part ? gen_total - gen_seed_len : gen_seed_len;
+                if (part) printf("\033[36m");
+                if (tb == 1) {
+                    for (int i = first; i < first + count; i++) { char c = (char)h[(size_t)i]; putchar((c >= 32 && c <= 126) ? c : '.'); }
+                } else {
+                    std::vector<uint32_t> toks((size_t)count);
+                    memcpy(toks.data(), h.data() + (size_t)first * 4, (size_t)count * 4);
+                    if (vocab) {
+                        std::vector<char> text((size_t)egg_detokenize(vocab, toks.data(), count, nullptr, 0) + 1);
+                        egg_detokenize(vocab, toks.data(), count, text.data(), (int64_t)text.size());
+                        fwrite(text.data(), 1, text.size() - 1, stdout);
+                    } else
+                        for (uint32_t t : toks) printf("<%u>", t);
+                }
             }
             printf("\033[0m\n\n");
         }
         if (save_every > 0 && step % save_every == 0) CK(egg_checkpoint_save(ctx, save_dir, step));
         seed = egg_next_seed(seed, (uint64_t)(step + 1));
     }
+    if (vocab) egg_vocab_free(vocab);
     if (d_gen) (void)hipFree(d_gen);
     if (gen_ctx) egg_ctx_destroy(gen_ctx);
     (void)hipFree(d_data);

@@ -43,6 +43,29 @@ def test_host_loop_eager_graph_adaptive_and_checkpoints(dev, tmp_path):
         assert resumed[0][1] != eager[0][1], "the resumed run started from the initialisation, not from the checkpoint"
 
 
+def test_host_loop_with_deggs_vocabulary_and_decoding_file(dev, tmp_path):
+    """d-eggs' loop shape: a vocabulary above 256 (uint32 tokens, like its input.bin), its sampler, and generated tokens
+    printed through a decoding.bin table."""
+    import struct
+    V = 512
+    with open(tmp_path / "decoding.bin", "wb") as f:
+        f.write(struct.pack("<I", V))
+        for i in range(V):
+            e = b"[%d]" % i
+            f.write(struct.pack("<I", len(e)) + e)
+    base = ["--population", "64", "--seq", "32", "--hidden", "64", "--layers", "1", "--steps", "3", "--vocab", str(V)]
+    plain, out = _run(base + ["--gen-every", "1"], tmp_path)
+    assert len(plain) == 3 and re.search(r"<\d+><\d+>", out), out[-600:]          # no table: ids in angle brackets
+    named, out2 = _run(base + ["--gen-every", "1", "--decoding", "decoding.bin", "--deggs-sampler"], tmp_path)
+    assert [(l, u) for _, l, u in named] == [(l, u) for _, l, u in plain]       # the sampler does not touch training
+    gens = re.findall(r"--- GENERATION ---\n(.*?)\n\n", out2, re.S)
+    assert len(gens) == 3 and all(re.search(r"\[\d+\]\[\d+\]", g) and "<" not in g for g in gens), out2[-600:]
+    ids = [int(x) for x in re.findall(r"\[(\d+)\]", gens[0])]
+    assert len(ids) == 32 and max(ids) < V        # 16 prompt tokens and 16 sampled ones
+    graph, _ = _run(base + ["--gen-every", "0", "--graph"], tmp_path)
+    assert [(l, u) for _, l, u in graph] == [(l, u) for _, l, u in plain]
+
+
 def test_mfma_probe_reports_plausible_rates(dev):
     """The measurement aid bench.py runs as a child process: one JSON line, rates between a fifth of the published int8
     peak and a little above it, zero operands not slower than random ones."""
