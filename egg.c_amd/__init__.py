@@ -50,7 +50,7 @@ EXPORTS = [
     "egg_shape_fitness", "egg_ternary_pack_size", "egg_ternary_pack", "egg_ternary_unpack",
     "egg_vocab_load", "egg_vocab_free", "egg_vocab_size", "egg_vocab_save", "egg_detokenize",
     "egg_checkpoint_save", "egg_checkpoint_load", "egg_eggc_save", "egg_eggc_load_latest",
-    "egg_learning_rate", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
+    "egg_learning_rate", "egg_learning_rate_deggs", "egg_model_info_save", "egg_next_seed", "egg_ctx_enable_taps", "egg_ctx_first_block_dedup", "egg_tap_download",
     "egg_ctx_enable_timing", "egg_timing_reset", "egg_timing_get",
     "egg_opt_state_bytes", "egg_tensor_state_offset", "egg_newton_schulz", "egg_describe_layout", "egg_muon_plan", "egg_ctx_generate_kv_cache", "egg_newton_schulz_static",
     "egg_gru_default_config", "egg_gru_create", "egg_gru_destroy", "egg_gru_last_error", "egg_gru_model_bytes",
@@ -76,6 +76,15 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise EggError("libegg_hip.so is not built (run __graft_entry__.build()); there is no CPU fallback")
+        # PyTorch brings a HIP runtime of its own.  When this library's runtime is loaded into the process first and torch
+        # initialises its devices afterwards, this library's first HIP call reports "no ROCm-capable device"; the other
+        # order works.  Callers hand over torch tensors' device pointers anyway, so torch goes first where it is installed.
+        import sys
+        if "torch" not in sys.modules:
+            try:
+                import torch  # noqa: F401
+            except ImportError:
+                pass
         L = C.CDLL(LIB_PATH)
         vp, i32, i64, u32 = C.c_void_p, C.c_int, C.c_int64, C.c_uint32
         L.egg_default_config.argtypes = [vp]
@@ -138,6 +147,9 @@ def lib():
         L.egg_eggc_load_latest.argtypes = [C.c_char_p, vp, vp, vp, C.c_uint64, vp]
         L.egg_learning_rate.restype = C.c_float
         L.egg_learning_rate.argtypes = [C.c_long]
+        L.egg_learning_rate_deggs.restype = C.c_float
+        L.egg_learning_rate_deggs.argtypes = [C.c_long]
+        L.egg_model_info_save.argtypes = [vp, C.c_char_p]
         L.egg_next_seed.restype = u32
         L.egg_next_seed.argtypes = [u32, C.c_uint64]
         L.egg_ctx_enable_taps.argtypes = [vp, i32]
@@ -407,6 +419,10 @@ class Context:
     def checkpoint_save(self, directory, step):
         self._ck(lib().egg_checkpoint_save(self._h, directory.encode() if directory else None, step), "egg_checkpoint_save")
 
+    def model_info_save(self, directory=None):
+        """<directory>/model.info, the reference's save_model_info text (egg_disk_utils.h:15-44)"""
+        self._ck(lib().egg_model_info_save(self._h, directory.encode() if directory else None), "egg_model_info_save")
+
     def checkpoint_load(self, model_path, state_path=None):
         self._ck(lib().egg_checkpoint_load(self._h, model_path.encode(), state_path.encode() if state_path else None), "egg_checkpoint_load")
 
@@ -583,6 +599,11 @@ def zipf_bytes(n, seed=1234, s=1.1):
 
 def learning_rate(step):
     return float(lib().egg_learning_rate(step))
+
+
+def learning_rate_deggs(step):
+    """d-eggs' schedule (d-eggs/include/utils/training.h:5-9)"""
+    return float(lib().egg_learning_rate_deggs(step))
 
 
 def next_seed(seed, step):

@@ -8,6 +8,7 @@
 #include <stdio.h>
 #include <string.h>
 #include <algorithm>
+#include <sys/stat.h>
 #include <string>
 #include <vector>
 
@@ -1013,6 +1014,37 @@ extern "C" float egg_learning_rate(long step) {
     if (step < 600) return 0.15f;
     if (step < 1000) return 0.075f;
     return 0.05f;
+}
+// d-eggs' schedule (d-eggs/include/utils/training.h:5-9)
+extern "C" float egg_learning_rate_deggs(long step) {
+    if (step < 100) return 0.5f;
+    if (step < 200) return 0.25f;
+    return 0.125f;
+}
+// save_model_info (egg_disk_utils.h:15-44, d-eggs/include/utils/io.h:24-53): "<dir>/model.info", the configuration and
+// sizes as text.  The reference's sizes are sizeof(TransformerModel) / sizeof(AdamModel): the blob and state sizes here.
+extern "C" int egg_model_info_save(egg_ctx *ctx, const char *dir) {
+    if (!ctx) return EGG_E_INVALID;
+    const std::string d = (dir && *dir) ? dir : "models";
+    (void)mkdir(d.c_str(), 0700);
+    FILE *f = fopen((d + "/model.info").c_str(), "w");
+    if (!f) return fail(ctx, EGG_E_INVALID, "cannot write model.info");
+    const egg_config &c = ctx->cfg;
+    const long params = (long)ctx->L.total, state = (long)egg_opt_state_bytes(ctx);
+    fprintf(f, "Model Configuration:\n");
+    fprintf(f, "HIDDEN_DIM: %d\n", c.hidden);
+    fprintf(f, "HEAD_DIM: %d\n", c.head_dim);
+    fprintf(f, "N_LAYERS: %d\n", c.n_layers);
+    fprintf(f, "SEQ_LEN: %d\n", c.seq_len);
+    fprintf(f, "VOCAB_SIZE: %d\n", c.vocab);
+    fprintf(f, "N_HEADS: %d\n", c.hidden / c.head_dim);
+    fprintf(f, "Weight Sharing: Yes\n");
+    fprintf(f, "Biases: Embedding(Yes) Output(No)\n");
+    fprintf(f, "Model Parameters: %ld (%.2f MB)\n", params, params / (1024.0 * 1024.0));
+    fprintf(f, "Adam State Size: %ld (%.2f MB)\n", state, state / (1024.0 * 1024.0));
+    fprintf(f, "Population: %d\n", c.population);
+    fprintf(f, "Softmax Scale: 2^%d\n", c.softmax_scale_bit);
+    return fclose(f) == 0 ? EGG_OK : fail(ctx, EGG_E_INVALID, "cannot write model.info");
 }
 // current_seed = hash_rng(current_seed, current_step) (d-eggs/src/worker.cu:542)
 extern "C" uint32_t egg_next_seed(uint32_t seed, uint64_t step) {

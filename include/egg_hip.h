@@ -231,6 +231,9 @@ int  egg_step_losses(egg_ctx *ctx, int32_t *host_loss, int32_t *host_fit);
 
 /* get_learning_rate (mgpu.cu:217-227) and the d-eggs seed chain seed' = hash_rng(seed, step) (de/src/worker.cu:542) */
 float    egg_learning_rate(long step);
+float    egg_learning_rate_deggs(long step);      /* d-eggs' schedule, de/include/utils/training.h:5-9 */
+/* save_model_info (egg_disk_utils.h:15-44, de/include/utils/io.h:24-53): writes <dir>/model.info (dir NULL = "models") */
+int      egg_model_info_save(egg_ctx *ctx, const char *dir);
 uint32_t egg_next_seed(uint32_t seed, uint64_t step);
 
 /* generate_sequence_kernel + its call site (mgpu.cu:1154-1283, :1701-1708): d_buffer holds seed_len prompt bytes

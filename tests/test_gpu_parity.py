@@ -801,6 +801,13 @@ def test_checkpoint_files_round_trip(pkg, orc, dev, tmp_path):
     ctx2.checkpoint_load(os.path.join(d, "egg_transformer_last.model.bin"), os.path.join(d, "egg_transformer_last.adam.bin"))
     assert np.array_equal(ctx2.model_download(), model)
     assert ctx2.opt_state_download().tobytes() == state.tobytes()
+    # save_model_info (egg_disk_utils.h:15-44): the configuration and sizes as text
+    ctx.model_info_save(d)
+    info = open(os.path.join(d, "model.info")).read().splitlines()
+    assert info[:7] == ["Model Configuration:", "HIDDEN_DIM: 64", "HEAD_DIM: 32", "N_LAYERS: 1", "SEQ_LEN: 32", "VOCAB_SIZE: 256", "N_HEADS: 2"]
+    assert f"Model Parameters: {model.size} ({model.size / 1048576:.2f} MB)" in info
+    assert f"Adam State Size: {12 * model.size} ({12 * model.size / 1048576:.2f} MB)" in info and "Population: 40" in info
+    assert "Softmax Scale: 2^18" in info
     ctx3 = pkg.Context(pkg.default_config(hidden=128, head_dim=32, n_layers=1, seq_len=32, population=40))
     with pytest.raises(pkg.EggError):
         ctx3.checkpoint_load(os.path.join(d, "egg_transformer_last.model.bin"))

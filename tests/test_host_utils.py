@@ -179,3 +179,10 @@ def test_token_vocabulary_file_and_detokenize(pkg, tmp_path):
         pkg.Vocabulary(huge)
     with pytest.raises(pkg.EggError):
         pkg.Vocabulary(tmp_path / "missing.bin")
+
+
+def test_learning_rate_schedules(pkg):
+    """get_learning_rate of the single-node trainer (mgpu.cu:217-227) and of d-eggs (d-eggs/include/utils/training.h:5-9)"""
+    f32 = lambda x: float(np.float32(x))
+    assert [pkg.learning_rate(s) for s in (0, 299, 300, 599, 600, 999, 1000, 10 ** 6)] == [f32(v) for v in (0.3, 0.3, 0.15, 0.15, 0.075, 0.075, 0.05, 0.05)]
+    assert [pkg.learning_rate_deggs(s) for s in (0, 99, 100, 199, 200, 10 ** 6)] == [0.5, 0.5, 0.25, 0.25, 0.125, 0.125]
